@@ -1,0 +1,143 @@
+"""ctypes binding of the C ABI declared in ``include/deconver_ndc.h``.
+
+The product library is ``libdeconver_ndc.so`` (hipcc, gfx950), built in-tree by
+``deconver_amd.build``.  There is no CPU fallback: if the library is missing,
+``get_library()`` raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+from typing import Optional, Sequence
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libdeconver_ndc.so")
+
+NDC_F32, NDC_BF16 = 0, 1
+PATH_AUTO, PATH_DIRECT, PATH_FUSED = 0, 1, 2
+
+EXPORTS = (
+    "ndc_version",
+    "ndc_status_string",
+    "ndc_fused_supported",
+    "ndc_check_geometry",
+    "ndc_forward",
+    "ndc_backward_workspace_bytes",
+    "ndc_backward",
+    "ndc_gconv",
+)
+
+
+class Geom(ctypes.Structure):
+    """Mirror of ``struct ndc_geom``."""
+
+    _fields_ = [
+        ("batch", ctypes.c_int32),
+        ("groups", ctypes.c_int32),
+        ("m", ctypes.c_int32),
+        ("sc", ctypes.c_int32),
+        ("size", ctypes.c_int32 * 3),
+        ("kernel", ctypes.c_int32 * 3),
+        ("dtype", ctypes.c_int32),
+        ("relu_input", ctypes.c_int32),
+        ("path", ctypes.c_int32),
+        ("eps", ctypes.c_float),
+    ]
+
+
+def make_geom(batch: int, groups: int, m: int, sc: int, spatial: Sequence[int],
+              kernel: Sequence[int], dtype: int, relu_input: bool, eps: float,
+              path: int = PATH_AUTO) -> Geom:
+    rank = len(spatial)
+    if not 1 <= rank <= 3 or len(kernel) != rank:
+        # same error class the reference raises for an unsupported rank
+        # (deconver/deconvolution/kernels.py:715-716)
+        raise ValueError(f"unsupported spatial rank {rank} / kernel rank {len(kernel)}")
+    size = (ctypes.c_int32 * 3)(*([1] * (3 - rank) + [int(v) for v in spatial]))
+    kern = (ctypes.c_int32 * 3)(*([1] * (3 - rank) + [int(v) for v in kernel]))
+    return Geom(int(batch), int(groups), int(m), int(sc), size, kern, int(dtype),
+                1 if relu_input else 0, int(path), float(eps))
+
+
+class NdcError(RuntimeError):
+    pass
+
+
+class NdcLibrary:
+    """A loaded build of the C ABI (the HIP product, or the host checker in CPU tests)."""
+
+    def __init__(self, path: str):
+        self.path = path
+        self._dll = ctypes.CDLL(path)
+        d = self._dll
+        vp, fp = ctypes.c_void_p, ctypes.c_void_p
+        gp = ctypes.POINTER(Geom)
+        d.ndc_version.restype = ctypes.c_int
+        d.ndc_status_string.restype = ctypes.c_char_p
+        d.ndc_status_string.argtypes = [ctypes.c_int]
+        d.ndc_fused_supported.argtypes = [gp]
+        d.ndc_check_geometry.argtypes = [gp]
+        d.ndc_forward.argtypes = [gp, vp, vp, fp, fp, vp, vp, vp]
+        d.ndc_backward_workspace_bytes.restype = ctypes.c_size_t
+        d.ndc_backward_workspace_bytes.argtypes = [gp] + [ctypes.c_int] * 4
+        d.ndc_backward.argtypes = [gp, vp, vp, vp, fp, fp, vp, vp, vp, fp, fp, vp,
+                                   ctypes.c_size_t, vp]
+        d.ndc_gconv.argtypes = [gp, vp, fp, fp, ctypes.c_int, vp, vp]
+
+    def _check(self, status: int, what: str) -> None:
+        if status != 0:
+            msg = self._dll.ndc_status_string(status).decode()
+            raise NdcError(f"{what} failed: {msg} (status {status})")
+
+    def version(self) -> int:
+        return self._dll.ndc_version()
+
+    def fused_supported(self, g: Geom) -> bool:
+        return bool(self._dll.ndc_fused_supported(ctypes.byref(g)))
+
+    def check_geometry(self, g: Geom) -> int:
+        return self._dll.ndc_check_geometry(ctypes.byref(g))
+
+    def forward(self, g: Geom, x: int, z: int, h: int, bias: Optional[int], out: int,
+                t1: Optional[int], stream: Optional[int]) -> None:
+        self._check(self._dll.ndc_forward(ctypes.byref(g), x, z, h, bias, out, t1, stream),
+                    "ndc_forward")
+
+    def backward_workspace_bytes(self, g: Geom, need_gx, need_gz, need_gh, need_gb) -> int:
+        return self._dll.ndc_backward_workspace_bytes(
+            ctypes.byref(g), int(need_gx), int(need_gz), int(need_gh), int(need_gb))
+
+    def backward(self, g: Geom, x, z, t1, h, bias, gout, gx, gz, gh, gb, ws, ws_bytes,
+                 stream) -> None:
+        self._check(
+            self._dll.ndc_backward(ctypes.byref(g), x, z, t1, h, bias, gout, gx, gz, gh, gb, ws,
+                                   ws_bytes, stream),
+            "ndc_backward")
+
+    def gconv(self, g: Geom, inp, h, bias, adjoint: bool, out, stream) -> None:
+        self._check(self._dll.ndc_gconv(ctypes.byref(g), inp, h, bias, int(adjoint), out, stream),
+                    "ndc_gconv")
+
+
+_lock = threading.Lock()
+_library: Optional[NdcLibrary] = None
+
+
+def library_available() -> bool:
+    return os.path.exists(LIB_PATH)
+
+
+def get_library() -> NdcLibrary:
+    """The HIP library; raises if it has not been built (there is no other backend)."""
+    global _library
+    if _library is None:
+        with _lock:
+            if _library is None:
+                if not os.path.exists(LIB_PATH):
+                    raise NdcError(
+                        f"{LIB_PATH} is missing: build it with `python -m deconver_amd.build` "
+                        "(hipcc, gfx950). The NDC update has no CPU or PyTorch fallback.")
+                _library = NdcLibrary(LIB_PATH)
+    return _library

@@ -1,0 +1,285 @@
+// Host-side logic of the C ABI (include/deconver_ndc.h): argument checks, path choice,
+// workspace carving, launch sequence.  Included by exactly two translation units, each of
+// which first defines a `Backend` with the launch primitives:
+//   ndc_capi.hip       -> HIP launches on gfx950 (the product)
+//   ndc_hostcheck.cpp  -> sequential host execution of the same kernel bodies (CPU tests)
+#pragma once
+
+#include "../../include/deconver_ndc.h"
+#include "ndc_common.h"
+#include "ndc_direct.h"
+#include "ndc_fused.h"
+
+namespace ndc {
+
+static inline int make_kgeom(const ndc_geom *g, KGeom &q)
+{
+    if (!g) return NDC_ERR_NULL;
+    if (g->dtype != NDC_F32 && g->dtype != NDC_BF16) return NDC_ERR_DTYPE;
+    if (g->batch < 1 || g->groups < 1 || g->m < 1 || g->sc < 1) return NDC_ERR_GEOMETRY;
+    long long taps = 1, sp = 1;
+    for (int a = 0; a < 3; ++a) {
+        if (g->size[a] < 1 || g->kernel[a] < 1 || (g->kernel[a] & 1) == 0) return NDC_ERR_GEOMETRY;
+        taps *= g->kernel[a];
+        sp *= g->size[a];
+    }
+    if (taps > 4096 || g->m > 1024 || g->sc > 1024) return NDC_ERR_GEOMETRY;
+    // element counts must stay well inside int64 and block counts inside int32
+    const long long cmax = (long long)g->groups * (g->m > g->sc ? g->m : g->sc);
+    if (sp > (1LL << 40) || (long double)sp * cmax * g->batch > 9.0e15L) return NDC_ERR_GEOMETRY;
+    if (g->path < NDC_PATH_AUTO || g->path > NDC_PATH_FUSED) return NDC_ERR_GEOMETRY;
+    q.B = g->batch;
+    q.G = g->groups;
+    q.m = g->m;
+    q.sc = g->sc;
+    q.D = g->size[0];
+    q.H = g->size[1];
+    q.W = g->size[2];
+    q.kD = g->kernel[0];
+    q.kH = g->kernel[1];
+    q.kW = g->kernel[2];
+    q.pD = q.kD / 2;
+    q.pH = q.kH / 2;
+    q.pW = q.kW / 2;
+    q.KT = (int)taps;
+    q.relu = g->relu_input ? 1 : 0;
+    q.eps = g->eps;
+    q.SP = sp;
+    return NDC_OK;
+}
+
+static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+// Decide which implementation serves a call.  Returns NDC_PATH_DIRECT / NDC_PATH_FUSED, or
+// a negative status when the caller forced a path that does not cover the geometry.
+static inline int choose_path(const ndc_geom *g, const KGeom &q)
+{
+    const bool fused_ok = fused::supported(q);
+    if (g->path == NDC_PATH_DIRECT) return NDC_PATH_DIRECT;
+    if (g->path == NDC_PATH_FUSED) return fused_ok ? (int)NDC_PATH_FUSED : (int)NDC_ERR_GEOMETRY;
+    return fused_ok ? (int)NDC_PATH_FUSED : (int)NDC_PATH_DIRECT;
+}
+
+// ------------------------------------------------------------------ direct path
+
+template <typename T>
+static int direct_forward(const KGeom &q, const T *x, const T *z, const float *h,
+                          const float *bias, T *out, T *t1, void *stream)
+{
+    // t1 = K(relu(z + b)) lands in the caller's t1; without one there is nowhere to put
+    // it, so the direct path asks for it (the fused path does not need it)
+    if (!t1) return NDC_ERR_NULL;
+    const long long n_x = (long long)q.B * q.C() * q.SP, n_s = (long long)q.B * q.CS() * q.SP;
+    int st = Backend::elementwise(n_x, stream, [=] NDC_LAMBDA(long long idx) {
+        direct::gconv<T, T, false>(idx, q, z, h, bias, true, t1);
+    });
+    if (st) return st;
+    return Backend::elementwise(n_s, stream, [=] NDC_LAMBDA(long long idx) {
+        direct::fwd<T>(idx, q, x, t1, z, h, bias, out);
+    });
+}
+
+static inline size_t direct_backward_ws(const KGeom &q)
+{
+    const size_t n_x = (size_t)q.B * q.C() * q.SP, n_s = (size_t)q.B * q.CS() * q.SP;
+    return align_up(n_s * 4, 256) * 2 + align_up(n_x * 4, 256);
+}
+
+template <typename T>
+static int direct_backward(const KGeom &q, const T *x, const T *z, const T *t1, const float *h,
+                           const float *bias, const T *gout, T *gx, T *gz, float *gh, float *gb,
+                           void *ws, void *stream)
+{
+    const long long n_x = (long long)q.B * q.C() * q.SP, n_s = (long long)q.B * q.CS() * q.SP;
+    char *w = (char *)ws;
+    float *gn = (float *)w;
+    w += align_up((size_t)n_s * 4, 256);
+    float *gd = (float *)w;
+    w += align_up((size_t)n_s * 4, 256);
+    float *gt1 = (float *)w;
+    KGeom qn = q;  // gn/gd/gt1 are plain tensors: no bias, no rectification on load
+    qn.relu = 0;
+    int st = Backend::elementwise(n_s, stream, [=] NDC_LAMBDA(long long idx) {
+        direct::bwd_gn_gd<T>(idx, q, x, t1, z, gout, h, bias, gn, gd);
+    });
+    if (st) return st;
+    st = Backend::elementwise(n_x, stream, [=] NDC_LAMBDA(long long idx) {
+        direct::gconv<float, float, false>(idx, qn, gd, h, nullptr, false, gt1);
+    });
+    if (st) return st;
+    if (gx) {
+        st = Backend::elementwise(n_x, stream, [=] NDC_LAMBDA(long long idx) {
+            direct::gconv<float, T, false>(idx, qn, gn, h, nullptr, false, gx);
+        });
+        if (st) return st;
+    }
+    if (gh) {
+        st = Backend::block_reduce(q.G * q.m * q.sc * q.KT, stream, gh,
+                                   [=] NDC_LAMBDA(int o, int tid, int nt) {
+                                       return direct::gh_partial<T>(o, tid, nt, q, x, t1, z, bias,
+                                                                    gn, gd, gt1);
+                                   });
+        if (st) return st;
+    }
+    if (gz || gb) {
+        // gz is needed to form gb; when the caller does not want gz it goes to the gn
+        // scratch (gn is dead by now), typed as T
+        T *gz_out = gz ? gz : (T *)gn;
+        st = Backend::elementwise(n_s, stream, [=] NDC_LAMBDA(long long idx) {
+            direct::bwd_gz<T>(idx, q, x, t1, z, gout, gt1, h, bias, gz_out);
+        });
+        if (st) return st;
+        if (gb) {
+            st = Backend::block_reduce(q.CS(), stream, gb, [=] NDC_LAMBDA(int o, int tid, int nt) {
+                return direct::gb_partial<T>(o, tid, nt, q, gz_out);
+            });
+            if (st) return st;
+        }
+    }
+    return NDC_OK;
+}
+
+template <typename TI, typename TO>
+static int direct_gconv(const KGeom &q, const TI *in, const float *h, const float *bias,
+                        int adjoint, TO *out, void *stream)
+{
+    const bool rectify = (bias != nullptr) || q.relu;
+    if (adjoint) {
+        const long long n = (long long)q.B * q.CS() * q.SP;
+        return Backend::elementwise(n, stream, [=] NDC_LAMBDA(long long idx) {
+            direct::gconv<TI, TO, true>(idx, q, in, h, bias, rectify, out);
+        });
+    }
+    const long long n = (long long)q.B * q.C() * q.SP;
+    return Backend::elementwise(n, stream, [=] NDC_LAMBDA(long long idx) {
+        direct::gconv<TI, TO, false>(idx, q, in, h, bias, rectify, out);
+    });
+}
+
+}  // namespace ndc
+
+// ============================================================================ C ABI
+
+extern "C" {
+
+int ndc_version(void) { return 100; }
+
+const char *ndc_status_string(int status)
+{
+    switch (status) {
+    case NDC_OK: return "ok";
+    case NDC_ERR_NULL: return "a required pointer is null";
+    case NDC_ERR_GEOMETRY: return "geometry not covered by the requested path";
+    case NDC_ERR_DTYPE: return "unknown dtype tag";
+    case NDC_ERR_WORKSPACE: return "workspace too small or misaligned";
+    case NDC_ERR_LAUNCH: return "kernel launch failed";
+    default: return "unknown status";
+    }
+}
+
+int ndc_fused_supported(const ndc_geom *g)
+{
+    ndc::KGeom q;
+    if (ndc::make_kgeom(g, q) != NDC_OK) return 0;
+    return ndc::fused::supported(q) ? 1 : 0;
+}
+
+int ndc_check_geometry(const ndc_geom *g)
+{
+    ndc::KGeom q;
+    int st = ndc::make_kgeom(g, q);
+    if (st) return st;
+    st = ndc::choose_path(g, q);
+    return st < 0 ? st : NDC_OK;
+}
+
+int ndc_forward(const ndc_geom *g, const void *x, const void *z, const float *h,
+                const float *bias, void *out, void *t1, void *stream)
+{
+    using namespace ndc;
+    KGeom q;
+    int st = make_kgeom(g, q);
+    if (st) return st;
+    if (!x || !z || !h || !out) return NDC_ERR_NULL;
+    const int path = choose_path(g, q);
+    if (path < 0) return path;
+    if (path == NDC_PATH_FUSED) {
+        return g->dtype == NDC_F32
+                   ? fused::forward<Backend, float>(q, (const float *)x, (const float *)z, h, bias,
+                                                    (float *)out, (float *)t1, stream)
+                   : fused::forward<Backend, bf16_t>(q, (const bf16_t *)x, (const bf16_t *)z, h,
+                                                     bias, (bf16_t *)out, (bf16_t *)t1, stream);
+    }
+    return g->dtype == NDC_F32
+               ? direct_forward<float>(q, (const float *)x, (const float *)z, h, bias,
+                                       (float *)out, (float *)t1, stream)
+               : direct_forward<bf16_t>(q, (const bf16_t *)x, (const bf16_t *)z, h, bias,
+                                        (bf16_t *)out, (bf16_t *)t1, stream);
+}
+
+size_t ndc_backward_workspace_bytes(const ndc_geom *g, int need_gx, int need_gz, int need_gh,
+                                    int need_gb)
+{
+    using namespace ndc;
+    KGeom q;
+    if (make_kgeom(g, q) != NDC_OK) return 0;
+    const int path = choose_path(g, q);
+    if (path < 0) return 0;
+    (void)need_gx;
+    (void)need_gz;
+    if (path == NDC_PATH_FUSED) return fused::backward_ws(q, g->dtype, need_gh, need_gb);
+    return direct_backward_ws(q);
+}
+
+int ndc_backward(const ndc_geom *g, const void *x, const void *z, const void *t1, const float *h,
+                 const float *bias, const void *gout, void *gx, void *gz, float *gh, float *gb,
+                 void *workspace, size_t workspace_bytes, void *stream)
+{
+    using namespace ndc;
+    KGeom q;
+    int st = make_kgeom(g, q);
+    if (st) return st;
+    if (!x || !z || !t1 || !h || !gout) return NDC_ERR_NULL;
+    if (!gx && !gz && !gh && !gb) return NDC_OK;
+    const int path = choose_path(g, q);
+    if (path < 0) return path;
+    const size_t need = ndc_backward_workspace_bytes(g, gx != nullptr, gz != nullptr,
+                                                     gh != nullptr, gb != nullptr);
+    if (need && (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255u)))
+        return NDC_ERR_WORKSPACE;
+    if (path == NDC_PATH_FUSED) {
+        return g->dtype == NDC_F32
+                   ? fused::backward<Backend, float>(q, (const float *)x, (const float *)z,
+                                                     (const float *)t1, h, bias,
+                                                     (const float *)gout, (float *)gx,
+                                                     (float *)gz, gh, gb, workspace, stream)
+                   : fused::backward<Backend, bf16_t>(q, (const bf16_t *)x, (const bf16_t *)z,
+                                                      (const bf16_t *)t1, h, bias,
+                                                      (const bf16_t *)gout, (bf16_t *)gx,
+                                                      (bf16_t *)gz, gh, gb, workspace, stream);
+    }
+    return g->dtype == NDC_F32
+               ? direct_backward<float>(q, (const float *)x, (const float *)z, (const float *)t1,
+                                        h, bias, (const float *)gout, (float *)gx, (float *)gz,
+                                        gh, gb, workspace, stream)
+               : direct_backward<bf16_t>(q, (const bf16_t *)x, (const bf16_t *)z,
+                                         (const bf16_t *)t1, h, bias, (const bf16_t *)gout,
+                                         (bf16_t *)gx, (bf16_t *)gz, gh, gb, workspace, stream);
+}
+
+int ndc_gconv(const ndc_geom *g, const void *in, const float *h, const float *bias, int adjoint,
+              void *out, void *stream)
+{
+    using namespace ndc;
+    KGeom q;
+    int st = make_kgeom(g, q);
+    if (st) return st;
+    if (!in || !h || !out) return NDC_ERR_NULL;
+    return g->dtype == NDC_F32
+               ? direct_gconv<float, float>(q, (const float *)in, h, bias, adjoint, (float *)out,
+                                            stream)
+               : direct_gconv<bf16_t, bf16_t>(q, (const bf16_t *)in, h, bias, adjoint,
+                                              (bf16_t *)out, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,103 @@
+"""Autograd node of one NDC source update, running on the HIP kernels.
+
+Mirrors ``deconver/deconvolution/functional.py:97-207`` of the reference
+(``DeconvUpdate`` / ``deconv_update``): same arguments, same saved tensors
+``(x, z, t1, h, bias)``, same returned gradients ``(gx, gz, gh, gb, None x5)``, same
+refusal of double backward.  The arithmetic is in ``libdeconver_ndc.so``; there is no
+PyTorch implementation behind this node.
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+from torch import Tensor
+
+from . import _lib, ops
+
+__all__ = ["deconv_update", "hip_kernels_apply", "DeconvUpdate"]
+
+
+def hip_kernels_apply(x: Tensor, m: int, sc: int, kernel_size, dtype=None) -> bool:
+    """Whether the HIP update can run for this input and filter geometry.
+
+    Counterpart of ``fused_kernels_apply`` (``functional.py:34-47``): device tensors only,
+    no active functorch transform, float32 or bfloat16 storage, rank 1-3, odd kernel.
+    """
+    try:
+        functorch = torch._C._are_functorch_transforms_active()
+    except AttributeError:  # pragma: no cover
+        functorch = False
+    dtype = x.dtype if dtype is None else dtype
+    if functorch or not x.is_cuda or dtype not in (torch.float32, torch.bfloat16):
+        return False
+    if not 1 <= len(kernel_size) <= 3 or x.dim() - 2 != len(kernel_size):
+        return False
+    if any(k % 2 == 0 for k in kernel_size):
+        return False
+    lib = _lib.get_library()  # raises when the library is missing: no silent fallback
+    g = _lib.make_geom(x.shape[0], x.shape[1] // m, m, sc, x.shape[2:], kernel_size,
+                       ops.dtype_tag(dtype), True, 0.0)
+    return lib.check_geometry(g) == 0
+
+
+class DeconvUpdate(torch.autograd.Function):
+    """``out = relu(z + b) * (A(x) + eps) / (A(K(relu(z + b))) + eps)``."""
+
+    @staticmethod
+    def forward(ctx, x, z, h, bias, groups, m, sc, eps, relu_input):
+        if not x.is_cuda:
+            raise RuntimeError("deconv_update runs on the GPU only (HIP kernels); "
+                               "CPU tensors take the layer's general PyTorch path")
+        lib = _lib.get_library()
+        x = x.contiguous()
+        z = z.contiguous()
+        hc = h.contiguous()
+        need_t1 = any(ctx.needs_input_grad[:4])
+        with torch.cuda.device(x.device):
+            out, t1 = ops.update_forward(lib, x, z, hc, bias, groups=groups, m=m, sc=sc,
+                                         eps=eps, relu_input=relu_input, need_t1=need_t1)
+        ctx.cfg = (groups, m, sc, eps, relu_input)
+        ctx.save_for_backward(x, z, t1, hc, bias)
+        return out
+
+    @staticmethod
+    def backward(ctx, gout):
+        # The gradients come from kernels autograd cannot see through, so a second
+        # differentiation would silently drop terms: refuse it, as the reference does.
+        if torch.is_grad_enabled():
+            raise RuntimeError(
+                "double backward through the fused Deconv update is not supported; "
+                "construct the layer with a convolution keyword argument (e.g. stride=1) "
+                "to force the general path, which is plain PyTorch and doubly differentiable")
+        x, z, t1, h, bias = ctx.saved_tensors
+        groups, m, sc, eps, relu_input = ctx.cfg
+        need_x, need_z, need_h, need_b = ctx.needs_input_grad[:4]
+        if t1 is None:
+            raise RuntimeError("backward called on an update that was run without gradients")
+        gout = gout.contiguous()
+        if gout.dtype != z.dtype:
+            gout = gout.to(z.dtype)
+        lib = _lib.get_library()
+        with torch.cuda.device(x.device):
+            gx, gz, gh, gb = ops.update_backward(
+                lib, x, z, t1, h, bias, gout, groups=groups, m=m, sc=sc, eps=eps,
+                relu_input=relu_input, need_x=need_x, need_z=need_z, need_h=need_h,
+                need_b=need_b and bias is not None)
+        return gx, gz, gh, gb, None, None, None, None, None
+
+
+def deconv_update(x: Tensor, z: Tensor, h: Tensor, bias: Optional[Tensor], *, groups: int,
+                  m: int, sc: int, eps: float, relu_input: bool) -> Tensor:
+    """One multiplicative source update.
+
+    Args:
+        x: input, ``(B, C, *S)``.
+        z: projection output ``(B, groups*sc, *S)``, pre-bias and pre-ReLU on the first
+            iteration (the kernels apply both on load); the rectified source afterwards.
+        h: rectified filter ``(C, sc, *k)``, float32.
+        bias: the projection's bias (float32) or ``None``.
+        eps: stabiliser added to numerator and denominator.
+    """
+    return DeconvUpdate.apply(x, z, h, bias, groups, m, sc, eps, relu_input)

@@ -1,0 +1,119 @@
+"""Tensor-level wrappers over the C ABI: shape/dtype checks, output allocation, pointers.
+
+These take the library explicitly.  The product passes ``_lib.get_library()`` (HIP) with
+CUDA tensors; the CPU test-suite passes the host checker with CPU tensors.  Nothing here
+computes anything in PyTorch.
+"""
+
+from __future__ import annotations
+
+from typing import Optional, Sequence, Tuple
+
+import torch
+from torch import Tensor
+
+from . import _lib
+
+_DTYPES = {torch.float32: _lib.NDC_F32, torch.bfloat16: _lib.NDC_BF16}
+
+
+def dtype_tag(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPES[dtype]
+    except KeyError:
+        raise TypeError(f"NDC kernels store activations as float32 or bfloat16, got {dtype}")
+
+
+def _stream_of(t: Tensor) -> Optional[int]:
+    if t.is_cuda:
+        return torch.cuda.current_stream(t.device).cuda_stream
+    return None
+
+
+def _ptr(t: Optional[Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _check_common(x: Tensor, z: Tensor, h: Tensor, bias: Optional[Tensor], groups: int, m: int,
+                  sc: int) -> Tuple[int, ...]:
+    if x.dim() < 3 or x.dim() > 5:
+        raise ValueError(f"expected a (B, C, *S) tensor with 1-3 spatial dims, got {tuple(x.shape)}")
+    if x.shape[1] != groups * m:
+        raise ValueError(f"x has {x.shape[1]} channels, expected groups*m = {groups * m}")
+    if tuple(z.shape) != (x.shape[0], groups * sc, *x.shape[2:]):
+        raise ValueError(f"z has shape {tuple(z.shape)}, expected "
+                         f"{(x.shape[0], groups * sc, *x.shape[2:])}")
+    if h.dim() != x.dim() or h.shape[0] * h.shape[1] != groups * m * sc:
+        raise ValueError(f"filter of shape {tuple(h.shape)} does not match groups={groups}, "
+                         f"m={m}, sc={sc}")
+    if x.dtype != z.dtype:
+        raise TypeError(f"x ({x.dtype}) and z ({z.dtype}) must share a dtype")
+    if h.dtype != torch.float32 or (bias is not None and bias.dtype != torch.float32):
+        raise TypeError("filter and bias must be float32")
+    for t in (x, z, h, bias):
+        if t is not None and (t.device != x.device or not t.is_contiguous()):
+            raise ValueError("all tensors must be contiguous and on one device")
+    if bias is not None and bias.numel() != groups * sc:
+        raise ValueError(f"bias has {bias.numel()} entries, expected {groups * sc}")
+    return tuple(h.shape[2:])
+
+
+def make_geom_for(x: Tensor, h: Tensor, groups: int, m: int, sc: int, eps: float,
+                  relu_input: bool, path: int = _lib.PATH_AUTO) -> _lib.Geom:
+    return _lib.make_geom(x.shape[0], groups, m, sc, x.shape[2:], h.shape[2:],
+                          dtype_tag(x.dtype), relu_input, eps, path)
+
+
+def update_forward(lib: _lib.NdcLibrary, x: Tensor, z: Tensor, h: Tensor,
+                   bias: Optional[Tensor], *, groups: int, m: int, sc: int, eps: float,
+                   relu_input: bool, need_t1: bool = True,
+                   path: int = _lib.PATH_AUTO) -> Tuple[Tensor, Optional[Tensor]]:
+    """``out = s*(A(x)+eps)/(A(K(s))+eps)`` with ``s = relu?(z+bias)``; returns ``(out, t1)``."""
+    _check_common(x, z, h, bias, groups, m, sc)
+    g = make_geom_for(x, h, groups, m, sc, eps, relu_input, path)
+    out = torch.empty_like(z)
+    want_t1 = need_t1 or not lib.fused_supported(g) or path == _lib.PATH_DIRECT
+    t1 = torch.empty_like(x) if want_t1 else None
+    lib.forward(g, _ptr(x), _ptr(z), _ptr(h), _ptr(bias), _ptr(out), _ptr(t1), _stream_of(x))
+    return out, t1
+
+
+def update_backward(lib: _lib.NdcLibrary, x: Tensor, z: Tensor, t1: Tensor, h: Tensor,
+                    bias: Optional[Tensor], gout: Tensor, *, groups: int, m: int, sc: int,
+                    eps: float, relu_input: bool, need_x: bool = True, need_z: bool = True,
+                    need_h: bool = True, need_b: bool = True,
+                    path: int = _lib.PATH_AUTO):
+    """Gradients ``(gx, gz, gh, gb)`` of the update; entries not asked for are ``None``."""
+    _check_common(x, z, h, bias, groups, m, sc)
+    if gout.shape != z.shape or gout.dtype != z.dtype or not gout.is_contiguous():
+        raise ValueError("gout must be contiguous with the shape and dtype of z")
+    if t1.shape != x.shape or t1.dtype != x.dtype or not t1.is_contiguous():
+        raise ValueError("t1 must be contiguous with the shape and dtype of x")
+    need_b = need_b and bias is not None
+    g = make_geom_for(x, h, groups, m, sc, eps, relu_input, path)
+    gx = torch.empty_like(x) if need_x else None
+    gz = torch.empty_like(z) if need_z else None
+    gh = torch.empty_like(h) if need_h else None
+    gb = torch.empty(groups * sc, dtype=torch.float32, device=x.device) if need_b else None
+    nbytes = lib.backward_workspace_bytes(g, need_x, need_z, need_h, need_b)
+    ws = torch.empty(max(nbytes, 1) + 256, dtype=torch.uint8, device=x.device)
+    ws_ptr = (ws.data_ptr() + 255) // 256 * 256
+    lib.backward(g, _ptr(x), _ptr(z), _ptr(t1), _ptr(h), _ptr(bias), _ptr(gout), _ptr(gx),
+                 _ptr(gz), _ptr(gh), _ptr(gb), ws_ptr, nbytes, _stream_of(x))
+    return gx, gz, gh, gb
+
+
+def gconv(lib: _lib.NdcLibrary, inp: Tensor, h: Tensor, *, groups: int, m: int, sc: int,
+          adjoint: bool, bias: Optional[Tensor] = None, relu_input: bool = False) -> Tensor:
+    """``K(inp)`` (adjoint=False, inp has groups*sc channels) or ``A(inp)`` (groups*m channels)."""
+    cin = groups * (m if adjoint else sc)
+    cout = groups * (sc if adjoint else m)
+    if inp.shape[1] != cin:
+        raise ValueError(f"input has {inp.shape[1]} channels, expected {cin}")
+    if not inp.is_contiguous() or not h.is_contiguous() or h.dtype != torch.float32:
+        raise ValueError("input and filter must be contiguous; filter float32")
+    g = _lib.make_geom(inp.shape[0], groups, m, sc, inp.shape[2:], h.shape[2:],
+                       dtype_tag(inp.dtype), relu_input, 0.0, _lib.PATH_DIRECT)
+    out = torch.empty((inp.shape[0], cout, *inp.shape[2:]), dtype=inp.dtype, device=inp.device)
+    lib.gconv(g, _ptr(inp), _ptr(h), _ptr(bias), adjoint, _ptr(out), _stream_of(inp))
+    return out

@@ -1,0 +1,123 @@
+/*
+ * deconver_ndc.h -- C ABI of the MI355X (gfx950) implementation of Deconver's
+ * nonnegative-deconvolution (NDC) source update.
+ *
+ * One call = one multiplicative update of the source, or its gradients:
+ *
+ *     s   = relu_input ? max(z + bias, 0) : z (+ bias)
+ *     t1  = K(s)                                  K(u)[o,p] = sum_{i,tau} u[i,p+tau-pad] h[o,i,tau]
+ *     out = s * (A(x) + eps) / (A(t1) + eps)      A(v)[i,p] = sum_{o,tau} v[o,p+pad-tau] h[o,i,tau]
+ *
+ * Conventions shared by every entry point
+ *   - plain pointers to DEVICE memory, sizes in the geometry struct, a hipStream_t passed
+ *     as void*; no framework types.  The caller owns every buffer (inputs, outputs,
+ *     workspace); the library never allocates, frees or retains pointers.
+ *   - launches are asynchronous on `stream`; nothing synchronises the host.
+ *   - return value: 0 on success, a negative ndc_status otherwise; nothing throws.
+ *   - layouts: x, t1, gx are (B, G*m, D, H, W); z, out, gout, gz are (B, G*sc, D, H, W),
+ *     contiguous, channel g*sc+i = group g, source i; h, gh are (G, m, sc, kD, kH, kW)
+ *     float32; bias, gb are (G*sc) float32.  Rank-1/2 problems use leading extents of 1
+ *     (size = {1,1,W} / {1,H,W}, kernel likewise).  Stride 1, zero padding k/2, odd k.
+ *   - dtype tags the storage of the activation tensors only; arithmetic and the
+ *     filter/bias and their gradients are float32.
+ */
+#ifndef DECONVER_NDC_H
+#define DECONVER_NDC_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum ndc_dtype { NDC_F32 = 0, NDC_BF16 = 1 };
+
+enum ndc_status {
+    NDC_OK = 0,
+    NDC_ERR_NULL = -1,        /* a required pointer is null */
+    NDC_ERR_GEOMETRY = -2,    /* extents/kernel/groups outside what the kernels cover */
+    NDC_ERR_DTYPE = -3,       /* unknown dtype tag */
+    NDC_ERR_WORKSPACE = -4,   /* workspace too small or misaligned */
+    NDC_ERR_LAUNCH = -5       /* hipGetLastError() reported a failure after a launch */
+};
+
+/* Which implementation a call may use.  AUTO picks the fused LDS-tiled kernels when the
+ * geometry is one they cover and the direct kernels otherwise. */
+enum ndc_path { NDC_PATH_AUTO = 0, NDC_PATH_DIRECT = 1, NDC_PATH_FUSED = 2 };
+
+typedef struct ndc_geom {
+    int32_t batch;       /* B */
+    int32_t groups;      /* G */
+    int32_t m;           /* filter channels per group, C = G*m */
+    int32_t sc;          /* source channels per group */
+    int32_t size[3];     /* D, H, W */
+    int32_t kernel[3];   /* kD, kH, kW (odd) */
+    int32_t dtype;       /* ndc_dtype of x, z, out, t1, gout, gx, gz */
+    int32_t relu_input;  /* 1: s = max(z + bias, 0); 0: s = z + bias (bias usually null) */
+    int32_t path;        /* ndc_path */
+    float eps;
+} ndc_geom;
+
+/* Library version (major*10000 + minor*100 + patch). */
+int ndc_version(void);
+
+/* Human-readable text for a status code (static storage). */
+const char *ndc_status_string(int status);
+
+/* 1 if the fused LDS-tiled kernels cover `g`, else 0.
+ * Counterpart of kernels_supported()/fused_kernels_apply()
+ * (deconver/deconvolution/kernels.py:143-163, functional.py:34-47). */
+int ndc_fused_supported(const ndc_geom *g);
+
+/* 0 if some path covers `g` (then every entry point below accepts it), else a status. */
+int ndc_check_geometry(const ndc_geom *g);
+
+/*
+ * Forward update.  Replaces DeconvUpdate.forward
+ * (deconver/deconvolution/functional.py:105-116), i.e. the pair
+ * kernels.gconv(z, K, relu, bias) + kernels.deconv_fwd(...)
+ * (deconver/deconvolution/kernels.py:728-788).
+ *   x, z, h       inputs;  bias may be null
+ *   out           output, same shape/dtype as z
+ *   t1            optional output K(s), same shape/dtype as x: pass it when a backward
+ *                 call will follow (it is what the reference saves for backward), null
+ *                 for inference
+ */
+int ndc_forward(const ndc_geom *g, const void *x, const void *z, const float *h,
+                const float *bias, void *out, void *t1, void *stream);
+
+/* Bytes of scratch `ndc_backward` needs for `g` with the requested outputs (each flag
+ * nonzero when the matching output pointer will be non-null). */
+size_t ndc_backward_workspace_bytes(const ndc_geom *g, int need_gx, int need_gz, int need_gh,
+                                    int need_gb);
+
+/*
+ * Backward of the update.  Replaces DeconvUpdate.backward
+ * (deconver/deconvolution/functional.py:118-182), i.e. kernels.deconv_bwd, gconv x2,
+ * wgrad x3, deconv_gz and the bias reduction (kernels.py:791-894).
+ *   x, z, t1, h, bias   what the forward call saw / produced (bias may be null)
+ *   gout                upstream gradient, shape/dtype of out
+ *   gx, gz, gh, gb      optional outputs (null = not needed); gh and gb are OVERWRITTEN,
+ *                       not accumulated into.  gx is only the NDC term K(gn); the
+ *                       projection's own input gradient is the caller's business.
+ *   workspace           >= ndc_backward_workspace_bytes(...) bytes, 256-byte aligned
+ */
+int ndc_backward(const ndc_geom *g, const void *x, const void *z, const void *t1,
+                 const float *h, const float *bias, const void *gout, void *gx, void *gz,
+                 float *gh, float *gb, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Plain grouped convolution with the same tap conventions (adjoint = 0: K, 1: A), input
+ * and output in g->dtype; optional on-load bias + ReLU of the input as in the forward.
+ * Replaces kernels.gconv (deconver/deconvolution/kernels.py:728-759); used for
+ * `reconstruct` and by tests that probe K and A separately.
+ */
+int ndc_gconv(const ndc_geom *g, const void *in, const float *h, const float *bias, int adjoint,
+              void *out, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* DECONVER_NDC_H */
