@@ -42,7 +42,7 @@ def build_hip(extra_flags=()) -> str:
 def build_hostcheck(sanitize: bool = False) -> str:
     out = os.path.join(_HERE, "libndc_hostcheck.so")
     flags = ["-O1", "-g", "-fsanitize=address,undefined"] if sanitize else ["-O2"]
-    _run(["g++", "-std=c++17", "-fPIC", "-shared", "-Wall", *flags, "-o", out,
+    _run(["g++", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wno-unknown-pragmas", *flags, "-o", out,
           os.path.join(CSRC, "ndc_hostcheck.cpp")])
     return out
 

@@ -8,7 +8,7 @@
 #include "../../include/deconver_ndc.h"
 #include "ndc_common.h"
 #include "ndc_direct.h"
-#include "ndc_fused.h"
+#include "ndc_fused_api.h"
 
 namespace ndc {
 

@@ -2,6 +2,7 @@
 #include <hip/hip_runtime.h>
 
 #include "ndc_common.h"
+#include "ndc_exec.h"
 
 #define NDC_LAMBDA __host__ __device__
 
@@ -29,8 +30,38 @@ __global__ void __launch_bounds__(256) block_reduce_kernel(float *out, F partial
     if (tid == 0) out[blockIdx.x] = buf[0];
 }
 
+// One workgroup of an LDS-tiled kernel.  512 threads at most, so up to 256 VGPRs per lane.
+template <class Kernel>
+__global__ void __launch_bounds__(512) block_kernel_entry(typename Kernel::Params p)
+{
+    extern __shared__ float ndc_lds[];
+    DeviceExec<typename Kernel::State> ex;
+    ex.lds = ndc_lds;
+    ex.tid = threadIdx.x;
+    ex.nthreads = blockDim.x;
+    Kernel::run(ex, p, (int)blockIdx.x);
+}
+
 struct Backend {
     static constexpr bool is_device = true;
+
+    template <class Kernel>
+    static int block_kernel(const typename Kernel::Params &p, int nblocks, int nthreads,
+                            int lds_floats, void *stream)
+    {
+        if (nblocks <= 0) return 0;
+        const size_t bytes = (size_t)lds_floats * sizeof(float);
+        if (bytes > 64 * 1024) {
+            // more dynamic LDS than the default cap: raise it for this kernel (idempotent)
+            if (hipFuncSetAttribute((const void *)block_kernel_entry<Kernel>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)bytes) != hipSuccess)
+                return -5;
+        }
+        hipLaunchKernelGGL(block_kernel_entry<Kernel>, dim3((unsigned)nblocks),
+                           dim3((unsigned)nthreads), bytes, (hipStream_t)stream, p);
+        return check();
+    }
 
     static int check()
     {

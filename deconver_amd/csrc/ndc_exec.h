@@ -1,0 +1,154 @@
+// Execution contexts of the block-cooperative (LDS-tiled) kernels.
+//
+// A kernel is written once as `Kernel::run(exec, params, block_id)`: a uniform sequence of
+// per-thread phases (`exec.each(f)`) separated by barriers (`exec.sync()`), with all LDS
+// traffic going through `exec.ld / exec.st`.  Two contexts implement that interface:
+//
+//   DeviceExec  one HIP thread: `each` runs the phase for this thread, `sync` is
+//               __syncthreads(), ld/st are plain LDS accesses.
+//   HostExec    a whole block on the CPU: `each` runs the phase for every thread in turn,
+//               `sync` opens a new epoch, and ld/st are bounds-checked and race-checked:
+//               two different threads touching one LDS word within an epoch, at least one
+//               of them writing, is reported (it would need a barrier on the GPU), as is a
+//               read of a word nobody has written.
+#pragma once
+
+#include "ndc_common.h"
+
+#if !NDC_DEVICE_BUILD
+#include <cstdio>
+#include <vector>
+#endif
+
+namespace ndc {
+
+#if NDC_DEVICE_BUILD
+
+template <class State> struct DeviceExec {
+    State st;
+    float *lds;
+    int tid;
+    int nthreads;
+    template <class F> NDC_D void each(F f) { f(st, tid); }
+    NDC_D void sync() { __syncthreads(); }
+    NDC_D float ld(int i) const { return lds[i]; }
+    NDC_D void st_(int i, float v) { lds[i] = v; }
+
+    // Sum N per-thread values over the workgroup: butterfly inside each wavefront, one LDS
+    // row per wavefront, then thread i < N adds the rows in a fixed order and hands the sum
+    // to `put`.  Reuses LDS from offset 0 (callers are done with their tiles by then).
+    template <int N, class Get, class Put> NDC_D void block_reduce(Get get, Put put)
+    {
+        __syncthreads();
+        const int lane = tid & 63, wave = tid >> 6, nw = nthreads >> 6;
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            float v = get(st, i);
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+            if (lane == 0) lds[wave * N + i] = v;
+        }
+        __syncthreads();
+        for (int i = tid; i < N; i += nthreads) {
+            float s = 0.f;
+            for (int w = 0; w < nw; ++w) s += lds[w * N + i];
+            put(i, s);
+        }
+    }
+};
+
+#else
+
+struct HostFaults {
+    long long races = 0, oob = 0, uninit = 0;
+    char first[256] = {0};
+    void note(const char *what, int idx, int tid, int other)
+    {
+        if (!first[0]) snprintf(first, sizeof first, "%s at lds[%d] tid %d vs %d", what, idx, tid, other);
+    }
+};
+
+inline HostFaults &host_faults()
+{
+    static HostFaults f;
+    return f;
+}
+
+template <class State> struct HostExec {
+    std::vector<State> states;
+    std::vector<float> mem;
+    std::vector<int> w_epoch, w_tid, r_epoch, r_tid;
+    int nthreads;
+    int cur = 0;
+    int epoch = 0;
+
+    HostExec(int nthreads_, int lds_floats)
+        : states(nthreads_), mem(lds_floats, 0.f), w_epoch(lds_floats, -1), w_tid(lds_floats, -1),
+          r_epoch(lds_floats, -1), r_tid(lds_floats, -1), nthreads(nthreads_)
+    {
+    }
+
+    template <class F> void each(F f)
+    {
+        for (cur = 0; cur < nthreads; ++cur) f(states[cur], cur);
+    }
+    void sync() { ++epoch; }
+
+    float ld(int i)
+    {
+        HostFaults &hf = host_faults();
+        if (i < 0 || i >= (int)mem.size()) {
+            ++hf.oob;
+            hf.note("out-of-bounds read", i, cur, -1);
+            return 0.f;
+        }
+        if (w_epoch[i] < 0) {
+            ++hf.uninit;
+            hf.note("uninitialised read", i, cur, -1);
+        } else if (w_epoch[i] == epoch && w_tid[i] != cur) {
+            ++hf.races;
+            hf.note("read-after-write race", i, cur, w_tid[i]);
+        }
+        if (r_epoch[i] != epoch) {
+            r_epoch[i] = epoch;
+            r_tid[i] = cur;
+        } else if (r_tid[i] != cur) {
+            r_tid[i] = -2;
+        }
+        return mem[i];
+    }
+    void st_(int i, float v)
+    {
+        HostFaults &hf = host_faults();
+        if (i < 0 || i >= (int)mem.size()) {
+            ++hf.oob;
+            hf.note("out-of-bounds write", i, cur, -1);
+            return;
+        }
+        if (w_epoch[i] == epoch && w_tid[i] != cur) {
+            ++hf.races;
+            hf.note("write-after-write race", i, cur, w_tid[i]);
+        }
+        if (r_epoch[i] == epoch && r_tid[i] != cur) {
+            ++hf.races;
+            hf.note("write-after-read race", i, cur, r_tid[i]);
+        }
+        w_epoch[i] = epoch;
+        w_tid[i] = cur;
+        mem[i] = v;
+    }
+
+    template <int N, class Get, class Put> void block_reduce(Get get, Put put)
+    {
+        sync();
+        for (int i = 0; i < N; ++i) {
+            float s = 0.f;
+            for (int t = 0; t < nthreads; ++t) s += get(states[t], i);
+            put(i, s);
+        }
+    }
+};
+
+#endif
+
+}  // namespace ndc

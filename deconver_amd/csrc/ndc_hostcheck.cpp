@@ -5,6 +5,7 @@
 #include <vector>
 
 #include "ndc_common.h"
+#include "ndc_exec.h"
 
 #define NDC_LAMBDA
 
@@ -12,6 +13,17 @@ namespace ndc {
 
 struct Backend {
     static constexpr bool is_device = false;
+
+    template <class Kernel>
+    static int block_kernel(const typename Kernel::Params &p, int nblocks, int nthreads,
+                            int lds_floats, void *)
+    {
+        for (int blk = 0; blk < nblocks; ++blk) {
+            HostExec<typename Kernel::State> ex(nthreads, lds_floats);
+            Kernel::run(ex, p, blk);
+        }
+        return 0;
+    }
 
     template <class F> static int elementwise(long long n, void *, F f)
     {
@@ -35,3 +47,16 @@ struct Backend {
 }  // namespace ndc
 
 #include "ndc_api_impl.h"
+
+// LDS faults (races, out-of-bounds, uninitialised reads) seen by the host execution since
+// the last call; `first` describes the first one.  Test hook of the host build only.
+extern "C" long long ndc_host_faults(char *first, int n)
+{
+    ndc::HostFaults &f = ndc::host_faults();
+    const long long total = f.races + f.oob + f.uninit;
+    if (first && n > 0) {
+        snprintf(first, (size_t)n, "%s", f.first);
+    }
+    f = ndc::HostFaults();
+    return total;
+}

@@ -33,3 +33,15 @@ def make_case(C, G, sc, ks, sp, B=2, seed=0, dtype=torch.float32, bias_shift=0.0
     gout = torch.randn(B, G * sc, *sp, generator=gen)
     x, z, gout = (t.to(dtype) for t in (x, z, gout))
     return [t.to(device) for t in (x, z, h, bias, gout)]
+
+
+def host_faults(lib) -> tuple:
+    """(count, first message) of LDS races / out-of-bounds / uninitialised reads the host
+    execution has seen since the last query."""
+    import ctypes
+
+    buf = ctypes.create_string_buffer(256)
+    fn = lib._dll.ndc_host_faults
+    fn.restype = ctypes.c_longlong
+    n = fn(buf, 256)
+    return n, buf.value.decode()

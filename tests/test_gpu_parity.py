@@ -1,0 +1,109 @@
+"""Parity of the HIP kernels (through the C ABI) with the oracle, on a real MI355X.
+
+Tolerances are north_star's: ``max|d| / max|ref|`` <= 1e-4 for float32 and <= 2e-2 for
+bfloat16 storage with float32 accumulation; the oracle is evaluated in float64 on the same
+(bf16-valued, where applicable) inputs.
+"""
+
+import pytest
+import torch
+
+from deconver_amd import _lib, ops
+from oracle import ndc_oracle as O
+from tests.helpers import make_case
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-4, torch.bfloat16: 2e-2}
+
+# (C, groups, sc, kernel, spatial, batch)
+DIRECT_GEOMS = [
+    (12, 3, 8, (3, 3, 3), (7, 6, 5), 2),
+    (8, 1, 1, (3, 3, 3), (6, 6, 6), 2),
+    (16, 16, 4, (3, 3), (17, 15), 2),
+    (6, 2, 6, (3, 5, 3), (6, 7, 5), 2),
+    (8, 8, 2, (5,), (11,), 2),
+    (10, 5, 6, (3, 3), (9, 8), 2),
+]
+FUSED_GEOMS = [
+    (32, 32, 4, (3, 3, 3), (12, 14, 13), 2),
+    (64, 64, 4, (3, 3, 3), (10, 9, 11), 2),
+    (128, 128, 4, (3, 3, 3), (8, 8, 8), 2),
+    (256, 256, 4, (3, 3, 3), (6, 5, 4), 2),
+    (512, 512, 4, (3, 3, 3), (3, 4, 3), 2),
+    (16, 16, 4, (3, 3, 3), (9, 8, 7), 3),
+    (4, 4, 4, (3, 3, 3), (5, 20, 70), 1),
+    (8, 8, 4, (3, 3, 3), (20, 33, 64), 1),
+    (32, 32, 4, (5, 5), (64, 64), 1),
+    (8, 8, 4, (5, 5), (40, 100), 2),
+    (16, 16, 4, (3, 3), (17, 15), 2),
+]
+
+
+def _lib_gpu():
+    return _lib.get_library()
+
+
+def _oracle(x, z, h, bias, gout, G, m, sc, eps, relu):
+    d = [t.detach().cpu().double() if t is not None else None for t in (x, z, h, bias, gout)]
+    out, t1 = O.update_grouped(d[0], d[1], d[2], d[3], G, m, sc, eps, relu)
+    grads = O.update_backward(d[0], d[1], d[2], d[3], d[4], G, m, sc, eps, relu)
+    return out, t1, grads
+
+
+def _run_case(geom, dtype, path, relu=True, with_bias=True):
+    C, G, sc, ks, sp, B = geom
+    m = C // G
+    x, z, h, bias, gout = make_case(C, G, sc, ks, sp, B=B, dtype=dtype, bias_shift=0.3,
+                                    positive_z=not relu, device="cuda")
+    if not with_bias:
+        bias = None
+    lib = _lib_gpu()
+    kw = dict(groups=G, m=m, sc=sc, eps=1e-16, relu_input=relu, path=path)
+    out, t1 = ops.update_forward(lib, x, z, h, bias, **kw)
+    gx, gz, gh, gb = ops.update_backward(lib, x, z, t1, h, bias, gout, **kw)
+    torch.cuda.synchronize()
+    ro, rt1, (rgx, rgz, rgh, rgb) = _oracle(x, z, h, bias, gout, G, m, sc, 1e-16, relu)
+    tol = TOL[dtype]
+    errs = dict(out=O.rel_err(out.cpu(), ro), t1=O.rel_err(t1.cpu(), rt1),
+                gx=O.rel_err(gx.cpu(), rgx), gz=O.rel_err(gz.cpu(), rgz),
+                gh=O.rel_err(gh.cpu(), rgh))
+    if with_bias:
+        errs["gb"] = O.rel_err(gb.cpu(), rgb)
+    bad = {k: v for k, v in errs.items() if not v < tol}
+    assert not bad, f"{geom} {dtype} path={path}: {bad} (all: {errs})"
+    return errs
+
+
+@pytest.mark.parametrize("geom", DIRECT_GEOMS)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_direct_kernels(geom, dtype):
+    _run_case(geom, dtype, _lib.PATH_DIRECT)
+
+
+@pytest.mark.parametrize("geom", FUSED_GEOMS)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_fused_kernels(geom, dtype):
+    print("case", geom, dtype, flush=True)
+    _run_case(geom, dtype, _lib.PATH_FUSED)
+
+
+@pytest.mark.parametrize("relu,with_bias", [(True, False), (False, False)])
+def test_fused_later_iteration_form(relu, with_bias):
+    _run_case(FUSED_GEOMS[0], torch.float32, _lib.PATH_FUSED, relu=relu, with_bias=with_bias)
+
+
+def test_fused_matches_direct_at_size():
+    """A size the CPU oracle would take minutes for: the two HIP paths check each other."""
+    C, sc, ks, sp = 16, 4, (3, 3, 3), (32, 64, 64)
+    x, z, h, bias, gout = make_case(C, C, sc, ks, sp, B=1, bias_shift=0.3, device="cuda")
+    lib = _lib_gpu()
+    res = {}
+    for path in (_lib.PATH_DIRECT, _lib.PATH_FUSED):
+        kw = dict(groups=C, m=1, sc=sc, eps=1e-16, relu_input=True, path=path)
+        out, t1 = ops.update_forward(lib, x, z, h, bias, **kw)
+        res[path] = (out, t1) + tuple(ops.update_backward(lib, x, z, t1, h, bias, gout, **kw))
+    torch.cuda.synchronize()
+    for name, a, b in zip(("out", "t1", "gx", "gz", "gh", "gb"), res[_lib.PATH_FUSED],
+                          res[_lib.PATH_DIRECT]):
+        assert O.rel_err(a, b) < 1e-4, name

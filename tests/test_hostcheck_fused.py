@@ -1,0 +1,118 @@
+"""The fused LDS-tiled kernels, executed on the host build (bounds-, race- and
+uninitialised-read-checked LDS), against the oracle in float64."""
+
+import pytest
+import torch
+
+from deconver_amd import _lib, ops
+from oracle import ndc_oracle as O
+from tests.helpers import host_faults, hostcheck_library, make_case
+
+# (C, sc, kernel, spatial, batch)
+FUSED_GEOMS = [
+    (3, 4, (3, 3, 3), (5, 9, 8), 2),      # several row bands, ragged last band
+    (2, 4, (3, 3, 3), (4, 16, 16), 1),
+    (2, 4, (3, 3, 3), (3, 7, 13), 2),     # odd extents, W not a multiple of anything
+    (1, 4, (3, 3, 3), (1, 4, 5), 1),      # single plane
+    (2, 4, (3, 3, 3), (6, 3, 70), 1),     # W > 64: two wavefronts per row
+    (3, 4, (5, 5), (9, 12), 2),           # 2-D 5x5 (marches along H)
+    (2, 4, (5, 5), (3, 70), 1),
+    (2, 4, (3, 3), (7, 9), 2),            # 2-D 3x3
+]
+
+
+def _oracle(x, z, h, bias, gout, C, sc, eps, relu):
+    d = [t.double() if t is not None else None for t in (x, z, h, bias, gout)]
+    out, t1 = O.update_grouped(d[0], d[1], d[2], d[3], C, 1, sc, eps, relu)
+    grads = O.update_backward(d[0], d[1], d[2], d[3], d[4], C, 1, sc, eps, relu)
+    return out, t1, grads
+
+
+def test_fused_coverage_predicate():
+    lib = hostcheck_library()
+    ok = _lib.make_geom(2, 8, 1, 4, (8, 8, 8), (3, 3, 3), _lib.NDC_F32, True, 1e-16)
+    assert lib.fused_supported(ok)
+    for bad in (
+        _lib.make_geom(2, 4, 2, 4, (8, 8, 8), (3, 3, 3), 0, True, 1e-16),     # m = 2
+        _lib.make_geom(2, 8, 1, 3, (8, 8, 8), (3, 3, 3), 0, True, 1e-16),     # sc = 3
+        _lib.make_geom(2, 8, 1, 4, (8, 8, 8), (3, 5, 3), 0, True, 1e-16),     # anisotropic
+        _lib.make_geom(2, 8, 1, 4, (8, 8, 600), (3, 3, 3), 0, True, 1e-16),   # row too wide
+    ):
+        assert not lib.fused_supported(bad)
+        bad.path = _lib.PATH_FUSED
+        assert lib.check_geometry(bad) == -2
+        bad.path = _lib.PATH_AUTO
+        assert lib.check_geometry(bad) == 0   # the direct kernels still cover it
+
+
+@pytest.mark.parametrize("geom", FUSED_GEOMS)
+@pytest.mark.parametrize("relu,with_bias", [(True, True), (False, False)])
+def test_fused_forward_backward_fp32(geom, relu, with_bias):
+    C, sc, ks, sp, B = geom
+    lib = hostcheck_library()
+    x, z, h, bias, gout = make_case(C, C, sc, ks, sp, B=B, bias_shift=0.3, positive_z=not relu)
+    if not with_bias:
+        bias = None
+    eps = 1e-16
+    host_faults(lib)
+    out, t1 = ops.update_forward(lib, x, z, h, bias, groups=C, m=1, sc=sc, eps=eps,
+                                 relu_input=relu, path=_lib.PATH_FUSED)
+    n, first = host_faults(lib)
+    assert n == 0, f"forward LDS faults: {n} ({first})"
+    ro, rt1, (rgx, rgz, rgh, rgb) = _oracle(x, z, h, bias, gout, C, sc, eps, relu)
+    assert O.rel_err(out, ro) < 1e-5
+    assert O.rel_err(t1, rt1) < 1e-5
+    gx, gz, gh, gb = ops.update_backward(lib, x, z, t1, h, bias, gout, groups=C, m=1, sc=sc,
+                                         eps=eps, relu_input=relu, path=_lib.PATH_FUSED)
+    n, first = host_faults(lib)
+    assert n == 0, f"backward LDS faults: {n} ({first})"
+    assert O.rel_err(gx, rgx) < 1e-4
+    assert O.rel_err(gz, rgz) < 1e-4
+    assert O.rel_err(gh, rgh) < 1e-4
+    if with_bias:
+        assert O.rel_err(gb, rgb) < 1e-4
+
+
+def test_fused_inference_needs_no_t1():
+    C, sc, ks, sp = 2, 4, (3, 3, 3), (4, 6, 8)
+    lib = hostcheck_library()
+    x, z, h, bias, _ = make_case(C, C, sc, ks, sp, bias_shift=0.3)
+    out, t1 = ops.update_forward(lib, x, z, h, bias, groups=C, m=1, sc=sc, eps=1e-16,
+                                 relu_input=True, need_t1=False)
+    assert t1 is None
+    ref, _ = O.update_grouped(x.double(), z.double(), h.double(), bias.double(), C, 1, sc, 1e-16, True)
+    assert O.rel_err(out, ref) < 1e-5
+
+
+@pytest.mark.parametrize("geom", [FUSED_GEOMS[0], FUSED_GEOMS[5]])
+def test_fused_bf16_storage(geom):
+    C, sc, ks, sp, B = geom
+    lib = hostcheck_library()
+    x, z, h, bias, gout = make_case(C, C, sc, ks, sp, B=B, dtype=torch.bfloat16, bias_shift=0.3)
+    out, t1 = ops.update_forward(lib, x, z, h, bias, groups=C, m=1, sc=sc, eps=1e-16,
+                                 relu_input=True, path=_lib.PATH_FUSED)
+    ro, rt1, (rgx, rgz, rgh, rgb) = _oracle(x, z, h, bias, gout, C, sc, 1e-16, True)
+    assert out.dtype == torch.bfloat16 and O.rel_err(out, ro) < 2e-2
+    gx, gz, gh, gb = ops.update_backward(lib, x, z, t1, h, bias, gout, groups=C, m=1, sc=sc,
+                                         eps=1e-16, relu_input=True, path=_lib.PATH_FUSED)
+    for got, ref in ((gx, rgx), (gz, rgz), (gh, rgh), (gb, rgb)):
+        assert O.rel_err(got, ref) < 2e-2
+    assert host_faults(lib)[0] == 0
+
+
+def test_fused_partial_outputs():
+    C, sc, ks, sp = 2, 4, (3, 3, 3), (4, 6, 8)
+    lib = hostcheck_library()
+    x, z, h, bias, gout = make_case(C, C, sc, ks, sp, bias_shift=0.3)
+    out, t1 = ops.update_forward(lib, x, z, h, bias, groups=C, m=1, sc=sc, eps=1e-16,
+                                 relu_input=True, path=_lib.PATH_FUSED)
+    kw = dict(groups=C, m=1, sc=sc, eps=1e-16, relu_input=True, path=_lib.PATH_FUSED)
+    full = ops.update_backward(lib, x, z, t1, h, bias, gout, **kw)
+    for mask in ((1, 0, 0, 0), (0, 1, 0, 0), (0, 0, 1, 0), (0, 0, 0, 1)):
+        part = ops.update_backward(lib, x, z, t1, h, bias, gout, need_x=bool(mask[0]),
+                                   need_z=bool(mask[1]), need_h=bool(mask[2]),
+                                   need_b=bool(mask[3]), **kw)
+        for want, a, b in zip(mask, part, full):
+            assert (a is None) == (not want)
+            if want:
+                assert torch.equal(a, b)
