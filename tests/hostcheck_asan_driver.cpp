@@ -1,0 +1,85 @@
+// Memory-safety driver of the host build: every buffer is heap-allocated at its exact size,
+// so AddressSanitizer reports any global access the kernels make outside a tensor.  Built and
+// run by tests/test_hostcheck_asan.py:
+//   g++ -fsanitize=address,undefined -g -O1 tests/hostcheck_asan_driver.cpp -o <tmp>/driver
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+
+#include "../deconver_amd/csrc/ndc_hostcheck.cpp"
+
+struct Case {
+    int B, G, m, sc, D, H, W, kD, kH, kW, dtype, path;
+};
+
+static int run_case(const Case &c)
+{
+    ndc_geom g;
+    g.batch = c.B;
+    g.groups = c.G;
+    g.m = c.m;
+    g.sc = c.sc;
+    g.size[0] = c.D;
+    g.size[1] = c.H;
+    g.size[2] = c.W;
+    g.kernel[0] = c.kD;
+    g.kernel[1] = c.kH;
+    g.kernel[2] = c.kW;
+    g.dtype = c.dtype;
+    g.relu_input = 1;
+    g.path = c.path;
+    g.eps = 1e-16f;
+    const size_t esz = c.dtype == NDC_BF16 ? 2 : 4;
+    const size_t sp = (size_t)c.D * c.H * c.W;
+    const size_t nx = (size_t)c.B * c.G * c.m * sp, ns = (size_t)c.B * c.G * c.sc * sp;
+    const size_t nh = (size_t)c.G * c.m * c.sc * c.kD * c.kH * c.kW;
+    auto fill = [&](size_t n) {
+        unsigned char *p = (unsigned char *)malloc(n * esz);
+        for (size_t i = 0; i < n; ++i) {
+            float v = (float)((i * 2654435761u) % 1000) / 1000.0f;
+            if (esz == 4) ((float *)p)[i] = v;
+            else ((unsigned short *)p)[i] = ndc::float_to_bf16(v);
+        }
+        return p;
+    };
+    unsigned char *x = fill(nx), *z = fill(ns), *gout = fill(ns);
+    unsigned char *out = (unsigned char *)malloc(ns * esz), *t1 = (unsigned char *)malloc(nx * esz);
+    unsigned char *gx = (unsigned char *)malloc(nx * esz), *gz = (unsigned char *)malloc(ns * esz);
+    std::vector<float> h(nh, 0.05f), bias((size_t)c.G * c.sc, 0.1f), gh(nh), gb((size_t)c.G * c.sc);
+    int st = ndc_forward(&g, x, z, h.data(), bias.data(), out, t1, nullptr);
+    if (st) return st;
+    const size_t wsb = ndc_backward_workspace_bytes(&g, 1, 1, 1, 1);
+    void *ws = nullptr;
+    if (posix_memalign(&ws, 256, wsb ? wsb : 256)) return -100;
+    st = ndc_backward(&g, x, z, t1, h.data(), bias.data(), gout, gx, gz, gh.data(), gb.data(), ws,
+                      wsb, nullptr);
+    free(ws);
+    free(x); free(z); free(gout); free(out); free(t1); free(gx); free(gz);
+    return st;
+}
+
+int main()
+{
+    const Case cases[] = {
+        {2, 3, 1, 4, 5, 9, 8, 3, 3, 3, NDC_F32, NDC_PATH_FUSED},
+        {1, 2, 1, 4, 3, 7, 13, 3, 3, 3, NDC_BF16, NDC_PATH_FUSED},
+        {1, 2, 1, 4, 6, 3, 70, 3, 3, 3, NDC_F32, NDC_PATH_FUSED},
+        {1, 1, 1, 4, 1, 1, 1, 3, 3, 3, NDC_F32, NDC_PATH_FUSED},
+        {2, 3, 1, 4, 1, 9, 12, 1, 5, 5, NDC_F32, NDC_PATH_FUSED},
+        {1, 2, 1, 4, 1, 3, 70, 1, 5, 5, NDC_BF16, NDC_PATH_FUSED},
+        {2, 2, 1, 4, 1, 7, 9, 1, 3, 3, NDC_F32, NDC_PATH_FUSED},
+        {1, 2, 1, 4, 2, 40, 33, 3, 3, 3, NDC_F32, NDC_PATH_FUSED},
+        {2, 3, 2, 2, 5, 4, 3, 3, 3, 3, NDC_F32, NDC_PATH_DIRECT},
+        {1, 2, 3, 2, 1, 6, 5, 1, 3, 5, NDC_BF16, NDC_PATH_DIRECT},
+    };
+    int bad = 0;
+    for (const Case &c : cases) {
+        const int st = run_case(c);
+        char first[256];
+        const long long faults = ndc_host_faults(first, sizeof first);
+        printf("case B%d G%d m%d sc%d %dx%dx%d k%dx%dx%d dtype%d path%d -> status %d, lds faults %lld %s\n",
+               c.B, c.G, c.m, c.sc, c.D, c.H, c.W, c.kD, c.kH, c.kW, c.dtype, c.path, st, faults, first);
+        if (st || faults) ++bad;
+    }
+    return bad ? 1 : 0;
+}
