@@ -67,6 +67,22 @@ NDC_HD float fast_rcp(float v)
 #endif
 }
 
+// Read-only, wave-uniform data (filter taps, bias): on the device the pointer is re-typed
+// into the constant address space, which lets the compiler fetch through the scalar unit
+// (s_load into SGPRs) instead of issuing a vector load per lane.  The data must not be
+// written by the kernel that reads it this way.
+#if NDC_DEVICE_BUILD && defined(__HIP_DEVICE_COMPILE__)
+typedef const float __attribute__((address_space(4))) *UniformF;
+NDC_D UniformF as_uniform(const float *p) { return (UniformF)(unsigned long long)p; }
+#else
+typedef const float *UniformF;
+NDC_HD UniformF as_uniform(const float *p) { return p; }
+#endif
+
+template <int N> struct IntTag {
+    static constexpr int value = N;
+};
+
 // Geometry as the kernels see it (derived once on the host from ndc_geom).
 struct KGeom {
     int B, G, m, sc;

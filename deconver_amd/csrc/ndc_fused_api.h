@@ -4,16 +4,20 @@
 #pragma once
 
 #include "../../include/deconver_ndc.h"
+#include <stdlib.h>
+
 #include "ndc_fused.h"
 
 namespace ndc {
 namespace fused {
 
 // Filter geometries with compiled instances, in the marching view (2-D k x k runs as
-// (k, 1, k)).  One row per (KD, KH, KW, SC); RHF / RHB are the rows per thread of the
-// forward and backward kernels.
+// (k, 1, k)).  One row per (KD, KH, KW, SC, RHF, RHB); RHF / RHB are the rows per thread of
+// the forward and backward kernels.  Several rows may share a filter geometry: the first
+// one whose row counts match the tuning choice (or, failing that, the first one) is used.
 #define NDC_FUSED_VARIANTS(X)  \
     X(3, 3, 3, 4, 4, 2)        \
+    X(3, 3, 3, 4, 2, 1)        \
     X(5, 1, 5, 4, 1, 1)        \
     X(3, 1, 3, 4, 1, 1)
 
@@ -21,17 +25,43 @@ struct Variant {
     int KD, KH, KW, SC, RHF, RHB;
 };
 
+// Launch-shape choices that are not dictated by the geometry.  Defaults are the measured
+// best; the environment variables exist for tuning runs only.
+struct Tuning {
+    int rhf, rhb, threads_f, threads_b;
+};
+
+static inline int env_int(const char *name, int dflt)
+{
+    const char *v = getenv(name);
+    return v && *v ? atoi(v) : dflt;
+}
+
+static inline Tuning tuning()
+{
+    Tuning t;
+    t.rhf = env_int("NDC_TUNE_RHF", 4);
+    t.rhb = env_int("NDC_TUNE_RHB", 2);
+    t.threads_f = env_int("NDC_TUNE_NTF", 256);
+    t.threads_b = env_int("NDC_TUNE_NTB", 256);
+    return t;
+}
+
 static inline bool find_variant(const KGeom &q, const March &m, Variant &v)
 {
     if (q.m != 1) return false;
-#define X(kd_, kh_, kw_, sc_, rhf_, rhb_)                                         \
+    const Tuning tn = tuning();
+    bool found = false;
+#define X(kd_, kh_, kw_, sc_, rhf_, rhb_)                                       \
     if (m.KD == kd_ && m.KH == kh_ && m.KW == kw_ && q.sc == sc_) {             \
-        v = Variant{kd_, kh_, kw_, sc_, rhf_, rhb_};                              \
-        return true;                                                        \
+        const bool exact = rhf_ == tn.rhf && rhb_ == tn.rhb;                    \
+        if (!found || exact) v = Variant{kd_, kh_, kw_, sc_, rhf_, rhb_};       \
+        if (exact) return true;                                                 \
+        found = true;                                                           \
     }
     NDC_FUSED_VARIANTS(X)
 #undef X
-    return false;
+    return found;
 }
 
 struct Plan {
@@ -54,10 +84,12 @@ static inline bool make_plan(const KGeom &q, Plan &pl)
 {
     pl.m = march_of(q);
     if (!find_variant(q, pl.m, pl.v)) return false;
-    if (!make_tile(pl.m, pl.v.RHF, 256, pl.tf)) return false;
-    if (!make_tile(pl.m, pl.v.RHB, 256, pl.tb)) return false;
+    const Tuning tn = tuning();
+    if (!make_tile(pl.m, pl.v.RHF, tn.threads_f, pl.tf)) return false;
+    if (!make_tile(pl.m, pl.v.RHB, tn.threads_b, pl.tb)) return false;
 #define X(kd_, kh_, kw_, sc_, rhf_, rhb_)                                                     \
-    if (pl.v.KD == kd_ && pl.v.KH == kh_ && pl.v.KW == kw_ && pl.v.SC == sc_)               \
+    if (pl.v.KD == kd_ && pl.v.KH == kh_ && pl.v.KW == kw_ && pl.v.SC == sc_ && pl.v.RHF == rhf_ &&  \
+        pl.v.RHB == rhb_)               \
         plan_lds<kd_, kh_, kw_, sc_, rhf_, rhb_>(pl);
     NDC_FUSED_VARIANTS(X)
 #undef X
@@ -112,7 +144,8 @@ static int forward(const KGeom &q, const T *x, const T *z, const float *h, const
     p.eps = q.eps;
     p.t = pl.tf;
 #define X(kd_, kh_, kw_, sc_, rhf_, rhb_)                                                        \
-    if (pl.v.KD == kd_ && pl.v.KH == kh_ && pl.v.KW == kw_ && pl.v.SC == sc_)                  \
+    if (pl.v.KD == kd_ && pl.v.KH == kh_ && pl.v.KW == kw_ && pl.v.SC == sc_ && pl.v.RHF == rhf_ &&  \
+        pl.v.RHB == rhb_)                  \
         return BE::template block_kernel<FwdKernel<kd_, kh_, kw_, sc_, rhf_, T>>(               \
             p, pl.nblk_f, pl.tf.NT, pl.lds_f, stream);
     NDC_FUSED_VARIANTS(X)
@@ -161,7 +194,8 @@ static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const f
     p.part = part1;
     p.part_stride = kt;
 #define X(kd_, kh_, kw_, sc_, rhf_, rhb_)                                                        \
-    if (pl.v.KD == kd_ && pl.v.KH == kh_ && pl.v.KW == kw_ && pl.v.SC == sc_)                  \
+    if (pl.v.KD == kd_ && pl.v.KH == kh_ && pl.v.KW == kw_ && pl.v.SC == sc_ && pl.v.RHF == rhf_ &&  \
+        pl.v.RHB == rhb_)                  \
         st = BE::template block_kernel<Bwd1Kernel<kd_, kh_, kw_, sc_, rhb_, T>>(                \
             p, pl.nblk_b, pl.tb.NT, pl.lds_b1, stream);
     NDC_FUSED_VARIANTS(X)
@@ -173,7 +207,8 @@ static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const f
     p.part_stride = kt + q.sc;
     st = NDC_ERR_GEOMETRY;
 #define X(kd_, kh_, kw_, sc_, rhf_, rhb_)                                                        \
-    if (pl.v.KD == kd_ && pl.v.KH == kh_ && pl.v.KW == kw_ && pl.v.SC == sc_)                  \
+    if (pl.v.KD == kd_ && pl.v.KH == kh_ && pl.v.KW == kw_ && pl.v.SC == sc_ && pl.v.RHF == rhf_ &&  \
+        pl.v.RHB == rhb_)                  \
         st = BE::template block_kernel<Bwd2Kernel<kd_, kh_, kw_, sc_, rhb_, T>>(                \
             p, pl.nblk_b, pl.tb.NT, pl.lds_b2, stream);
     NDC_FUSED_VARIANTS(X)
