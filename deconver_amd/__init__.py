@@ -1,4 +1,9 @@
-"""MI355X-native implementation of Deconver's nonnegative-deconvolution (NDC) update."""
+"""MI355X-native implementation of Deconver's nonnegative-deconvolution (NDC) update.
+
+``Deconv`` / ``NDC`` is the drop-in layer; ``deconv_update`` is the operator boundary
+(one multiplicative update as an autograd node over ``libdeconver_ndc.so``)."""
 
 from . import _lib, ops  # noqa: F401
-from .functional import deconv_update, hip_kernels_apply  # noqa: F401
+from .functional import DeconvUpdate, deconv_update, hip_kernels_apply  # noqa: F401
+from .layers import MLP, LayerNorm, Linear  # noqa: F401
+from .ndc import NDC, Deconv, Initializer  # noqa: F401

@@ -1,0 +1,236 @@
+"""The layer on a real MI355X (HIP route) against the oracle; the case list follows the
+reference's own equivalence tests (tests/test_deconv_equivalence.py:112-281)."""
+
+import pytest
+import torch
+
+import deconver_amd as dc
+from oracle import ndc_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+BRATS_STAGES = [(32, (12, 14, 13)), (64, (10, 9, 11)), (128, (8, 8, 8)), (256, (6, 5, 4)),
+                (512, (3, 4, 3))]
+
+
+def _layer(kwargs, seed=0, bias=1.0):
+    torch.manual_seed(seed)
+    layer = dc.Deconv(**kwargs)
+    with torch.no_grad():
+        layer.init.linear.linear.bias.add_(bias)
+    return layer.cuda()
+
+
+def _oracle_run(layer, kwargs, x, g, need=("x", "w", "b", "h")):
+    """Oracle forward/backward in float64 on the CPU with the layer's parameters."""
+    oracle = O.OracleNDC(kwargs["channels"], kwargs["kernel_size"],
+                         source_channels=kwargs.get("source_channels"),
+                         ratio=kwargs.get("ratio", 1), groups=kwargs.get("groups", -1),
+                         num_iters=kwargs.get("num_iters", 1),
+                         num_grad_iters=kwargs.get("num_grad_iters"))
+    w = layer.init.linear.linear.weight.detach().cpu().double().squeeze(-1).requires_grad_(True)
+    b = layer.init.linear.linear.bias.detach().cpu().double().requires_grad_(True)
+    h0 = layer.init.h0.detach().cpu().double().requires_grad_(True)
+    xr = x.detach().cpu().double().requires_grad_(True)
+    y = oracle.forward(xr, w, b, h0)
+    if y.requires_grad:
+        y.backward(g.detach().cpu().double())
+    return y.detach(), dict(x=xr.grad, w=w.grad, b=b.grad, h=h0.grad)
+
+
+def _compare(kwargs, batch, spatial, tol=1e-4, seed=0, bias=1.0, dtype=torch.float32):
+    layer = _layer(kwargs, seed, bias)
+    torch.manual_seed(seed + 1)
+    x0 = torch.rand(batch, kwargs["channels"], *spatial).to(dtype)
+    x = x0.cuda().requires_grad_(True)
+    assert layer.fast_path_applicable(x), "expected the HIP route"
+    y = layer(x)
+    torch.manual_seed(seed + 2)
+    g = torch.randn(y.shape).to(y.dtype)
+    if y.requires_grad:
+        y.backward(g.cuda())
+    yr, gr = _oracle_run(layer, kwargs, x0.float(), g.float())
+    assert y.shape == yr.shape
+    assert O.rel_err(y.detach().cpu(), yr) < tol, "forward"
+    got = dict(x=x.grad, w=layer.init.linear.linear.weight.grad,
+               b=layer.init.linear.linear.bias.grad, h=layer.init.h0.grad)
+    for name, ref in gr.items():
+        if ref is None:
+            assert got[name] is None, f"{name} should have no gradient"
+            continue
+        assert got[name] is not None, f"missing gradient for {name}"
+        e = O.rel_err(got[name].detach().cpu().reshape(ref.shape), ref)
+        assert e < tol, f"{name} grad rel err {e:.3e}"
+
+
+@pytest.mark.parametrize("channels,spatial", BRATS_STAGES)
+def test_brats_stage_geometries(channels, spatial):
+    _compare(dict(channels=channels, ratio=4, groups=-1, kernel_size=(3, 3, 3), num_iters=1), 2, spatial)
+
+
+@pytest.mark.parametrize("kwargs,spatial", [
+    (dict(channels=12, ratio=2, groups=3, kernel_size=(3, 3, 3)), (7, 6, 5)),
+    (dict(channels=8, ratio=1, groups=1, kernel_size=(3, 3, 3)), (6, 6, 6)),
+    (dict(channels=16, ratio=4, groups=-1, kernel_size=(3, 3)), (17, 15)),
+    (dict(channels=6, ratio=2, groups=2, kernel_size=(3, 5, 3)), (6, 7, 5)),
+    (dict(channels=8, ratio=2, groups=-1, kernel_size=(5,)), (11,)),
+    (dict(channels=10, ratio=3, groups=5, kernel_size=(3, 3)), (9, 8)),
+    (dict(channels=32, ratio=4, groups=-1, kernel_size=(5, 5)), (24, 40)),
+])
+def test_geometries(kwargs, spatial):
+    _compare(dict(num_iters=1, **kwargs), 2, spatial)
+
+
+@pytest.mark.parametrize("batch", [1, 3])
+def test_batch_sizes(batch):
+    _compare(dict(channels=16, ratio=4, groups=-1, kernel_size=(3, 3, 3), num_iters=1), batch, (9, 8, 7))
+
+
+@pytest.mark.parametrize("iters", [(3, 1), (5, 1), (2, 2), (3, 3)])
+def test_multiple_iterations(iters):
+    kwargs = dict(channels=8, ratio=4, groups=-1, kernel_size=(3, 3, 3), num_iters=iters[0],
+                  num_grad_iters=iters[1])
+    _compare(kwargs, 2, (6, 6, 6), tol=5e-4)
+
+
+def test_bf16_autocast_route_and_tolerance():
+    kwargs = dict(channels=16, ratio=4, groups=-1, kernel_size=(3, 3, 3))
+    layer = _layer(kwargs)
+    torch.manual_seed(1)
+    x0 = torch.rand(2, 16, 9, 8, 10)
+    x = x0.cuda().requires_grad_(True)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        assert layer.fast_path_applicable(x)
+        y = layer(x)
+    assert y.dtype == torch.bfloat16
+    g = torch.randn(y.shape)
+    y.backward(g.cuda().to(y.dtype))
+    # oracle on the bf16-rounded operands the HIP route saw (x and the projection weight)
+    ref_layer = _layer(kwargs)
+    with torch.no_grad():
+        ref_layer.init.linear.linear.weight.copy_(layer.init.linear.linear.weight.bfloat16().float())
+    yr, gr = _oracle_run(ref_layer, kwargs, x0.bfloat16().float(), g.bfloat16().float())
+    assert O.rel_err(y.detach().float().cpu(), yr) < 2e-2
+    assert x.grad.dtype == torch.float32 and layer.init.h0.grad.dtype == torch.float32
+    assert O.rel_err(x.grad.cpu(), gr["x"]) < 2e-2
+    assert O.rel_err(layer.init.h0.grad.cpu(), gr["h"]) < 2e-2
+    assert O.rel_err(layer.init.linear.linear.bias.grad.cpu(), gr["b"]) < 2e-2
+    assert O.rel_err(layer.init.linear.linear.weight.grad.cpu().squeeze(-1), gr["w"]) < 2e-2
+
+
+def test_partial_gradient_requests():
+    kwargs = dict(channels=16, ratio=4, groups=-1, kernel_size=(3, 3, 3), num_iters=1)
+    names = ["init.h0", "init.linear.linear.weight", "init.linear.linear.bias"]
+    key = {"init.h0": "h", "init.linear.linear.weight": "w", "init.linear.linear.bias": "b"}
+    for wanted in ([], ["init.h0"], ["init.linear.linear.bias"], names):
+        for input_grad in (False, True):
+            layer = _layer(kwargs)
+            for name, p in layer.named_parameters():
+                p.requires_grad_(name in wanted)
+            torch.manual_seed(3)
+            x0 = torch.rand(2, 16, 7, 6, 8)
+            x = x0.cuda().requires_grad_(input_grad)
+            y = layer(x)
+            g = torch.ones_like(y)
+            if wanted or input_grad:
+                y.backward(g)
+            yr, gr = _oracle_run(layer, kwargs, x0, g)
+            assert O.rel_err(y.detach().cpu(), yr) < 1e-4
+            assert (x.grad is not None) == input_grad
+            if input_grad:
+                assert O.rel_err(x.grad.cpu(), gr["x"]) < 1e-4
+            for name, p in layer.named_parameters():
+                assert (p.grad is not None) == (name in wanted), name
+                if name in wanted:
+                    assert O.rel_err(p.grad.cpu().reshape(gr[key[name]].shape), gr[key[name]]) < 1e-4
+
+
+def test_non_contiguous_input_and_fit_reconstruct():
+    kwargs = dict(channels=8, ratio=2, groups=-1, kernel_size=(3, 3, 3), num_iters=1)
+    layer = _layer(kwargs, bias=0.0)
+    base = torch.rand(2, 8, 6, 6, 12).cuda()
+    x = base[..., ::2]
+    assert not x.is_contiguous()
+    yr, _ = _oracle_run(layer, kwargs, x, torch.zeros(2, 16, 6, 6, 6))
+    assert O.rel_err(layer(x).cpu(), yr) < 1e-4
+    s, h = layer.fit(x)
+    assert h.shape == (2, 8, 2, 3, 3, 3) and h.is_contiguous()
+    assert torch.equal(h[0], torch.relu(layer.init.h0))
+    xh = layer.reconstruct(s, h)
+    ref = O.op_K(s.cpu().double(), torch.relu(layer.init.h0).cpu().double(), 8, 1, 2)
+    assert O.rel_err(xh.cpu(), ref) < 1e-5
+
+
+def test_double_backward_is_refused():
+    layer = _layer(dict(channels=4, ratio=2, groups=-1, kernel_size=(3, 3)))
+    x = torch.rand(1, 4, 6, 6, device="cuda", requires_grad=True)
+    y = layer(x)
+    with pytest.raises(RuntimeError, match="double backward"):
+        torch.autograd.grad(y.sum(), x, create_graph=True)
+
+
+def test_general_route_on_gpu_for_unsupported_regimes():
+    kwargs = dict(channels=8, ratio=2, groups=-1, kernel_size=(3, 3), update_filter=True, num_iters=2)
+    layer = _layer(kwargs, bias=0.0)
+    x = torch.rand(2, 8, 6, 6, device="cuda")
+    assert not layer.fast_path_applicable(x)
+    cpu = _layer(kwargs, bias=0.0).cpu()
+    assert O.rel_err(layer(x).cpu(), cpu(x.cpu())) < 1e-4
+
+
+def test_config1_single_layer_2d_sum_of_squares():
+    """Batch 1, 32 channels, 64x64, depthwise, ratio 4, 5x5, softplus-positive kernel."""
+    torch.manual_seed(0)
+    kwargs = dict(channels=32, kernel_size=(5, 5), ratio=4, groups=-1)
+    layer = dc.Deconv(**kwargs)
+    with torch.no_grad():
+        layer.init.h0.copy_(torch.nn.functional.softplus(0.1 * torch.randn(32, 4, 5, 5)))
+    x0 = torch.rand(1, 32, 64, 64)
+    layer = layer.cuda()
+    x = x0.cuda().requires_grad_(True)
+    y = layer(x)
+    (y ** 2).sum().backward()
+    oracle = O.OracleNDC(32, (5, 5), ratio=4)
+    w = layer.init.linear.linear.weight.detach().cpu().double().squeeze(-1).requires_grad_(True)
+    b = layer.init.linear.linear.bias.detach().cpu().double().requires_grad_(True)
+    h0 = layer.init.h0.detach().cpu().double().requires_grad_(True)
+    xr = x0.double().requires_grad_(True)
+    yr = oracle.forward(xr, w, b, h0)
+    (yr ** 2).sum().backward()
+    assert O.rel_err(y.detach().cpu(), yr.detach()) < 1e-4
+    assert O.rel_err(x.grad.cpu(), xr.grad) < 1e-4
+    assert O.rel_err(layer.init.h0.grad.cpu(), h0.grad) < 1e-4
+    assert O.rel_err(layer.init.linear.linear.weight.grad.cpu().squeeze(-1), w.grad) < 1e-4
+    assert O.rel_err(layer.init.linear.linear.bias.grad.cpu(), b.grad) < 1e-4
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.bfloat16, 2e-2), (torch.float32, 1e-4)])
+def test_headline_size_channel_slices_match_oracle(dtype, tol):
+    """Config 3 at full size (B=2, C=128, 64^3, 3x3x3, ratio 4).  Depthwise channels are
+    independent, so any channel slice of the full-size result must equal the oracle run on
+    that slice alone -- which the CPU does in seconds."""
+    from deconver_amd import _lib, ops
+    B, C, sc, sp = 2, 128, 4, (64, 64, 64)
+    gen = torch.Generator().manual_seed(0)
+    h = torch.nn.functional.softplus(0.1 * torch.randn(C, sc, 3, 3, 3, generator=gen))
+    x = torch.randn(B, C, *sp, generator=gen).abs().to(dtype)
+    z = (0.5 * torch.randn(B, C * sc, *sp, generator=gen)).to(dtype)
+    bias = 0.1 * torch.randn(C * sc, generator=gen)
+    gout = torch.randn(B, C * sc, *sp, generator=gen).to(dtype)
+    lib = _lib.get_library()
+    dev = [t.cuda() for t in (x, z, h, bias, gout)]
+    kw = dict(groups=C, m=1, sc=sc, eps=1e-16, relu_input=True)
+    out, t1 = ops.update_forward(lib, dev[0], dev[1], dev[2], dev[3], **kw)
+    gx, gz, gh, gb = ops.update_backward(lib, dev[0], dev[1], t1, dev[2], dev[3], dev[4], **kw)
+    torch.cuda.synchronize()
+    for c in (0, 77, 127):
+        cs = slice(c * sc, (c + 1) * sc)
+        xs, zs, hs, bs, gs = (x[:, c:c + 1].double(), z[:, cs].double(), h[c:c + 1].double(),
+                              bias[cs].double(), gout[:, cs].double())
+        ro, _ = O.update_grouped(xs, zs, hs, bs, 1, 1, sc, 1e-16, True)
+        rgx, rgz, rgh, rgb = O.update_backward(xs, zs, hs, bs, gs, 1, 1, sc, 1e-16, True)
+        assert O.rel_err(out[:, cs].cpu(), ro) < tol, f"out channel {c}"
+        assert O.rel_err(gx[:, c:c + 1].cpu(), rgx) < tol, f"gx channel {c}"
+        assert O.rel_err(gz[:, cs].cpu(), rgz) < tol, f"gz channel {c}"
+        assert O.rel_err(gh[c:c + 1].cpu(), rgh) < tol, f"gh channel {c}"
+        assert O.rel_err(gb[cs].cpu(), rgb) < tol, f"gb channel {c}"

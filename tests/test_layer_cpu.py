@@ -1,0 +1,160 @@
+"""The layer module on CPU: general route against the oracle, API and checkpoint contract,
+route choice, error behaviour.  (The HIP route is exercised in the gpu-marked tests.)"""
+
+import pytest
+import torch
+
+import deconver_amd as dc
+from deconver_amd import operations as G
+from oracle import ndc_oracle as O
+
+
+def _pair(kwargs, seed=0, bias=0.0, dtype=torch.float64):
+    torch.manual_seed(seed)
+    layer = dc.Deconv(**kwargs).to(dtype)
+    with torch.no_grad():
+        layer.init.linear.linear.bias.add_(bias)
+    oracle = O.OracleNDC(kwargs["channels"], kwargs["kernel_size"],
+                         source_channels=kwargs.get("source_channels"),
+                         ratio=kwargs.get("ratio", 1), groups=kwargs.get("groups", -1),
+                         num_iters=kwargs.get("num_iters", 1),
+                         num_grad_iters=kwargs.get("num_grad_iters"))
+    return layer, oracle
+
+
+CASES = [
+    (dict(channels=12, ratio=2, groups=3, kernel_size=(3, 3, 3)), (7, 6, 5)),
+    (dict(channels=8, ratio=1, groups=1, kernel_size=(3, 3, 3)), (6, 6, 6)),
+    (dict(channels=16, ratio=4, groups=-1, kernel_size=(3, 3)), (17, 15)),
+    (dict(channels=6, ratio=2, groups=2, kernel_size=(3, 5, 3)), (6, 7, 5)),
+    (dict(channels=8, ratio=2, groups=-1, kernel_size=(5,)), (11,)),
+    (dict(channels=8, ratio=2, groups=-1, kernel_size=(3, 3, 3), num_iters=3, num_grad_iters=1), (6, 6, 6)),
+    (dict(channels=8, ratio=2, groups=-1, kernel_size=(3, 3, 3), num_iters=3, num_grad_iters=3), (6, 6, 6)),
+]
+
+
+@pytest.mark.parametrize("kwargs,spatial", CASES)
+def test_general_route_matches_oracle(kwargs, spatial):
+    layer, oracle = _pair(kwargs, bias=1.0)
+    torch.manual_seed(1)
+    x = torch.rand(2, kwargs["channels"], *spatial, dtype=torch.float64)
+    xa, xb = x.clone().requires_grad_(True), x.clone().requires_grad_(True)
+    params = [layer.init.linear.linear.weight, layer.init.linear.linear.bias, layer.init.h0]
+    ref_params = [p.detach().clone().requires_grad_(True) for p in params]
+    y = layer(xa)
+    yr = oracle.forward(xb, ref_params[0].squeeze(-1), ref_params[1], ref_params[2])
+    assert y.shape == (2, layer.groups * layer.source_channels, *spatial)
+    assert O.rel_err(y, yr) < 1e-12
+    g = torch.randn_like(y)
+    y.backward(g)
+    yr.backward(g)
+    assert O.rel_err(xa.grad, xb.grad) < 1e-10
+    for p, r in zip(params, ref_params):
+        if r.grad is None:
+            assert p.grad is None
+        else:
+            assert O.rel_err(p.grad, r.grad.view_as(p.grad)) < 1e-10
+
+
+def test_constructor_arithmetic_and_state_dict_contract():
+    layer = dc.Deconv(channels=16, kernel_size=(3, 3, 3), ratio=4, groups=-1)
+    assert (layer.groups, layer.source_channels, layer.filter_channels) == (16, 4, 1)
+    assert layer.num_iters == 1 and layer.num_grad_iters == 1 and layer.eps == 1e-16
+    sd = layer.state_dict()
+    assert list(sd) == ["init.h0", "init.linear.linear.weight", "init.linear.linear.bias"]
+    assert sd["init.h0"].shape == (16, 4, 3, 3, 3)
+    assert sd["init.linear.linear.weight"].shape == (64, 16, 1)
+    assert sd["init.linear.linear.bias"].shape == (64,)
+    other = dc.NDC(channels=16, kernel_size=(3, 3, 3), ratio=4)
+    other.load_state_dict(sd, strict=True)
+    grouped = dc.Deconv(channels=12, kernel_size=(3, 3), ratio=2, groups=3)
+    assert (grouped.groups, grouped.source_channels, grouped.filter_channels) == (3, 8, 4)
+    assert grouped.init.h0.shape == (12, 8, 3, 3)
+    assert grouped.init.linear.linear.weight.shape == (24, 12, 1)
+    with pytest.raises(AssertionError):
+        dc.Deconv(channels=10, kernel_size=(3,), groups=4)
+    # kaiming-uniform(a=sqrt(5)) bound of h0: 1/sqrt(fan_in), fan_in = sc * taps
+    assert layer.init.h0.abs().max() <= 1 / (4 * 27) ** 0.5
+
+
+def test_route_choice():
+    base = dict(channels=8, ratio=2, groups=-1, kernel_size=(3, 3, 3))
+    assert dc.Deconv(**base).fast_path_applicable()
+    for extra in (dict(update_filter=True), dict(update_source=False), dict(verbose=True),
+                  dict(stride=1), dict(num_iters=0)):
+        assert not dc.Deconv(**base, **extra).fast_path_applicable()
+    assert not dc.Deconv(channels=8, kernel_size=(4, 4)).fast_path_applicable()
+
+    class Custom(dc.Deconv):
+        def update_s(self, x, s, h):
+            return super().update_s(x, s, h)
+
+    assert not Custom(**base).fast_path_applicable()
+    layer = dc.Deconv(**base)
+    assert not layer.fast_path_applicable(torch.rand(1, 8, 4, 4, 4))        # CPU tensor
+    assert not layer.fast_path_applicable(torch.rand(1, 8, 4, 4, 4).double())
+
+
+def test_update_op_refuses_cpu_tensors():
+    x, z = torch.rand(1, 2, 4, 4), torch.rand(1, 4, 4, 4)
+    h = torch.rand(2, 2, 3, 3)
+    with pytest.raises(RuntimeError):
+        dc.deconv_update(x, z, h, None, groups=2, m=1, sc=2, eps=1e-16, relu_input=True)
+
+
+def test_filter_update_fit_reconstruct_loss_and_verbose(capsys):
+    kwargs = dict(channels=6, ratio=2, groups=3, kernel_size=(3, 3), update_filter=True, num_iters=3)
+    torch.manual_seed(0)
+    layer = dc.Deconv(**kwargs).double()
+    x = torch.rand(2, 6, 7, 6, dtype=torch.float64)
+    s, h = layer.fit(x)
+    assert s.shape == (2, 12, 7, 6) and h.shape == (2, 6, 4, 3, 3)
+    assert (s >= 0).all() and (h >= 0).all()
+    xh = layer.reconstruct(s, h)
+    assert xh.shape == x.shape
+    # the multiplicative updates must not increase the reconstruction error
+    s0, h0 = layer.init(x)
+    args0 = [layer.split_channels(v) for v in (x, s0, h0)]
+    args1 = [layer.split_channels(v) for v in (x, s, h)]
+    assert (layer.loss(*args1) <= layer.loss(*args0) + 1e-12).all()
+    nh = layer.normalize_h(layer.split_channels(h))
+    assert torch.allclose(nh.sum(dim=[1, 3, 4]), torch.ones(6, 4, dtype=torch.float64), atol=1e-9)
+    loud = dc.Deconv(channels=4, kernel_size=(3,), num_iters=2, verbose=True)
+    loud(torch.rand(1, 4, 9))
+    assert capsys.readouterr().out.count("loss") == 2
+
+
+def test_sconv_matches_definition():
+    torch.manual_seed(0)
+    a = torch.rand(2, 3, 5, 4, dtype=torch.float64)
+    b = torch.rand(2, 2, 5, 4, dtype=torch.float64)
+    out = G.sconv(a, b, padding=(1, 1))
+    assert out.shape == (2, 3, 2, 3, 3)
+    ap = torch.nn.functional.pad(a, (1, 1, 1, 1))
+    for n in range(2):
+        for i in range(3):
+            for o in range(2):
+                for u in range(3):
+                    for v in range(3):
+                        want = (ap[n, i, u:u + 5, v:v + 4] * b[n, o]).sum()
+                        assert abs(out[n, i, o, u, v] - want) < 1e-12
+
+
+def test_helper_ops():
+    x = torch.rand(2, 3, 4, 5)
+    sm = G.softmax(x, dim=(1, 3))
+    assert torch.allclose(sm.sum(dim=(1, 3)), torch.ones(2, 4), atol=1e-6)
+    assert torch.allclose(G.softmax(x, 2), torch.softmax(x, 2))
+    assert torch.allclose(G.relative_error(x, x), torch.full((2,), 1e-16) / (G.norm2(x) + 1e-16))
+    assert (G.kl_divergence(x, x).abs() < 1e-7).all()
+    lin = dc.Linear(3, 6)
+    assert lin(x).shape == (2, 6, 4, 5)
+    assert list(lin.state_dict()) == ["linear.weight", "linear.bias"]
+    mlp = dc.MLP(3, ratio=4)
+    assert mlp(x).shape == x.shape
+    assert list(mlp.state_dict()) == ["block.0.linear.weight", "block.0.linear.bias",
+                                      "block.3.linear.weight", "block.3.linear.bias"]
+    ln = dc.LayerNorm(3)
+    y = ln(x)
+    assert torch.allclose(y.mean(1), torch.zeros(2, 4, 5), atol=1e-5)
+    assert list(ln.state_dict()) == ["norm.weight", "norm.bias"]
