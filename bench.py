@@ -1,0 +1,241 @@
+#!/usr/bin/env python3
+"""Benchmark of the NDC update hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bf16|fp32] [--no-cpu]
+
+One step = one forward + one backward (input-, source-, filter- and bias-gradient) of the
+update node on config 3 of the baseline: batch 2, 128 depthwise channels, 64^3 voxels,
+3x3x3 filter, ratio 4, bfloat16 storage with float32 accumulation; inputs resident in HBM.
+Prints ONE JSON line: whole-step throughput in Gvoxel/s, plus a ``roofline`` object for the
+slowest kernel (device time from events on the launch stream, algorithmic bytes as stated
+below) and a ``cpu_baseline`` object (the oracle timed on the host cores on a bounded
+sample of the same workload).
+
+Algorithmic bytes (each compulsory tensor once, re-reads and temporaries zero), with
+U = B*C*D*H*W channel-voxels and e bytes per element:
+    forward      9 U e   (read x, z; write out)
+    backward    14 U e   (read gout, re-read x, z; write gx, gz), attributed to its two
+                          passes as pass 1 = 10 U e (x, z, gout in; gx out) and
+                          pass 2 = 4 U e (gz out; its inputs are re-reads)
+    whole step  23 U e
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+WORKLOAD = dict(batch=2, channels=128, spatial=(64, 64, 64), kernel=(3, 3, 3), ratio=4)
+
+
+def make_inputs(torch, dtype, device, batch, channels, spatial, kernel, ratio, seed=0):
+    """Config-3 style tensors: h = softplus(0.1 N(0,1)) > 0, x = |N(0,1)|, z = W x with the
+    projection's default initialisation (bias withheld: the kernels add it), g = N(0,1)."""
+    import deconver_amd as dc
+
+    torch.manual_seed(seed)
+    layer = dc.Deconv(channels=channels, kernel_size=kernel, ratio=ratio, groups=-1)
+    sc = layer.source_channels
+    h = torch.nn.functional.softplus(0.1 * torch.randn(channels, sc, *kernel))
+    x = torch.randn(batch, channels, *spatial).abs()
+    proj = layer.init.linear.linear
+    x = x.to(device=device, dtype=dtype)
+    w = proj.weight.detach().to(device=device, dtype=dtype)
+    z = torch.nn.functional.conv1d(x.flatten(2), w, None).view(batch, channels * sc, *spatial)
+    torch.manual_seed(seed + 2)
+    g = torch.randn(batch, channels * sc, *spatial).to(device=device, dtype=dtype)
+    bias = proj.bias.detach().float().to(device)
+    return x.contiguous(), z.contiguous(), h.float().to(device).contiguous(), bias, g.contiguous(), sc
+
+
+def cpu_baseline(torch, budget_channels=32):
+    """The oracle (literal restatement of the reference's update, autograd backward) on the
+    host cores, float32, on a channel slice of the workload: depthwise channels are
+    independent, so the rate scales linearly to the full channel count."""
+    from oracle import ndc_oracle as O
+
+    w = WORKLOAD
+    b, c, sp, ks = 1, budget_channels, w["spatial"], w["kernel"]
+    sc = w["ratio"]
+    gen = torch.Generator().manual_seed(0)
+    x = torch.randn(b, c, *sp, generator=gen).abs()
+    s = torch.randn(b, c * sc, *sp, generator=gen).abs()
+    h = torch.nn.functional.softplus(0.1 * torch.randn(c, sc, *ks, generator=gen))
+    g = torch.randn(b, c * sc, *sp, generator=gen)
+    layer = O.OracleNDC(c, ks, ratio=sc)
+
+    def step():
+        xs = layer.split(x.clone().requires_grad_(True))
+        ss = layer.split(s.clone().requires_grad_(True))
+        hs = layer.split(h.clone().requires_grad_(True).expand(b, *h.shape))
+        out = layer.merge(layer.update_s(xs, ss, hs))
+        out.backward(g)
+
+    step()
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        step()
+        times.append(time.perf_counter() - t0)
+    t = statistics.median(times)
+    vox = b * sp[0] * sp[1] * sp[2]
+    # voxels/s this slice sustains, rescaled to the workload's channel count
+    gvox = vox / t / 1e9 * (c / w["channels"])
+    return {
+        "value": gvox,
+        "unit": "Gvoxel/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"oracle update fwd+bwd (autograd), float32, B={b}, {c} of {w['channels']} "
+                  f"depthwise channels, {sp[0]}^3, median of 3 ({t:.2f} s each); rate rescaled "
+                  f"to {w['channels']} channels",
+        "channel_voxels_per_s": vox * c / t,
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--dtype", choices=("bf16", "fp32"), default="bf16")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain 1 GiB device copy (reference point for the "
+                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures the one-GPU hot path only: this build has no multi-GPU code "
+              "path (every box has one GPU); run with --gpus 1", file=sys.stderr)
+        return 2
+
+    import torch
+
+    from deconver_amd import _lib, ops
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (the NDC update has no CPU path)", file=sys.stderr)
+        return 2
+    lib = _lib.get_library()
+    dev = torch.device("cuda:0")
+    dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float32
+    esz = 2 if dtype == torch.bfloat16 else 4
+    w = WORKLOAD
+    x, z, h, bias, g, sc = make_inputs(torch, dtype, dev, w["batch"], w["channels"], w["spatial"],
+                                       w["kernel"], w["ratio"])
+    C = w["channels"]
+    kw = dict(groups=C, m=1, sc=sc, eps=1e-16, relu_input=True)
+    geom = ops.make_geom_for(x, h, C, 1, sc, 1e-16, True)
+    assert lib.fused_supported(geom), "the headline workload must run on the fused kernels"
+
+    def step():
+        out, t1 = ops.update_forward(lib, x, z, h, bias, **kw)
+        return ops.update_backward(lib, x, z, t1, h, bias, g, **kw)
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+
+    # per-kernel device time: events on the stream the library launches on
+    n_probe = max(3, min(10, args.steps))
+    fwd_ms, pass_ms = [], []
+    for _ in range(n_probe):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        out, t1 = ops.update_forward(lib, x, z, h, bias, **kw)
+        e1.record()
+        pt = []
+        ops.update_backward(lib, x, z, t1, h, bias, g, pass_times=pt, **kw)
+        torch.cuda.synchronize()
+        fwd_ms.append(e0.elapsed_time(e1))
+        pass_ms.append(pt)
+    k_ms = {
+        "forward": statistics.mean(fwd_ms),
+        "backward_pass1": statistics.mean(p[0] for p in pass_ms),
+        "backward_pass2": statistics.mean(p[1] for p in pass_ms),
+        "backward_reduce": statistics.mean(p[2] for p in pass_ms),
+    }
+
+    sp = w["spatial"]
+    vox = w["batch"] * sp[0] * sp[1] * sp[2]
+    U = vox * C
+    alg = {"forward": 9 * U * esz, "backward_pass1": 10 * U * esz, "backward_pass2": 4 * U * esz}
+    dominant = max(alg, key=lambda k: k_ms[k])
+    achieved = alg[dominant] / (k_ms[dominant] * 1e-3) / 1e9
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        try:
+            traffic = json.load(open(tpath)).get(args.dtype, {}).get(dominant)
+        except (ValueError, OSError):
+            traffic = None
+    roofline = {
+        "kernel": dominant,
+        "bound": "hbm",
+        "achieved": achieved,
+        "peak": HBM_PEAK_GBS,
+        "unit": "GB/s",
+        "frac": achieved / HBM_PEAK_GBS,
+        "traffic": traffic,
+        "algorithmic_bytes": alg[dominant],
+        "avg_launch_ms": k_ms[dominant],
+    }
+    step_bytes = 23 * U * esz
+    result = {
+        "metric": "NDC mixer fwd+bwd Gvoxel/s",
+        "value": vox / (ms_per_step * 1e-3) / 1e9,
+        "unit": "Gvoxel/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if dtype == torch.bfloat16 else "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "config 3: one NDC source update, 3-D, batch 2, 128 depthwise channels, "
+                        "64^3 voxels, 3x3x3 filter, ratio 4 (512 source channels), "
+                        f"{args.dtype} storage / float32 accumulation; forward + input-, source-, "
+                        "filter- and bias-gradient",
+            "batch": w["batch"], "channels": C, "spatial": list(sp), "kernel": list(w["kernel"]),
+            "ratio": w["ratio"], "num_iters": 1,
+        },
+        "channel_voxels_per_s": U / (ms_per_step * 1e-3),
+        "step_algorithmic_bytes": step_bytes,
+        "step_hbm_frac": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "kernel_ms": k_ms,
+        "roofline": roofline,
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(torch)
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -26,6 +26,7 @@ EXPORTS = (
     "ndc_forward",
     "ndc_backward_workspace_bytes",
     "ndc_backward",
+    "ndc_backward_profiled",
     "ndc_gconv",
 )
 
@@ -84,6 +85,7 @@ class NdcLibrary:
         d.ndc_backward_workspace_bytes.argtypes = [gp] + [ctypes.c_int] * 4
         d.ndc_backward.argtypes = [gp, vp, vp, vp, fp, fp, vp, vp, vp, fp, fp, vp,
                                    ctypes.c_size_t, vp]
+        d.ndc_backward_profiled.argtypes = d.ndc_backward.argtypes + [ctypes.POINTER(ctypes.c_float)]
         d.ndc_gconv.argtypes = [gp, vp, fp, fp, ctypes.c_int, vp, vp]
 
     def _check(self, status: int, what: str) -> None:
@@ -115,6 +117,16 @@ class NdcLibrary:
             self._dll.ndc_backward(ctypes.byref(g), x, z, t1, h, bias, gout, gx, gz, gh, gb, ws,
                                    ws_bytes, stream),
             "ndc_backward")
+
+    def backward_profiled(self, g: Geom, x, z, t1, h, bias, gout, gx, gz, gh, gb, ws, ws_bytes,
+                          stream):
+        """``backward`` plus the device time (ms) of pass 1, pass 2 and the reduction."""
+        ms = (ctypes.c_float * 3)()
+        self._check(
+            self._dll.ndc_backward_profiled(ctypes.byref(g), x, z, t1, h, bias, gout, gx, gz, gh,
+                                            gb, ws, ws_bytes, stream, ms),
+            "ndc_backward_profiled")
+        return tuple(ms)
 
     def gconv(self, g: Geom, inp, h, bias, adjoint: bool, out, stream) -> None:
         self._check(self._dll.ndc_gconv(ctypes.byref(g), inp, h, bias, int(adjoint), out, stream),

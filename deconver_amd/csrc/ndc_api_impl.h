@@ -231,9 +231,9 @@ size_t ndc_backward_workspace_bytes(const ndc_geom *g, int need_gx, int need_gz,
     return direct_backward_ws(q);
 }
 
-int ndc_backward(const ndc_geom *g, const void *x, const void *z, const void *t1, const float *h,
+static int backward_impl(const ndc_geom *g, const void *x, const void *z, const void *t1, const float *h,
                  const float *bias, const void *gout, void *gx, void *gz, float *gh, float *gb,
-                 void *workspace, size_t workspace_bytes, void *stream)
+                 void *workspace, size_t workspace_bytes, void *stream, float *pass_ms)
 {
     using namespace ndc;
     KGeom q;
@@ -252,11 +252,11 @@ int ndc_backward(const ndc_geom *g, const void *x, const void *z, const void *t1
                    ? fused::backward<Backend, float>(q, (const float *)x, (const float *)z,
                                                      (const float *)t1, h, bias,
                                                      (const float *)gout, (float *)gx,
-                                                     (float *)gz, gh, gb, workspace, stream)
+                                                     (float *)gz, gh, gb, workspace, stream, pass_ms)
                    : fused::backward<Backend, bf16_t>(q, (const bf16_t *)x, (const bf16_t *)z,
                                                       (const bf16_t *)t1, h, bias,
                                                       (const bf16_t *)gout, (bf16_t *)gx,
-                                                      (bf16_t *)gz, gh, gb, workspace, stream);
+                                                      (bf16_t *)gz, gh, gb, workspace, stream, pass_ms);
     }
     return g->dtype == NDC_F32
                ? direct_backward<float>(q, (const float *)x, (const float *)z, (const float *)t1,
@@ -265,6 +265,25 @@ int ndc_backward(const ndc_geom *g, const void *x, const void *z, const void *t1
                : direct_backward<bf16_t>(q, (const bf16_t *)x, (const bf16_t *)z,
                                          (const bf16_t *)t1, h, bias, (const bf16_t *)gout,
                                          (bf16_t *)gx, (bf16_t *)gz, gh, gb, workspace, stream);
+}
+
+int ndc_backward(const ndc_geom *g, const void *x, const void *z, const void *t1, const float *h,
+                 const float *bias, const void *gout, void *gx, void *gz, float *gh, float *gb,
+                 void *workspace, size_t workspace_bytes, void *stream)
+{
+    return backward_impl(g, x, z, t1, h, bias, gout, gx, gz, gh, gb, workspace, workspace_bytes,
+                         stream, nullptr);
+}
+
+int ndc_backward_profiled(const ndc_geom *g, const void *x, const void *z, const void *t1,
+                          const float *h, const float *bias, const void *gout, void *gx,
+                          void *gz, float *gh, float *gb, void *workspace,
+                          size_t workspace_bytes, void *stream, float *pass_ms)
+{
+    if (!pass_ms) return NDC_ERR_NULL;
+    pass_ms[0] = pass_ms[1] = pass_ms[2] = 0.f;
+    return backward_impl(g, x, z, t1, h, bias, gout, gx, gz, gh, gb, workspace, workspace_bytes,
+                         stream, pass_ms);
 }
 
 int ndc_gconv(const ndc_geom *g, const void *in, const float *h, const float *bias, int adjoint,

@@ -42,8 +42,41 @@ __global__ void __launch_bounds__(512) block_kernel_entry(typename Kernel::Param
     Kernel::run(ex, p, (int)blockIdx.x);
 }
 
+// Event stopwatch on one stream: mark() after each stage, finish() synchronises and
+// reports the stage durations in milliseconds.
+struct HipTimer {
+    static const int kMax = 8;
+    hipEvent_t ev[kMax + 1];
+    int n = 0;
+    bool on;
+    hipStream_t stream;
+    HipTimer(bool enable, void *s) : on(enable), stream((hipStream_t)s)
+    {
+        if (!on) return;
+        for (int i = 0; i <= kMax; ++i) (void)hipEventCreate(&ev[i]);
+        (void)hipEventRecord(ev[0], stream);
+    }
+    void mark()
+    {
+        if (on && n < kMax) (void)hipEventRecord(ev[++n], stream);
+    }
+    void finish(float *ms, int count)
+    {
+        if (!on) return;
+        (void)hipEventSynchronize(ev[n]);
+        for (int i = 0; i < count; ++i) {
+            ms[i] = 0.f;
+            if (i < n) (void)hipEventElapsedTime(&ms[i], ev[i], ev[i + 1]);
+        }
+        for (int i = 0; i <= kMax; ++i) (void)hipEventDestroy(ev[i]);
+        on = false;
+    }
+    ~HipTimer() { if (on) for (int i = 0; i <= kMax; ++i) (void)hipEventDestroy(ev[i]); }
+};
+
 struct Backend {
     static constexpr bool is_device = true;
+    typedef HipTimer Timer;
 
     template <class Kernel>
     static int block_kernel(const typename Kernel::Params &p, int nblocks, int nthreads,

@@ -156,8 +156,11 @@ static int forward(const KGeom &q, const T *x, const T *z, const float *h, const
 template <class BE, typename T>
 static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const float *h,
                     const float *bias, const T *gout, T *gx, T *gz, float *gh, float *gb,
-                    void *ws, void *stream)
+                    void *ws, void *stream, float *pass_ms = nullptr)
 {
+    // pass_ms (optional, 3 floats): device time of pass 1, pass 2 and the partial-sum
+    // reduction, taken with events on `stream`; makes the call synchronous
+    typename BE::Timer tm(pass_ms != nullptr, stream);
     Plan pl;
     if (!make_plan(q, pl)) return NDC_ERR_GEOMETRY;
     const size_t n_x = (size_t)q.B * q.G * q.SP;
@@ -201,7 +204,11 @@ static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const f
     NDC_FUSED_VARIANTS(X)
 #undef X
     if (st) return st;
-    if (!gz && !gh && !gb) return NDC_OK;
+    tm.mark();
+    if (!gz && !gh && !gb) {
+        tm.finish(pass_ms, 3);
+        return NDC_OK;
+    }
 
     p.part = part2;
     p.part_stride = kt + q.sc;
@@ -214,6 +221,7 @@ static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const f
     NDC_FUSED_VARIANTS(X)
 #undef X
     if (st) return st;
+    tm.mark();
 
     // combine the per-workgroup partial sums: fixed order, so results are reproducible
     const int C = q.G, SC = q.sc, ntile = pl.tb.ntile, B = q.B;
@@ -243,6 +251,8 @@ static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const f
         });
         if (st) return st;
     }
+    tm.mark();
+    tm.finish(pass_ms, 3);
     return NDC_OK;
 }
 

@@ -82,8 +82,11 @@ def update_backward(lib: _lib.NdcLibrary, x: Tensor, z: Tensor, t1: Tensor, h: T
                     bias: Optional[Tensor], gout: Tensor, *, groups: int, m: int, sc: int,
                     eps: float, relu_input: bool, need_x: bool = True, need_z: bool = True,
                     need_h: bool = True, need_b: bool = True,
-                    path: int = _lib.PATH_AUTO):
-    """Gradients ``(gx, gz, gh, gb)`` of the update; entries not asked for are ``None``."""
+                    path: int = _lib.PATH_AUTO, pass_times: Optional[list] = None):
+    """Gradients ``(gx, gz, gh, gb)`` of the update; entries not asked for are ``None``.
+
+    ``pass_times``: a list that, if given, receives the device milliseconds of the three
+    backward stages (the call then synchronises)."""
     _check_common(x, z, h, bias, groups, m, sc)
     if gout.shape != z.shape or gout.dtype != z.dtype or not gout.is_contiguous():
         raise ValueError("gout must be contiguous with the shape and dtype of z")
@@ -98,8 +101,12 @@ def update_backward(lib: _lib.NdcLibrary, x: Tensor, z: Tensor, t1: Tensor, h: T
     nbytes = lib.backward_workspace_bytes(g, need_x, need_z, need_h, need_b)
     ws = torch.empty(max(nbytes, 1) + 256, dtype=torch.uint8, device=x.device)
     ws_ptr = (ws.data_ptr() + 255) // 256 * 256
-    lib.backward(g, _ptr(x), _ptr(z), _ptr(t1), _ptr(h), _ptr(bias), _ptr(gout), _ptr(gx),
-                 _ptr(gz), _ptr(gh), _ptr(gb), ws_ptr, nbytes, _stream_of(x))
+    args = (g, _ptr(x), _ptr(z), _ptr(t1), _ptr(h), _ptr(bias), _ptr(gout), _ptr(gx),
+            _ptr(gz), _ptr(gh), _ptr(gb), ws_ptr, nbytes, _stream_of(x))
+    if pass_times is None:
+        lib.backward(*args)
+    else:
+        pass_times[:] = lib.backward_profiled(*args)
     return gx, gz, gh, gb
 
 

@@ -108,6 +108,19 @@ int ndc_backward(const ndc_geom *g, const void *x, const void *z, const void *t1
                  float *gh, float *gb, void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * ndc_backward with a stopwatch: same arguments and results, plus pass_ms[3] = device time in
+ * milliseconds of (pass 1: gn/gd, gx, gt1, A-side filter terms), (pass 2: gz, gb, K-side
+ * filter term) and (the partial-sum reduction), taken with events on `stream`.  The call
+ * synchronises the host with `stream`.  Measurement aid for the benchmark harness; it has no
+ * counterpart in the reference (its benchmarks time whole calls, benchmarks/bench_deconv.py:109-121).
+ * The direct path is not instrumented and reports zeros.
+ */
+int ndc_backward_profiled(const ndc_geom *g, const void *x, const void *z, const void *t1,
+                          const float *h, const float *bias, const void *gout, void *gx,
+                          void *gz, float *gh, float *gb, void *workspace,
+                          size_t workspace_bytes, void *stream, float *pass_ms);
+
+/*
  * Plain grouped convolution with the same tap conventions (adjoint = 0: K, 1: A), input
  * and output in g->dtype; optional on-load bias + ReLU of the input as in the forward.
  * Replaces kernels.gconv (deconver/deconvolution/kernels.py:728-759); used for

@@ -93,29 +93,67 @@ def test_multiple_iterations(iters):
     _compare(kwargs, 2, (6, 6, 6), tol=5e-4)
 
 
-def test_bf16_autocast_route_and_tolerance():
+class _GeneralRoute(dc.Deconv):
+    """Same layer, forced onto the PyTorch general route (an overridden update method)."""
+
+    def update_s(self, x, s, h):
+        return super().update_s(x, s, h)
+
+
+def test_bf16_autocast_layer_no_further_from_exact_than_pytorch():
+    """Whole layer under bfloat16 autocast (which the reference's fused path declines).  The
+    bf16 projection feeds a rounded z into the update, so neither route is within 2e-2 of a
+    float64 evaluation of the unrounded layer; as in the reference's own network test
+    (test_deconv_equivalence.py:332-379) the HIP route must be no further from exact than
+    the PyTorch route is (x1.5)."""
     kwargs = dict(channels=16, ratio=4, groups=-1, kernel_size=(3, 3, 3))
-    layer = _layer(kwargs)
     torch.manual_seed(1)
     x0 = torch.rand(2, 16, 9, 8, 10)
-    x = x0.cuda().requires_grad_(True)
-    with torch.autocast("cuda", dtype=torch.bfloat16):
-        assert layer.fast_path_applicable(x)
-        y = layer(x)
-    assert y.dtype == torch.bfloat16
-    g = torch.randn(y.shape)
-    y.backward(g.cuda().to(y.dtype))
-    # oracle on the bf16-rounded operands the HIP route saw (x and the projection weight)
-    ref_layer = _layer(kwargs)
-    with torch.no_grad():
-        ref_layer.init.linear.linear.weight.copy_(layer.init.linear.linear.weight.bfloat16().float())
-    yr, gr = _oracle_run(ref_layer, kwargs, x0.bfloat16().float(), g.bfloat16().float())
-    assert O.rel_err(y.detach().float().cpu(), yr) < 2e-2
-    assert x.grad.dtype == torch.float32 and layer.init.h0.grad.dtype == torch.float32
-    assert O.rel_err(x.grad.cpu(), gr["x"]) < 2e-2
-    assert O.rel_err(layer.init.h0.grad.cpu(), gr["h"]) < 2e-2
-    assert O.rel_err(layer.init.linear.linear.bias.grad.cpu(), gr["b"]) < 2e-2
-    assert O.rel_err(layer.init.linear.linear.weight.grad.cpu().squeeze(-1), gr["w"]) < 2e-2
+    g0 = torch.randn(2, 64, 9, 8, 10)
+    errs = {}
+    for name, cls in (("hip", dc.Deconv), ("torch", _GeneralRoute)):
+        torch.manual_seed(0)
+        layer = cls(**kwargs)
+        with torch.no_grad():
+            layer.init.linear.linear.bias.add_(1.0)
+        layer = layer.cuda()
+        x = x0.cuda().requires_grad_(True)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            assert layer.fast_path_applicable(x) == (name == "hip")
+            y = layer(x)
+        assert y.dtype == torch.bfloat16
+        y.backward(g0.cuda().to(y.dtype))
+        assert x.grad.dtype == torch.float32 and layer.init.h0.grad.dtype == torch.float32
+        yr, gr = _oracle_run(layer, kwargs, x0, g0)
+        errs[name] = dict(out=O.rel_err(y.detach().float().cpu(), yr),
+                          x=O.rel_err(x.grad.cpu(), gr["x"]),
+                          h=O.rel_err(layer.init.h0.grad.cpu(), gr["h"]),
+                          b=O.rel_err(layer.init.linear.linear.bias.grad.cpu(), gr["b"]),
+                          w=O.rel_err(layer.init.linear.linear.weight.grad.cpu().squeeze(-1), gr["w"]))
+    for k, e in errs["hip"].items():
+        assert e <= max(1.5 * errs["torch"][k], 2e-2), (k, errs)
+
+
+def test_bf16_update_node_autograd():
+    """The autograd node on bfloat16 tensors: outputs and all four gradients within 2e-2 of
+    the oracle evaluated on the same bf16-valued operands."""
+    gen = torch.Generator().manual_seed(1)
+    C, sc, sp = 16, 4, (9, 8, 10)
+    xb = torch.rand(2, C, *sp, generator=gen).bfloat16()
+    zb = (torch.rand(2, C * sc, *sp, generator=gen) - 0.3).bfloat16()
+    hb = torch.nn.functional.softplus(0.1 * torch.randn(C, sc, 3, 3, 3, generator=gen))
+    bb = 0.2 * torch.rand(C * sc, generator=gen)
+    gb = torch.randn(2, C * sc, *sp, generator=gen).bfloat16()
+    leaves = [t.cuda().requires_grad_(True) for t in (xb, zb, hb, bb)]
+    out = dc.deconv_update(*leaves, groups=C, m=1, sc=sc, eps=1e-16, relu_input=True)
+    out.backward(gb.cuda())
+    d = [t.double() for t in (xb, zb, hb, bb, gb)]
+    ro, _ = O.update_grouped(d[0], d[1], d[2], d[3], C, 1, sc, 1e-16, True)
+    refs = O.update_backward(d[0], d[1], d[2], d[3], d[4], C, 1, sc, 1e-16, True)
+    assert out.dtype == torch.bfloat16 and O.rel_err(out.detach().float().cpu(), ro) < 2e-2
+    assert leaves[0].grad.dtype == torch.bfloat16 and leaves[2].grad.dtype == torch.float32
+    for leaf, ref in zip(leaves, refs):
+        assert O.rel_err(leaf.grad.float().cpu(), ref) < 2e-2
 
 
 def test_partial_gradient_requests():
