@@ -37,15 +37,15 @@ NDC_HD float bf16_to_float(bf16_t v)
 // round-to-nearest-even, NaN kept quiet
 NDC_HD bf16_t float_to_bf16(float f)
 {
-    uint32_t u;
 #if NDC_DEVICE_BUILD && defined(__HIP_DEVICE_COMPILE__)
-    u = __float_as_uint(f);
+    return __builtin_bit_cast(bf16_t, (__bf16)f);   // v_cvt_pk_bf16_f32
 #else
+    uint32_t u;
     memcpy(&u, &f, 4);
-#endif
     if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40u);
     u += 0x7fffu + ((u >> 16) & 1u);
     return (bf16_t)(u >> 16);
+#endif
 }
 
 template <typename T> struct Elem;
@@ -57,6 +57,78 @@ template <> struct Elem<bf16_t> {
     static NDC_HD float load(const bf16_t *p) { return bf16_to_float(*p); }
     static NDC_HD void store(bf16_t *p, float v) { *p = float_to_bf16(v); }
 };
+
+// two floats -> packed bf16 pair (lo in bits 0-15): one v_cvt_pk_bf16_f32 on gfx950
+NDC_HD uint32_t pack_bf16x2(float lo, float hi)
+{
+#if NDC_DEVICE_BUILD && defined(__HIP_DEVICE_COMPILE__)
+    typedef __attribute__((ext_vector_type(2))) float f2_t;
+    typedef __attribute__((ext_vector_type(2))) __bf16 bf2_t;
+    const f2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf2_t));
+#else
+    return (uint32_t)float_to_bf16(lo) | ((uint32_t)float_to_bf16(hi) << 16);
+#endif
+}
+
+NDC_HD float bits_to_float(uint32_t u)
+{
+    float f;
+#if NDC_DEVICE_BUILD && defined(__HIP_DEVICE_COMPILE__)
+    f = __uint_as_float(u);
+#else
+    memcpy(&f, &u, 4);
+#endif
+    return f;
+}
+
+// N consecutive elements <-> N floats with one memory access (N = 1 or 2; the address must
+// be aligned to N elements)
+template <typename T, int N> struct VecIO;
+template <typename T> struct VecIO<T, 1> {
+    static NDC_HD void load(const T *p, float (&v)[1]) { v[0] = Elem<T>::load(p); }
+    static NDC_HD void store(T *p, const float (&v)[1]) { Elem<T>::store(p, v[0]); }
+};
+template <> struct VecIO<float, 2> {
+    struct alignas(8) Pair {
+        float a, b;
+    };
+    static NDC_HD void load(const float *p, float (&v)[2])
+    {
+        const Pair q = *reinterpret_cast<const Pair *>(p);
+        v[0] = q.a;
+        v[1] = q.b;
+    }
+    static NDC_HD void store(float *p, const float (&v)[2])
+    {
+        Pair q;
+        q.a = v[0];
+        q.b = v[1];
+        *reinterpret_cast<Pair *>(p) = q;
+    }
+};
+template <> struct VecIO<bf16_t, 2> {
+    static NDC_HD void load(const bf16_t *p, float (&v)[2])
+    {
+        const uint32_t w = *reinterpret_cast<const uint32_t *>(p);
+        v[0] = bits_to_float(w << 16);
+        v[1] = bits_to_float(w & 0xffff0000u);
+    }
+    static NDC_HD void store(bf16_t *p, const float (&v)[2])
+    {
+        *reinterpret_cast<uint32_t *>(p) = pack_bf16x2(v[0], v[1]);
+    }
+};
+
+// max(v, 0): one v_max_f32 (a compare + select pair otherwise)
+NDC_HD float relu_f(float v)
+{
+#if NDC_DEVICE_BUILD && defined(__HIP_DEVICE_COMPILE__)
+    return __builtin_fmaxf(v, 0.f);
+#else
+    return v > 0.f ? v : 0.f;
+#endif
+}
 
 NDC_HD float fast_rcp(float v)
 {

@@ -3,8 +3,9 @@
 // Work decomposition (all three kernels):
 //   - one workgroup owns one (sample, channel) volume and a band of TH = S*RH output rows
 //     over the FULL width W, and marches along the slowest spatial axis ("planes", k);
-//   - lanes run along W (coalesced global traffic, conflict-free LDS rows); a thread owns
-//     column `col` of row strip `strip` (RH consecutive rows);
+//   - lanes run along W (coalesced global traffic, conflict-free LDS rows); a thread owns a
+//     register tile of RH consecutive rows x RW consecutive columns, and moves its RW
+//     columns with one global access per row (32-bit for bf16 pairs, 64-bit for fp32);
 //   - operands that are read with spatial neighbours live in LDS rings of a few planes
 //     with zero halo columns / rows (so the tap loops carry no bounds checks); operands
 //     that are only read at the thread's own position come straight from global memory;
@@ -49,10 +50,12 @@ namespace fused {
 
 struct Tile {
     int S;       // row strips per workgroup
-    int NT;      // threads per workgroup (multiple of 64, >= S*W)
+    int NT;      // threads per workgroup (multiple of 64, >= S*CPW)
     int TH;      // output rows per workgroup
     int ntile;   // row bands per volume
-    int P;       // LDS row pitch in floats (W + 2*PW)
+    int P;       // LDS row pitch in words
+    int PL;      // zero words to the left of column 0 in an LDS row (>= PW, multiple of RW)
+    int CPW;     // column groups per row = W / RW
 };
 
 // the marching view of a problem: 2-D inputs march along H
@@ -86,22 +89,27 @@ static inline int round_up(int v, int a) { return (v + a - 1) / a * a; }
 static const int kMaxThreads = 512;
 static const int kMaxLdsBytes = 160 * 1024;
 
-// S strips of RH rows; S >= 2*PH so that the halo rows fit the fixed per-thread bounds
-static inline bool make_tile(const March &m, int RH, int target_threads, Tile &t)
+// S strips of RH rows, RW columns per thread; S >= 2*PH so that the halo rows fit the
+// fixed per-thread bounds
+static inline bool make_tile(const March &m, int RH, int RW, int target_threads, Tile &t)
 {
     const int PH = m.KH / 2, PW = m.KW / 2;
-    if (m.W > kMaxThreads) return false;
+    if (m.W % RW) return false;
+    const int cpw = m.W / RW;
+    if (cpw > kMaxThreads) return false;
     int smin = PH > 0 ? 2 * PH : 1;
-    int s = target_threads / m.W;
+    int s = target_threads / cpw;
     const int srows = (m.H + RH - 1) / RH;
     if (s > srows) s = srows;
     if (s < smin) s = smin;
-    if (s * m.W > kMaxThreads) return false;
+    if (s * cpw > kMaxThreads) return false;
     t.S = s;
-    t.NT = round_up(s * m.W, 64);
+    t.CPW = cpw;
+    t.NT = round_up(s * cpw, 64);
     t.TH = s * RH;
     t.ntile = (m.H + t.TH - 1) / t.TH;
-    t.P = m.W + 2 * PW;
+    t.PL = round_up(PW, RW);
+    t.P = round_up(t.PL + m.W + PW, RW);
     return true;
 }
 
@@ -157,34 +165,108 @@ NDC_HD int clampi(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? hi : v
 // is image row r0 - PH + j: the PH rows above the band, then the PH rows below it.
 NDC_HD int halo_row(int s, int PH, int TH) { return s < PH ? s : TH + s; }
 
-// One K-type pass over NR consecutive output rows: `base` addresses, in a staged plane of
-// ONE source channel, the element (first output row, own column - PW); the input rows
-// base .. base + NR + 2*PH - 1 feed the NR output rows, and every tap plane jd of the KD
-// pending output planes.  w = taps of that source channel, (KD, KH, KW) order.
-template <int KD, int KH, int KW, int NR, int STRIDE, class Exec>
-NDC_D void k_rows(Exec &ex, int base, int P, UniformF w, float (*acc)[STRIDE], int r_off)
+// One K-type pass over an NR x RW register tile of outputs.  `base` addresses, in a staged
+// plane of ONE source channel, the word (first input row, first own column - PW); input
+// rows base .. base + NR + KH - 2 feed the NR output rows and every tap plane jd of the KD
+// pending output planes.  w = taps of that source channel in (KD, KH, KW) order.
+template <int KD, int KH, int KW, int NR, int RW, int STRIDE, class Exec>
+NDC_D void k_rows(Exec &ex, int base, int P, const float (&w)[KD * KH * KW],
+                  float (*acc)[STRIDE][RW], int r_off)
 {
     NDC_UNROLL
     for (int q = 0; q < NR + KH - 1; ++q) {
+        float v[RW + KW - 1];
         NDC_UNROLL
-        for (int tw = 0; tw < KW; ++tw) {
-            const float v = ex.ld(base + q * P + tw);
+        for (int u = 0; u < RW + KW - 1; ++u) v[u] = ex.ld(base + q * P + u);
+        NDC_UNROLL
+        for (int th = 0; th < KH; ++th) {
+            const int rr = q - th;
+            if (rr < 0 || rr >= NR) continue;
             NDC_UNROLL
-            for (int th = 0; th < KH; ++th) {
-                const int rr = q - th;
-                if (rr < 0 || rr >= NR) continue;
+            for (int tw = 0; tw < KW; ++tw)
                 NDC_UNROLL
-                for (int jd = 0; jd < KD; ++jd)
-                    acc[jd][r_off + rr] += v * w[((KD - 1 - jd) * KH + th) * KW + tw];
-            }
+                for (int jd = 0; jd < KD; ++jd) {
+                    const float wv = w[((KD - 1 - jd) * KH + th) * KW + tw];
+                    NDC_UNROLL
+                    for (int c = 0; c < RW; ++c) acc[jd][r_off + rr][c] += v[c + tw] * wv;
+                }
         }
     }
 }
 
+// One tap plane of an A-type gather for NT tensors at once over an NR x RW register tile:
+// base[t] addresses, in plane-slot form, the word (first input row, first own column - PW)
+// of tensor t; wt = taps of tap plane td, indexed wt[i][th*KW + tw].
+template <int KH, int KW, int KT, int SC, int NR, int RW, int NTEN, class Exec>
+NDC_D void a_plane(Exec &ex, const int (&base)[NTEN], int P, const float (&wt)[SC][KH * KW],
+                   float (&acc)[NTEN][SC][NR][RW])
+{
+    constexpr int PH = KH / 2;
+    NDC_UNROLL
+    for (int q = 0; q < NR + 2 * PH; ++q) {
+        float v[NTEN][RW + KW - 1];
+        NDC_UNROLL
+        for (int t = 0; t < NTEN; ++t)
+            NDC_UNROLL
+            for (int u = 0; u < RW + KW - 1; ++u) v[t][u] = ex.ld(base[t] + q * P + u);
+        NDC_UNROLL
+        for (int th = 0; th < KH; ++th) {
+            const int rr = q - 2 * PH + th;
+            if (rr < 0 || rr >= NR) continue;
+            NDC_UNROLL
+            for (int tw = 0; tw < KW; ++tw)
+                NDC_UNROLL
+                for (int i = 0; i < SC; ++i) {
+                    const float wv = wt[i][th * KW + tw];
+                    NDC_UNROLL
+                    for (int t = 0; t < NTEN; ++t)
+                        NDC_UNROLL
+                        for (int c = 0; c < RW; ++c) acc[t][i][rr][c] += v[t][c + KW - 1 - tw] * wv;
+                }
+        }
+    }
+}
+
+// Filter slices, fetched one loop iteration ahead so that the scalar loads of the next slice
+// overlap the multiply-adds of the current one.
+template <int N> NDC_D void load_taps(UniformF src, float (&dst)[N])
+{
+    NDC_UNROLL
+    for (int a = 0; a < N; ++a) dst[a] = src[a];
+}
+
+template <int SC, int KT, int N> NDC_D void load_plane_taps(UniformF src, float (&dst)[SC][N])
+{
+    NDC_UNROLL
+    for (int i = 0; i < SC; ++i)
+        NDC_UNROLL
+        for (int a = 0; a < N; ++a) dst[i][a] = src[i * KT + a];
+}
+
+template <int N> NDC_D void copy_taps(const float (&src)[N], float (&dst)[N])
+{
+    NDC_UNROLL
+    for (int a = 0; a < N; ++a) dst[a] = src[a];
+}
+
+// thread coordinates shared by the three kernels
+struct Lane {
+    int strip, c0, active;
+};
+
+NDC_HD Lane make_lane(int tid, const Tile &t, int RW)
+{
+    Lane l;
+    l.strip = tid / t.CPW;
+    l.c0 = (tid - l.strip * t.CPW) * RW;
+    l.active = l.strip < t.S;
+    return l;
+}
+
 // =================================================================== forward
 
-template <int KD_, int KH_, int KW_, int SC_, int RH_, typename T> struct FwdKernel {
-    static constexpr int KD = KD_, KH = KH_, KW = KW_, SC = SC_, RH = RH_;
+template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> struct FwdKernel {
+    static constexpr int KD = KD_, KH = KH_, KW = KW_, SC = SC_, RH = RH_, RW = RW_;
     static constexpr int PD = KD / 2, PH = KH / 2, PW = KW / 2, KT = KD * KH * KW;
     static constexpr int XT = PH > 0 ? 1 : 0;            // one extra halo row for strips < 2*PH
     static constexpr int RHK = RH + XT;
@@ -192,12 +274,16 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, typename T> struct FwdKer
     static constexpr int NXR = RH + (PH > 0 ? 1 : 0);    // rows of x a thread stages
     static constexpr int XR = KD + 1;                    // x ring slots
     typedef FwdParams<T> Params;
+    typedef VecIO<T, RW> IO;
 
     struct State {
-        int strip, col, active;
-        float t1acc[KD][RHK];
-        float pz[SC][NZR];
-        float px[NXR];
+        Lane ln;
+        int zoff[NZR], xoff[NXR], ooff[RH];   // element offsets inside one plane (rows clamped)
+        unsigned zok, xok, ook;               // bit n: that row is inside the image
+        float bv[SC];
+        float t1acc[KD][RHK][RW];
+        float pz[SC][NZR][RW];
+        float px[NXR][RW];
     };
 
     // tile rows: s has TH + 4*PH (row j = image r0 - 2*PH + j); x and t1 have TH + 2*PH
@@ -213,18 +299,17 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, typename T> struct FwdKer
     {
         const Tile t = p.t;
         const BlockId id = decode_block(block_id, p.C, t);
-        const int S = t.S, P = t.P, TH = t.TH, W = p.W, H = p.H, D = p.D;
+        const int S = t.S, P = t.P, PL = t.PL, TH = t.TH, W = p.W, H = p.H, D = p.D;
         const int RS = rows_s(TH), RX = rows_x(TH);
         const int off_s = 0, off_x = SC * RS * P, off_t = off_x + XR * RX * P;
         const int total = off_t + KD * RX * P;
-        const long long plane = (long long)H * W;
+        const int plane = H * W;
         const long long cplane = (long long)D * plane;   // one channel volume
         const T *xg = p.x + ((long long)id.b * p.C + id.c) * cplane;
         const T *zg = p.z + ((long long)id.b * p.C + id.c) * SC * cplane;
         T *og = p.out + ((long long)id.b * p.C + id.c) * SC * cplane;
         T *t1g = p.t1 ? p.t1 + ((long long)id.b * p.C + id.c) * cplane : nullptr;
         UniformF hw = as_uniform(p.h + (long long)id.c * SC * KT);
-        UniformF bias = as_uniform(p.bias ? p.bias + id.c * SC : nullptr);
         const int r0 = id.r0;
         const int nthreads = ex.nthreads;
         const int relu = p.relu;
@@ -233,72 +318,102 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, typename T> struct FwdKer
         // global -> registers: plane k of s (bias / ReLU applied) and plane k - PD of x.
         // Rows outside the image read a clamped address and are zeroed by a select.
         auto load_plane = [&](State &st, int k) {
-            if (!st.active) return;
+            if (!st.ln.active) return;
             if (k < D) {
                 const T *zk = zg + (long long)k * plane;
                 NDC_UNROLL
                 for (int n = 0; n < NZR; ++n) {
-                    const int j = st.strip + n * S, row = r0 - 2 * PH + j;
-                    const bool ok = j < RS && row >= 0 && row < H;
-                    const int o = clampi(row, 0, H - 1) * W + st.col;
                     NDC_UNROLL
                     for (int i = 0; i < SC; ++i) {
-                        float v = Elem<T>::load(zk + i * cplane + o) + (bias ? bias[i] : 0.f);
-                        if (relu) v = v > 0.f ? v : 0.f;
-                        st.pz[i][n] = ok ? v : 0.f;
+                        float v[RW];
+                        IO::load(zk + i * cplane + st.zoff[n], v);
+                        NDC_UNROLL
+                        for (int c = 0; c < RW; ++c) {
+                            float s = v[c] + st.bv[i];
+                            if (relu) s = relu_f(s);
+                            st.pz[i][n][c] = s;
+                        }
                     }
                 }
             } else {
                 NDC_UNROLL
                 for (int n = 0; n < NZR; ++n)
                     NDC_UNROLL
-                    for (int i = 0; i < SC; ++i) st.pz[i][n] = 0.f;
+                    for (int i = 0; i < SC; ++i)
+                        NDC_UNROLL
+                        for (int c = 0; c < RW; ++c) st.pz[i][n][c] = 0.f;
             }
             const int kx = k - PD;
             if (kx >= 0 && kx < D) {
                 const T *xk = xg + (long long)kx * plane;
                 NDC_UNROLL
-                for (int n = 0; n < NXR; ++n) {
-                    const int j = st.strip + n * S, row = r0 - PH + j;
-                    const bool ok = j < RX && row >= 0 && row < H;
-                    const float v = Elem<T>::load(xk + clampi(row, 0, H - 1) * W + st.col);
-                    st.px[n] = ok ? v : 0.f;
-                }
+                for (int n = 0; n < NXR; ++n) IO::load(xk + st.xoff[n], st.px[n]);
             } else {
                 NDC_UNROLL
-                for (int n = 0; n < NXR; ++n) st.px[n] = 0.f;
+                for (int n = 0; n < NXR; ++n)
+                    NDC_UNROLL
+                    for (int c = 0; c < RW; ++c) st.px[n][c] = 0.f;
             }
         };
 
         auto store_plane = [&](State &st, int k) {
-            if (!st.active) return;
+            if (!st.ln.active) return;
+            const int lb = PL + st.ln.c0;
+            // rows outside the image are never written: they keep the zeros of the set-up
             NDC_UNROLL
             for (int n = 0; n < NZR; ++n) {
-                const int j = st.strip + n * S;
-                if (j < RS) {
+                const int j = st.ln.strip + n * S;
+                if ((st.zok >> n) & 1u) {
                     NDC_UNROLL
                     for (int i = 0; i < SC; ++i)
-                        ex.st_(off_s + (i * RS + j) * P + PW + st.col, st.pz[i][n]);
+                        NDC_UNROLL
+                        for (int c = 0; c < RW; ++c)
+                            ex.st_(off_s + (i * RS + j) * P + lb + c, st.pz[i][n][c]);
                 }
             }
             const int slot = wrap((k - PD) % XR, XR);
             NDC_UNROLL
             for (int n = 0; n < NXR; ++n) {
-                const int j = st.strip + n * S;
-                if (j < RX) ex.st_(off_x + (slot * RX + j) * P + PW + st.col, st.px[n]);
+                const int j = st.ln.strip + n * S;
+                if ((st.xok >> n) & 1u) {
+                    NDC_UNROLL
+                    for (int c = 0; c < RW; ++c)
+                        ex.st_(off_x + (slot * RX + j) * P + lb + c, st.px[n][c]);
+                }
             }
         };
 
-        // ---- set-up: thread coordinates, zeroed accumulators, zeroed LDS (halo columns and
-        //      never-staged rows stay zero for the whole march)
+        // ---- set-up: thread coordinates, row offsets, zeroed accumulators, zeroed LDS (halo
+        //      columns and never-staged rows stay zero for the whole march)
         ex.each([&](State &st, int tid) {
-            st.strip = tid / W;
-            st.col = tid - st.strip * W;
-            st.active = st.strip < S;
+            st.ln = make_lane(tid, t, RW);
+            st.zok = st.xok = st.ook = 0u;
+            NDC_UNROLL
+            for (int n = 0; n < NZR; ++n) {
+                const int j = st.ln.strip + n * S, row = r0 - 2 * PH + j;
+                if (j < RS && row >= 0 && row < H) st.zok |= 1u << n;
+                st.zoff[n] = clampi(row, 0, H - 1) * W + st.ln.c0;
+            }
+            NDC_UNROLL
+            for (int n = 0; n < NXR; ++n) {
+                const int j = st.ln.strip + n * S, row = r0 - PH + j;
+                if (j < RX && row >= 0 && row < H) st.xok |= 1u << n;
+                st.xoff[n] = clampi(row, 0, H - 1) * W + st.ln.c0;
+            }
+            NDC_UNROLL
+            for (int r = 0; r < RH; ++r) {
+                const int row = r0 + st.ln.strip * RH + r;
+                if (row < H) st.ook |= 1u << r;
+                st.ooff[r] = clampi(row, 0, H - 1) * W + st.ln.c0;
+            }
+            NDC_UNROLL
+            for (int i = 0; i < SC; ++i) st.bv[i] = p.bias ? p.bias[id.c * SC + i] : 0.f;
             NDC_UNROLL
             for (int a = 0; a < KD; ++a)
                 NDC_UNROLL
-                for (int r = 0; r < RHK; ++r) st.t1acc[a][r] = 0.f;
+                for (int r = 0; r < RHK; ++r)
+                    NDC_UNROLL
+                    for (int c = 0; c < RW; ++c) st.t1acc[a][r][c] = 0.f;
             for (int i = tid; i < total; i += nthreads) ex.st_(i, 0.f);
             load_plane(st, 0);
         });
@@ -310,99 +425,111 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, typename T> struct FwdKer
 
             // ---- K-scatter: plane k of s feeds the KD pending planes of t1
             ex.each([&](State &st, int) {
-                if (!st.active) return;
-                const bool extra = XT && st.strip < 2 * PH;
-                const int jx = halo_row(st.strip, PH, TH);
+                if (!st.ln.active) return;
+#ifdef NDC_EXP_NOEXTRA
+                const bool extra = false;
+#else
+                const bool extra = XT && st.ln.strip < 2 * PH;
+#endif
+                const int jx = halo_row(st.ln.strip, PH, TH);
+                const int cb = PL + st.ln.c0 - PW;
                 if (k < D) {
+                    float wi[KT], wn[KT];
+                    load_taps<KT>(hw, wi);
                     NDC_ROLLED
                     for (int i = 0; i < SC; ++i) {
-                        UniformF wi = hw + i * KT;
-                        const int sb = off_s + i * RS * P + st.col;
-                        k_rows<KD, KH, KW, RH, RHK>(ex, sb + (PH + st.strip * RH) * P, P, wi, st.t1acc, 0);
-                        if (extra) k_rows<KD, KH, KW, 1, RHK>(ex, sb + jx * P, P, wi, st.t1acc, RH);
+                        load_taps<KT>(hw + (i + 1 < SC ? i + 1 : 0) * KT, wn);
+                        const int sb = off_s + i * RS * P + cb;
+                        k_rows<KD, KH, KW, RH, RW, RHK>(ex, sb + (PH + st.ln.strip * RH) * P, P, wi,
+                                                        st.t1acc, 0);
+                        if (extra) k_rows<KD, KH, KW, 1, RW, RHK>(ex, sb + jx * P, P, wi, st.t1acc, RH);
+                        copy_taps<KT>(wn, wi);
                     }
                 }
                 // plane k - PD of t1 is complete: publish it (zero outside the volume)
                 const int pf = k - PD;
                 const bool inplane = pf >= 0 && pf < D;
-                const int tb = off_t + wrap(pf % KD, KD) * RX * P + PW + st.col;
+                const int tb = off_t + wrap(pf % KD, KD) * RX * P + PL + st.ln.c0;
                 NDC_UNROLL
                 for (int r = 0; r < RHK; ++r) {
                     const bool mine = r < RH || extra;
-                    const int j = r < RH ? PH + st.strip * RH + r : jx;
+                    const int j = r < RH ? PH + st.ln.strip * RH + r : jx;
                     const int row = r0 - PH + j;
                     const bool live = inplane && row >= 0 && row < H;
-                    const float v = live ? st.t1acc[0][r] : 0.f;
-                    if (mine) ex.st_(tb + j * P, v);
-                    if (r < RH && t1g && live)
-                        Elem<T>::store(t1g + (long long)pf * plane + row * W + st.col, v);
+                    float v[RW];
                     NDC_UNROLL
-                    for (int a = 0; a + 1 < KD; ++a) st.t1acc[a][r] = st.t1acc[a + 1][r];
-                    st.t1acc[KD - 1][r] = 0.f;
+                    for (int c = 0; c < RW; ++c) {
+                        v[c] = live ? st.t1acc[0][r][c] : 0.f;
+                        if (mine) ex.st_(tb + j * P + c, v[c]);
+                    }
+                    if (r < RH && t1g && live) IO::store(t1g + (long long)pf * plane + st.ooff[r < RH ? r : 0], v);
+                    NDC_UNROLL
+                    for (int c = 0; c < RW; ++c) {
+                        NDC_UNROLL
+                        for (int a = 0; a + 1 < KD; ++a) st.t1acc[a][r][c] = st.t1acc[a + 1][r][c];
+                        st.t1acc[KD - 1][r][c] = 0.f;
+                    }
                 }
             });
+#ifndef NDC_EXP_NOSYNC2
             ex.sync();
+#endif
 
             // ---- prefetch of the next plane, then A-gather + epilogue for plane k - 2*PD
             ex.each([&](State &st, int) {
-                if (!st.active) return;
+                if (!st.ln.active) return;
                 load_plane(st, k + 1);
                 const int j0 = k - 2 * PD;
                 if (j0 < 0) return;
                 // the thread's own source values: re-read from global (an L2 hit) rather
                 // than carried in registers across 2*PD planes
-                float sv[SC][RH];
+                float sv[SC][RH][RW];
                 const T *zk = zg + (long long)j0 * plane;
                 NDC_UNROLL
-                for (int r = 0; r < RH; ++r) {
-                    const int row = r0 + st.strip * RH + r;
-                    const int o = clampi(row, 0, H - 1) * W + st.col;
+                for (int r = 0; r < RH; ++r)
                     NDC_UNROLL
                     for (int i = 0; i < SC; ++i) {
-                        float v = Elem<T>::load(zk + i * cplane + o) + (bias ? bias[i] : 0.f);
-                        if (relu) v = v > 0.f ? v : 0.f;
-                        sv[i][r] = v;
+                        IO::load(zk + i * cplane + st.ooff[r], sv[i][r]);
+                        NDC_UNROLL
+                        for (int c = 0; c < RW; ++c) {
+                            float s = sv[i][r][c] + st.bv[i];
+                            if (relu) s = relu_f(s);
+                            sv[i][r][c] = s;
+                        }
                     }
-                }
-                float an[SC][RH], ad[SC][RH];
+                float acc[2][SC][RH][RW];
                 NDC_UNROLL
-                for (int i = 0; i < SC; ++i)
+                for (int a = 0; a < 2; ++a)
                     NDC_UNROLL
-                    for (int r = 0; r < RH; ++r) an[i][r] = ad[i][r] = 0.f;
+                    for (int i = 0; i < SC; ++i)
+                        NDC_UNROLL
+                        for (int r = 0; r < RH; ++r)
+                            NDC_UNROLL
+                            for (int c = 0; c < RW; ++c) acc[a][i][r][c] = 0.f;
+                float wt[SC][KH * KW], wn[SC][KH * KW];
+                load_plane_taps<SC, KT, KH * KW>(hw, wt);
                 NDC_ROLLED
                 for (int td = 0; td < KD; ++td) {
+                    load_plane_taps<SC, KT, KH * KW>(hw + (td + 1 < KD ? td + 1 : 0) * KH * KW, wn);
                     const int pl = j0 + PD - td;
-                    const int ob = (st.strip * RH) * P + st.col + 2 * PW;
-                    const int bx = off_x + wrap(pl % XR, XR) * RX * P + ob;
-                    const int bt = off_t + wrap(pl % KD, KD) * RX * P + ob;
-                    UniformF wt = hw + td * KH * KW;
+                    const int ob = (st.ln.strip * RH) * P + PL + st.ln.c0 - PW;
+                    const int base[2] = {off_x + wrap(pl % XR, XR) * RX * P + ob,
+                                         off_t + wrap(pl % KD, KD) * RX * P + ob};
+                    a_plane<KH, KW, KT, SC, RH, RW, 2>(ex, base, P, wt, acc);
                     NDC_UNROLL
-                    for (int q = 0; q < RH + 2 * PH; ++q)
-                        NDC_UNROLL
-                        for (int tw = 0; tw < KW; ++tw) {
-                            const float vx = ex.ld(bx + q * P - tw), vt = ex.ld(bt + q * P - tw);
-                            NDC_UNROLL
-                            for (int th = 0; th < KH; ++th) {
-                                const int rr = q - 2 * PH + th;
-                                if (rr < 0 || rr >= RH) continue;
-                                NDC_UNROLL
-                                for (int i = 0; i < SC; ++i) {
-                                    const float wv = wt[i * KT + th * KW + tw];
-                                    an[i][rr] += vx * wv;
-                                    ad[i][rr] += vt * wv;
-                                }
-                            }
-                        }
+                    for (int i = 0; i < SC; ++i) copy_taps<KH * KW>(wn[i], wt[i]);
                 }
                 T *ok_ = og + (long long)j0 * plane;
                 NDC_UNROLL
                 for (int r = 0; r < RH; ++r) {
-                    const int row = r0 + st.strip * RH + r;
-                    if (row >= H) continue;
+                    if (!((st.ook >> r) & 1u)) continue;
                     NDC_UNROLL
                     for (int i = 0; i < SC; ++i) {
-                        const float v = sv[i][r] * (an[i][r] + eps) * fast_rcp(ad[i][r] + eps);
-                        Elem<T>::store(ok_ + i * cplane + row * W + st.col, v);
+                        float v[RW];
+                        NDC_UNROLL
+                        for (int c = 0; c < RW; ++c)
+                            v[c] = sv[i][r][c] * (acc[0][i][r][c] + eps) * fast_rcp(acc[1][i][r][c] + eps);
+                        IO::store(ok_ + i * cplane + st.ooff[r], v);
                     }
                 }
             });
@@ -412,21 +539,25 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, typename T> struct FwdKer
 
 // =================================================================== backward, pass 1
 
-template <int KD_, int KH_, int KW_, int SC_, int RH_, typename T> struct Bwd1Kernel {
-    static constexpr int KD = KD_, KH = KH_, KW = KW_, SC = SC_, RH = RH_;
+template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> struct Bwd1Kernel {
+    static constexpr int KD = KD_, KH = KH_, KW = KW_, SC = SC_, RH = RH_, RW = RW_;
     static constexpr int PD = KD / 2, PH = KH / 2, PW = KW / 2, KT = KD * KH * KW;
     static constexpr int XT = PH > 0 ? 1 : 0;
     static constexpr int NXR = RH + (PH > 0 ? 2 : 0);   // rows of x/t1 a thread stages
     static constexpr int XR = KD + 1;
     static constexpr int NRED = SC * KT;
     typedef BwdParams<T> Params;
+    typedef VecIO<T, RW> IO;
 
     struct State {
-        int strip, col, active;
-        float gacc[SC][KT];      // A-side filter-gradient terms
-        float accx[KD][RH];      // pending planes of gx
-        float acct[KD][RH];      // pending planes of gt1
-        float px[NXR], pt[NXR];
+        Lane ln;
+        int xoff[NXR], ooff[RH];
+        unsigned xok, ook;
+        float bv[SC];
+        float gacc[SC][KT];          // A-side filter-gradient terms
+        float accx[KD][RH][RW];      // pending planes of gx
+        float acct[KD][RH][RW];      // pending planes of gt1
+        float px[NXR][RW], pt[NXR][RW];
     };
 
     // tile rows: x / t1 have TH + 4*PH (row j = image r0 - 2*PH + j); gn / gd have
@@ -440,39 +571,15 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, typename T> struct Bwd1Ke
         return main_ > red ? main_ : red;
     }
 
-    // n, d (numerator / denominator sums) of NR rows whose first x/t1 tile row is `base`
-    template <int NR, class Exec>
-    static NDC_D void gather_nd(Exec &ex, int bx, int bt, int P, UniformF wt,
-                                float (&an)[SC][NR], float (&ad)[SC][NR])
-    {
-        NDC_UNROLL
-        for (int q = 0; q < NR + 2 * PH; ++q)
-            NDC_UNROLL
-            for (int tw = 0; tw < KW; ++tw) {
-                const float vx = ex.ld(bx + q * P - tw), vt = ex.ld(bt + q * P - tw);
-                NDC_UNROLL
-                for (int th = 0; th < KH; ++th) {
-                    const int rr = q - 2 * PH + th;
-                    if (rr < 0 || rr >= NR) continue;
-                    NDC_UNROLL
-                    for (int i = 0; i < SC; ++i) {
-                        const float wv = wt[i * KT + th * KW + tw];
-                        an[i][rr] += vx * wv;
-                        ad[i][rr] += vt * wv;
-                    }
-                }
-            }
-    }
-
     template <class Exec> static NDC_D void run(Exec &ex, const Params &p, int block_id)
     {
         const Tile t = p.t;
         const BlockId id = decode_block(block_id, p.C, t);
-        const int S = t.S, P = t.P, TH = t.TH, W = p.W, H = p.H, D = p.D;
+        const int S = t.S, P = t.P, PL = t.PL, TH = t.TH, W = p.W, H = p.H, D = p.D;
         const int RX = rows_x(TH), RG = rows_g(TH);
         const int off_x = 0, off_t = XR * RX * P, off_g = 2 * XR * RX * P;
         const int total = off_g + 2 * SC * RG * P;
-        const long long plane = (long long)H * W;
+        const int plane = H * W;
         const long long cplane = (long long)D * plane;
         const long long cbase = ((long long)id.b * p.C + id.c) * cplane;
         const T *xg = p.x + cbase, *t1g = p.t1 + cbase;
@@ -480,7 +587,6 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, typename T> struct Bwd1Ke
         T *gxg = p.gx ? p.gx + cbase : nullptr;
         T *gt1g = p.gt1 + cbase;
         UniformF hw = as_uniform(p.h + (long long)id.c * SC * KT);
-        UniformF bias = as_uniform(p.bias ? p.bias + id.c * SC : nullptr);
         const int r0 = id.r0;
         const int nthreads = ex.nthreads;
         const int relu = p.relu;
@@ -488,92 +594,127 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, typename T> struct Bwd1Ke
         const int need_gh = p.need_gh;
 
         auto load_plane = [&](State &st, int k) {
-            if (!st.active) return;
+            if (!st.ln.active) return;
             if (k < D) {
                 const long long ko = (long long)k * plane;
                 NDC_UNROLL
                 for (int n = 0; n < NXR; ++n) {
-                    const int j = st.strip + n * S, row = r0 - 2 * PH + j;
-                    const bool ok = j < RX && row >= 0 && row < H;
-                    const long long o = ko + clampi(row, 0, H - 1) * W + st.col;
-                    const float vx = Elem<T>::load(xg + o), vt = Elem<T>::load(t1g + o);
-                    st.px[n] = ok ? vx : 0.f;
-                    st.pt[n] = ok ? vt : 0.f;
+                    IO::load(xg + ko + st.xoff[n], st.px[n]);
+                    IO::load(t1g + ko + st.xoff[n], st.pt[n]);
                 }
             } else {
                 NDC_UNROLL
-                for (int n = 0; n < NXR; ++n) st.px[n] = st.pt[n] = 0.f;
+                for (int n = 0; n < NXR; ++n)
+                    NDC_UNROLL
+                    for (int c = 0; c < RW; ++c) st.px[n][c] = st.pt[n][c] = 0.f;
             }
         };
         auto store_plane = [&](State &st, int k) {
-            if (!st.active) return;
+            if (!st.ln.active) return;
             const int slot = wrap(k % XR, XR);
+            // rows outside the image are never written: they keep the zeros of the set-up
             NDC_UNROLL
             for (int n = 0; n < NXR; ++n) {
-                const int j = st.strip + n * S;
-                if (j < RX) {
-                    ex.st_(off_x + (slot * RX + j) * P + PW + st.col, st.px[n]);
-                    ex.st_(off_t + (slot * RX + j) * P + PW + st.col, st.pt[n]);
+                const int j = st.ln.strip + n * S;
+                if ((st.xok >> n) & 1u) {
+                    NDC_UNROLL
+                    for (int c = 0; c < RW; ++c) {
+                        const int o = (slot * RX + j) * P + PL + st.ln.c0 + c;
+                        ex.st_(off_x + o, st.px[n][c]);
+                        ex.st_(off_t + o, st.pt[n][c]);
+                    }
                 }
             }
         };
 
-        // gn, gd of NR rows starting at gn/gd tile row j; published to LDS; returned in an/ad
-        auto gn_gd_rows = [&](State &st, int j1, int j, auto nr_tag, float (&an)[SC][decltype(nr_tag)::value],
-                              float (&ad)[SC][decltype(nr_tag)::value]) {
+        // gn, gd of NR rows starting at gn/gd tile row j (image row r0 - PH + j): computed,
+        // published to LDS, and returned in acc[0] / acc[1]
+        auto gn_gd_rows = [&](State &st, int j1, int j, auto nr_tag,
+                              float (&acc)[2][SC][decltype(nr_tag)::value][RW]) {
             constexpr int NR = decltype(nr_tag)::value;
-            float sv[SC][NR], gv[SC][NR];
+            float sv[SC][NR][RW], gv[SC][NR][RW];
             const long long ko = (long long)j1 * plane;
             NDC_UNROLL
             for (int r = 0; r < NR; ++r) {
                 const int row = r0 - PH + j + r;
                 const bool ok = row >= 0 && row < H;
-                const long long o = ko + clampi(row, 0, H - 1) * W + st.col;
+                const int o = clampi(row, 0, H - 1) * W + st.ln.c0;
                 NDC_UNROLL
                 for (int i = 0; i < SC; ++i) {
-                    float s = Elem<T>::load(zg + i * cplane + o) + (bias ? bias[i] : 0.f);
-                    if (relu) s = s > 0.f ? s : 0.f;
-                    const float g = Elem<T>::load(gg + i * cplane + o);
-                    sv[i][r] = s;
-                    gv[i][r] = ok ? g : 0.f;
+                    IO::load(zg + i * cplane + ko + o, sv[i][r]);
+                    IO::load(gg + i * cplane + ko + o, gv[i][r]);
+                    NDC_UNROLL
+                    for (int c = 0; c < RW; ++c) {
+                        float s = sv[i][r][c] + st.bv[i];
+                        if (relu) s = relu_f(s);
+                        sv[i][r][c] = s;
+                        gv[i][r][c] = ok ? gv[i][r][c] : 0.f;
+                    }
                 }
             }
             NDC_UNROLL
-            for (int i = 0; i < SC; ++i)
+            for (int a = 0; a < 2; ++a)
                 NDC_UNROLL
-                for (int r = 0; r < NR; ++r) an[i][r] = ad[i][r] = 0.f;
+                for (int i = 0; i < SC; ++i)
+                    NDC_UNROLL
+                    for (int r = 0; r < NR; ++r)
+                        NDC_UNROLL
+                        for (int c = 0; c < RW; ++c) acc[a][i][r][c] = 0.f;
+            float wt[SC][KH * KW], wn[SC][KH * KW];
+            load_plane_taps<SC, KT, KH * KW>(hw, wt);
             NDC_ROLLED
             for (int td = 0; td < KD; ++td) {
+                load_plane_taps<SC, KT, KH * KW>(hw + (td + 1 < KD ? td + 1 : 0) * KH * KW, wn);
                 const int slot = wrap((j1 + PD - td) % XR, XR);
-                const int ob = (slot * RX + j) * P + st.col + 2 * PW;
-                gather_nd<NR>(ex, off_x + ob, off_t + ob, P, hw + td * KH * KW, an, ad);
+                const int ob = (slot * RX + j) * P + PL + st.ln.c0 - PW;
+                const int base[2] = {off_x + ob, off_t + ob};
+                a_plane<KH, KW, KT, SC, NR, RW, 2>(ex, base, P, wt, acc);
+                NDC_UNROLL
+                for (int i = 0; i < SC; ++i) copy_taps<KH * KW>(wn[i], wt[i]);
             }
             NDC_UNROLL
             for (int r = 0; r < NR; ++r)
                 NDC_UNROLL
-                for (int i = 0; i < SC; ++i) {
-                    const float inv = fast_rcp(ad[i][r] + eps);
-                    const float gn = gv[i][r] * sv[i][r] * inv;
-                    const float gd = -(gn * (an[i][r] + eps)) * inv;
-                    ex.st_(off_g + (i * RG + j + r) * P + PW + st.col, gn);
-                    ex.st_(off_g + ((SC + i) * RG + j + r) * P + PW + st.col, gd);
-                    an[i][r] = gn;
-                    ad[i][r] = gd;
-                }
+                for (int i = 0; i < SC; ++i)
+                    NDC_UNROLL
+                    for (int c = 0; c < RW; ++c) {
+                        const float inv = fast_rcp(acc[1][i][r][c] + eps);
+                        const float gn = gv[i][r][c] * sv[i][r][c] * inv;
+                        const float gd = -(gn * (acc[0][i][r][c] + eps)) * inv;
+                        ex.st_(off_g + (i * RG + j + r) * P + PL + st.ln.c0 + c, gn);
+                        ex.st_(off_g + ((SC + i) * RG + j + r) * P + PL + st.ln.c0 + c, gd);
+                        acc[0][i][r][c] = gn;
+                        acc[1][i][r][c] = gd;
+                    }
         };
 
         ex.each([&](State &st, int tid) {
-            st.strip = tid / W;
-            st.col = tid - st.strip * W;
-            st.active = st.strip < S;
+            st.ln = make_lane(tid, t, RW);
+            st.xok = st.ook = 0u;
             NDC_UNROLL
-            for (int i = 0; i < SC; ++i)
+            for (int n = 0; n < NXR; ++n) {
+                const int j = st.ln.strip + n * S, row = r0 - 2 * PH + j;
+                if (j < RX && row >= 0 && row < H) st.xok |= 1u << n;
+                st.xoff[n] = clampi(row, 0, H - 1) * W + st.ln.c0;
+            }
+            NDC_UNROLL
+            for (int r = 0; r < RH; ++r) {
+                const int row = r0 + st.ln.strip * RH + r;
+                if (row < H) st.ook |= 1u << r;
+                st.ooff[r] = clampi(row, 0, H - 1) * W + st.ln.c0;
+            }
+            NDC_UNROLL
+            for (int i = 0; i < SC; ++i) {
+                st.bv[i] = p.bias ? p.bias[id.c * SC + i] : 0.f;
                 NDC_UNROLL
                 for (int a = 0; a < KT; ++a) st.gacc[i][a] = 0.f;
+            }
             NDC_UNROLL
             for (int a = 0; a < KD; ++a)
                 NDC_UNROLL
-                for (int r = 0; r < RH; ++r) st.accx[a][r] = st.acct[a][r] = 0.f;
+                for (int r = 0; r < RH; ++r)
+                    NDC_UNROLL
+                    for (int c = 0; c < RW; ++c) st.accx[a][r][c] = st.acct[a][r][c] = 0.f;
             for (int i = tid; i < total; i += nthreads) ex.st_(i, 0.f);
             load_plane(st, 0);
         });
@@ -587,72 +728,84 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, typename T> struct Bwd1Ke
             const int j1 = k - PD;
             const bool live1 = j1 >= 0 && j1 < D;
             ex.each([&](State &st, int) {
-                if (!st.active || !live1) return;
+                if (!st.ln.active || !live1) return;
                 {
-                    float an[SC][RH], ad[SC][RH];
-                    const int j = PH + st.strip * RH;
-                    gn_gd_rows(st, j1, j, IntTag<RH>(), an, ad);
+                    float acc[2][SC][RH][RW];
+                    const int j = PH + st.ln.strip * RH;
+                    gn_gd_rows(st, j1, j, IntTag<RH>(), acc);
                     if (need_gh) {
                         // own rows: A-side filter-gradient terms, re-reading the x / t1 windows
                         NDC_UNROLL
                         for (int td = 0; td < KD; ++td) {
                             const int slot = wrap((j1 + PD - td) % XR, XR);
-                            const int ob = (slot * RX + j) * P + st.col + 2 * PW;
+                            const int ob = (slot * RX + j) * P + PL + st.ln.c0 - PW;
                             NDC_UNROLL
-                            for (int q = 0; q < RH + 2 * PH; ++q)
+                            for (int q = 0; q < RH + 2 * PH; ++q) {
+                                float vx[RW + KW - 1], vt[RW + KW - 1];
                                 NDC_UNROLL
-                                for (int tw = 0; tw < KW; ++tw) {
-                                    const float vx = ex.ld(off_x + ob + q * P - tw);
-                                    const float vt = ex.ld(off_t + ob + q * P - tw);
+                                for (int u = 0; u < RW + KW - 1; ++u) {
+                                    vx[u] = ex.ld(off_x + ob + q * P + u);
+                                    vt[u] = ex.ld(off_t + ob + q * P + u);
+                                }
+                                NDC_UNROLL
+                                for (int th = 0; th < KH; ++th) {
+                                    const int rr = q - 2 * PH + th;
+                                    if (rr < 0 || rr >= RH) continue;
                                     NDC_UNROLL
-                                    for (int th = 0; th < KH; ++th) {
-                                        const int rr = q - 2 * PH + th;
-                                        if (rr < 0 || rr >= RH) continue;
+                                    for (int tw = 0; tw < KW; ++tw)
                                         NDC_UNROLL
                                         for (int i = 0; i < SC; ++i)
-                                            st.gacc[i][(td * KH + th) * KW + tw] +=
-                                                an[i][rr] * vx + ad[i][rr] * vt;
-                                    }
+                                            NDC_UNROLL
+                                            for (int c = 0; c < RW; ++c)
+                                                st.gacc[i][(td * KH + th) * KW + tw] +=
+                                                    acc[0][i][rr][c] * vx[c + KW - 1 - tw] +
+                                                    acc[1][i][rr][c] * vt[c + KW - 1 - tw];
                                 }
+                            }
                         }
                     }
                 }
-                if (XT && st.strip < 2 * PH) {
-                    float an[SC][1], ad[SC][1];
-                    gn_gd_rows(st, j1, halo_row(st.strip, PH, TH), IntTag<1>(), an, ad);
+                if (XT && st.ln.strip < 2 * PH) {
+                    float acc[2][SC][1][RW];
+                    gn_gd_rows(st, j1, halo_row(st.ln.strip, PH, TH), IntTag<1>(), acc);
                 }
             });
             ex.sync();
 
             // ---- prefetch, then scatter: plane k - PD of gn/gd feeds pending planes of gx / gt1
             ex.each([&](State &st, int) {
-                if (!st.active) return;
+                if (!st.ln.active) return;
                 load_plane(st, k + 1);
                 if (live1) {
+                    float wi[KT], wn[KT];
+                    load_taps<KT>(hw, wi);
                     NDC_ROLLED
                     for (int i = 0; i < SC; ++i) {
-                        UniformF wi = hw + i * KT;
-                        const int gb_ = off_g + (st.strip * RH) * P + st.col;
-                        k_rows<KD, KH, KW, RH, RH>(ex, gb_ + i * RG * P, P, wi, st.accx, 0);
-                        k_rows<KD, KH, KW, RH, RH>(ex, gb_ + (SC + i) * RG * P, P, wi, st.acct, 0);
+                        load_taps<KT>(hw + (i + 1 < SC ? i + 1 : 0) * KT, wn);
+                        const int gb_ = off_g + (st.ln.strip * RH) * P + PL + st.ln.c0 - PW;
+                        k_rows<KD, KH, KW, RH, RW, RH>(ex, gb_ + i * RG * P, P, wi, st.accx, 0);
+                        k_rows<KD, KH, KW, RH, RW, RH>(ex, gb_ + (SC + i) * RG * P, P, wi, st.acct, 0);
+                        copy_taps<KT>(wn, wi);
                     }
                 }
                 const int pf = k - 2 * PD;
                 NDC_UNROLL
                 for (int r = 0; r < RH; ++r) {
-                    const int row = r0 + st.strip * RH + r;
-                    if (pf >= 0 && row < H) {
-                        const long long o = (long long)pf * plane + row * W + st.col;
-                        if (gxg) Elem<T>::store(gxg + o, st.accx[0][r]);
-                        Elem<T>::store(gt1g + o, st.acct[0][r]);
+                    if (pf >= 0 && ((st.ook >> r) & 1u)) {
+                        const long long o = (long long)pf * plane + st.ooff[r];
+                        if (gxg) IO::store(gxg + o, st.accx[0][r]);
+                        IO::store(gt1g + o, st.acct[0][r]);
                     }
                     NDC_UNROLL
-                    for (int a = 0; a + 1 < KD; ++a) {
-                        st.accx[a][r] = st.accx[a + 1][r];
-                        st.acct[a][r] = st.acct[a + 1][r];
+                    for (int c = 0; c < RW; ++c) {
+                        NDC_UNROLL
+                        for (int a = 0; a + 1 < KD; ++a) {
+                            st.accx[a][r][c] = st.accx[a + 1][r][c];
+                            st.acct[a][r][c] = st.acct[a + 1][r][c];
+                        }
+                        st.accx[KD - 1][r][c] = 0.f;
+                        st.acct[KD - 1][r][c] = 0.f;
                     }
-                    st.accx[KD - 1][r] = 0.f;
-                    st.acct[KD - 1][r] = 0.f;
                 }
             });
         }
@@ -668,19 +821,23 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, typename T> struct Bwd1Ke
 
 // =================================================================== backward, pass 2
 
-template <int KD_, int KH_, int KW_, int SC_, int RH_, typename T> struct Bwd2Kernel {
-    static constexpr int KD = KD_, KH = KH_, KW = KW_, SC = SC_, RH = RH_;
+template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> struct Bwd2Kernel {
+    static constexpr int KD = KD_, KH = KH_, KW = KW_, SC = SC_, RH = RH_, RW = RW_;
     static constexpr int PD = KD / 2, PH = KH / 2, PW = KW / 2, KT = KD * KH * KW;
     static constexpr int NXR = RH + (PH > 0 ? 1 : 0);
     static constexpr int XR = KD + 1;
     static constexpr int NRED = SC * KT + SC;
     typedef BwdParams<T> Params;
+    typedef VecIO<T, RW> IO;
 
     struct State {
-        int strip, col, active;
+        Lane ln;
+        int xoff[NXR], ooff[RH];
+        unsigned xok, ook;
+        float bv[SC];
         float gacc[SC][KT];   // K-side filter-gradient term
         float gbacc[SC];
-        float px[NXR], pt[NXR], pg[NXR];
+        float px[NXR][RW], pt[NXR][RW], pg[NXR][RW];
     };
 
     static NDC_HD int rows_x(int TH) { return TH + 2 * PH; }
@@ -695,18 +852,17 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, typename T> struct Bwd2Ke
     {
         const Tile t = p.t;
         const BlockId id = decode_block(block_id, p.C, t);
-        const int S = t.S, P = t.P, TH = t.TH, W = p.W, H = p.H, D = p.D;
+        const int S = t.S, P = t.P, PL = t.PL, TH = t.TH, W = p.W, H = p.H, D = p.D;
         const int RX = rows_x(TH);
         const int off_x = 0, off_t = XR * RX * P, off_g = 2 * XR * RX * P;
         const int total = 3 * XR * RX * P;
-        const long long plane = (long long)H * W;
+        const int plane = H * W;
         const long long cplane = (long long)D * plane;
         const long long cbase = ((long long)id.b * p.C + id.c) * cplane;
         const T *xg = p.x + cbase, *t1g = p.t1 + cbase, *gt1g = p.gt1 + cbase;
         const T *zg = p.z + cbase * SC, *gg = p.gout + cbase * SC;
         T *gzg = p.gz ? p.gz + cbase * SC : nullptr;
         UniformF hw = as_uniform(p.h + (long long)id.c * SC * KT);
-        UniformF bias = as_uniform(p.bias ? p.bias + id.c * SC : nullptr);
         const int r0 = id.r0;
         const int nthreads = ex.nthreads;
         const int relu = p.relu;
@@ -714,46 +870,58 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, typename T> struct Bwd2Ke
         const int need_gh = p.need_gh;
 
         auto load_plane = [&](State &st, int k) {
-            if (!st.active) return;
+            if (!st.ln.active) return;
             if (k < D) {
                 const long long ko = (long long)k * plane;
                 NDC_UNROLL
                 for (int n = 0; n < NXR; ++n) {
-                    const int j = st.strip + n * S, row = r0 - PH + j;
-                    const bool ok = j < RX && row >= 0 && row < H;
-                    const long long o = ko + clampi(row, 0, H - 1) * W + st.col;
-                    const float vx = Elem<T>::load(xg + o), vt = Elem<T>::load(t1g + o),
-                                vg = Elem<T>::load(gt1g + o);
-                    st.px[n] = ok ? vx : 0.f;
-                    st.pt[n] = ok ? vt : 0.f;
-                    st.pg[n] = ok ? vg : 0.f;
+                    IO::load(xg + ko + st.xoff[n], st.px[n]);
+                    IO::load(t1g + ko + st.xoff[n], st.pt[n]);
+                    IO::load(gt1g + ko + st.xoff[n], st.pg[n]);
                 }
             } else {
                 NDC_UNROLL
-                for (int n = 0; n < NXR; ++n) st.px[n] = st.pt[n] = st.pg[n] = 0.f;
+                for (int n = 0; n < NXR; ++n)
+                    NDC_UNROLL
+                    for (int c = 0; c < RW; ++c) st.px[n][c] = st.pt[n][c] = st.pg[n][c] = 0.f;
             }
         };
         auto store_plane = [&](State &st, int k) {
-            if (!st.active) return;
+            if (!st.ln.active) return;
             const int slot = wrap(k % XR, XR);
             NDC_UNROLL
             for (int n = 0; n < NXR; ++n) {
-                const int j = st.strip + n * S;
-                if (j < RX) {
-                    const int o = (slot * RX + j) * P + PW + st.col;
-                    ex.st_(off_x + o, st.px[n]);
-                    ex.st_(off_t + o, st.pt[n]);
-                    ex.st_(off_g + o, st.pg[n]);
+                const int j = st.ln.strip + n * S;
+                if ((st.xok >> n) & 1u) {
+                    NDC_UNROLL
+                    for (int c = 0; c < RW; ++c) {
+                        const int o = (slot * RX + j) * P + PL + st.ln.c0 + c;
+                        ex.st_(off_x + o, st.px[n][c]);
+                        ex.st_(off_t + o, st.pt[n][c]);
+                        ex.st_(off_g + o, st.pg[n][c]);
+                    }
                 }
             }
         };
 
         ex.each([&](State &st, int tid) {
-            st.strip = tid / W;
-            st.col = tid - st.strip * W;
-            st.active = st.strip < S;
+            st.ln = make_lane(tid, t, RW);
+            st.xok = st.ook = 0u;
+            NDC_UNROLL
+            for (int n = 0; n < NXR; ++n) {
+                const int j = st.ln.strip + n * S, row = r0 - PH + j;
+                if (j < RX && row >= 0 && row < H) st.xok |= 1u << n;
+                st.xoff[n] = clampi(row, 0, H - 1) * W + st.ln.c0;
+            }
+            NDC_UNROLL
+            for (int r = 0; r < RH; ++r) {
+                const int row = r0 + st.ln.strip * RH + r;
+                if (row < H) st.ook |= 1u << r;
+                st.ooff[r] = clampi(row, 0, H - 1) * W + st.ln.c0;
+            }
             NDC_UNROLL
             for (int i = 0; i < SC; ++i) {
+                st.bv[i] = p.bias ? p.bias[id.c * SC + i] : 0.f;
                 st.gbacc[i] = 0.f;
                 NDC_UNROLL
                 for (int a = 0; a < KT; ++a) st.gacc[i][a] = 0.f;
@@ -769,66 +937,91 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, typename T> struct Bwd2Ke
 
             const int j0 = k - PD;
             ex.each([&](State &st, int) {
-                if (!st.active) return;
+                if (!st.ln.active) return;
                 load_plane(st, k + 1);
                 if (j0 < 0) return;
-                float sv[SC][RH], gv[SC][RH];
+                float sv[SC][RH][RW], gv[SC][RH][RW];
                 const long long ko = (long long)j0 * plane;
                 NDC_UNROLL
                 for (int r = 0; r < RH; ++r) {
-                    const int row = r0 + st.strip * RH + r;
-                    const bool ok = row < H;
-                    const long long o = ko + clampi(row, 0, H - 1) * W + st.col;
+                    const bool ok = (st.ook >> r) & 1u;
                     NDC_UNROLL
                     for (int i = 0; i < SC; ++i) {
-                        // s <= 0 marks "masked" (ReLU inactive); with relu off nothing is masked
-                        float s = Elem<T>::load(zg + i * cplane + o) + (bias ? bias[i] : 0.f);
-                        const float g = Elem<T>::load(gg + i * cplane + o);
-                        if (relu) s = s > 0.f ? s : 0.f;
-                        sv[i][r] = ok ? s : 0.f;
-                        gv[i][r] = ok ? g : 0.f;
+                        IO::load(zg + i * cplane + ko + st.ooff[r], sv[i][r]);
+                        IO::load(gg + i * cplane + ko + st.ooff[r], gv[i][r]);
+                        NDC_UNROLL
+                        for (int c = 0; c < RW; ++c) {
+                            // with the ReLU on, s <= 0 marks a masked element
+                            float s = sv[i][r][c] + st.bv[i];
+                            if (relu) s = relu_f(s);
+                            sv[i][r][c] = ok ? s : 0.f;
+                            gv[i][r][c] = ok ? gv[i][r][c] : 0.f;
+                        }
                     }
                 }
-                float an[SC][RH], ad[SC][RH], ag[SC][RH];
+                float acc[3][SC][RH][RW];
                 NDC_UNROLL
-                for (int i = 0; i < SC; ++i)
+                for (int a = 0; a < 3; ++a)
                     NDC_UNROLL
-                    for (int r = 0; r < RH; ++r) an[i][r] = ad[i][r] = ag[i][r] = 0.f;
-                NDC_UNROLL
-                for (int td = 0; td < KD; ++td) {
-                    const int slot = wrap((j0 + PD - td) % XR, XR);
-                    const int ob = (slot * RX + st.strip * RH) * P + st.col + 2 * PW;
-                    NDC_UNROLL
-                    for (int q = 0; q < RH + 2 * PH; ++q)
+                    for (int i = 0; i < SC; ++i)
                         NDC_UNROLL
-                        for (int tw = 0; tw < KW; ++tw) {
-                            const int o = ob + q * P - tw;
-                            const float vx = ex.ld(off_x + o), vt = ex.ld(off_t + o), vg = ex.ld(off_g + o);
+                        for (int r = 0; r < RH; ++r)
+                            NDC_UNROLL
+                            for (int c = 0; c < RW; ++c) acc[a][i][r][c] = 0.f;
+                float wt[SC][KH * KW], wn[SC][KH * KW];
+                load_plane_taps<SC, KT, KH * KW>(hw, wt);
+                NDC_ROLLED
+                for (int td = 0; td < KD; ++td) {
+                    load_plane_taps<SC, KT, KH * KW>(hw + (td + 1 < KD ? td + 1 : 0) * KH * KW, wn);
+                    const int slot = wrap((j0 + PD - td) % XR, XR);
+                    const int ob = (slot * RX + st.ln.strip * RH) * P + PL + st.ln.c0 - PW;
+                    const int base[3] = {off_x + ob, off_t + ob, off_g + ob};
+                    a_plane<KH, KW, KT, SC, RH, RW, 3>(ex, base, P, wt, acc);
+                    NDC_UNROLL
+                    for (int i = 0; i < SC; ++i) copy_taps<KH * KW>(wn[i], wt[i]);
+                }
+                if (need_gh) {
+                    // K-side filter-gradient term: re-read the gt1 window
+                    NDC_UNROLL
+                    for (int td = 0; td < KD; ++td) {
+                        const int slot = wrap((j0 + PD - td) % XR, XR);
+                        const int ob = (slot * RX + st.ln.strip * RH) * P + PL + st.ln.c0 - PW;
+                        NDC_UNROLL
+                        for (int q = 0; q < RH + 2 * PH; ++q) {
+                            float vg[RW + KW - 1];
+                            NDC_UNROLL
+                            for (int u = 0; u < RW + KW - 1; ++u) vg[u] = ex.ld(off_g + ob + q * P + u);
                             NDC_UNROLL
                             for (int th = 0; th < KH; ++th) {
                                 const int rr = q - 2 * PH + th;
                                 if (rr < 0 || rr >= RH) continue;
                                 NDC_UNROLL
-                                for (int i = 0; i < SC; ++i) {
-                                    const float wv = hw[((i * KD + td) * KH + th) * KW + tw];
-                                    an[i][rr] += vx * wv;
-                                    ad[i][rr] += vt * wv;
-                                    ag[i][rr] += vg * wv;
-                                    if (need_gh) st.gacc[i][(td * KH + th) * KW + tw] += sv[i][rr] * vg;
-                                }
+                                for (int tw = 0; tw < KW; ++tw)
+                                    NDC_UNROLL
+                                    for (int i = 0; i < SC; ++i)
+                                        NDC_UNROLL
+                                        for (int c = 0; c < RW; ++c)
+                                            st.gacc[i][(td * KH + th) * KW + tw] +=
+                                                sv[i][rr][c] * vg[c + KW - 1 - tw];
                             }
                         }
+                    }
                 }
                 NDC_UNROLL
                 for (int r = 0; r < RH; ++r) {
-                    const int row = r0 + st.strip * RH + r;
-                    if (row >= H) continue;
+                    if (!((st.ook >> r) & 1u)) continue;
                     NDC_UNROLL
                     for (int i = 0; i < SC; ++i) {
-                        float v = gv[i][r] * (an[i][r] + eps) * fast_rcp(ad[i][r] + eps) + ag[i][r];
-                        if (relu && !(sv[i][r] > 0.f)) v = 0.f;
-                        st.gbacc[i] += v;
-                        if (gzg) Elem<T>::store(gzg + i * cplane + ko + row * W + st.col, v);
+                        float v[RW];
+                        NDC_UNROLL
+                        for (int c = 0; c < RW; ++c) {
+                            float gzv = gv[i][r][c] * (acc[0][i][r][c] + eps) * fast_rcp(acc[1][i][r][c] + eps) +
+                                        acc[2][i][r][c];
+                            if (relu && !(sv[i][r][c] > 0.f)) gzv = 0.f;
+                            st.gbacc[i] += gzv;
+                            v[c] = gzv;
+                        }
+                        if (gzg) IO::store(gzg + i * cplane + ko + st.ooff[r], v);
                     }
                 }
             });

@@ -11,24 +11,29 @@
 namespace ndc {
 namespace fused {
 
-// Filter geometries with compiled instances, in the marching view (2-D k x k runs as
-// (k, 1, k)).  One row per (KD, KH, KW, SC, RHF, RHB); RHF / RHB are the rows per thread of
-// the forward and backward kernels.  Several rows may share a filter geometry: the first
-// one whose row counts match the tuning choice (or, failing that, the first one) is used.
-#define NDC_FUSED_VARIANTS(X)  \
-    X(3, 3, 3, 4, 4, 2)        \
-    X(3, 3, 3, 4, 2, 1)        \
-    X(5, 1, 5, 4, 1, 1)        \
-    X(3, 1, 3, 4, 1, 1)
+// Compiled instances, in the marching view (2-D k x k runs as (k, 1, k)).  One row per
+// (KD, KH, KW, SC, RHF, RWF, RHB, RWB): RHF x RWF is the register tile (rows x columns per
+// thread) of the forward kernel, RHB x RWB that of the two backward kernels.  Rows of one
+// filter geometry are listed in order of preference; a row with RW = 2 needs an even W and
+// tensors aligned to two elements, so every geometry also has an RW = 1 row.
+#define NDC_FUSED_VARIANTS(X)        \
+    X(3, 3, 3, 4, 2, 2, 2, 2)        \
+    X(3, 3, 3, 4, 2, 2, 1, 2)        \
+    X(3, 3, 3, 4, 4, 1, 2, 1)        \
+    X(3, 3, 3, 4, 2, 1, 1, 1)        \
+    X(5, 1, 5, 4, 1, 2, 1, 2)        \
+    X(5, 1, 5, 4, 1, 1, 1, 1)        \
+    X(3, 1, 3, 4, 1, 2, 1, 2)        \
+    X(3, 1, 3, 4, 1, 1, 1, 1)
 
 struct Variant {
-    int KD, KH, KW, SC, RHF, RHB;
+    int KD, KH, KW, SC, RHF, RWF, RHB, RWB;
 };
 
 // Launch-shape choices that are not dictated by the geometry.  Defaults are the measured
 // best; the environment variables exist for tuning runs only.
 struct Tuning {
-    int rhf, rhb, threads_f, threads_b;
+    int rhf, rwf, rhb, rwb, threads_f, threads_b;
 };
 
 static inline int env_int(const char *name, int dflt)
@@ -40,24 +45,40 @@ static inline int env_int(const char *name, int dflt)
 static inline Tuning tuning()
 {
     Tuning t;
-    t.rhf = env_int("NDC_TUNE_RHF", 4);
-    t.rhb = env_int("NDC_TUNE_RHB", 2);
+    t.rhf = env_int("NDC_TUNE_RHF", 0);
+    t.rwf = env_int("NDC_TUNE_RWF", 0);
+    t.rhb = env_int("NDC_TUNE_RHB", 0);
+    t.rwb = env_int("NDC_TUNE_RWB", 0);
     t.threads_f = env_int("NDC_TUNE_NTF", 256);
-    t.threads_b = env_int("NDC_TUNE_NTB", 256);
+    t.threads_b = env_int("NDC_TUNE_NTB", 512);
     return t;
 }
 
-static inline bool find_variant(const KGeom &q, const March &m, Variant &v)
+// first listed row of this filter geometry that the width / alignment allow (and, in a
+// tuning run, that matches the requested register tiles)
+static inline bool find_variant(const KGeom &q, const March &m, bool pairs_ok, Variant &v)
 {
     if (q.m != 1) return false;
     const Tuning tn = tuning();
+    const bool even = pairs_ok && m.W % 2 == 0;
     bool found = false;
-#define X(kd_, kh_, kw_, sc_, rhf_, rhb_)                                       \
-    if (m.KD == kd_ && m.KH == kh_ && m.KW == kw_ && q.sc == sc_) {             \
-        const bool exact = rhf_ == tn.rhf && rhb_ == tn.rhb;                    \
-        if (!found || exact) v = Variant{kd_, kh_, kw_, sc_, rhf_, rhb_};       \
-        if (exact) return true;                                                 \
-        found = true;                                                           \
+#define X(kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_)                                        \
+    if (!found && m.KD == kd_ && m.KH == kh_ && m.KW == kw_ && q.sc == sc_ &&                \
+        (even || (rwf_ == 1 && rwb_ == 1)) && (!tn.rhf || tn.rhf == rhf_) &&                 \
+        (!tn.rwf || tn.rwf == rwf_) && (!tn.rhb || tn.rhb == rhb_) &&                        \
+        (!tn.rwb || tn.rwb == rwb_)) {                                                       \
+        v = Variant{kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_};                             \
+        found = true;                                                                        \
+    }
+    NDC_FUSED_VARIANTS(X)
+#undef X
+    if (found) return true;
+    // no row matches a tuning request: fall back to the plain order of preference
+#define X(kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_)                                        \
+    if (!found && m.KD == kd_ && m.KH == kh_ && m.KW == kw_ && q.sc == sc_ &&                \
+        (even || (rwf_ == 1 && rwb_ == 1))) {                                                \
+        v = Variant{kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_};                             \
+        found = true;                                                                        \
     }
     NDC_FUSED_VARIANTS(X)
 #undef X
@@ -72,25 +93,31 @@ struct Plan {
     int nblk_f, nblk_b;
 };
 
-template <int KD, int KH, int KW, int SC, int RHF, int RHB>
+template <int KD, int KH, int KW, int SC, int RHF, int RWF, int RHB, int RWB>
 static inline void plan_lds(Plan &pl)
 {
-    pl.lds_f = FwdKernel<KD, KH, KW, SC, RHF, float>::lds_floats(pl.tf);
-    pl.lds_b1 = Bwd1Kernel<KD, KH, KW, SC, RHB, float>::lds_floats(pl.tb);
-    pl.lds_b2 = Bwd2Kernel<KD, KH, KW, SC, RHB, float>::lds_floats(pl.tb);
+    pl.lds_f = FwdKernel<KD, KH, KW, SC, RHF, RWF, float>::lds_floats(pl.tf);
+    pl.lds_b1 = Bwd1Kernel<KD, KH, KW, SC, RHB, RWB, float>::lds_floats(pl.tb);
+    pl.lds_b2 = Bwd2Kernel<KD, KH, KW, SC, RHB, RWB, float>::lds_floats(pl.tb);
 }
 
-static inline bool make_plan(const KGeom &q, Plan &pl)
+#define NDC_IS_VARIANT(pl, kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_)                          \
+    ((pl).v.KD == kd_ && (pl).v.KH == kh_ && (pl).v.KW == kw_ && (pl).v.SC == sc_ &&            \
+     (pl).v.RHF == rhf_ && (pl).v.RWF == rwf_ && (pl).v.RHB == rhb_ && (pl).v.RWB == rwb_)
+
+// pairs_ok: every activation pointer of the call is aligned to two elements
+static inline bool make_plan(const KGeom &q, Plan &pl, bool pairs_ok = true)
 {
     pl.m = march_of(q);
-    if (!find_variant(q, pl.m, pl.v)) return false;
+    // 32-bit offsets inside one (sample, channel) volume
+    if ((long long)q.sc * q.SP >= (1LL << 31)) return false;
+    if (!find_variant(q, pl.m, pairs_ok, pl.v)) return false;
     const Tuning tn = tuning();
-    if (!make_tile(pl.m, pl.v.RHF, tn.threads_f, pl.tf)) return false;
-    if (!make_tile(pl.m, pl.v.RHB, tn.threads_b, pl.tb)) return false;
-#define X(kd_, kh_, kw_, sc_, rhf_, rhb_)                                                     \
-    if (pl.v.KD == kd_ && pl.v.KH == kh_ && pl.v.KW == kw_ && pl.v.SC == sc_ && pl.v.RHF == rhf_ &&  \
-        pl.v.RHB == rhb_)               \
-        plan_lds<kd_, kh_, kw_, sc_, rhf_, rhb_>(pl);
+    if (!make_tile(pl.m, pl.v.RHF, pl.v.RWF, tn.threads_f, pl.tf)) return false;
+    if (!make_tile(pl.m, pl.v.RHB, pl.v.RWB, tn.threads_b, pl.tb)) return false;
+#define X(kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_)                                        \
+    if (NDC_IS_VARIANT(pl, kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_))                      \
+        plan_lds<kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_>(pl);
     NDC_FUSED_VARIANTS(X)
 #undef X
     const int cap = kMaxLdsBytes / 4;
@@ -105,7 +132,12 @@ static inline bool make_plan(const KGeom &q, Plan &pl)
 static inline bool supported(const KGeom &q)
 {
     Plan pl;
-    return make_plan(q, pl);
+    return make_plan(q, pl, false);
+}
+
+template <typename T> static inline bool pair_aligned(const void *p)
+{
+    return p == nullptr || ((uintptr_t)p % (2 * sizeof(T))) == 0;
 }
 
 static inline size_t align256(size_t v) { return (v + 255) / 256 * 256; }
@@ -113,13 +145,15 @@ static inline size_t align256(size_t v) { return (v + 255) / 256 * 256; }
 // scratch: gt1 (activation dtype) | pass-1 partials | pass-2 partials
 static inline size_t backward_ws(const KGeom &q, int dtype, int /*need_gh*/, int /*need_gb*/)
 {
-    Plan pl;
-    if (!make_plan(q, pl)) return 0;
+    // sized for whichever variant the call ends up with (aligned pairs or not)
+    Plan a, b;
+    if (!make_plan(q, a, false)) return 0;
+    const bool has_b = make_plan(q, b, true);
+    const size_t nblk = has_b && b.nblk_b > a.nblk_b ? b.nblk_b : a.nblk_b;
     const size_t esz = dtype == NDC_BF16 ? 2 : 4;
     const size_t n_x = (size_t)q.B * q.G * q.SP;
     const size_t kt = (size_t)q.sc * q.KT;
-    return align256(n_x * esz) + align256((size_t)pl.nblk_b * kt * 4) +
-           align256((size_t)pl.nblk_b * (kt + q.sc) * 4);
+    return align256(n_x * esz) + align256(nblk * kt * 4) + align256(nblk * (kt + q.sc) * 4);
 }
 
 template <class BE, typename T>
@@ -127,7 +161,9 @@ static int forward(const KGeom &q, const T *x, const T *z, const float *h, const
                    T *out, T *t1, void *stream)
 {
     Plan pl;
-    if (!make_plan(q, pl)) return NDC_ERR_GEOMETRY;
+    const bool pairs = pair_aligned<T>(x) && pair_aligned<T>(z) && pair_aligned<T>(out) &&
+                       pair_aligned<T>(t1);
+    if (!make_plan(q, pl, pairs)) return NDC_ERR_GEOMETRY;
     FwdParams<T> p;
     p.x = x;
     p.z = z;
@@ -143,10 +179,9 @@ static int forward(const KGeom &q, const T *x, const T *z, const float *h, const
     p.relu = q.relu;
     p.eps = q.eps;
     p.t = pl.tf;
-#define X(kd_, kh_, kw_, sc_, rhf_, rhb_)                                                        \
-    if (pl.v.KD == kd_ && pl.v.KH == kh_ && pl.v.KW == kw_ && pl.v.SC == sc_ && pl.v.RHF == rhf_ &&  \
-        pl.v.RHB == rhb_)                  \
-        return BE::template block_kernel<FwdKernel<kd_, kh_, kw_, sc_, rhf_, T>>(               \
+#define X(kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_)                                          \
+    if (NDC_IS_VARIANT(pl, kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_))                        \
+        return BE::template block_kernel<FwdKernel<kd_, kh_, kw_, sc_, rhf_, rwf_, T>>(        \
             p, pl.nblk_f, pl.tf.NT, pl.lds_f, stream);
     NDC_FUSED_VARIANTS(X)
 #undef X
@@ -162,7 +197,9 @@ static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const f
     // reduction, taken with events on `stream`; makes the call synchronous
     typename BE::Timer tm(pass_ms != nullptr, stream);
     Plan pl;
-    if (!make_plan(q, pl)) return NDC_ERR_GEOMETRY;
+    const bool pairs = pair_aligned<T>(x) && pair_aligned<T>(z) && pair_aligned<T>(t1) &&
+                       pair_aligned<T>(gout) && pair_aligned<T>(gx) && pair_aligned<T>(gz);
+    if (!make_plan(q, pl, pairs)) return NDC_ERR_GEOMETRY;
     const size_t n_x = (size_t)q.B * q.G * q.SP;
     const int kt = q.sc * q.KT;
     char *w = (char *)ws;
@@ -196,10 +233,9 @@ static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const f
     int st = NDC_ERR_GEOMETRY;
     p.part = part1;
     p.part_stride = kt;
-#define X(kd_, kh_, kw_, sc_, rhf_, rhb_)                                                        \
-    if (pl.v.KD == kd_ && pl.v.KH == kh_ && pl.v.KW == kw_ && pl.v.SC == sc_ && pl.v.RHF == rhf_ &&  \
-        pl.v.RHB == rhb_)                  \
-        st = BE::template block_kernel<Bwd1Kernel<kd_, kh_, kw_, sc_, rhb_, T>>(                \
+#define X(kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_)                                          \
+    if (NDC_IS_VARIANT(pl, kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_))                        \
+        st = BE::template block_kernel<Bwd1Kernel<kd_, kh_, kw_, sc_, rhb_, rwb_, T>>(         \
             p, pl.nblk_b, pl.tb.NT, pl.lds_b1, stream);
     NDC_FUSED_VARIANTS(X)
 #undef X
@@ -213,10 +249,9 @@ static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const f
     p.part = part2;
     p.part_stride = kt + q.sc;
     st = NDC_ERR_GEOMETRY;
-#define X(kd_, kh_, kw_, sc_, rhf_, rhb_)                                                        \
-    if (pl.v.KD == kd_ && pl.v.KH == kh_ && pl.v.KW == kw_ && pl.v.SC == sc_ && pl.v.RHF == rhf_ &&  \
-        pl.v.RHB == rhb_)                  \
-        st = BE::template block_kernel<Bwd2Kernel<kd_, kh_, kw_, sc_, rhb_, T>>(                \
+#define X(kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_)                                          \
+    if (NDC_IS_VARIANT(pl, kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_))                        \
+        st = BE::template block_kernel<Bwd2Kernel<kd_, kh_, kw_, sc_, rhb_, rwb_, T>>(         \
             p, pl.nblk_b, pl.tb.NT, pl.lds_b2, stream);
     NDC_FUSED_VARIANTS(X)
 #undef X
