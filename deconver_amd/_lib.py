@@ -24,6 +24,7 @@ EXPORTS = (
     "ndc_fused_supported",
     "ndc_check_geometry",
     "ndc_forward",
+    "ndc_forward_workspace_bytes",
     "ndc_backward_workspace_bytes",
     "ndc_backward",
     "ndc_backward_profiled",
@@ -80,7 +81,9 @@ class NdcLibrary:
         d.ndc_status_string.argtypes = [ctypes.c_int]
         d.ndc_fused_supported.argtypes = [gp]
         d.ndc_check_geometry.argtypes = [gp]
-        d.ndc_forward.argtypes = [gp, vp, vp, fp, fp, vp, vp, vp]
+        d.ndc_forward.argtypes = [gp, vp, vp, fp, fp, vp, vp, vp, ctypes.c_size_t, vp]
+        d.ndc_forward_workspace_bytes.restype = ctypes.c_size_t
+        d.ndc_forward_workspace_bytes.argtypes = [gp]
         d.ndc_backward_workspace_bytes.restype = ctypes.c_size_t
         d.ndc_backward_workspace_bytes.argtypes = [gp] + [ctypes.c_int] * 4
         d.ndc_backward.argtypes = [gp, vp, vp, vp, fp, fp, vp, vp, vp, fp, fp, vp,
@@ -102,10 +105,14 @@ class NdcLibrary:
     def check_geometry(self, g: Geom) -> int:
         return self._dll.ndc_check_geometry(ctypes.byref(g))
 
+    def forward_workspace_bytes(self, g: Geom) -> int:
+        return self._dll.ndc_forward_workspace_bytes(ctypes.byref(g))
+
     def forward(self, g: Geom, x: int, z: int, h: int, bias: Optional[int], out: int,
-                t1: Optional[int], stream: Optional[int]) -> None:
-        self._check(self._dll.ndc_forward(ctypes.byref(g), x, z, h, bias, out, t1, stream),
-                    "ndc_forward")
+                t1: Optional[int], ws: Optional[int], ws_bytes: int,
+                stream: Optional[int]) -> None:
+        self._check(self._dll.ndc_forward(ctypes.byref(g), x, z, h, bias, out, t1, ws, ws_bytes,
+                                          stream), "ndc_forward")
 
     def backward_workspace_bytes(self, g: Geom, need_gx, need_gz, need_gh, need_gb) -> int:
         return self._dll.ndc_backward_workspace_bytes(

@@ -193,8 +193,19 @@ int ndc_check_geometry(const ndc_geom *g)
     return st < 0 ? st : NDC_OK;
 }
 
+size_t ndc_forward_workspace_bytes(const ndc_geom *g)
+{
+    using namespace ndc;
+    KGeom q;
+    if (make_kgeom(g, q) != NDC_OK) return 0;
+    const int path = choose_path(g, q);
+    if (path != NDC_PATH_FUSED) return 0;
+    return fused::forward_ws(q, g->dtype);
+}
+
 int ndc_forward(const ndc_geom *g, const void *x, const void *z, const float *h,
-                const float *bias, void *out, void *t1, void *stream)
+                const float *bias, void *out, void *t1, void *workspace, size_t workspace_bytes,
+                void *stream)
 {
     using namespace ndc;
     KGeom q;
@@ -204,11 +215,15 @@ int ndc_forward(const ndc_geom *g, const void *x, const void *z, const float *h,
     const int path = choose_path(g, q);
     if (path < 0) return path;
     if (path == NDC_PATH_FUSED) {
+        const size_t need = fused::forward_ws(q, g->dtype);
+        if (need && (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255u)))
+            return NDC_ERR_WORKSPACE;
+        void *ws = need ? workspace : nullptr;
         return g->dtype == NDC_F32
                    ? fused::forward<Backend, float>(q, (const float *)x, (const float *)z, h, bias,
-                                                    (float *)out, (float *)t1, stream)
+                                                    (float *)out, (float *)t1, ws, stream)
                    : fused::forward<Backend, bf16_t>(q, (const bf16_t *)x, (const bf16_t *)z, h,
-                                                     bias, (bf16_t *)out, (bf16_t *)t1, stream);
+                                                     bias, (bf16_t *)out, (bf16_t *)t1, ws, stream);
     }
     return g->dtype == NDC_F32
                ? direct_forward<float>(q, (const float *)x, (const float *)z, h, bias,

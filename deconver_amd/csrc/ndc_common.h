@@ -82,6 +82,32 @@ NDC_HD float bits_to_float(uint32_t u)
     return f;
 }
 
+NDC_HD uint32_t float_to_bits(float f)
+{
+    uint32_t u;
+#if NDC_DEVICE_BUILD && defined(__HIP_DEVICE_COMPILE__)
+    u = __float_as_uint(f);
+#else
+    memcpy(&u, &f, 4);
+#endif
+    return u;
+}
+
+// acc + a.lo*b.lo + a.hi*b.hi on packed bf16 pairs, float32 accumulate: one
+// v_dot2c_f32_bf16 (issues at the rate of an fp32 FMA, i.e. two MACs per lane-instruction)
+NDC_HD float dot2_bf16(uint32_t a, uint32_t b, float acc)
+{
+#if NDC_DEVICE_BUILD && defined(__HIP_DEVICE_COMPILE__)
+    typedef __attribute__((ext_vector_type(2))) __bf16 bf2_t;
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf2_t, a), __builtin_bit_cast(bf2_t, b),
+                                           acc, false);
+#else
+    const float alo = bits_to_float(a << 16), ahi = bits_to_float(a & 0xffff0000u);
+    const float blo = bits_to_float(b << 16), bhi = bits_to_float(b & 0xffff0000u);
+    return acc + alo * blo + ahi * bhi;
+#endif
+}
+
 // N consecutive elements <-> N floats with one memory access (N = 1 or 2; the address must
 // be aligned to N elements)
 template <typename T, int N> struct VecIO;
@@ -150,6 +176,17 @@ NDC_D UniformF as_uniform(const float *p) { return (UniformF)(unsigned long long
 typedef const float *UniformF;
 NDC_HD UniformF as_uniform(const float *p) { return p; }
 #endif
+
+// Tell the compiler that a value is the same in every lane (so that addresses derived from
+// it stay on the scalar unit).
+NDC_HD int uniform_int(int v)
+{
+#if NDC_DEVICE_BUILD && defined(__HIP_DEVICE_COMPILE__)
+    return __builtin_amdgcn_readfirstlane(v);
+#else
+    return v;
+#endif
+}
 
 template <int N> struct IntTag {
     static constexpr int value = N;

@@ -118,6 +118,7 @@ static inline bool make_tile(const March &m, int RH, int RW, int target_threads,
 template <typename T> struct FwdParams {
     const T *x, *z;
     const float *h, *bias;
+    const float *wtab;   // packed bf16 tap tables (bf16 dot2 kernels only)
     T *out, *t1;
     int B, C, D, H, W;
     int relu;
@@ -128,6 +129,7 @@ template <typename T> struct FwdParams {
 template <typename T> struct BwdParams {
     const T *x, *z, *t1, *gout;
     const float *h, *bias;
+    const float *wtab;   // packed bf16 tap tables (bf16 dot2 kernels only)
     T *gx, *gz;
     T *gt1;        // scratch (B, C, S): written by pass 1, read by pass 2
     float *part;   // per-workgroup partial sums, [nblocks][part_stride]

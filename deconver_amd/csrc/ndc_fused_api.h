@@ -7,6 +7,7 @@
 #include <stdlib.h>
 
 #include "ndc_fused.h"
+#include "ndc_fused_bf16.h"
 
 namespace ndc {
 namespace fused {
@@ -88,6 +89,7 @@ static inline bool find_variant(const KGeom &q, const March &m, bool pairs_ok, V
 struct Plan {
     Variant v;
     March m;
+    bool dot2;            // bf16 dot2 kernels (3x3x3, SC = 4, even W, aligned pairs)
     Tile tf, tb;          // forward / backward launch shapes
     int lds_f, lds_b1, lds_b2;
     int nblk_f, nblk_b;
@@ -106,9 +108,12 @@ static inline void plan_lds(Plan &pl)
      (pl).v.RHF == rhf_ && (pl).v.RWF == rwf_ && (pl).v.RHB == rhb_ && (pl).v.RWB == rwb_)
 
 // pairs_ok: every activation pointer of the call is aligned to two elements
-static inline bool make_plan(const KGeom &q, Plan &pl, bool pairs_ok = true)
+static const int kDot2RH = 2;   // rows per thread of the bf16 dot2 kernels (columns: 2)
+
+static inline bool make_plan(const KGeom &q, Plan &pl, bool pairs_ok = true, int dtype = NDC_F32)
 {
     pl.m = march_of(q);
+    pl.dot2 = false;
     // 32-bit offsets inside one (sample, channel) volume
     if ((long long)q.sc * q.SP >= (1LL << 31)) return false;
     if (!find_variant(q, pl.m, pairs_ok, pl.v)) return false;
@@ -120,6 +125,18 @@ static inline bool make_plan(const KGeom &q, Plan &pl, bool pairs_ok = true)
         plan_lds<kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_>(pl);
     NDC_FUSED_VARIANTS(X)
 #undef X
+    if (dtype == NDC_BF16 && pairs_ok && pl.m.W % 2 == 0 && q.sc == 4 && pl.m.KD == 3 &&
+        pl.m.KH == 3 && pl.m.KW == 3 && env_int("NDC_TUNE_DOT2", 1)) {
+        Tile tf;
+        if (make_tile(pl.m, kDot2RH, 2, tn.threads_f, tf)) {
+            const int lds = FwdKernelB<kDot2RH>::lds_floats(tf);
+            if (lds <= kMaxLdsBytes / 4) {
+                pl.dot2 = true;
+                pl.tf = tf;
+                pl.lds_f = lds;
+            }
+        }
+    }
     const int cap = kMaxLdsBytes / 4;
     if (pl.lds_f > cap || pl.lds_b1 > cap || pl.lds_b2 > cap) return false;
     const long long nbc = (long long)q.B * q.G;
@@ -156,15 +173,35 @@ static inline size_t backward_ws(const KGeom &q, int dtype, int /*need_gh*/, int
     return align256(n_x * esz) + align256(nblk * kt * 4) + align256(nblk * (kt + q.sc) * 4);
 }
 
+// bytes of scratch the forward call needs (the packed tap tables of the bf16 dot2 kernels)
+static inline size_t forward_ws(const KGeom &q, int dtype)
+{
+    Plan pl;
+    if (!make_plan(q, pl, true, dtype) || !pl.dot2) return 0;
+    return align256((size_t)q.G * kTabWords * 4);
+}
+
+template <class BE, typename T> struct Dot2Launch {
+    static int fwd(const FwdParams<T> &, const Plan &, void *) { return NDC_ERR_GEOMETRY; }
+};
+template <class BE> struct Dot2Launch<BE, bf16_t> {
+    static int fwd(const FwdParams<bf16_t> &p, const Plan &pl, void *stream)
+    {
+        return BE::template block_kernel<FwdKernelB<kDot2RH>>(p, pl.nblk_f, pl.tf.NT, pl.lds_f, stream);
+    }
+};
+
 template <class BE, typename T>
 static int forward(const KGeom &q, const T *x, const T *z, const float *h, const float *bias,
-                   T *out, T *t1, void *stream)
+                   T *out, T *t1, void *ws, void *stream)
 {
     Plan pl;
     const bool pairs = pair_aligned<T>(x) && pair_aligned<T>(z) && pair_aligned<T>(out) &&
                        pair_aligned<T>(t1);
-    if (!make_plan(q, pl, pairs)) return NDC_ERR_GEOMETRY;
+    const int dtype = sizeof(T) == 2 ? NDC_BF16 : NDC_F32;
+    if (!make_plan(q, pl, pairs, ws ? dtype : NDC_F32)) return NDC_ERR_GEOMETRY;
     FwdParams<T> p;
+    p.wtab = nullptr;
     p.x = x;
     p.z = z;
     p.h = h;
@@ -179,6 +216,14 @@ static int forward(const KGeom &q, const T *x, const T *z, const float *h, const
     p.relu = q.relu;
     p.eps = q.eps;
     p.t = pl.tf;
+    if (pl.dot2) {
+        float *tab = (float *)ws;
+        const int st = BE::elementwise((long long)q.G * kTabWords, stream,
+                                       [=] NDC_LAMBDA(long long idx) { prep_tables(idx, h, tab); });
+        if (st) return st;
+        p.wtab = tab;
+        return Dot2Launch<BE, T>::fwd(p, pl, stream);
+    }
 #define X(kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_)                                          \
     if (NDC_IS_VARIANT(pl, kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_))                        \
         return BE::template block_kernel<FwdKernel<kd_, kh_, kw_, sc_, rhf_, rwf_, T>>(        \
@@ -219,6 +264,7 @@ static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const f
     p.gx = gx;
     p.gz = gz;
     p.gt1 = gt1;
+    p.wtab = nullptr;
     p.need_gh = gh != nullptr;
     p.need_gb = gb != nullptr;
     p.B = q.B;

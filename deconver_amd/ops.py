@@ -74,7 +74,13 @@ def update_forward(lib: _lib.NdcLibrary, x: Tensor, z: Tensor, h: Tensor,
     out = torch.empty_like(z)
     want_t1 = need_t1 or not lib.fused_supported(g) or path == _lib.PATH_DIRECT
     t1 = torch.empty_like(x) if want_t1 else None
-    lib.forward(g, _ptr(x), _ptr(z), _ptr(h), _ptr(bias), _ptr(out), _ptr(t1), _stream_of(x))
+    nbytes = lib.forward_workspace_bytes(g)
+    ws_ptr = None
+    if nbytes:
+        ws = torch.empty(nbytes + 256, dtype=torch.uint8, device=x.device)
+        ws_ptr = (ws.data_ptr() + 255) // 256 * 256
+    lib.forward(g, _ptr(x), _ptr(z), _ptr(h), _ptr(bias), _ptr(out), _ptr(t1), ws_ptr, nbytes,
+                _stream_of(x))
     return out, t1
 
 

@@ -73,6 +73,10 @@ int ndc_fused_supported(const ndc_geom *g);
 /* 0 if some path covers `g` (then every entry point below accepts it), else a status. */
 int ndc_check_geometry(const ndc_geom *g);
 
+/* Bytes of scratch `ndc_forward` needs for `g` (0 for most geometries; the bfloat16 3x3x3
+ * kernels keep their packed filter tables there). */
+size_t ndc_forward_workspace_bytes(const ndc_geom *g);
+
 /*
  * Forward update.  Replaces DeconvUpdate.forward
  * (deconver/deconvolution/functional.py:105-116), i.e. the pair
@@ -83,9 +87,12 @@ int ndc_check_geometry(const ndc_geom *g);
  *   t1            optional output K(s), same shape/dtype as x: pass it when a backward
  *                 call will follow (it is what the reference saves for backward), null
  *                 for inference
+ *   workspace     >= ndc_forward_workspace_bytes(g) bytes, 256-byte aligned (may be null
+ *                 when that is 0)
  */
 int ndc_forward(const ndc_geom *g, const void *x, const void *z, const float *h,
-                const float *bias, void *out, void *t1, void *stream);
+                const float *bias, void *out, void *t1, void *workspace, size_t workspace_bytes,
+                void *stream);
 
 /* Bytes of scratch `ndc_backward` needs for `g` with the requested outputs (each flag
  * nonzero when the matching output pointer will be non-null). */

