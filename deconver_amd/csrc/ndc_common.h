@@ -156,6 +156,16 @@ NDC_HD float relu_f(float v)
 #endif
 }
 
+// max(v, lo): one v_max_f32
+NDC_HD float floor_f(float v, float lo)
+{
+#if NDC_DEVICE_BUILD && defined(__HIP_DEVICE_COMPILE__)
+    return __builtin_fmaxf(v, lo);
+#else
+    return v > lo ? v : lo;
+#endif
+}
+
 NDC_HD float fast_rcp(float v)
 {
 #if NDC_DEVICE_BUILD && defined(__HIP_DEVICE_COMPILE__)

@@ -314,7 +314,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
         UniformF hw = as_uniform(p.h + (long long)id.c * SC * KT);
         const int r0 = id.r0;
         const int nthreads = ex.nthreads;
-        const int relu = p.relu;
+        const float floor_ = p.relu ? 0.f : -3.0e38f;   // max(s, floor_) rectifies or passes through
         const float eps = p.eps;
 
         // global -> registers: plane k of s (bias / ReLU applied) and plane k - PD of x.
@@ -332,7 +332,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                         NDC_UNROLL
                         for (int c = 0; c < RW; ++c) {
                             float s = v[c] + st.bv[i];
-                            if (relu) s = relu_f(s);
+                            s = floor_f(s, floor_);
                             st.pz[i][n][c] = s;
                         }
                     }
@@ -495,7 +495,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                         NDC_UNROLL
                         for (int c = 0; c < RW; ++c) {
                             float s = sv[i][r][c] + st.bv[i];
-                            if (relu) s = relu_f(s);
+                            s = floor_f(s, floor_);
                             sv[i][r][c] = s;
                         }
                     }
@@ -591,7 +591,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
         UniformF hw = as_uniform(p.h + (long long)id.c * SC * KT);
         const int r0 = id.r0;
         const int nthreads = ex.nthreads;
-        const int relu = p.relu;
+        const float floor_ = p.relu ? 0.f : -3.0e38f;   // max(s, floor_) rectifies or passes through
         const float eps = p.eps;
         const int need_gh = p.need_gh;
 
@@ -648,7 +648,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                     NDC_UNROLL
                     for (int c = 0; c < RW; ++c) {
                         float s = sv[i][r][c] + st.bv[i];
-                        if (relu) s = relu_f(s);
+                        s = floor_f(s, floor_);
                         sv[i][r][c] = s;
                         gv[i][r][c] = ok ? gv[i][r][c] : 0.f;
                     }
@@ -867,7 +867,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
         UniformF hw = as_uniform(p.h + (long long)id.c * SC * KT);
         const int r0 = id.r0;
         const int nthreads = ex.nthreads;
-        const int relu = p.relu;
+        const float floor_ = p.relu ? 0.f : -3.0e38f;   // max(s, floor_) rectifies or passes through
         const float eps = p.eps;
         const int need_gh = p.need_gh;
 
@@ -955,7 +955,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                         for (int c = 0; c < RW; ++c) {
                             // with the ReLU on, s <= 0 marks a masked element
                             float s = sv[i][r][c] + st.bv[i];
-                            if (relu) s = relu_f(s);
+                            s = floor_f(s, floor_);
                             sv[i][r][c] = ok ? s : 0.f;
                             gv[i][r][c] = ok ? gv[i][r][c] : 0.f;
                         }
@@ -1019,7 +1019,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                         for (int c = 0; c < RW; ++c) {
                             float gzv = gv[i][r][c] * (acc[0][i][r][c] + eps) * fast_rcp(acc[1][i][r][c] + eps) +
                                         acc[2][i][r][c];
-                            if (relu && !(sv[i][r][c] > 0.f)) gzv = 0.f;
+                            if (p.relu && !(sv[i][r][c] > 0.f)) gzv = 0.f;
                             st.gbacc[i] += gzv;
                             v[c] = gzv;
                         }

@@ -127,13 +127,20 @@ static inline bool make_plan(const KGeom &q, Plan &pl, bool pairs_ok = true, int
 #undef X
     if (dtype == NDC_BF16 && pairs_ok && pl.m.W % 2 == 0 && q.sc == 4 && pl.m.KD == 3 &&
         pl.m.KH == 3 && pl.m.KW == 3 && env_int("NDC_TUNE_DOT2", 1)) {
-        Tile tf;
-        if (make_tile(pl.m, kDot2RH, 2, tn.threads_f, tf)) {
-            const int lds = FwdKernelB<kDot2RH>::lds_floats(tf);
-            if (lds <= kMaxLdsBytes / 4) {
+        Tile tf, tb;
+        if (make_tile(pl.m, kDot2RH, 2, tn.threads_f, tf) &&
+            make_tile(pl.m, kDot2RH, 2, tn.threads_b, tb)) {
+            const int lf = FwdKernelB<kDot2RH>::lds_floats(tf);
+            const int l1 = Bwd1KernelB<kDot2RH>::lds_floats(tb);
+            const int l2 = Bwd2KernelB<kDot2RH>::lds_floats(tb);
+            const int cap2 = kMaxLdsBytes / 4;
+            if (lf <= cap2 && l1 <= cap2 && l2 <= cap2) {
                 pl.dot2 = true;
                 pl.tf = tf;
-                pl.lds_f = lds;
+                pl.tb = tb;
+                pl.lds_f = lf;
+                pl.lds_b1 = l1;
+                pl.lds_b2 = l2;
             }
         }
     }
@@ -164,13 +171,14 @@ static inline size_t backward_ws(const KGeom &q, int dtype, int /*need_gh*/, int
 {
     // sized for whichever variant the call ends up with (aligned pairs or not)
     Plan a, b;
-    if (!make_plan(q, a, false)) return 0;
-    const bool has_b = make_plan(q, b, true);
+    if (!make_plan(q, a, false, dtype)) return 0;
+    const bool has_b = make_plan(q, b, true, dtype);
     const size_t nblk = has_b && b.nblk_b > a.nblk_b ? b.nblk_b : a.nblk_b;
     const size_t esz = dtype == NDC_BF16 ? 2 : 4;
     const size_t n_x = (size_t)q.B * q.G * q.SP;
     const size_t kt = (size_t)q.sc * q.KT;
-    return align256(n_x * esz) + align256(nblk * kt * 4) + align256(nblk * (kt + q.sc) * 4);
+    const size_t tabs = has_b && b.dot2 ? align256((size_t)q.G * kTabWords * 4) : 0;
+    return align256(n_x * esz) + align256(nblk * kt * 4) + align256(nblk * (kt + q.sc) * 4) + tabs;
 }
 
 // bytes of scratch the forward call needs (the packed tap tables of the bf16 dot2 kernels)
@@ -183,11 +191,21 @@ static inline size_t forward_ws(const KGeom &q, int dtype)
 
 template <class BE, typename T> struct Dot2Launch {
     static int fwd(const FwdParams<T> &, const Plan &, void *) { return NDC_ERR_GEOMETRY; }
+    static int bwd1(const BwdParams<T> &, const Plan &, void *) { return NDC_ERR_GEOMETRY; }
+    static int bwd2(const BwdParams<T> &, const Plan &, void *) { return NDC_ERR_GEOMETRY; }
 };
 template <class BE> struct Dot2Launch<BE, bf16_t> {
     static int fwd(const FwdParams<bf16_t> &p, const Plan &pl, void *stream)
     {
         return BE::template block_kernel<FwdKernelB<kDot2RH>>(p, pl.nblk_f, pl.tf.NT, pl.lds_f, stream);
+    }
+    static int bwd1(const BwdParams<bf16_t> &p, const Plan &pl, void *stream)
+    {
+        return BE::template block_kernel<Bwd1KernelB<kDot2RH>>(p, pl.nblk_b, pl.tb.NT, pl.lds_b1, stream);
+    }
+    static int bwd2(const BwdParams<bf16_t> &p, const Plan &pl, void *stream)
+    {
+        return BE::template block_kernel<Bwd2KernelB<kDot2RH>>(p, pl.nblk_b, pl.tb.NT, pl.lds_b2, stream);
     }
 };
 
@@ -244,7 +262,8 @@ static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const f
     Plan pl;
     const bool pairs = pair_aligned<T>(x) && pair_aligned<T>(z) && pair_aligned<T>(t1) &&
                        pair_aligned<T>(gout) && pair_aligned<T>(gx) && pair_aligned<T>(gz);
-    if (!make_plan(q, pl, pairs)) return NDC_ERR_GEOMETRY;
+    const int dtype = sizeof(T) == 2 ? NDC_BF16 : NDC_F32;
+    if (!make_plan(q, pl, pairs, dtype)) return NDC_ERR_GEOMETRY;
     const size_t n_x = (size_t)q.B * q.G * q.SP;
     const int kt = q.sc * q.KT;
     char *w = (char *)ws;
@@ -253,6 +272,8 @@ static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const f
     float *part1 = (float *)w;
     w += align256((size_t)pl.nblk_b * kt * 4);
     float *part2 = (float *)w;
+    w += align256((size_t)pl.nblk_b * (kt + q.sc) * 4);
+    float *tab = (float *)w;
 
     BwdParams<T> p;
     p.x = x;
@@ -279,12 +300,20 @@ static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const f
     int st = NDC_ERR_GEOMETRY;
     p.part = part1;
     p.part_stride = kt;
+    if (pl.dot2) {
+        st = BE::elementwise((long long)q.G * kTabWords, stream,
+                             [=] NDC_LAMBDA(long long idx) { prep_tables(idx, h, tab); });
+        if (st) return st;
+        p.wtab = tab;
+        st = Dot2Launch<BE, T>::bwd1(p, pl, stream);
+    } else {
 #define X(kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_)                                          \
     if (NDC_IS_VARIANT(pl, kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_))                        \
         st = BE::template block_kernel<Bwd1Kernel<kd_, kh_, kw_, sc_, rhb_, rwb_, T>>(         \
             p, pl.nblk_b, pl.tb.NT, pl.lds_b1, stream);
-    NDC_FUSED_VARIANTS(X)
+        NDC_FUSED_VARIANTS(X)
 #undef X
+    }
     if (st) return st;
     tm.mark();
     if (!gz && !gh && !gb) {
@@ -295,12 +324,16 @@ static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const f
     p.part = part2;
     p.part_stride = kt + q.sc;
     st = NDC_ERR_GEOMETRY;
+    if (pl.dot2) {
+        st = Dot2Launch<BE, T>::bwd2(p, pl, stream);
+    } else {
 #define X(kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_)                                          \
     if (NDC_IS_VARIANT(pl, kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_))                        \
         st = BE::template block_kernel<Bwd2Kernel<kd_, kh_, kw_, sc_, rhb_, rwb_, T>>(         \
             p, pl.nblk_b, pl.tb.NT, pl.lds_b2, stream);
-    NDC_FUSED_VARIANTS(X)
+        NDC_FUSED_VARIANTS(X)
 #undef X
+    }
     if (st) return st;
     tm.mark();
 

@@ -65,6 +65,15 @@ NDC_HD uint32_t zip_hi(uint32_t a, uint32_t b)
     return (a >> 16) | (b & 0xffff0000u);
 #endif
 }
+// one 32-bit global access at a uniform base plus a 32-bit byte offset
+template <typename T> NDC_HD uint32_t ld_word(const T *base, unsigned byte_off)
+{
+    return *reinterpret_cast<const uint32_t *>(reinterpret_cast<const char *>(base) + byte_off);
+}
+template <typename T> NDC_HD void st_word(T *base, unsigned byte_off, uint32_t w)
+{
+    *reinterpret_cast<uint32_t *>(reinterpret_cast<char *>(base) + byte_off) = w;
+}
 NDC_HD float bf_lo(uint32_t w) { return bits_to_float(w << 16); }
 NDC_HD float bf_hi(uint32_t w) { return bits_to_float(w & 0xffff0000u); }
 
@@ -140,7 +149,7 @@ template <int RH_> struct FwdKernelB {
 
     struct State {
         Lane ln;
-        int zoff[NZR], xoff[NXR], ooff[RH];
+        unsigned zoff[NZR], xoff[NXR], ooff[RH];   // BYTE offsets inside one plane (rows clamped)
         unsigned zok, xok, ook;
         float bv[SC];
         float t1acc[KD][RHK][RW];
@@ -174,7 +183,7 @@ template <int RH_> struct FwdKernelB {
         UniformF tab = as_uniform(p.wtab + (long long)id.c * kTabWords);
         const int r0 = id.r0;
         const int nthreads = ex.nthreads;
-        const int relu = p.relu;
+        const float floor_ = p.relu ? 0.f : -3.0e38f;   // max(s, floor_) rectifies or passes through
         const float eps = p.eps;
 
         auto load_plane = [&](State &st, int k) {
@@ -185,14 +194,14 @@ template <int RH_> struct FwdKernelB {
                 for (int n = 0; n < NZR; ++n)
                     NDC_UNROLL
                     for (int i = 0; i < SC; ++i)
-                        st.pz[i][n] = *reinterpret_cast<const uint32_t *>(zk + i * cplane + st.zoff[n]);
+                        st.pz[i][n] = ld_word(zk + i * cplane, st.zoff[n]);
             }
             const int kx = k - PD;
             if (kx >= 0 && kx < D) {
                 const T *xk = xg + (long long)kx * plane;
                 NDC_UNROLL
                 for (int n = 0; n < NXR; ++n)
-                    st.px[n] = *reinterpret_cast<const uint32_t *>(xk + st.xoff[n]);
+                    st.px[n] = ld_word(xk, st.xoff[n]);
             } else {
                 NDC_UNROLL
                 for (int n = 0; n < NXR; ++n) st.px[n] = 0u;
@@ -205,27 +214,23 @@ template <int RH_> struct FwdKernelB {
             if (!st.ln.active) return;
             const int lb = PL + st.ln.c0;
             const int sb = off_s + wrap(k % NS, NS) * 2 * RS * P;
-            const bool zin = k < D;
+            // planes past the end are never K-scattered, so their slot may keep stale words
             NDC_UNROLL
             for (int n = 0; n < NZR; ++n) {
-                if (!((st.zok >> n) & 1u)) continue;
+                if (k >= D || !((st.zok >> n) & 1u)) continue;
                 const int j = st.ln.strip + n * S;
                 float s[SC][RW];
                 NDC_UNROLL
                 for (int i = 0; i < SC; ++i) {
                     s[i][0] = bf_lo(st.pz[i][n]) + st.bv[i];
                     s[i][1] = bf_hi(st.pz[i][n]) + st.bv[i];
-                    if (relu) {
-                        s[i][0] = relu_f(s[i][0]);
-                        s[i][1] = relu_f(s[i][1]);
-                    }
+                    s[i][0] = floor_f(s[i][0], floor_);
+                    s[i][1] = floor_f(s[i][1], floor_);
                 }
                 NDC_UNROLL
                 for (int c = 0; c < RW; ++c) {
-                    const uint32_t w01 = zin ? pack_bf16x2(s[0][c], s[1][c]) : 0u;
-                    const uint32_t w23 = zin ? pack_bf16x2(s[2][c], s[3][c]) : 0u;
-                    ex.st_(sb + j * P + lb + c, bits_to_float(w01));
-                    ex.st_(sb + (RS + j) * P + lb + c, bits_to_float(w23));
+                    ex.st_(sb + j * P + lb + c, bits_to_float(pack_bf16x2(s[0][c], s[1][c])));
+                    ex.st_(sb + (RS + j) * P + lb + c, bits_to_float(pack_bf16x2(s[2][c], s[3][c])));
                 }
             }
             const int xb = off_x + wrap((k - 2) % NX, NX) * RX * P;
@@ -247,7 +252,7 @@ template <int RH_> struct FwdKernelB {
             for (int n = 0; n < NZR; ++n) {
                 const int j = st.ln.strip + n * S, row = r0 - 2 * PH + j;
                 if (j < RS && row >= 0 && row < H) st.zok |= 1u << n;
-                st.zoff[n] = clampi(row, 0, H - 1) * W + st.ln.c0;
+                st.zoff[n] = (unsigned)(clampi(row, 0, H - 1) * W + st.ln.c0) * 2u;
                 NDC_UNROLL
                 for (int i = 0; i < SC; ++i) st.pz[i][n] = 0u;
             }
@@ -255,14 +260,14 @@ template <int RH_> struct FwdKernelB {
             for (int n = 0; n < NXR; ++n) {
                 const int j = st.ln.strip + n * S, row = r0 - PH + j;
                 if (j < RX && row >= 0 && row < H) st.xok |= 1u << n;
-                st.xoff[n] = clampi(row, 0, H - 1) * W + st.ln.c0;
+                st.xoff[n] = (unsigned)(clampi(row, 0, H - 1) * W + st.ln.c0) * 2u;
                 st.px[n] = st.pxprev[n] = 0u;
             }
             NDC_UNROLL
             for (int r = 0; r < RH; ++r) {
                 const int row = r0 + st.ln.strip * RH + r;
                 if (row < H) st.ook |= 1u << r;
-                st.ooff[r] = clampi(row, 0, H - 1) * W + st.ln.c0;
+                st.ooff[r] = (unsigned)(clampi(row, 0, H - 1) * W + st.ln.c0) * 2u;
             }
             NDC_UNROLL
             for (int i = 0; i < SC; ++i) st.bv[i] = p.bias ? p.bias[id.c * SC + i] : 0.f;
@@ -330,7 +335,7 @@ template <int RH_> struct FwdKernelB {
                         if (mine) ex.st_(tb + j * P + c, bits_to_float(pack_bf16x2(st.t1prev[r][c], v[c])));
                         st.t1prev[r][c] = v[c];
                     }
-                    if (r < RH && t1g && live) IO::store(t1g + (long long)pf * plane + st.ooff[r < RH ? r : 0], v);
+                    if (r < RH && t1g && live) st_word(t1g + (long long)pf * plane, st.ooff[r < RH ? r : 0], pack_bf16x2(v[0], v[1]));
                     NDC_UNROLL
                     for (int c = 0; c < RW; ++c) {
                         st.t1acc[0][r][c] = st.t1acc[1][r][c];
@@ -355,7 +360,7 @@ template <int RH_> struct FwdKernelB {
                         NDC_UNROLL
                         for (int r = 0; r < RH; ++r)
                             NDC_UNROLL
-                            for (int c = 0; c < RW; ++c) acc[a][i][r][c] = 0.f;
+                            for (int c = 0; c < RW; ++c) acc[a][i][r][c] = eps;   // n, d start at eps
                 NDC_ROLLED
                 for (int s = 0; s < 2; ++s) {
                     float wt[SC][9];
@@ -377,12 +382,536 @@ template <int RH_> struct FwdKernelB {
                         for (int c = 0; c < RW; ++c) {
                             const uint32_t w = st.own[i >> 1][r][c];
                             const float s = (i & 1) ? bf_hi(w) : bf_lo(w);
-                            v[c] = s * (acc[0][i][r][c] + eps) * fast_rcp(acc[1][i][r][c] + eps);
+                            v[c] = s * acc[0][i][r][c] * fast_rcp(acc[1][i][r][c]);
                         }
-                        IO::store(ok_ + i * cplane + st.ooff[r], v);
+                        st_word(ok_ + i * cplane, st.ooff[r], pack_bf16x2(v[0], v[1]));
                     }
                 }
             });
+        }
+    }
+};
+
+// =================================================================== backward pass 1 (bf16, dot2)
+
+template <int RH_> struct Bwd1KernelB {
+    static constexpr int KD = 3, KH = 3, KW = 3, SC = 4, RH = RH_, RW = 2;
+    static constexpr int PD = 1, PH = 1, PW = 1, KT = 27;
+    static constexpr int NXR = RH + 2;
+    static constexpr int NP = 2, NXT = 3;   // ring slots: plane pairs of x / t1; (x, t1) words
+    static constexpr int NRED = SC * KT;
+    typedef bf16_t T;
+    typedef BwdParams<T> Params;
+
+    struct State {
+        Lane ln;
+        unsigned xoff[NXR], ooff[RH];   // byte offsets inside one plane
+        unsigned xok, ook;
+        float bv[SC];
+        float gacc[SC][KT];
+        float accx[KD][RH][RW], acct[KD][RH][RW];
+        uint32_t px[NXR], pt[NXR], pxprev[NXR], ptprev[NXR];
+    };
+
+    static NDC_HD int rows_x(int TH) { return TH + 4; }
+    static NDC_HD int rows_g(int TH) { return TH + 2; }
+    static NDC_HD int lds_floats(const Tile &t)
+    {
+        const int main_ = ((2 * NP + NXT) * rows_x(t.TH) + 4 * rows_g(t.TH)) * t.P;
+        const int red = (t.NT / 64) * NRED;
+        return main_ > red ? main_ : red;
+    }
+
+    template <class Exec> static NDC_D void run(Exec &ex, const Params &p, int block_id)
+    {
+        const Tile t = p.t;
+        const BlockId id = decode_block(block_id, p.C, t);
+        const int S = t.S, P = t.P, PL = t.PL, TH = t.TH, W = p.W, H = p.H, D = p.D;
+        const int RX = rows_x(TH), RG = rows_g(TH);
+        const int off_xp = 0, off_tp = NP * RX * P, off_xt = 2 * NP * RX * P;
+        const int off_g = off_xt + NXT * RX * P;
+        const int total = off_g + 4 * RG * P;
+        const int plane = H * W;
+        const long long cplane = (long long)D * plane;
+        const long long cbase = ((long long)id.b * p.C + id.c) * cplane;
+        const T *xg = p.x + cbase, *t1g = p.t1 + cbase;
+        const T *zg = p.z + cbase * SC, *gg = p.gout + cbase * SC;
+        T *gxg = p.gx ? p.gx + cbase : nullptr;
+        T *gt1g = p.gt1 + cbase;
+        UniformF tab = as_uniform(p.wtab + (long long)id.c * kTabWords);
+        const int r0 = id.r0;
+        const int nthreads = ex.nthreads;
+        const float floor_ = p.relu ? 0.f : -3.0e38f;
+        const float eps = p.eps;
+        const int need_gh = p.need_gh;
+
+        auto load_plane = [&](State &st, int k) {
+            if (!st.ln.active) return;
+            if (k < D) {
+                const T *xk = xg + (long long)k * plane, *tk = t1g + (long long)k * plane;
+                NDC_UNROLL
+                for (int n = 0; n < NXR; ++n) {
+                    st.px[n] = ld_word(xk, st.xoff[n]);
+                    st.pt[n] = ld_word(tk, st.xoff[n]);
+                }
+            } else {
+                NDC_UNROLL
+                for (int n = 0; n < NXR; ++n) st.px[n] = st.pt[n] = 0u;
+            }
+        };
+        // plane k arrives: plane-pair words (v[k-1], v[k]) into pair slot (k-1) % 2 and the
+        // operand-pair words (x[k], t1[k]) into slot k % 3
+        auto store_plane = [&](State &st, int k) {
+            if (!st.ln.active) return;
+            const int ps = wrap((k - 1) % NP, NP) * RX * P, xs = wrap(k % NXT, NXT) * RX * P;
+            NDC_UNROLL
+            for (int n = 0; n < NXR; ++n) {
+                if ((st.xok >> n) & 1u) {
+                    const int o = (st.ln.strip + n * S) * P + PL + st.ln.c0;
+                    ex.st_(off_xp + ps + o, bits_to_float(zip_lo(st.pxprev[n], st.px[n])));
+                    ex.st_(off_xp + ps + o + 1, bits_to_float(zip_hi(st.pxprev[n], st.px[n])));
+                    ex.st_(off_tp + ps + o, bits_to_float(zip_lo(st.ptprev[n], st.pt[n])));
+                    ex.st_(off_tp + ps + o + 1, bits_to_float(zip_hi(st.ptprev[n], st.pt[n])));
+                    ex.st_(off_xt + xs + o, bits_to_float(zip_lo(st.px[n], st.pt[n])));
+                    ex.st_(off_xt + xs + o + 1, bits_to_float(zip_hi(st.px[n], st.pt[n])));
+                }
+                st.pxprev[n] = st.px[n];
+                st.ptprev[n] = st.pt[n];
+            }
+        };
+
+        // gn, gd of NR rows from gn/gd tile row j (image row r0 - 1 + j): published to LDS as
+        // channel-pair words; returned as operand pairs GG[i][r][c] = (gn_i, gd_i)
+        auto gn_gd_rows = [&](State &st, int j1, int j, auto nr_tag,
+                              uint32_t (&gg_out)[SC][decltype(nr_tag)::value][RW]) {
+            constexpr int NR = decltype(nr_tag)::value;
+            uint32_t zw[SC][NR], gw[SC][NR];
+            const T *zk = zg + (long long)j1 * plane, *gk = gg + (long long)j1 * plane;
+            bool ok[NR];
+            NDC_UNROLL
+            for (int r = 0; r < NR; ++r) {
+                const int row = r0 - PH + j + r;
+                ok[r] = row >= 0 && row < H;
+                const unsigned o = (unsigned)(clampi(row, 0, H - 1) * W + st.ln.c0) * 2u;
+                NDC_UNROLL
+                for (int i = 0; i < SC; ++i) {
+                    zw[i][r] = ld_word(zk + i * cplane, o);
+                    gw[i][r] = ld_word(gk + i * cplane, o);
+                }
+            }
+            float acc[2][SC][NR][RW];
+            NDC_UNROLL
+            for (int a = 0; a < 2; ++a)
+                NDC_UNROLL
+                for (int i = 0; i < SC; ++i)
+                    NDC_UNROLL
+                    for (int r = 0; r < NR; ++r)
+                        NDC_UNROLL
+                        for (int c = 0; c < RW; ++c) acc[a][i][r][c] = eps;
+            NDC_ROLLED
+            for (int s = 0; s < 2; ++s) {
+                float wt[SC][9];
+                load_plane_taps<SC, 9, 9>(tab + 54 + s * 36, wt);
+                const int m = j1 - 1 + s;
+                const int ob = (wrap(m % NP, NP) * RX + j) * P + PL + st.ln.c0 - PW;
+                const int base[2] = {off_xp + ob, off_tp + ob};
+                a_plane_d2<NR, RW, 2>(ex, base, P, wt, acc);
+            }
+            NDC_UNROLL
+            for (int r = 0; r < NR; ++r) {
+                float gn[SC][RW], gd[SC][RW];
+                NDC_UNROLL
+                for (int i = 0; i < SC; ++i)
+                    NDC_UNROLL
+                    for (int c = 0; c < RW; ++c) {
+                        const float sv = floor_f((c ? bf_hi(zw[i][r]) : bf_lo(zw[i][r])) + st.bv[i], floor_);
+                        const float gv = ok[r] ? (c ? bf_hi(gw[i][r]) : bf_lo(gw[i][r])) : 0.f;
+                        const float inv = fast_rcp(acc[1][i][r][c]);
+                        gn[i][c] = gv * sv * inv;
+                        gd[i][c] = -(gn[i][c] * acc[0][i][r][c]) * inv;
+                        gg_out[i][r][c] = pack_bf16x2(gn[i][c], gd[i][c]);
+                    }
+                NDC_UNROLL
+                for (int c = 0; c < RW; ++c) {
+                    const int o = off_g + (j + r) * P + PL + st.ln.c0 + c;
+                    ex.st_(o, bits_to_float(pack_bf16x2(gn[0][c], gn[1][c])));
+                    ex.st_(o + RG * P, bits_to_float(pack_bf16x2(gn[2][c], gn[3][c])));
+                    ex.st_(o + 2 * RG * P, bits_to_float(pack_bf16x2(gd[0][c], gd[1][c])));
+                    ex.st_(o + 3 * RG * P, bits_to_float(pack_bf16x2(gd[2][c], gd[3][c])));
+                }
+            }
+        };
+
+        ex.each([&](State &st, int tid) {
+            st.ln = make_lane(tid, t, RW);
+            st.xok = st.ook = 0u;
+            NDC_UNROLL
+            for (int n = 0; n < NXR; ++n) {
+                const int j = st.ln.strip + n * S, row = r0 - 2 * PH + j;
+                if (j < RX && row >= 0 && row < H) st.xok |= 1u << n;
+                st.xoff[n] = (unsigned)(clampi(row, 0, H - 1) * W + st.ln.c0) * 2u;
+                st.px[n] = st.pt[n] = st.pxprev[n] = st.ptprev[n] = 0u;
+            }
+            NDC_UNROLL
+            for (int r = 0; r < RH; ++r) {
+                const int row = r0 + st.ln.strip * RH + r;
+                if (row < H) st.ook |= 1u << r;
+                st.ooff[r] = (unsigned)(clampi(row, 0, H - 1) * W + st.ln.c0) * 2u;
+            }
+            NDC_UNROLL
+            for (int i = 0; i < SC; ++i) {
+                st.bv[i] = p.bias ? p.bias[id.c * SC + i] : 0.f;
+                NDC_UNROLL
+                for (int a = 0; a < KT; ++a) st.gacc[i][a] = 0.f;
+            }
+            NDC_UNROLL
+            for (int a = 0; a < KD; ++a)
+                NDC_UNROLL
+                for (int r = 0; r < RH; ++r)
+                    NDC_UNROLL
+                    for (int c = 0; c < RW; ++c) st.accx[a][r][c] = st.acct[a][r][c] = 0.f;
+            for (int i = tid; i < total; i += nthreads) ex.st_(i, 0.f);
+            load_plane(st, 0);
+        });
+        ex.sync();
+
+        for (int k = 0; k < D + 2; ++k) {
+            ex.each([&](State &st, int) { store_plane(st, k); });
+            ex.sync();
+
+            const int j1 = k - 1;
+            const bool live1 = j1 >= 0 && j1 < D;
+            ex.each([&](State &st, int) {
+                if (!st.ln.active || !live1) return;
+                {
+                    uint32_t gg2[SC][RH][RW];
+                    const int j = PH + st.ln.strip * RH;
+                    gn_gd_rows(st, j1, j, IntTag<RH>(), gg2);
+                    if (need_gh) {
+                        // A-side filter-gradient terms: (gn_i, gd_i) . (x, t1)[neighbour]
+                        NDC_UNROLL
+                        for (int td = 0; td < KD; ++td) {
+                            const int ob = off_xt + (wrap((j1 + 1 - td) % NXT, NXT) * RX + j) * P + PL +
+                                           st.ln.c0 - PW;
+                            NDC_UNROLL
+                            for (int q = 0; q < RH + 2; ++q) {
+                                uint32_t v[RW + 2];
+                                NDC_UNROLL
+                                for (int u = 0; u < RW + 2; ++u) v[u] = float_to_bits(ex.ld(ob + q * P + u));
+                                NDC_UNROLL
+                                for (int th = 0; th < KH; ++th) {
+                                    const int rr = q - 2 + th;
+                                    if (rr < 0 || rr >= RH) continue;
+                                    NDC_UNROLL
+                                    for (int tw = 0; tw < KW; ++tw)
+                                        NDC_UNROLL
+                                        for (int i = 0; i < SC; ++i)
+                                            NDC_UNROLL
+                                            for (int c = 0; c < RW; ++c)
+                                                st.gacc[i][(td * KH + th) * KW + tw] = dot2_bf16(
+                                                    v[c + 2 - tw], gg2[i][rr][c],
+                                                    st.gacc[i][(td * KH + th) * KW + tw]);
+                                }
+                            }
+                        }
+                    }
+                }
+                if (st.ln.strip < 2) {
+                    uint32_t gg1[SC][1][RW];
+                    gn_gd_rows(st, j1, halo_row(st.ln.strip, PH, TH), IntTag<1>(), gg1);
+                }
+            });
+            ex.sync();
+
+            ex.each([&](State &st, int) {
+                if (!st.ln.active) return;
+                load_plane(st, k + 1);
+                if (live1) {
+                    const int gb_ = off_g + (st.ln.strip * RH) * P + PL + st.ln.c0 - PW;
+                    float wp[KT], wn[KT];
+                    load_taps<KT>(tab, wp);
+                    NDC_ROLLED
+                    for (int pr = 0; pr < 2; ++pr) {
+                        load_taps<KT>(tab + uniform_int((pr + 1) & 1) * KT, wn);
+                        k_rows_d2<RH, RW, RH>(ex, gb_ + pr * RG * P, P, wp, st.accx, 0);
+                        k_rows_d2<RH, RW, RH>(ex, gb_ + (2 + pr) * RG * P, P, wp, st.acct, 0);
+                        copy_taps<KT>(wn, wp);
+                    }
+                }
+                const int pf = k - 2;
+                NDC_UNROLL
+                for (int r = 0; r < RH; ++r) {
+                    if (pf >= 0 && ((st.ook >> r) & 1u)) {
+                        if (gxg) st_word(gxg + (long long)pf * plane, st.ooff[r],
+                                         pack_bf16x2(st.accx[0][r][0], st.accx[0][r][1]));
+                        st_word(gt1g + (long long)pf * plane, st.ooff[r],
+                                pack_bf16x2(st.acct[0][r][0], st.acct[0][r][1]));
+                    }
+                    NDC_UNROLL
+                    for (int c = 0; c < RW; ++c) {
+                        st.accx[0][r][c] = st.accx[1][r][c];
+                        st.accx[1][r][c] = st.accx[2][r][c];
+                        st.accx[2][r][c] = 0.f;
+                        st.acct[0][r][c] = st.acct[1][r][c];
+                        st.acct[1][r][c] = st.acct[2][r][c];
+                        st.acct[2][r][c] = 0.f;
+                    }
+                }
+            });
+        }
+
+        if (need_gh) {
+            float *dst = p.part + (long long)block_id * p.part_stride;
+            ex.template block_reduce<NRED>(
+                [](State &st, int i) { return st.gacc[i / KT][i % KT]; },
+                [&](int i, float v) { dst[i] = v; });
+        }
+    }
+};
+
+// =================================================================== backward pass 2 (bf16, dot2)
+
+template <int RH_> struct Bwd2KernelB {
+    static constexpr int KD = 3, KH = 3, KW = 3, SC = 4, RH = RH_, RW = 2;
+    static constexpr int PD = 1, PH = 1, PW = 1, KT = 27;
+    static constexpr int NXR = RH + 1;
+    static constexpr int NP = 3, NG = 4;   // ring slots: plane pairs of x / t1; of gt1
+    static constexpr int NRED = SC * KT + SC;
+    typedef bf16_t T;
+    typedef BwdParams<T> Params;
+
+    struct State {
+        Lane ln;
+        unsigned xoff[NXR], ooff[RH];
+        unsigned xok, ook;
+        float bv[SC];
+        float gacc[SC][KT];
+        float gbacc[SC];
+        float sprev[SC][RH][RW];   // own source values of the previous plane
+        uint32_t px[NXR], pt[NXR], pg[NXR], pxprev[NXR], ptprev[NXR], pgprev[NXR];
+    };
+
+    static NDC_HD int rows_x(int TH) { return TH + 2; }
+    static NDC_HD int lds_floats(const Tile &t)
+    {
+        const int main_ = (2 * NP + NG) * rows_x(t.TH) * t.P;
+        const int red = (t.NT / 64) * NRED;
+        return main_ > red ? main_ : red;
+    }
+
+    template <class Exec> static NDC_D void run(Exec &ex, const Params &p, int block_id)
+    {
+        const Tile t = p.t;
+        const BlockId id = decode_block(block_id, p.C, t);
+        const int S = t.S, P = t.P, PL = t.PL, TH = t.TH, W = p.W, H = p.H, D = p.D;
+        const int RX = rows_x(TH);
+        const int off_xp = 0, off_tp = NP * RX * P, off_gp = 2 * NP * RX * P;
+        const int total = off_gp + NG * RX * P;
+        const int plane = H * W;
+        const long long cplane = (long long)D * plane;
+        const long long cbase = ((long long)id.b * p.C + id.c) * cplane;
+        const T *xg = p.x + cbase, *t1g = p.t1 + cbase, *gt1g = p.gt1 + cbase;
+        const T *zg = p.z + cbase * SC, *gg = p.gout + cbase * SC;
+        T *gzg = p.gz ? p.gz + cbase * SC : nullptr;
+        UniformF tab = as_uniform(p.wtab + (long long)id.c * kTabWords);
+        const int r0 = id.r0;
+        const int nthreads = ex.nthreads;
+        const float floor_ = p.relu ? 0.f : -3.0e38f;
+        const float eps = p.eps;
+        const int need_gh = p.need_gh;
+
+        auto load_plane = [&](State &st, int k) {
+            if (!st.ln.active) return;
+            if (k < D) {
+                const long long ko = (long long)k * plane;
+                NDC_UNROLL
+                for (int n = 0; n < NXR; ++n) {
+                    st.px[n] = ld_word(xg + ko, st.xoff[n]);
+                    st.pt[n] = ld_word(t1g + ko, st.xoff[n]);
+                    st.pg[n] = ld_word(gt1g + ko, st.xoff[n]);
+                }
+            } else {
+                NDC_UNROLL
+                for (int n = 0; n < NXR; ++n) st.px[n] = st.pt[n] = st.pg[n] = 0u;
+            }
+        };
+        // plane k arrives: plane-pair words (v[k-1], v[k]) into slot (k-1) % ring
+        auto store_plane = [&](State &st, int k) {
+            if (!st.ln.active) return;
+            const int ps = wrap((k - 1) % NP, NP) * RX * P, gs = wrap((k - 1) % NG, NG) * RX * P;
+            NDC_UNROLL
+            for (int n = 0; n < NXR; ++n) {
+                if ((st.xok >> n) & 1u) {
+                    const int o = (st.ln.strip + n * S) * P + PL + st.ln.c0;
+                    ex.st_(off_xp + ps + o, bits_to_float(zip_lo(st.pxprev[n], st.px[n])));
+                    ex.st_(off_xp + ps + o + 1, bits_to_float(zip_hi(st.pxprev[n], st.px[n])));
+                    ex.st_(off_tp + ps + o, bits_to_float(zip_lo(st.ptprev[n], st.pt[n])));
+                    ex.st_(off_tp + ps + o + 1, bits_to_float(zip_hi(st.ptprev[n], st.pt[n])));
+                    ex.st_(off_gp + gs + o, bits_to_float(zip_lo(st.pgprev[n], st.pg[n])));
+                    ex.st_(off_gp + gs + o + 1, bits_to_float(zip_hi(st.pgprev[n], st.pg[n])));
+                }
+                st.pxprev[n] = st.px[n];
+                st.ptprev[n] = st.pt[n];
+                st.pgprev[n] = st.pg[n];
+            }
+        };
+
+        ex.each([&](State &st, int tid) {
+            st.ln = make_lane(tid, t, RW);
+            st.xok = st.ook = 0u;
+            NDC_UNROLL
+            for (int n = 0; n < NXR; ++n) {
+                const int j = st.ln.strip + n * S, row = r0 - PH + j;
+                if (j < RX && row >= 0 && row < H) st.xok |= 1u << n;
+                st.xoff[n] = (unsigned)(clampi(row, 0, H - 1) * W + st.ln.c0) * 2u;
+                st.px[n] = st.pt[n] = st.pg[n] = st.pxprev[n] = st.ptprev[n] = st.pgprev[n] = 0u;
+            }
+            NDC_UNROLL
+            for (int r = 0; r < RH; ++r) {
+                const int row = r0 + st.ln.strip * RH + r;
+                if (row < H) st.ook |= 1u << r;
+                st.ooff[r] = (unsigned)(clampi(row, 0, H - 1) * W + st.ln.c0) * 2u;
+            }
+            NDC_UNROLL
+            for (int i = 0; i < SC; ++i) {
+                st.bv[i] = p.bias ? p.bias[id.c * SC + i] : 0.f;
+                st.gbacc[i] = 0.f;
+                NDC_UNROLL
+                for (int a = 0; a < KT; ++a) st.gacc[i][a] = 0.f;
+                NDC_UNROLL
+                for (int r = 0; r < RH; ++r)
+                    NDC_UNROLL
+                    for (int c = 0; c < RW; ++c) st.sprev[i][r][c] = 0.f;
+            }
+            for (int i = tid; i < total; i += nthreads) ex.st_(i, 0.f);
+            load_plane(st, 0);
+        });
+        ex.sync();
+
+        // one step past the usual end so that an unpaired last plane still gets its
+        // filter-gradient contribution (paired with a zero plane)
+        for (int k = 0; k < D + 2; ++k) {
+            ex.each([&](State &st, int) { store_plane(st, k); });
+            ex.sync();
+
+            const int j0 = k - 1;
+            ex.each([&](State &st, int) {
+                if (!st.ln.active) return;
+                load_plane(st, k + 1);
+                if (j0 < 0) return;
+                float sv[SC][RH][RW];
+                if (j0 < D) {
+                    uint32_t zw[SC][RH], gw[SC][RH];
+                    const T *zk = zg + (long long)j0 * plane, *gk = gg + (long long)j0 * plane;
+                    NDC_UNROLL
+                    for (int r = 0; r < RH; ++r)
+                        NDC_UNROLL
+                        for (int i = 0; i < SC; ++i) {
+                            zw[i][r] = ld_word(zk + i * cplane, st.ooff[r]);
+                            gw[i][r] = ld_word(gk + i * cplane, st.ooff[r]);
+                        }
+                    float acc[3][SC][RH][RW];
+                    NDC_UNROLL
+                    for (int a = 0; a < 3; ++a)
+                        NDC_UNROLL
+                        for (int i = 0; i < SC; ++i)
+                            NDC_UNROLL
+                            for (int r = 0; r < RH; ++r)
+                                NDC_UNROLL
+                                for (int c = 0; c < RW; ++c) acc[a][i][r][c] = a < 2 ? eps : 0.f;
+                    NDC_ROLLED
+                    for (int s = 0; s < 2; ++s) {
+                        float wt[SC][9];
+                        load_plane_taps<SC, 9, 9>(tab + 54 + s * 36, wt);
+                        const int m = j0 - 1 + s;
+                        const int ob = (st.ln.strip * RH) * P + PL + st.ln.c0 - PW;
+                        const int base[3] = {off_xp + wrap(m % NP, NP) * RX * P + ob,
+                                             off_tp + wrap(m % NP, NP) * RX * P + ob,
+                                             off_gp + wrap(m % NG, NG) * RX * P + ob};
+                        a_plane_d2<RH, RW, 3>(ex, base, P, wt, acc);
+                    }
+                    T *gzk = gzg ? gzg + (long long)j0 * plane : nullptr;
+                    NDC_UNROLL
+                    for (int r = 0; r < RH; ++r) {
+                        const bool ok = (st.ook >> r) & 1u;
+                        NDC_UNROLL
+                        for (int i = 0; i < SC; ++i) {
+                            float v[RW];
+                            NDC_UNROLL
+                            for (int c = 0; c < RW; ++c) {
+                                const float s = floor_f((c ? bf_hi(zw[i][r]) : bf_lo(zw[i][r])) + st.bv[i], floor_);
+                                const float g = c ? bf_hi(gw[i][r]) : bf_lo(gw[i][r]);
+                                float gzv = g * acc[0][i][r][c] * fast_rcp(acc[1][i][r][c]) + acc[2][i][r][c];
+                                if (p.relu && !(s > 0.f)) gzv = 0.f;
+                                if (!ok) gzv = 0.f;
+                                sv[i][r][c] = ok ? s : 0.f;
+                                st.gbacc[i] += gzv;
+                                v[c] = gzv;
+                            }
+                            if (gzk && ok) st_word(gzk + i * cplane, st.ooff[r], pack_bf16x2(v[0], v[1]));
+                        }
+                    }
+                } else {
+                    NDC_UNROLL
+                    for (int i = 0; i < SC; ++i)
+                        NDC_UNROLL
+                        for (int r = 0; r < RH; ++r)
+                            NDC_UNROLL
+                            for (int c = 0; c < RW; ++c) sv[i][r][c] = 0.f;
+                }
+                if (need_gh && (j0 & 1) && j0 <= D) {
+                    // K-side filter-gradient term for the plane pair (j0 - 1, j0):
+                    // (s_i[j0-1], s_i[j0]) . (gt1[m], gt1[m+1])[neighbour], m = j0 - td
+                    uint32_t ss[SC][RH][RW];
+                    NDC_UNROLL
+                    for (int i = 0; i < SC; ++i)
+                        NDC_UNROLL
+                        for (int r = 0; r < RH; ++r)
+                            NDC_UNROLL
+                            for (int c = 0; c < RW; ++c) ss[i][r][c] = pack_bf16x2(st.sprev[i][r][c], sv[i][r][c]);
+                    NDC_UNROLL
+                    for (int td = 0; td < KD; ++td) {
+                        const int ob = off_gp + (wrap((j0 - td) % NG, NG) * RX + st.ln.strip * RH) * P + PL +
+                                       st.ln.c0 - PW;
+                        NDC_UNROLL
+                        for (int q = 0; q < RH + 2; ++q) {
+                            uint32_t v[RW + 2];
+                            NDC_UNROLL
+                            for (int u = 0; u < RW + 2; ++u) v[u] = float_to_bits(ex.ld(ob + q * P + u));
+                            NDC_UNROLL
+                            for (int th = 0; th < KH; ++th) {
+                                const int rr = q - 2 + th;
+                                if (rr < 0 || rr >= RH) continue;
+                                NDC_UNROLL
+                                for (int tw = 0; tw < KW; ++tw)
+                                    NDC_UNROLL
+                                    for (int i = 0; i < SC; ++i)
+                                        NDC_UNROLL
+                                        for (int c = 0; c < RW; ++c)
+                                            st.gacc[i][(td * KH + th) * KW + tw] = dot2_bf16(
+                                                v[c + 2 - tw], ss[i][rr][c],
+                                                st.gacc[i][(td * KH + th) * KW + tw]);
+                            }
+                        }
+                    }
+                }
+                NDC_UNROLL
+                for (int i = 0; i < SC; ++i)
+                    NDC_UNROLL
+                    for (int r = 0; r < RH; ++r)
+                        NDC_UNROLL
+                        for (int c = 0; c < RW; ++c) st.sprev[i][r][c] = sv[i][r][c];
+            });
+        }
+
+        if (p.need_gh || p.need_gb) {
+            float *dst = p.part + (long long)block_id * p.part_stride;
+            ex.template block_reduce<NRED>(
+                [](State &st, int i) {
+                    return i < SC * KT ? st.gacc[(i < SC * KT ? i : 0) / KT][i % KT]
+                                       : st.gbacc[i >= SC * KT ? i - SC * KT : 0];
+                },
+                [&](int i, float v) { dst[i] = v; });
         }
     }
 };

@@ -68,6 +68,8 @@ int main()
         {2, 3, 1, 4, 5, 9, 8, 3, 3, 3, NDC_F32, NDC_PATH_FUSED},
         {1, 2, 1, 4, 3, 7, 13, 3, 3, 3, NDC_BF16, NDC_PATH_FUSED},
         {1, 2, 1, 4, 6, 3, 70, 3, 3, 3, NDC_F32, NDC_PATH_FUSED},
+        {1, 2, 1, 4, 5, 9, 8, 3, 3, 3, NDC_BF16, NDC_PATH_FUSED},
+        {2, 1, 1, 4, 4, 5, 70, 3, 3, 3, NDC_BF16, NDC_PATH_FUSED},
         {1, 1, 1, 4, 1, 1, 1, 3, 3, 3, NDC_F32, NDC_PATH_FUSED},
         {2, 3, 1, 4, 1, 9, 12, 1, 5, 5, NDC_F32, NDC_PATH_FUSED},
         {1, 2, 1, 4, 1, 3, 70, 1, 5, 5, NDC_BF16, NDC_PATH_FUSED},

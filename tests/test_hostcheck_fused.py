@@ -84,7 +84,17 @@ def test_fused_inference_needs_no_t1():
     assert O.rel_err(out, ref) < 1e-5
 
 
-@pytest.mark.parametrize("geom", [FUSED_GEOMS[0], FUSED_GEOMS[5]])
+BF16_GEOMS = [
+    FUSED_GEOMS[0],                       # dot2 kernels: odd plane count, ragged last band
+    FUSED_GEOMS[5],                       # 2-D 5x5 (FMA kernels, bf16 storage)
+    (2, 4, (3, 3, 3), (4, 16, 16), 1),    # dot2: even plane count
+    (1, 4, (3, 3, 3), (1, 4, 6), 1),      # dot2: single plane
+    (2, 4, (3, 3, 3), (6, 3, 70), 1),     # dot2: two wavefronts per row
+    (2, 4, (3, 3, 3), (3, 7, 13), 2),     # odd width: unpaired FMA kernels
+]
+
+
+@pytest.mark.parametrize("geom", BF16_GEOMS)
 def test_fused_bf16_storage(geom):
     C, sc, ks, sp, B = geom
     lib = hostcheck_library()
