@@ -19,6 +19,9 @@ HIPCC_FLAGS = [
     "-ffp-contract=fast",
     # packed-fp32 VALU forms are kept out of the generated code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # LLVM's VectorCombine widens scalar loads of the per-thread state into overlapping
+    # two-element loads, which pins that state in private memory instead of registers
+    "-mllvm", "-disable-vector-combine",
 ]
 
 

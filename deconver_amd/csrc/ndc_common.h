@@ -12,10 +12,14 @@
 #define NDC_HD __host__ __device__ __forceinline__
 #define NDC_D __device__ __forceinline__
 #define NDC_DEVICE_BUILD 1
+// kernel-body lambdas are inlined before any per-function optimisation, so that the
+// per-thread state they take by reference is promoted to registers as one object
+#define NDC_LAMBDA __attribute__((always_inline))
 #else
 #define NDC_HD inline
 #define NDC_D inline
 #define NDC_DEVICE_BUILD 0
+#define NDC_LAMBDA
 #endif
 
 namespace ndc {

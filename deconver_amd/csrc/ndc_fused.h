@@ -319,7 +319,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
 
         // global -> registers: plane k of s (bias / ReLU applied) and plane k - PD of x.
         // Rows outside the image read a clamped address and are zeroed by a select.
-        auto load_plane = [&](State &st, int k) {
+        auto load_plane = [&](State &st, int k) NDC_LAMBDA {
             if (!st.ln.active) return;
             if (k < D) {
                 const T *zk = zg + (long long)k * plane;
@@ -358,7 +358,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
             }
         };
 
-        auto store_plane = [&](State &st, int k) {
+        auto store_plane = [&](State &st, int k) NDC_LAMBDA {
             if (!st.ln.active) return;
             const int lb = PL + st.ln.c0;
             // rows outside the image are never written: they keep the zeros of the set-up
@@ -387,7 +387,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
 
         // ---- set-up: thread coordinates, row offsets, zeroed accumulators, zeroed LDS (halo
         //      columns and never-staged rows stay zero for the whole march)
-        ex.each([&](State &st, int tid) {
+        ex.each([&](State &st, int tid) NDC_LAMBDA {
             st.ln = make_lane(tid, t, RW);
             st.zok = st.xok = st.ook = 0u;
             NDC_UNROLL
@@ -422,11 +422,11 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
         ex.sync();
 
         for (int k = 0; k < D + 2 * PD; ++k) {
-            ex.each([&](State &st, int) { store_plane(st, k); });
+            ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k); });
             ex.sync();
 
             // ---- K-scatter: plane k of s feeds the KD pending planes of t1
-            ex.each([&](State &st, int) {
+            ex.each([&](State &st, int) NDC_LAMBDA {
                 if (!st.ln.active) return;
 #ifdef NDC_EXP_NOEXTRA
                 const bool extra = false;
@@ -478,7 +478,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
 #endif
 
             // ---- prefetch of the next plane, then A-gather + epilogue for plane k - 2*PD
-            ex.each([&](State &st, int) {
+            ex.each([&](State &st, int) NDC_LAMBDA {
                 if (!st.ln.active) return;
                 load_plane(st, k + 1);
                 const int j0 = k - 2 * PD;
@@ -595,7 +595,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
         const float eps = p.eps;
         const int need_gh = p.need_gh;
 
-        auto load_plane = [&](State &st, int k) {
+        auto load_plane = [&](State &st, int k) NDC_LAMBDA {
             if (!st.ln.active) return;
             if (k < D) {
                 const long long ko = (long long)k * plane;
@@ -611,7 +611,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                     for (int c = 0; c < RW; ++c) st.px[n][c] = st.pt[n][c] = 0.f;
             }
         };
-        auto store_plane = [&](State &st, int k) {
+        auto store_plane = [&](State &st, int k) NDC_LAMBDA {
             if (!st.ln.active) return;
             const int slot = wrap(k % XR, XR);
             // rows outside the image are never written: they keep the zeros of the set-up
@@ -632,7 +632,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
         // gn, gd of NR rows starting at gn/gd tile row j (image row r0 - PH + j): computed,
         // published to LDS, and returned in acc[0] / acc[1]
         auto gn_gd_rows = [&](State &st, int j1, int j, auto nr_tag,
-                              float (&acc)[2][SC][decltype(nr_tag)::value][RW]) {
+                              float (&acc)[2][SC][decltype(nr_tag)::value][RW]) NDC_LAMBDA {
             constexpr int NR = decltype(nr_tag)::value;
             float sv[SC][NR][RW], gv[SC][NR][RW];
             const long long ko = (long long)j1 * plane;
@@ -690,7 +690,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                     }
         };
 
-        ex.each([&](State &st, int tid) {
+        ex.each([&](State &st, int tid) NDC_LAMBDA {
             st.ln = make_lane(tid, t, RW);
             st.xok = st.ook = 0u;
             NDC_UNROLL
@@ -723,13 +723,13 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
         ex.sync();
 
         for (int k = 0; k < D + 2 * PD; ++k) {
-            ex.each([&](State &st, int) { store_plane(st, k); });
+            ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k); });
             ex.sync();
 
             // ---- gather: gn, gd of plane k - PD on the band plus PH halo rows each side
             const int j1 = k - PD;
             const bool live1 = j1 >= 0 && j1 < D;
-            ex.each([&](State &st, int) {
+            ex.each([&](State &st, int) NDC_LAMBDA {
                 if (!st.ln.active || !live1) return;
                 {
                     float acc[2][SC][RH][RW];
@@ -775,7 +775,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
             ex.sync();
 
             // ---- prefetch, then scatter: plane k - PD of gn/gd feeds pending planes of gx / gt1
-            ex.each([&](State &st, int) {
+            ex.each([&](State &st, int) NDC_LAMBDA {
                 if (!st.ln.active) return;
                 load_plane(st, k + 1);
                 if (live1) {
@@ -815,8 +815,8 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
         if (need_gh) {
             float *dst = p.part + (long long)block_id * p.part_stride;
             ex.template block_reduce<NRED>(
-                [](State &st, int i) { return st.gacc[i / KT][i % KT]; },
-                [&](int i, float v) { dst[i] = v; });
+                [](State &st, int i) NDC_LAMBDA { return st.gacc[i / KT][i % KT]; },
+                [&](int i, float v) NDC_LAMBDA { dst[i] = v; });
         }
     }
 };
@@ -871,7 +871,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
         const float eps = p.eps;
         const int need_gh = p.need_gh;
 
-        auto load_plane = [&](State &st, int k) {
+        auto load_plane = [&](State &st, int k) NDC_LAMBDA {
             if (!st.ln.active) return;
             if (k < D) {
                 const long long ko = (long long)k * plane;
@@ -888,7 +888,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                     for (int c = 0; c < RW; ++c) st.px[n][c] = st.pt[n][c] = st.pg[n][c] = 0.f;
             }
         };
-        auto store_plane = [&](State &st, int k) {
+        auto store_plane = [&](State &st, int k) NDC_LAMBDA {
             if (!st.ln.active) return;
             const int slot = wrap(k % XR, XR);
             NDC_UNROLL
@@ -906,7 +906,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
             }
         };
 
-        ex.each([&](State &st, int tid) {
+        ex.each([&](State &st, int tid) NDC_LAMBDA {
             st.ln = make_lane(tid, t, RW);
             st.xok = st.ook = 0u;
             NDC_UNROLL
@@ -934,11 +934,11 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
         ex.sync();
 
         for (int k = 0; k < D + PD; ++k) {
-            ex.each([&](State &st, int) { store_plane(st, k); });
+            ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k); });
             ex.sync();
 
             const int j0 = k - PD;
-            ex.each([&](State &st, int) {
+            ex.each([&](State &st, int) NDC_LAMBDA {
                 if (!st.ln.active) return;
                 load_plane(st, k + 1);
                 if (j0 < 0) return;
@@ -1032,11 +1032,11 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
         if (p.need_gh || p.need_gb) {
             float *dst = p.part + (long long)block_id * p.part_stride;
             ex.template block_reduce<NRED>(
-                [](State &st, int i) {
+                [](State &st, int i) NDC_LAMBDA {
                     return i < SC * KT ? st.gacc[(i < SC * KT ? i : 0) / KT][i % KT]
                                        : st.gbacc[i >= SC * KT ? i - SC * KT : 0];
                 },
-                [&](int i, float v) { dst[i] = v; });
+                [&](int i, float v) NDC_LAMBDA { dst[i] = v; });
         }
     }
 };

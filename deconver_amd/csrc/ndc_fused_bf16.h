@@ -186,7 +186,7 @@ template <int RH_> struct FwdKernelB {
         const float floor_ = p.relu ? 0.f : -3.0e38f;   // max(s, floor_) rectifies or passes through
         const float eps = p.eps;
 
-        auto load_plane = [&](State &st, int k) {
+        auto load_plane = [&](State &st, int k) NDC_LAMBDA {
             if (!st.ln.active) return;
             if (k < D) {
                 const T *zk = zg + (long long)k * plane;
@@ -196,21 +196,21 @@ template <int RH_> struct FwdKernelB {
                     for (int i = 0; i < SC; ++i)
                         st.pz[i][n] = ld_word(zk + i * cplane, st.zoff[n]);
             }
+            // planes outside the volume: load a clamped plane and select zero (a store in each
+            // arm of a branch would push the staging registers into private memory)
             const int kx = k - PD;
-            if (kx >= 0 && kx < D) {
-                const T *xk = xg + (long long)kx * plane;
-                NDC_UNROLL
-                for (int n = 0; n < NXR; ++n)
-                    st.px[n] = ld_word(xk, st.xoff[n]);
-            } else {
-                NDC_UNROLL
-                for (int n = 0; n < NXR; ++n) st.px[n] = 0u;
+            const bool xlive = kx >= 0 && kx < D;
+            const T *xk = xg + (long long)clampi(kx, 0, D - 1) * plane;
+            NDC_UNROLL
+            for (int n = 0; n < NXR; ++n) {
+                const uint32_t v = ld_word(xk, st.xoff[n]);
+                st.px[n] = xlive ? v : 0u;
             }
         };
 
         // registers -> LDS: source plane k as channel-pair words into slot k % 3; x plane
         // k - 1 completes the plane-pair word (x[k-2], x[k-1]) of slot (k - 2) % 3
-        auto store_plane = [&](State &st, int k) {
+        auto store_plane = [&](State &st, int k) NDC_LAMBDA {
             if (!st.ln.active) return;
             const int lb = PL + st.ln.c0;
             const int sb = off_s + wrap(k % NS, NS) * 2 * RS * P;
@@ -245,7 +245,7 @@ template <int RH_> struct FwdKernelB {
             }
         };
 
-        ex.each([&](State &st, int tid) {
+        ex.each([&](State &st, int tid) NDC_LAMBDA {
             st.ln = make_lane(tid, t, RW);
             st.zok = st.xok = st.ook = 0u;
             NDC_UNROLL
@@ -285,11 +285,11 @@ template <int RH_> struct FwdKernelB {
         ex.sync();
 
         for (int k = 0; k < D + 2; ++k) {
-            ex.each([&](State &st, int) { store_plane(st, k); });
+            ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k); });
             ex.sync();
 
             // ---- K-scatter of source plane k; own source words of plane k - 2; t1 plane k - 1
-            ex.each([&](State &st, int) {
+            ex.each([&](State &st, int) NDC_LAMBDA {
                 if (!st.ln.active) return;
                 const bool extra = st.ln.strip < 2;
                 const int jx = halo_row(st.ln.strip, PH, TH);
@@ -347,7 +347,7 @@ template <int RH_> struct FwdKernelB {
             ex.sync();
 
             // ---- prefetch, then A-gather + epilogue of plane k - 2
-            ex.each([&](State &st, int) {
+            ex.each([&](State &st, int) NDC_LAMBDA {
                 if (!st.ln.active) return;
                 load_plane(st, k + 1);
                 const int j0 = k - 2;
@@ -445,23 +445,23 @@ template <int RH_> struct Bwd1KernelB {
         const float eps = p.eps;
         const int need_gh = p.need_gh;
 
-        auto load_plane = [&](State &st, int k) {
+        auto load_plane = [&](State &st, int k) NDC_LAMBDA {
             if (!st.ln.active) return;
-            if (k < D) {
-                const T *xk = xg + (long long)k * plane, *tk = t1g + (long long)k * plane;
-                NDC_UNROLL
-                for (int n = 0; n < NXR; ++n) {
-                    st.px[n] = ld_word(xk, st.xoff[n]);
-                    st.pt[n] = ld_word(tk, st.xoff[n]);
-                }
-            } else {
-                NDC_UNROLL
-                for (int n = 0; n < NXR; ++n) st.px[n] = st.pt[n] = 0u;
+            // planes past the end: load the last plane and select zero (a store in each arm of
+            // a branch would push the staging registers into private memory)
+            const bool live = k < D;
+            const long long ko = (long long)clampi(k, 0, D - 1) * plane;
+            NDC_UNROLL
+            for (int n = 0; n < NXR; ++n) {
+                const uint32_t vx = ld_word(xg + ko, st.xoff[n]);
+                const uint32_t vt = ld_word(t1g + ko, st.xoff[n]);
+                st.px[n] = live ? vx : 0u;
+                st.pt[n] = live ? vt : 0u;
             }
         };
         // plane k arrives: plane-pair words (v[k-1], v[k]) into pair slot (k-1) % 2 and the
         // operand-pair words (x[k], t1[k]) into slot k % 3
-        auto store_plane = [&](State &st, int k) {
+        auto store_plane = [&](State &st, int k) NDC_LAMBDA {
             if (!st.ln.active) return;
             const int ps = wrap((k - 1) % NP, NP) * RX * P, xs = wrap(k % NXT, NXT) * RX * P;
             NDC_UNROLL
@@ -483,7 +483,7 @@ template <int RH_> struct Bwd1KernelB {
         // gn, gd of NR rows from gn/gd tile row j (image row r0 - 1 + j): published to LDS as
         // channel-pair words; returned as operand pairs GG[i][r][c] = (gn_i, gd_i)
         auto gn_gd_rows = [&](State &st, int j1, int j, auto nr_tag,
-                              uint32_t (&gg_out)[SC][decltype(nr_tag)::value][RW]) {
+                              uint32_t (&gg_out)[SC][decltype(nr_tag)::value][RW]) NDC_LAMBDA {
             constexpr int NR = decltype(nr_tag)::value;
             uint32_t zw[SC][NR], gw[SC][NR];
             const T *zk = zg + (long long)j1 * plane, *gk = gg + (long long)j1 * plane;
@@ -542,7 +542,7 @@ template <int RH_> struct Bwd1KernelB {
             }
         };
 
-        ex.each([&](State &st, int tid) {
+        ex.each([&](State &st, int tid) NDC_LAMBDA {
             st.ln = make_lane(tid, t, RW);
             st.xok = st.ook = 0u;
             NDC_UNROLL
@@ -576,12 +576,12 @@ template <int RH_> struct Bwd1KernelB {
         ex.sync();
 
         for (int k = 0; k < D + 2; ++k) {
-            ex.each([&](State &st, int) { store_plane(st, k); });
+            ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k); });
             ex.sync();
 
             const int j1 = k - 1;
             const bool live1 = j1 >= 0 && j1 < D;
-            ex.each([&](State &st, int) {
+            ex.each([&](State &st, int) NDC_LAMBDA {
                 if (!st.ln.active || !live1) return;
                 {
                     uint32_t gg2[SC][RH][RW];
@@ -623,7 +623,7 @@ template <int RH_> struct Bwd1KernelB {
             });
             ex.sync();
 
-            ex.each([&](State &st, int) {
+            ex.each([&](State &st, int) NDC_LAMBDA {
                 if (!st.ln.active) return;
                 load_plane(st, k + 1);
                 if (live1) {
@@ -663,8 +663,8 @@ template <int RH_> struct Bwd1KernelB {
         if (need_gh) {
             float *dst = p.part + (long long)block_id * p.part_stride;
             ex.template block_reduce<NRED>(
-                [](State &st, int i) { return st.gacc[i / KT][i % KT]; },
-                [&](int i, float v) { dst[i] = v; });
+                [](State &st, int i) NDC_LAMBDA { return st.gacc[i / KT][i % KT]; },
+                [&](int i, float v) NDC_LAMBDA { dst[i] = v; });
         }
     }
 };
@@ -720,23 +720,24 @@ template <int RH_> struct Bwd2KernelB {
         const float eps = p.eps;
         const int need_gh = p.need_gh;
 
-        auto load_plane = [&](State &st, int k) {
+        auto load_plane = [&](State &st, int k) NDC_LAMBDA {
             if (!st.ln.active) return;
-            if (k < D) {
-                const long long ko = (long long)k * plane;
-                NDC_UNROLL
-                for (int n = 0; n < NXR; ++n) {
-                    st.px[n] = ld_word(xg + ko, st.xoff[n]);
-                    st.pt[n] = ld_word(t1g + ko, st.xoff[n]);
-                    st.pg[n] = ld_word(gt1g + ko, st.xoff[n]);
-                }
-            } else {
-                NDC_UNROLL
-                for (int n = 0; n < NXR; ++n) st.px[n] = st.pt[n] = st.pg[n] = 0u;
+            // planes past the end: load the last plane and select zero (a store in each arm of
+            // a branch would push the staging registers into private memory)
+            const bool live = k < D;
+            const long long ko = (long long)clampi(k, 0, D - 1) * plane;
+            NDC_UNROLL
+            for (int n = 0; n < NXR; ++n) {
+                const uint32_t vx = ld_word(xg + ko, st.xoff[n]);
+                const uint32_t vt = ld_word(t1g + ko, st.xoff[n]);
+                const uint32_t vg = ld_word(gt1g + ko, st.xoff[n]);
+                st.px[n] = live ? vx : 0u;
+                st.pt[n] = live ? vt : 0u;
+                st.pg[n] = live ? vg : 0u;
             }
         };
         // plane k arrives: plane-pair words (v[k-1], v[k]) into slot (k-1) % ring
-        auto store_plane = [&](State &st, int k) {
+        auto store_plane = [&](State &st, int k) NDC_LAMBDA {
             if (!st.ln.active) return;
             const int ps = wrap((k - 1) % NP, NP) * RX * P, gs = wrap((k - 1) % NG, NG) * RX * P;
             NDC_UNROLL
@@ -756,7 +757,7 @@ template <int RH_> struct Bwd2KernelB {
             }
         };
 
-        ex.each([&](State &st, int tid) {
+        ex.each([&](State &st, int tid) NDC_LAMBDA {
             st.ln = make_lane(tid, t, RW);
             st.xok = st.ook = 0u;
             NDC_UNROLL
@@ -791,15 +792,21 @@ template <int RH_> struct Bwd2KernelB {
         // one step past the usual end so that an unpaired last plane still gets its
         // filter-gradient contribution (paired with a zero plane)
         for (int k = 0; k < D + 2; ++k) {
-            ex.each([&](State &st, int) { store_plane(st, k); });
+            ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k); });
             ex.sync();
 
             const int j0 = k - 1;
-            ex.each([&](State &st, int) {
+            ex.each([&](State &st, int) NDC_LAMBDA {
                 if (!st.ln.active) return;
                 load_plane(st, k + 1);
                 if (j0 < 0) return;
                 float sv[SC][RH][RW];
+                NDC_UNROLL
+                for (int i = 0; i < SC; ++i)
+                    NDC_UNROLL
+                    for (int r = 0; r < RH; ++r)
+                        NDC_UNROLL
+                        for (int c = 0; c < RW; ++c) sv[i][r][c] = 0.f;
                 if (j0 < D) {
                     uint32_t zw[SC][RH], gw[SC][RH];
                     const T *zk = zg + (long long)j0 * plane, *gk = gg + (long long)j0 * plane;
@@ -851,13 +858,6 @@ template <int RH_> struct Bwd2KernelB {
                             if (gzk && ok) st_word(gzk + i * cplane, st.ooff[r], pack_bf16x2(v[0], v[1]));
                         }
                     }
-                } else {
-                    NDC_UNROLL
-                    for (int i = 0; i < SC; ++i)
-                        NDC_UNROLL
-                        for (int r = 0; r < RH; ++r)
-                            NDC_UNROLL
-                            for (int c = 0; c < RW; ++c) sv[i][r][c] = 0.f;
                 }
                 if (need_gh && (j0 & 1) && j0 <= D) {
                     // K-side filter-gradient term for the plane pair (j0 - 1, j0):
@@ -907,11 +907,11 @@ template <int RH_> struct Bwd2KernelB {
         if (p.need_gh || p.need_gb) {
             float *dst = p.part + (long long)block_id * p.part_stride;
             ex.template block_reduce<NRED>(
-                [](State &st, int i) {
+                [](State &st, int i) NDC_LAMBDA {
                     return i < SC * KT ? st.gacc[(i < SC * KT ? i : 0) / KT][i % KT]
                                        : st.gbacc[i >= SC * KT ? i - SC * KT : 0];
                 },
-                [&](int i, float v) { dst[i] = v; });
+                [&](int i, float v) NDC_LAMBDA { dst[i] = v; });
         }
     }
 };
