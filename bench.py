@@ -110,6 +110,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--dtype", choices=("bf16", "fp32"), default="bf16")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--recompute", action="store_true",
+                    help="backward re-gathers the denominator and ratio (as the reference does) "
+                         "instead of reading the forward's copies")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -138,9 +141,12 @@ def main() -> int:
     geom = ops.make_geom_for(x, h, C, 1, sc, 1e-16, True)
     assert lib.fused_supported(geom), "the headline workload must run on the fused kernels"
 
+    keep = (not args.recompute) and lib.backward_uses_saved(geom)
+
     def step():
-        out, t1 = ops.update_forward(lib, x, z, h, bias, **kw)
-        return ops.update_backward(lib, x, z, t1, h, bias, g, **kw)
+        res = ops.update_forward(lib, x, z, h, bias, save_ratio=keep, **kw)
+        return ops.update_backward(lib, x, z, res[1], h, bias, g,
+                                   saved=res[2] if keep else None, **kw)
 
     if args.calibrate_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
@@ -165,10 +171,11 @@ def main() -> int:
     for _ in range(n_probe):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
-        out, t1 = ops.update_forward(lib, x, z, h, bias, **kw)
+        res = ops.update_forward(lib, x, z, h, bias, save_ratio=keep, **kw)
         e1.record()
         pt = []
-        ops.update_backward(lib, x, z, t1, h, bias, g, pass_times=pt, **kw)
+        ops.update_backward(lib, x, z, res[1], h, bias, g, pass_times=pt,
+                            saved=res[2] if keep else None, **kw)
         torch.cuda.synchronize()
         fwd_ms.append(e0.elapsed_time(e1))
         pass_ms.append(pt)
@@ -229,6 +236,7 @@ def main() -> int:
         "step_algorithmic_bytes": step_bytes,
         "step_hbm_frac": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "kernel_ms": k_ms,
+        "backward_reads_forward_ratio": bool(keep),
         "roofline": roofline,
     }
     if not args.no_cpu:

@@ -23,6 +23,7 @@ EXPORTS = (
     "ndc_status_string",
     "ndc_fused_supported",
     "ndc_check_geometry",
+    "ndc_backward_uses_saved",
     "ndc_forward",
     "ndc_forward_workspace_bytes",
     "ndc_backward_workspace_bytes",
@@ -81,12 +82,13 @@ class NdcLibrary:
         d.ndc_status_string.argtypes = [ctypes.c_int]
         d.ndc_fused_supported.argtypes = [gp]
         d.ndc_check_geometry.argtypes = [gp]
-        d.ndc_forward.argtypes = [gp, vp, vp, fp, fp, vp, vp, vp, ctypes.c_size_t, vp]
+        d.ndc_backward_uses_saved.argtypes = [gp]
+        d.ndc_forward.argtypes = [gp, vp, vp, fp, fp, vp, vp, vp, vp, vp, ctypes.c_size_t, vp]
         d.ndc_forward_workspace_bytes.restype = ctypes.c_size_t
         d.ndc_forward_workspace_bytes.argtypes = [gp]
         d.ndc_backward_workspace_bytes.restype = ctypes.c_size_t
         d.ndc_backward_workspace_bytes.argtypes = [gp] + [ctypes.c_int] * 4
-        d.ndc_backward.argtypes = [gp, vp, vp, vp, fp, fp, vp, vp, vp, fp, fp, vp,
+        d.ndc_backward.argtypes = [gp, vp, vp, vp, vp, vp, fp, fp, vp, vp, vp, fp, fp, vp,
                                    ctypes.c_size_t, vp]
         d.ndc_backward_profiled.argtypes = d.ndc_backward.argtypes + [ctypes.POINTER(ctypes.c_float)]
         d.ndc_gconv.argtypes = [gp, vp, fp, fp, ctypes.c_int, vp, vp]
@@ -105,33 +107,36 @@ class NdcLibrary:
     def check_geometry(self, g: Geom) -> int:
         return self._dll.ndc_check_geometry(ctypes.byref(g))
 
+    def backward_uses_saved(self, g: Geom) -> bool:
+        return bool(self._dll.ndc_backward_uses_saved(ctypes.byref(g)))
+
     def forward_workspace_bytes(self, g: Geom) -> int:
         return self._dll.ndc_forward_workspace_bytes(ctypes.byref(g))
 
     def forward(self, g: Geom, x: int, z: int, h: int, bias: Optional[int], out: int,
-                t1: Optional[int], ws: Optional[int], ws_bytes: int,
-                stream: Optional[int]) -> None:
-        self._check(self._dll.ndc_forward(ctypes.byref(g), x, z, h, bias, out, t1, ws, ws_bytes,
-                                          stream), "ndc_forward")
+                t1: Optional[int], inv_den: Optional[int], ratio: Optional[int],
+                ws: Optional[int], ws_bytes: int, stream: Optional[int]) -> None:
+        self._check(self._dll.ndc_forward(ctypes.byref(g), x, z, h, bias, out, t1, inv_den, ratio,
+                                          ws, ws_bytes, stream), "ndc_forward")
 
     def backward_workspace_bytes(self, g: Geom, need_gx, need_gz, need_gh, need_gb) -> int:
         return self._dll.ndc_backward_workspace_bytes(
             ctypes.byref(g), int(need_gx), int(need_gz), int(need_gh), int(need_gb))
 
-    def backward(self, g: Geom, x, z, t1, h, bias, gout, gx, gz, gh, gb, ws, ws_bytes,
-                 stream) -> None:
+    def backward(self, g: Geom, x, z, t1, inv_den, ratio, h, bias, gout, gx, gz, gh, gb, ws,
+                 ws_bytes, stream) -> None:
         self._check(
-            self._dll.ndc_backward(ctypes.byref(g), x, z, t1, h, bias, gout, gx, gz, gh, gb, ws,
-                                   ws_bytes, stream),
+            self._dll.ndc_backward(ctypes.byref(g), x, z, t1, inv_den, ratio, h, bias, gout, gx,
+                                   gz, gh, gb, ws, ws_bytes, stream),
             "ndc_backward")
 
-    def backward_profiled(self, g: Geom, x, z, t1, h, bias, gout, gx, gz, gh, gb, ws, ws_bytes,
-                          stream):
+    def backward_profiled(self, g: Geom, x, z, t1, inv_den, ratio, h, bias, gout, gx, gz, gh, gb,
+                          ws, ws_bytes, stream):
         """``backward`` plus the device time (ms) of pass 1, pass 2 and the reduction."""
         ms = (ctypes.c_float * 3)()
         self._check(
-            self._dll.ndc_backward_profiled(ctypes.byref(g), x, z, t1, h, bias, gout, gx, gz, gh,
-                                            gb, ws, ws_bytes, stream, ms),
+            self._dll.ndc_backward_profiled(ctypes.byref(g), x, z, t1, inv_den, ratio, h, bias,
+                                            gout, gx, gz, gh, gb, ws, ws_bytes, stream, ms),
             "ndc_backward_profiled")
         return tuple(ms)
 

@@ -120,6 +120,7 @@ template <typename T> struct FwdParams {
     const float *h, *bias;
     const float *wtab;   // packed bf16 tap tables (bf16 dot2 kernels only)
     T *out, *t1;
+    T *inv_den, *ratio;   // optional: 1/(A(t1)+eps) and (A(x)+eps)/(A(t1)+eps), shape of out
     int B, C, D, H, W;
     int relu;
     float eps;
@@ -128,6 +129,7 @@ template <typename T> struct FwdParams {
 
 template <typename T> struct BwdParams {
     const T *x, *z, *t1, *gout;
+    const T *inv_den, *ratio;   // optional: what the forward call saved (both or neither)
     const float *h, *bias;
     const float *wtab;   // packed bf16 tap tables (bf16 dot2 kernels only)
     T *gx, *gz;
@@ -421,7 +423,8 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
         });
         ex.sync();
 
-        for (int k = 0; k < D + 2 * PD; ++k) {
+        for (int kk = 0; kk < D + 2 * PD; ++kk) {
+            const int k = uniform_int(kk);   // the plane index stays on the scalar unit
             ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k); });
             ex.sync();
 
@@ -522,16 +525,25 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                     for (int i = 0; i < SC; ++i) copy_taps<KH * KW>(wn[i], wt[i]);
                 }
                 T *ok_ = og + (long long)j0 * plane;
+                T *dk_ = p.inv_den ? p.inv_den + (og - p.out) + (long long)j0 * plane : nullptr;
+                T *rk_ = p.ratio ? p.ratio + (og - p.out) + (long long)j0 * plane : nullptr;
                 NDC_UNROLL
                 for (int r = 0; r < RH; ++r) {
                     if (!((st.ook >> r) & 1u)) continue;
                     NDC_UNROLL
                     for (int i = 0; i < SC; ++i) {
-                        float v[RW];
+                        float v[RW], rd[RW], rt[RW];
                         NDC_UNROLL
-                        for (int c = 0; c < RW; ++c)
-                            v[c] = sv[i][r][c] * (acc[0][i][r][c] + eps) * fast_rcp(acc[1][i][r][c] + eps);
+                        for (int c = 0; c < RW; ++c) {
+                            rd[c] = fast_rcp(acc[1][i][r][c] + eps);
+                            rt[c] = (acc[0][i][r][c] + eps) * rd[c];
+                            v[c] = sv[i][r][c] * rt[c];
+                        }
                         IO::store(ok_ + i * cplane + st.ooff[r], v);
+                        if (dk_) {
+                            IO::store(dk_ + i * cplane + st.ooff[r], rd);
+                            IO::store(rk_ + i * cplane + st.ooff[r], rt);
+                        }
                     }
                 }
             });
@@ -722,7 +734,8 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
         });
         ex.sync();
 
-        for (int k = 0; k < D + 2 * PD; ++k) {
+        for (int kk = 0; kk < D + 2 * PD; ++kk) {
+            const int k = uniform_int(kk);   // the plane index stays on the scalar unit
             ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k); });
             ex.sync();
 
@@ -933,7 +946,8 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
         });
         ex.sync();
 
-        for (int k = 0; k < D + PD; ++k) {
+        for (int kk = 0; kk < D + PD; ++kk) {
+            const int k = uniform_int(kk);   // the plane index stays on the scalar unit
             ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k); });
             ex.sync();
 

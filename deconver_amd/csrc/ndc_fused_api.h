@@ -189,33 +189,48 @@ static inline size_t forward_ws(const KGeom &q, int dtype)
     return align256((size_t)q.G * kTabWords * 4);
 }
 
+// whether backward() reads the forward's 1/d and n/d for this geometry (aligned pointers
+// assumed): only the bf16 dot2 kernels have that form
+static inline bool backward_uses_saved(const KGeom &q, int dtype)
+{
+    Plan pl;
+    return make_plan(q, pl, true, dtype) && pl.dot2;
+}
+
 template <class BE, typename T> struct Dot2Launch {
     static int fwd(const FwdParams<T> &, const Plan &, void *) { return NDC_ERR_GEOMETRY; }
-    static int bwd1(const BwdParams<T> &, const Plan &, void *) { return NDC_ERR_GEOMETRY; }
-    static int bwd2(const BwdParams<T> &, const Plan &, void *) { return NDC_ERR_GEOMETRY; }
+    static int bwd1(const BwdParams<T> &, const Plan &, void *, bool) { return NDC_ERR_GEOMETRY; }
+    static int bwd2(const BwdParams<T> &, const Plan &, void *, bool) { return NDC_ERR_GEOMETRY; }
 };
 template <class BE> struct Dot2Launch<BE, bf16_t> {
     static int fwd(const FwdParams<bf16_t> &p, const Plan &pl, void *stream)
     {
         return BE::template block_kernel<FwdKernelB<kDot2RH>>(p, pl.nblk_f, pl.tf.NT, pl.lds_f, stream);
     }
-    static int bwd1(const BwdParams<bf16_t> &p, const Plan &pl, void *stream)
+    // saved: the call brought the forward's 1/d and n/d
+    static int bwd1(const BwdParams<bf16_t> &p, const Plan &pl, void *stream, bool saved)
     {
+        if (saved)
+            return BE::template block_kernel<Bwd1KernelB<kDot2RH, true>>(
+                p, pl.nblk_b, pl.tb.NT, Bwd1KernelB<kDot2RH, true>::lds_floats(pl.tb), stream);
         return BE::template block_kernel<Bwd1KernelB<kDot2RH>>(p, pl.nblk_b, pl.tb.NT, pl.lds_b1, stream);
     }
-    static int bwd2(const BwdParams<bf16_t> &p, const Plan &pl, void *stream)
+    static int bwd2(const BwdParams<bf16_t> &p, const Plan &pl, void *stream, bool saved)
     {
+        if (saved)
+            return BE::template block_kernel<Bwd2KernelB<kDot2RH, true>>(
+                p, pl.nblk_b, pl.tb.NT, Bwd2KernelB<kDot2RH, true>::lds_floats(pl.tb), stream);
         return BE::template block_kernel<Bwd2KernelB<kDot2RH>>(p, pl.nblk_b, pl.tb.NT, pl.lds_b2, stream);
     }
 };
 
 template <class BE, typename T>
 static int forward(const KGeom &q, const T *x, const T *z, const float *h, const float *bias,
-                   T *out, T *t1, void *ws, void *stream)
+                   T *out, T *t1, T *inv_den, T *ratio, void *ws, void *stream)
 {
     Plan pl;
     const bool pairs = pair_aligned<T>(x) && pair_aligned<T>(z) && pair_aligned<T>(out) &&
-                       pair_aligned<T>(t1);
+                       pair_aligned<T>(t1) && pair_aligned<T>(inv_den) && pair_aligned<T>(ratio);
     const int dtype = sizeof(T) == 2 ? NDC_BF16 : NDC_F32;
     if (!make_plan(q, pl, pairs, ws ? dtype : NDC_F32)) return NDC_ERR_GEOMETRY;
     FwdParams<T> p;
@@ -226,6 +241,8 @@ static int forward(const KGeom &q, const T *x, const T *z, const float *h, const
     p.bias = bias;
     p.out = out;
     p.t1 = t1;
+    p.inv_den = inv_den;
+    p.ratio = ratio;
     p.B = q.B;
     p.C = q.G;
     p.D = pl.m.D;
@@ -252,16 +269,18 @@ static int forward(const KGeom &q, const T *x, const T *z, const float *h, const
 }
 
 template <class BE, typename T>
-static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const float *h,
-                    const float *bias, const T *gout, T *gx, T *gz, float *gh, float *gb,
-                    void *ws, void *stream, float *pass_ms = nullptr)
+static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const T *inv_den,
+                    const T *ratio, const float *h, const float *bias, const T *gout, T *gx,
+                    T *gz, float *gh, float *gb, void *ws, void *stream, float *pass_ms = nullptr)
 {
     // pass_ms (optional, 3 floats): device time of pass 1, pass 2 and the partial-sum
     // reduction, taken with events on `stream`; makes the call synchronous
     typename BE::Timer tm(pass_ms != nullptr, stream);
     Plan pl;
     const bool pairs = pair_aligned<T>(x) && pair_aligned<T>(z) && pair_aligned<T>(t1) &&
-                       pair_aligned<T>(gout) && pair_aligned<T>(gx) && pair_aligned<T>(gz);
+                       pair_aligned<T>(gout) && pair_aligned<T>(gx) && pair_aligned<T>(gz) &&
+                       pair_aligned<T>(inv_den) && pair_aligned<T>(ratio);
+    const bool saved = inv_den != nullptr && ratio != nullptr;
     const int dtype = sizeof(T) == 2 ? NDC_BF16 : NDC_F32;
     if (!make_plan(q, pl, pairs, dtype)) return NDC_ERR_GEOMETRY;
     const size_t n_x = (size_t)q.B * q.G * q.SP;
@@ -280,6 +299,8 @@ static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const f
     p.z = z;
     p.t1 = t1;
     p.gout = gout;
+    p.inv_den = inv_den;
+    p.ratio = ratio;
     p.h = h;
     p.bias = bias;
     p.gx = gx;
@@ -305,7 +326,7 @@ static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const f
                              [=] NDC_LAMBDA(long long idx) { prep_tables(idx, h, tab); });
         if (st) return st;
         p.wtab = tab;
-        st = Dot2Launch<BE, T>::bwd1(p, pl, stream);
+        st = Dot2Launch<BE, T>::bwd1(p, pl, stream, saved);
     } else {
 #define X(kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_)                                          \
     if (NDC_IS_VARIANT(pl, kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_))                        \
@@ -325,7 +346,7 @@ static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const f
     p.part_stride = kt + q.sc;
     st = NDC_ERR_GEOMETRY;
     if (pl.dot2) {
-        st = Dot2Launch<BE, T>::bwd2(p, pl, stream);
+        st = Dot2Launch<BE, T>::bwd2(p, pl, stream, saved);
     } else {
 #define X(kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_)                                          \
     if (NDC_IS_VARIANT(pl, kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_))                        \

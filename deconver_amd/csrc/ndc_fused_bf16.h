@@ -284,7 +284,8 @@ template <int RH_> struct FwdKernelB {
         });
         ex.sync();
 
-        for (int k = 0; k < D + 2; ++k) {
+        for (int kk = 0; kk < D + 2; ++kk) {
+            const int k = uniform_int(kk);   // the plane index stays on the scalar unit
             ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k); });
             ex.sync();
 
@@ -372,19 +373,27 @@ template <int RH_> struct FwdKernelB {
                     a_plane_d2<RH, RW, 2>(ex, base, P, wt, acc);
                 }
                 T *ok_ = og + (long long)j0 * plane;
+                T *dk_ = p.inv_den ? p.inv_den + (og - p.out) + (long long)j0 * plane : nullptr;
+                T *rk_ = p.ratio ? p.ratio + (og - p.out) + (long long)j0 * plane : nullptr;
                 NDC_UNROLL
                 for (int r = 0; r < RH; ++r) {
                     if (!((st.ook >> r) & 1u)) continue;
                     NDC_UNROLL
                     for (int i = 0; i < SC; ++i) {
-                        float v[RW];
+                        float v[RW], rd[RW], rt[RW];
                         NDC_UNROLL
                         for (int c = 0; c < RW; ++c) {
                             const uint32_t w = st.own[i >> 1][r][c];
                             const float s = (i & 1) ? bf_hi(w) : bf_lo(w);
-                            v[c] = s * acc[0][i][r][c] * fast_rcp(acc[1][i][r][c]);
+                            rd[c] = fast_rcp(acc[1][i][r][c]);
+                            rt[c] = acc[0][i][r][c] * rd[c];
+                            v[c] = s * rt[c];
                         }
                         st_word(ok_ + i * cplane, st.ooff[r], pack_bf16x2(v[0], v[1]));
+                        if (dk_) {
+                            st_word(dk_ + i * cplane, st.ooff[r], pack_bf16x2(rd[0], rd[1]));
+                            st_word(rk_ + i * cplane, st.ooff[r], pack_bf16x2(rt[0], rt[1]));
+                        }
                     }
                 }
             });
@@ -394,7 +403,10 @@ template <int RH_> struct FwdKernelB {
 
 // =================================================================== backward pass 1 (bf16, dot2)
 
-template <int RH_> struct Bwd1KernelB {
+// SAVED: the call brings the forward's 1/d and n/d, so gn = g s (1/d), gd = -gn (n/d) are
+// elementwise and the plane-pair rings of x and t1 (for re-gathering n and d) are not kept.
+template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
+    static constexpr bool SAVED = SAVED_;
     static constexpr int KD = 3, KH = 3, KW = 3, SC = 4, RH = RH_, RW = 2;
     static constexpr int PD = 1, PH = 1, PW = 1, KT = 27;
     static constexpr int NXR = RH + 2;
@@ -417,7 +429,7 @@ template <int RH_> struct Bwd1KernelB {
     static NDC_HD int rows_g(int TH) { return TH + 2; }
     static NDC_HD int lds_floats(const Tile &t)
     {
-        const int main_ = ((2 * NP + NXT) * rows_x(t.TH) + 4 * rows_g(t.TH)) * t.P;
+        const int main_ = (((SAVED ? 0 : 2 * NP) + NXT) * rows_x(t.TH) + 4 * rows_g(t.TH)) * t.P;
         const int red = (t.NT / 64) * NRED;
         return main_ > red ? main_ : red;
     }
@@ -428,7 +440,7 @@ template <int RH_> struct Bwd1KernelB {
         const BlockId id = decode_block(block_id, p.C, t);
         const int S = t.S, P = t.P, PL = t.PL, TH = t.TH, W = p.W, H = p.H, D = p.D;
         const int RX = rows_x(TH), RG = rows_g(TH);
-        const int off_xp = 0, off_tp = NP * RX * P, off_xt = 2 * NP * RX * P;
+        const int off_xp = 0, off_tp = NP * RX * P, off_xt = SAVED ? 0 : 2 * NP * RX * P;
         const int off_g = off_xt + NXT * RX * P;
         const int total = off_g + 4 * RG * P;
         const int plane = H * W;
@@ -436,6 +448,8 @@ template <int RH_> struct Bwd1KernelB {
         const long long cbase = ((long long)id.b * p.C + id.c) * cplane;
         const T *xg = p.x + cbase, *t1g = p.t1 + cbase;
         const T *zg = p.z + cbase * SC, *gg = p.gout + cbase * SC;
+        const T *dg = SAVED ? p.inv_den + cbase * SC : nullptr;
+        const T *rg = SAVED ? p.ratio + cbase * SC : nullptr;
         T *gxg = p.gx ? p.gx + cbase : nullptr;
         T *gt1g = p.gt1 + cbase;
         UniformF tab = as_uniform(p.wtab + (long long)id.c * kTabWords);
@@ -468,10 +482,12 @@ template <int RH_> struct Bwd1KernelB {
             for (int n = 0; n < NXR; ++n) {
                 if ((st.xok >> n) & 1u) {
                     const int o = (st.ln.strip + n * S) * P + PL + st.ln.c0;
-                    ex.st_(off_xp + ps + o, bits_to_float(zip_lo(st.pxprev[n], st.px[n])));
-                    ex.st_(off_xp + ps + o + 1, bits_to_float(zip_hi(st.pxprev[n], st.px[n])));
-                    ex.st_(off_tp + ps + o, bits_to_float(zip_lo(st.ptprev[n], st.pt[n])));
-                    ex.st_(off_tp + ps + o + 1, bits_to_float(zip_hi(st.ptprev[n], st.pt[n])));
+                    if (!SAVED) {
+                        ex.st_(off_xp + ps + o, bits_to_float(zip_lo(st.pxprev[n], st.px[n])));
+                        ex.st_(off_xp + ps + o + 1, bits_to_float(zip_hi(st.pxprev[n], st.px[n])));
+                        ex.st_(off_tp + ps + o, bits_to_float(zip_lo(st.ptprev[n], st.pt[n])));
+                        ex.st_(off_tp + ps + o + 1, bits_to_float(zip_hi(st.ptprev[n], st.pt[n])));
+                    }
                     ex.st_(off_xt + xs + o, bits_to_float(zip_lo(st.px[n], st.pt[n])));
                     ex.st_(off_xt + xs + o + 1, bits_to_float(zip_hi(st.px[n], st.pt[n])));
                 }
@@ -485,7 +501,7 @@ template <int RH_> struct Bwd1KernelB {
         auto gn_gd_rows = [&](State &st, int j1, int j, auto nr_tag,
                               uint32_t (&gg_out)[SC][decltype(nr_tag)::value][RW]) NDC_LAMBDA {
             constexpr int NR = decltype(nr_tag)::value;
-            uint32_t zw[SC][NR], gw[SC][NR];
+            uint32_t zw[SC][NR], gw[SC][NR], dw[SC][NR], rw[SC][NR];
             const T *zk = zg + (long long)j1 * plane, *gk = gg + (long long)j1 * plane;
             bool ok[NR];
             NDC_UNROLL
@@ -497,6 +513,12 @@ template <int RH_> struct Bwd1KernelB {
                 for (int i = 0; i < SC; ++i) {
                     zw[i][r] = ld_word(zk + i * cplane, o);
                     gw[i][r] = ld_word(gk + i * cplane, o);
+                    if (SAVED) {
+                        dw[i][r] = ld_word(dg + (long long)j1 * plane + i * cplane, o);
+                        rw[i][r] = ld_word(rg + (long long)j1 * plane + i * cplane, o);
+                    } else {
+                        dw[i][r] = rw[i][r] = 0u;
+                    }
                 }
             }
             float acc[2][SC][NR][RW];
@@ -508,14 +530,16 @@ template <int RH_> struct Bwd1KernelB {
                     for (int r = 0; r < NR; ++r)
                         NDC_UNROLL
                         for (int c = 0; c < RW; ++c) acc[a][i][r][c] = eps;
-            NDC_ROLLED
-            for (int s = 0; s < 2; ++s) {
-                float wt[SC][9];
-                load_plane_taps<SC, 9, 9>(tab + 54 + s * 36, wt);
-                const int m = j1 - 1 + s;
-                const int ob = (wrap(m % NP, NP) * RX + j) * P + PL + st.ln.c0 - PW;
-                const int base[2] = {off_xp + ob, off_tp + ob};
-                a_plane_d2<NR, RW, 2>(ex, base, P, wt, acc);
+            if (!SAVED) {
+                NDC_ROLLED
+                for (int s = 0; s < 2; ++s) {
+                    float wt[SC][9];
+                    load_plane_taps<SC, 9, 9>(tab + 54 + s * 36, wt);
+                    const int m = j1 - 1 + s;
+                    const int ob = (wrap(m % NP, NP) * RX + j) * P + PL + st.ln.c0 - PW;
+                    const int base[2] = {off_xp + ob, off_tp + ob};
+                    a_plane_d2<NR, RW, 2>(ex, base, P, wt, acc);
+                }
             }
             NDC_UNROLL
             for (int r = 0; r < NR; ++r) {
@@ -526,9 +550,14 @@ template <int RH_> struct Bwd1KernelB {
                     for (int c = 0; c < RW; ++c) {
                         const float sv = floor_f((c ? bf_hi(zw[i][r]) : bf_lo(zw[i][r])) + st.bv[i], floor_);
                         const float gv = ok[r] ? (c ? bf_hi(gw[i][r]) : bf_lo(gw[i][r])) : 0.f;
-                        const float inv = fast_rcp(acc[1][i][r][c]);
-                        gn[i][c] = gv * sv * inv;
-                        gd[i][c] = -(gn[i][c] * acc[0][i][r][c]) * inv;
+                        if (SAVED) {
+                            gn[i][c] = gv * sv * (c ? bf_hi(dw[i][r]) : bf_lo(dw[i][r]));
+                            gd[i][c] = -(gn[i][c] * (c ? bf_hi(rw[i][r]) : bf_lo(rw[i][r])));
+                        } else {
+                            const float inv = fast_rcp(acc[1][i][r][c]);
+                            gn[i][c] = gv * sv * inv;
+                            gd[i][c] = -(gn[i][c] * acc[0][i][r][c]) * inv;
+                        }
                         gg_out[i][r][c] = pack_bf16x2(gn[i][c], gd[i][c]);
                     }
                 NDC_UNROLL
@@ -575,7 +604,8 @@ template <int RH_> struct Bwd1KernelB {
         });
         ex.sync();
 
-        for (int k = 0; k < D + 2; ++k) {
+        for (int kk = 0; kk < D + 2; ++kk) {
+            const int k = uniform_int(kk);   // the plane index stays on the scalar unit
             ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k); });
             ex.sync();
 
@@ -671,7 +701,10 @@ template <int RH_> struct Bwd1KernelB {
 
 // =================================================================== backward pass 2 (bf16, dot2)
 
-template <int RH_> struct Bwd2KernelB {
+// SAVED: gz = [s > 0] (g (n/d) + A(gt1)) with the forward's n/d, so only the gt1 ring is kept.
+template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
+    static constexpr bool SAVED = SAVED_;
+    static constexpr int NA = SAVED ? 1 : 3;   // gathered operands: (x, t1,) gt1
     static constexpr int KD = 3, KH = 3, KW = 3, SC = 4, RH = RH_, RW = 2;
     static constexpr int PD = 1, PH = 1, PW = 1, KT = 27;
     static constexpr int NXR = RH + 1;
@@ -694,7 +727,7 @@ template <int RH_> struct Bwd2KernelB {
     static NDC_HD int rows_x(int TH) { return TH + 2; }
     static NDC_HD int lds_floats(const Tile &t)
     {
-        const int main_ = (2 * NP + NG) * rows_x(t.TH) * t.P;
+        const int main_ = ((SAVED ? 0 : 2 * NP) + NG) * rows_x(t.TH) * t.P;
         const int red = (t.NT / 64) * NRED;
         return main_ > red ? main_ : red;
     }
@@ -705,13 +738,14 @@ template <int RH_> struct Bwd2KernelB {
         const BlockId id = decode_block(block_id, p.C, t);
         const int S = t.S, P = t.P, PL = t.PL, TH = t.TH, W = p.W, H = p.H, D = p.D;
         const int RX = rows_x(TH);
-        const int off_xp = 0, off_tp = NP * RX * P, off_gp = 2 * NP * RX * P;
+        const int off_xp = 0, off_tp = NP * RX * P, off_gp = SAVED ? 0 : 2 * NP * RX * P;
         const int total = off_gp + NG * RX * P;
         const int plane = H * W;
         const long long cplane = (long long)D * plane;
         const long long cbase = ((long long)id.b * p.C + id.c) * cplane;
         const T *xg = p.x + cbase, *t1g = p.t1 + cbase, *gt1g = p.gt1 + cbase;
         const T *zg = p.z + cbase * SC, *gg = p.gout + cbase * SC;
+        const T *rg = SAVED ? p.ratio + cbase * SC : nullptr;
         T *gzg = p.gz ? p.gz + cbase * SC : nullptr;
         UniformF tab = as_uniform(p.wtab + (long long)id.c * kTabWords);
         const int r0 = id.r0;
@@ -728,8 +762,8 @@ template <int RH_> struct Bwd2KernelB {
             const long long ko = (long long)clampi(k, 0, D - 1) * plane;
             NDC_UNROLL
             for (int n = 0; n < NXR; ++n) {
-                const uint32_t vx = ld_word(xg + ko, st.xoff[n]);
-                const uint32_t vt = ld_word(t1g + ko, st.xoff[n]);
+                const uint32_t vx = SAVED ? 0u : ld_word(xg + ko, st.xoff[n]);
+                const uint32_t vt = SAVED ? 0u : ld_word(t1g + ko, st.xoff[n]);
                 const uint32_t vg = ld_word(gt1g + ko, st.xoff[n]);
                 st.px[n] = live ? vx : 0u;
                 st.pt[n] = live ? vt : 0u;
@@ -744,10 +778,12 @@ template <int RH_> struct Bwd2KernelB {
             for (int n = 0; n < NXR; ++n) {
                 if ((st.xok >> n) & 1u) {
                     const int o = (st.ln.strip + n * S) * P + PL + st.ln.c0;
-                    ex.st_(off_xp + ps + o, bits_to_float(zip_lo(st.pxprev[n], st.px[n])));
-                    ex.st_(off_xp + ps + o + 1, bits_to_float(zip_hi(st.pxprev[n], st.px[n])));
-                    ex.st_(off_tp + ps + o, bits_to_float(zip_lo(st.ptprev[n], st.pt[n])));
-                    ex.st_(off_tp + ps + o + 1, bits_to_float(zip_hi(st.ptprev[n], st.pt[n])));
+                    if (!SAVED) {
+                        ex.st_(off_xp + ps + o, bits_to_float(zip_lo(st.pxprev[n], st.px[n])));
+                        ex.st_(off_xp + ps + o + 1, bits_to_float(zip_hi(st.pxprev[n], st.px[n])));
+                        ex.st_(off_tp + ps + o, bits_to_float(zip_lo(st.ptprev[n], st.pt[n])));
+                        ex.st_(off_tp + ps + o + 1, bits_to_float(zip_hi(st.ptprev[n], st.pt[n])));
+                    }
                     ex.st_(off_gp + gs + o, bits_to_float(zip_lo(st.pgprev[n], st.pg[n])));
                     ex.st_(off_gp + gs + o + 1, bits_to_float(zip_hi(st.pgprev[n], st.pg[n])));
                 }
@@ -791,7 +827,8 @@ template <int RH_> struct Bwd2KernelB {
 
         // one step past the usual end so that an unpaired last plane still gets its
         // filter-gradient contribution (paired with a zero plane)
-        for (int k = 0; k < D + 2; ++k) {
+        for (int kk = 0; kk < D + 2; ++kk) {
+            const int k = uniform_int(kk);   // the plane index stays on the scalar unit
             ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k); });
             ex.sync();
 
@@ -808,7 +845,7 @@ template <int RH_> struct Bwd2KernelB {
                         NDC_UNROLL
                         for (int c = 0; c < RW; ++c) sv[i][r][c] = 0.f;
                 if (j0 < D) {
-                    uint32_t zw[SC][RH], gw[SC][RH];
+                    uint32_t zw[SC][RH], gw[SC][RH], rw[SC][RH];
                     const T *zk = zg + (long long)j0 * plane, *gk = gg + (long long)j0 * plane;
                     NDC_UNROLL
                     for (int r = 0; r < RH; ++r)
@@ -816,26 +853,30 @@ template <int RH_> struct Bwd2KernelB {
                         for (int i = 0; i < SC; ++i) {
                             zw[i][r] = ld_word(zk + i * cplane, st.ooff[r]);
                             gw[i][r] = ld_word(gk + i * cplane, st.ooff[r]);
+                            rw[i][r] = SAVED ? ld_word(rg + (long long)j0 * plane + i * cplane, st.ooff[r]) : 0u;
                         }
-                    float acc[3][SC][RH][RW];
+                    float acc[NA][SC][RH][RW];
                     NDC_UNROLL
-                    for (int a = 0; a < 3; ++a)
+                    for (int a = 0; a < NA; ++a)
                         NDC_UNROLL
                         for (int i = 0; i < SC; ++i)
                             NDC_UNROLL
                             for (int r = 0; r < RH; ++r)
                                 NDC_UNROLL
-                                for (int c = 0; c < RW; ++c) acc[a][i][r][c] = a < 2 ? eps : 0.f;
+                                for (int c = 0; c < RW; ++c) acc[a][i][r][c] = a < NA - 1 ? eps : 0.f;
                     NDC_ROLLED
                     for (int s = 0; s < 2; ++s) {
                         float wt[SC][9];
                         load_plane_taps<SC, 9, 9>(tab + 54 + s * 36, wt);
                         const int m = j0 - 1 + s;
                         const int ob = (st.ln.strip * RH) * P + PL + st.ln.c0 - PW;
-                        const int base[3] = {off_xp + wrap(m % NP, NP) * RX * P + ob,
-                                             off_tp + wrap(m % NP, NP) * RX * P + ob,
-                                             off_gp + wrap(m % NG, NG) * RX * P + ob};
-                        a_plane_d2<RH, RW, 3>(ex, base, P, wt, acc);
+                        int base[NA];
+                        base[NA - 1] = off_gp + wrap(m % NG, NG) * RX * P + ob;
+                        if (!SAVED) {
+                            base[0] = off_xp + wrap(m % NP, NP) * RX * P + ob;
+                            base[NA > 1 ? 1 : 0] = off_tp + wrap(m % NP, NP) * RX * P + ob;
+                        }
+                        a_plane_d2<RH, RW, NA>(ex, base, P, wt, acc);
                     }
                     T *gzk = gzg ? gzg + (long long)j0 * plane : nullptr;
                     NDC_UNROLL
@@ -848,7 +889,12 @@ template <int RH_> struct Bwd2KernelB {
                             for (int c = 0; c < RW; ++c) {
                                 const float s = floor_f((c ? bf_hi(zw[i][r]) : bf_lo(zw[i][r])) + st.bv[i], floor_);
                                 const float g = c ? bf_hi(gw[i][r]) : bf_lo(gw[i][r]);
-                                float gzv = g * acc[0][i][r][c] * fast_rcp(acc[1][i][r][c]) + acc[2][i][r][c];
+                                float gzv;
+                                if (SAVED)
+                                    gzv = g * (c ? bf_hi(rw[i][r]) : bf_lo(rw[i][r])) + acc[NA - 1][i][r][c];
+                                else
+                                    gzv = g * acc[0][i][r][c] * fast_rcp(acc[NA > 1 ? 1 : 0][i][r][c]) +
+                                          acc[NA - 1][i][r][c];
                                 if (p.relu && !(s > 0.f)) gzv = 0.f;
                                 if (!ok) gzv = 0.f;
                                 sv[i][r][c] = ok ? s : 0.f;

@@ -1,14 +1,18 @@
 """Autograd node of one NDC source update, running on the HIP kernels.
 
 Mirrors ``deconver/deconvolution/functional.py:97-207`` of the reference
-(``DeconvUpdate`` / ``deconv_update``): same arguments, same saved tensors
-``(x, z, t1, h, bias)``, same returned gradients ``(gx, gz, gh, gb, None x5)``, same
-refusal of double backward.  The arithmetic is in ``libdeconver_ndc.so``; there is no
-PyTorch implementation behind this node.
+(``DeconvUpdate`` / ``deconv_update``): same arguments, same returned gradients
+``(gx, gz, gh, gb, None x5)``, same refusal of double backward.  It saves the reference's
+``(x, z, t1, h, bias)`` plus, unless ``save_ratio(False)`` was called, the forward's
+``1/(A(t1)+eps)`` and ``(A(x)+eps)/(A(t1)+eps)``: two tensors of the size of the output
+kept until backward, which then does not gather ``A(x)`` and ``A(t1)`` a second time.
+The arithmetic is in ``libdeconver_ndc.so``; there is no PyTorch implementation behind
+this node.
 """
 
 from __future__ import annotations
 
+import os
 from typing import Optional
 
 import torch
@@ -16,7 +20,22 @@ from torch import Tensor
 
 from . import _lib, ops
 
-__all__ = ["deconv_update", "hip_kernels_apply", "DeconvUpdate"]
+__all__ = ["deconv_update", "hip_kernels_apply", "DeconvUpdate", "save_ratio"]
+
+_SAVE_RATIO = os.environ.get("DECONVER_NDC_SAVE_RATIO", "1") != "0"
+
+
+def save_ratio(enabled: Optional[bool] = None) -> bool:
+    """Get or set whether training keeps the forward's denominator and ratio for backward.
+
+    On (the default; environment ``DECONVER_NDC_SAVE_RATIO=0`` turns it off): each update
+    node holds two more tensors of the size of its output until backward, and backward is
+    shorter.  Off: backward re-gathers them from ``x`` and ``t1`` as the reference does.
+    """
+    global _SAVE_RATIO
+    if enabled is not None:
+        _SAVE_RATIO = bool(enabled)
+    return _SAVE_RATIO
 
 
 def hip_kernels_apply(x: Tensor, m: int, sc: int, kernel_size, dtype=None) -> bool:
@@ -55,11 +74,18 @@ class DeconvUpdate(torch.autograd.Function):
         z = z.contiguous()
         hc = h.contiguous()
         need_t1 = any(ctx.needs_input_grad[:4])
+        keep = need_t1 and _SAVE_RATIO
+        if keep:
+            # only where the backward kernels for this geometry read them
+            keep = lib.backward_uses_saved(
+                ops.make_geom_for(x, hc, groups, m, sc, eps, relu_input))
         with torch.cuda.device(x.device):
-            out, t1 = ops.update_forward(lib, x, z, hc, bias, groups=groups, m=m, sc=sc,
-                                         eps=eps, relu_input=relu_input, need_t1=need_t1)
+            res = ops.update_forward(lib, x, z, hc, bias, groups=groups, m=m, sc=sc, eps=eps,
+                                     relu_input=relu_input, need_t1=need_t1, save_ratio=keep)
+        out, t1 = res[0], res[1]
+        inv_den, ratio = res[2] if keep else (None, None)
         ctx.cfg = (groups, m, sc, eps, relu_input)
-        ctx.save_for_backward(x, z, t1, hc, bias)
+        ctx.save_for_backward(x, z, t1, hc, bias, inv_den, ratio)
         return out
 
     @staticmethod
@@ -71,7 +97,7 @@ class DeconvUpdate(torch.autograd.Function):
                 "double backward through the fused Deconv update is not supported; "
                 "construct the layer with a convolution keyword argument (e.g. stride=1) "
                 "to force the general path, which is plain PyTorch and doubly differentiable")
-        x, z, t1, h, bias = ctx.saved_tensors
+        x, z, t1, h, bias, inv_den, ratio = ctx.saved_tensors
         groups, m, sc, eps, relu_input = ctx.cfg
         need_x, need_z, need_h, need_b = ctx.needs_input_grad[:4]
         if t1 is None:
@@ -84,7 +110,8 @@ class DeconvUpdate(torch.autograd.Function):
             gx, gz, gh, gb = ops.update_backward(
                 lib, x, z, t1, h, bias, gout, groups=groups, m=m, sc=sc, eps=eps,
                 relu_input=relu_input, need_x=need_x, need_z=need_z, need_h=need_h,
-                need_b=need_b and bias is not None)
+                need_b=need_b and bias is not None,
+                saved=None if inv_den is None else (inv_den, ratio))
         return gx, gz, gh, gb, None, None, None, None, None
 
 

@@ -66,9 +66,13 @@ def make_geom_for(x: Tensor, h: Tensor, groups: int, m: int, sc: int, eps: float
 
 def update_forward(lib: _lib.NdcLibrary, x: Tensor, z: Tensor, h: Tensor,
                    bias: Optional[Tensor], *, groups: int, m: int, sc: int, eps: float,
-                   relu_input: bool, need_t1: bool = True,
-                   path: int = _lib.PATH_AUTO) -> Tuple[Tensor, Optional[Tensor]]:
-    """``out = s*(A(x)+eps)/(A(K(s))+eps)`` with ``s = relu?(z+bias)``; returns ``(out, t1)``."""
+                   relu_input: bool, need_t1: bool = True, save_ratio: bool = False,
+                   path: int = _lib.PATH_AUTO):
+    """``out = s*(A(x)+eps)/(A(K(s))+eps)`` with ``s = relu?(z+bias)``.
+
+    Returns ``(out, t1)``, or ``(out, t1, (inv_den, ratio))`` with ``save_ratio``: the two
+    extra tensors (shape of ``out``) that let :func:`update_backward` skip re-gathering
+    ``A(x)`` and ``A(t1)``."""
     _check_common(x, z, h, bias, groups, m, sc)
     g = make_geom_for(x, h, groups, m, sc, eps, relu_input, path)
     out = torch.empty_like(z)
@@ -79,8 +83,12 @@ def update_forward(lib: _lib.NdcLibrary, x: Tensor, z: Tensor, h: Tensor,
     if nbytes:
         ws = torch.empty(nbytes + 256, dtype=torch.uint8, device=x.device)
         ws_ptr = (ws.data_ptr() + 255) // 256 * 256
-    lib.forward(g, _ptr(x), _ptr(z), _ptr(h), _ptr(bias), _ptr(out), _ptr(t1), ws_ptr, nbytes,
-                _stream_of(x))
+    inv_den = torch.empty_like(z) if save_ratio else None
+    ratio = torch.empty_like(z) if save_ratio else None
+    lib.forward(g, _ptr(x), _ptr(z), _ptr(h), _ptr(bias), _ptr(out), _ptr(t1), _ptr(inv_den),
+                _ptr(ratio), ws_ptr, nbytes, _stream_of(x))
+    if save_ratio:
+        return out, t1, (inv_den, ratio)
     return out, t1
 
 
@@ -88,8 +96,12 @@ def update_backward(lib: _lib.NdcLibrary, x: Tensor, z: Tensor, t1: Tensor, h: T
                     bias: Optional[Tensor], gout: Tensor, *, groups: int, m: int, sc: int,
                     eps: float, relu_input: bool, need_x: bool = True, need_z: bool = True,
                     need_h: bool = True, need_b: bool = True,
-                    path: int = _lib.PATH_AUTO, pass_times: Optional[list] = None):
+                    path: int = _lib.PATH_AUTO, pass_times: Optional[list] = None,
+                    saved: Optional[Tuple[Tensor, Tensor]] = None):
     """Gradients ``(gx, gz, gh, gb)`` of the update; entries not asked for are ``None``.
+
+    ``saved``: the ``(inv_den, ratio)`` pair a ``save_ratio`` forward call returned for the
+    same inputs.
 
     ``pass_times``: a list that, if given, receives the device milliseconds of the three
     backward stages (the call then synchronises)."""
@@ -98,6 +110,12 @@ def update_backward(lib: _lib.NdcLibrary, x: Tensor, z: Tensor, t1: Tensor, h: T
         raise ValueError("gout must be contiguous with the shape and dtype of z")
     if t1.shape != x.shape or t1.dtype != x.dtype or not t1.is_contiguous():
         raise ValueError("t1 must be contiguous with the shape and dtype of x")
+    inv_den = ratio = None
+    if saved is not None:
+        inv_den, ratio = saved
+        for t in (inv_den, ratio):
+            if t.shape != z.shape or t.dtype != z.dtype or not t.is_contiguous():
+                raise ValueError("saved tensors must be contiguous with the shape and dtype of z")
     need_b = need_b and bias is not None
     g = make_geom_for(x, h, groups, m, sc, eps, relu_input, path)
     gx = torch.empty_like(x) if need_x else None
@@ -107,7 +125,8 @@ def update_backward(lib: _lib.NdcLibrary, x: Tensor, z: Tensor, t1: Tensor, h: T
     nbytes = lib.backward_workspace_bytes(g, need_x, need_z, need_h, need_b)
     ws = torch.empty(max(nbytes, 1) + 256, dtype=torch.uint8, device=x.device)
     ws_ptr = (ws.data_ptr() + 255) // 256 * 256
-    args = (g, _ptr(x), _ptr(z), _ptr(t1), _ptr(h), _ptr(bias), _ptr(gout), _ptr(gx),
+    args = (g, _ptr(x), _ptr(z), _ptr(t1), _ptr(inv_den), _ptr(ratio), _ptr(h), _ptr(bias),
+            _ptr(gout), _ptr(gx),
             _ptr(gz), _ptr(gh), _ptr(gb), ws_ptr, nbytes, _stream_of(x))
     if pass_times is None:
         lib.backward(*args)

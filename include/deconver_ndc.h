@@ -73,6 +73,11 @@ int ndc_fused_supported(const ndc_geom *g);
 /* 0 if some path covers `g` (then every entry point below accepts it), else a status. */
 int ndc_check_geometry(const ndc_geom *g);
 
+/* 1 if `ndc_backward` for `g` reads the forward's inv_den / ratio when they are passed (so
+ * that keeping them pays), 0 if its kernels re-gather regardless.  No counterpart in the
+ * reference. */
+int ndc_backward_uses_saved(const ndc_geom *g);
+
 /* Bytes of scratch `ndc_forward` needs for `g` (0 for most geometries; the bfloat16 3x3x3
  * kernels keep their packed filter tables there). */
 size_t ndc_forward_workspace_bytes(const ndc_geom *g);
@@ -87,12 +92,17 @@ size_t ndc_forward_workspace_bytes(const ndc_geom *g);
  *   t1            optional output K(s), same shape/dtype as x: pass it when a backward
  *                 call will follow (it is what the reference saves for backward), null
  *                 for inference
+ *   inv_den,      optional outputs 1/(A(t1)+eps) and (A(x)+eps)/(A(t1)+eps), same shape/dtype
+ *   ratio         as out; both or neither.  Handing them to ndc_backward lets it skip
+ *                 re-gathering A(x) and A(t1): more memory kept between the two calls
+ *                 (two tensors of the size of out) for fewer multiplications.  The
+ *                 reference has no counterpart (it re-gathers, kernels.py:791-838).
  *   workspace     >= ndc_forward_workspace_bytes(g) bytes, 256-byte aligned (may be null
  *                 when that is 0)
  */
 int ndc_forward(const ndc_geom *g, const void *x, const void *z, const float *h,
-                const float *bias, void *out, void *t1, void *workspace, size_t workspace_bytes,
-                void *stream);
+                const float *bias, void *out, void *t1, void *inv_den, void *ratio,
+                void *workspace, size_t workspace_bytes, void *stream);
 
 /* Bytes of scratch `ndc_backward` needs for `g` with the requested outputs (each flag
  * nonzero when the matching output pointer will be non-null). */
@@ -104,6 +114,8 @@ size_t ndc_backward_workspace_bytes(const ndc_geom *g, int need_gx, int need_gz,
  * (deconver/deconvolution/functional.py:118-182), i.e. kernels.deconv_bwd, gconv x2,
  * wgrad x3, deconv_gz and the bias reduction (kernels.py:791-894).
  *   x, z, t1, h, bias   what the forward call saw / produced (bias may be null)
+ *   inv_den, ratio      what the forward call wrote for the same inputs, or both null (then
+ *                       the kernels re-gather A(x) and A(t1)); results agree to rounding
  *   gout                upstream gradient, shape/dtype of out
  *   gx, gz, gh, gb      optional outputs (null = not needed); gh and gb are OVERWRITTEN,
  *                       not accumulated into.  gx is only the NDC term K(gn); the
@@ -111,8 +123,9 @@ size_t ndc_backward_workspace_bytes(const ndc_geom *g, int need_gx, int need_gz,
  *   workspace           >= ndc_backward_workspace_bytes(...) bytes, 256-byte aligned
  */
 int ndc_backward(const ndc_geom *g, const void *x, const void *z, const void *t1,
-                 const float *h, const float *bias, const void *gout, void *gx, void *gz,
-                 float *gh, float *gb, void *workspace, size_t workspace_bytes, void *stream);
+                 const void *inv_den, const void *ratio, const float *h, const float *bias,
+                 const void *gout, void *gx, void *gz, float *gh, float *gb, void *workspace,
+                 size_t workspace_bytes, void *stream);
 
 /*
  * ndc_backward with a stopwatch: same arguments and results, plus pass_ms[3] = device time in
@@ -123,9 +136,10 @@ int ndc_backward(const ndc_geom *g, const void *x, const void *z, const void *t1
  * The direct path is not instrumented and reports zeros.
  */
 int ndc_backward_profiled(const ndc_geom *g, const void *x, const void *z, const void *t1,
-                          const float *h, const float *bias, const void *gout, void *gx,
-                          void *gz, float *gh, float *gb, void *workspace,
-                          size_t workspace_bytes, void *stream, float *pass_ms);
+                          const void *inv_den, const void *ratio, const float *h,
+                          const float *bias, const void *gout, void *gx, void *gz, float *gh,
+                          float *gb, void *workspace, size_t workspace_bytes, void *stream,
+                          float *pass_ms);
 
 /*
  * Plain grouped convolution with the same tap conventions (adjoint = 0: K, 1: A), input

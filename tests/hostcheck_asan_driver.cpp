@@ -45,20 +45,25 @@ static int run_case(const Case &c)
     unsigned char *x = fill(nx), *z = fill(ns), *gout = fill(ns);
     unsigned char *out = (unsigned char *)malloc(ns * esz), *t1 = (unsigned char *)malloc(nx * esz);
     unsigned char *gx = (unsigned char *)malloc(nx * esz), *gz = (unsigned char *)malloc(ns * esz);
+    unsigned char *inv = (unsigned char *)malloc(ns * esz), *rat = (unsigned char *)malloc(ns * esz);
     std::vector<float> h(nh, 0.05f), bias((size_t)c.G * c.sc, 0.1f), gh(nh), gb((size_t)c.G * c.sc);
     const size_t fws = ndc_forward_workspace_bytes(&g);
     void *fw = nullptr;
     if (posix_memalign(&fw, 256, fws ? fws : 256)) return -100;
-    int st = ndc_forward(&g, x, z, h.data(), bias.data(), out, t1, fw, fws, nullptr);
+    int st = ndc_forward(&g, x, z, h.data(), bias.data(), out, t1, inv, rat, fw, fws, nullptr);
     free(fw);
     if (st) return st;
     const size_t wsb = ndc_backward_workspace_bytes(&g, 1, 1, 1, 1);
     void *ws = nullptr;
     if (posix_memalign(&ws, 256, wsb ? wsb : 256)) return -100;
-    st = ndc_backward(&g, x, z, t1, h.data(), bias.data(), gout, gx, gz, gh.data(), gb.data(), ws,
-                      wsb, nullptr);
+    // once re-gathering the denominator and ratio, once with the forward's copies
+    st = ndc_backward(&g, x, z, t1, nullptr, nullptr, h.data(), bias.data(), gout, gx, gz,
+                      gh.data(), gb.data(), ws, wsb, nullptr);
+    if (!st)
+        st = ndc_backward(&g, x, z, t1, inv, rat, h.data(), bias.data(), gout, gx, gz, gh.data(),
+                          gb.data(), ws, wsb, nullptr);
     free(ws);
-    free(x); free(z); free(gout); free(out); free(t1); free(gx); free(gz);
+    free(x); free(z); free(gout); free(out); free(t1); free(gx); free(gz); free(inv); free(rat);
     return st;
 }
 

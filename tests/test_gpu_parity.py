@@ -51,7 +51,7 @@ def _oracle(x, z, h, bias, gout, G, m, sc, eps, relu):
     return out, t1, grads
 
 
-def _run_case(geom, dtype, path, relu=True, with_bias=True):
+def _run_case(geom, dtype, path, relu=True, with_bias=True, saved=False):
     C, G, sc, ks, sp, B = geom
     m = C // G
     x, z, h, bias, gout = make_case(C, G, sc, ks, sp, B=B, dtype=dtype, bias_shift=0.3,
@@ -60,8 +60,10 @@ def _run_case(geom, dtype, path, relu=True, with_bias=True):
         bias = None
     lib = _lib_gpu()
     kw = dict(groups=G, m=m, sc=sc, eps=1e-16, relu_input=relu, path=path)
-    out, t1 = ops.update_forward(lib, x, z, h, bias, **kw)
-    gx, gz, gh, gb = ops.update_backward(lib, x, z, t1, h, bias, gout, **kw)
+    res = ops.update_forward(lib, x, z, h, bias, save_ratio=saved, **kw)
+    out, t1 = res[0], res[1]
+    gx, gz, gh, gb = ops.update_backward(lib, x, z, t1, h, bias, gout,
+                                         saved=res[2] if saved else None, **kw)
     torch.cuda.synchronize()
     ro, rt1, (rgx, rgz, rgh, rgb) = _oracle(x, z, h, bias, gout, G, m, sc, 1e-16, relu)
     tol = TOL[dtype]
@@ -71,7 +73,14 @@ def _run_case(geom, dtype, path, relu=True, with_bias=True):
     if with_bias:
         errs["gb"] = O.rel_err(gb.cpu(), rgb)
     bad = {k: v for k, v in errs.items() if not v < tol}
-    assert not bad, f"{geom} {dtype} path={path}: {bad} (all: {errs})"
+    assert not bad, f"{geom} {dtype} path={path} saved={saved}: {bad} (all: {errs})"
+    if saved:
+        # the kept tensors themselves: 1/(A(t1)+eps) and (A(x)+eps)/(A(t1)+eps)
+        d = [t.detach().cpu().double() for t in (x, z, h)]
+        s = O.rectified_source(d[1], None if bias is None else bias.cpu().double(), relu)
+        den = O.op_A(O.op_K(s, d[2], G, m, sc), d[2], G, m, sc) + 1e-16
+        assert O.rel_err(res[2][0].cpu(), 1.0 / den) < tol
+        assert O.rel_err(res[2][1].cpu(), (O.op_A(d[0], d[2], G, m, sc) + 1e-16) / den) < tol
     return errs
 
 
@@ -86,6 +95,20 @@ def test_direct_kernels(geom, dtype):
 def test_fused_kernels(geom, dtype):
     print("case", geom, dtype, flush=True)
     _run_case(geom, dtype, _lib.PATH_FUSED)
+
+
+@pytest.mark.parametrize("geom", FUSED_GEOMS)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_fused_kernels_with_saved_ratio(geom, dtype):
+    """Backward fed with the forward's denominator and ratio instead of re-gathering them."""
+    print("case saved", geom, dtype, flush=True)
+    _run_case(geom, dtype, _lib.PATH_FUSED, saved=True)
+
+
+def test_saved_ratio_later_iteration_form():
+    _run_case(FUSED_GEOMS[0], torch.bfloat16, _lib.PATH_FUSED, relu=False, with_bias=False,
+              saved=True)
+    _run_case(DIRECT_GEOMS[0], torch.float32, _lib.PATH_DIRECT, saved=True)
 
 
 @pytest.mark.parametrize("relu,with_bias", [(True, False), (False, False)])

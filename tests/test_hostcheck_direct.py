@@ -102,6 +102,6 @@ def test_c_abi_error_codes():
     assert lib.check_geometry(g) == -3
     g.dtype = 0
     with pytest.raises(_lib.NdcError):
-        lib.forward(g, None, None, None, None, None, None, None, 0, None)
+        lib.forward(g, None, None, None, None, None, None, None, None, None, 0, None)
     with pytest.raises(ValueError):
         _lib.make_geom(1, 1, 1, 1, (2, 2, 2, 2), (3, 3, 3, 3), 0, True, 0.0)

@@ -45,6 +45,15 @@ def test_fused_coverage_predicate():
         assert lib.check_geometry(bad) == 0   # the direct kernels still cover it
 
 
+def _saved_refs(x, z, h, bias, C, sc, eps, relu):
+    """1/(A(t1)+eps) and (A(x)+eps)/(A(t1)+eps) from the oracle's operators, float64."""
+    xd, zd, hd = x.double(), z.double(), h.double()
+    s = O.rectified_source(zd, None if bias is None else bias.double(), relu)
+    t1 = O.op_K(s, hd, C, 1, sc)
+    den = O.op_A(t1, hd, C, 1, sc) + eps
+    return 1.0 / den, (O.op_A(xd, hd, C, 1, sc) + eps) / den
+
+
 @pytest.mark.parametrize("geom", FUSED_GEOMS)
 @pytest.mark.parametrize("relu,with_bias", [(True, True), (False, False)])
 def test_fused_forward_backward_fp32(geom, relu, with_bias):
@@ -71,6 +80,15 @@ def test_fused_forward_backward_fp32(geom, relu, with_bias):
     assert O.rel_err(gh, rgh) < 1e-4
     if with_bias:
         assert O.rel_err(gb, rgb) < 1e-4
+
+
+def test_backward_uses_saved_predicate():
+    lib = hostcheck_library()
+    mk = lambda dt, ks, sp: _lib.make_geom(2, 8, 1, 4, sp, ks, dt, True, 1e-16)
+    assert lib.backward_uses_saved(mk(_lib.NDC_BF16, (3, 3, 3), (8, 8, 8)))
+    assert not lib.backward_uses_saved(mk(_lib.NDC_F32, (3, 3, 3), (8, 8, 8)))
+    assert not lib.backward_uses_saved(mk(_lib.NDC_BF16, (5, 5), (8, 8)))
+    assert not lib.backward_uses_saved(mk(_lib.NDC_BF16, (3, 3, 3), (8, 8, 7)))   # odd width
 
 
 def test_fused_inference_needs_no_t1():
@@ -108,6 +126,36 @@ def test_fused_bf16_storage(geom):
     for got, ref in ((gx, rgx), (gz, rgz), (gh, rgh), (gb, rgb)):
         assert O.rel_err(got, ref) < 2e-2
     assert host_faults(lib)[0] == 0
+
+
+@pytest.mark.parametrize("geom", FUSED_GEOMS[:3] + FUSED_GEOMS[5:6])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("relu", [True, False])
+def test_fused_saved_denominator_and_ratio(geom, dtype, relu):
+    """The forward's optional 1/d and n/d outputs, and a backward that consumes them."""
+    C, sc, ks, sp, B = geom
+    tol_f, tol_b = (1e-5, 1e-4) if dtype == torch.float32 else (2e-2, 2e-2)
+    lib = hostcheck_library()
+    x, z, h, bias, gout = make_case(C, C, sc, ks, sp, B=B, dtype=dtype, bias_shift=0.3,
+                                    positive_z=not relu)
+    kw = dict(groups=C, m=1, sc=sc, eps=1e-6, relu_input=relu, path=_lib.PATH_FUSED)
+    host_faults(lib)
+    out, t1, saved = ops.update_forward(lib, x, z, h, bias, save_ratio=True, **kw)
+    out0, t10 = ops.update_forward(lib, x, z, h, bias, **kw)
+    assert torch.equal(out, out0) and torch.equal(t1, t10)
+    r_inv, r_ratio = _saved_refs(x, z, h, bias, C, sc, 1e-6, relu)
+    assert O.rel_err(saved[0], r_inv) < tol_f
+    assert O.rel_err(saved[1], r_ratio) < tol_f
+    _, _, refs = _oracle(x, z, h, bias, gout, C, sc, 1e-6, relu)
+    got = ops.update_backward(lib, x, z, t1, h, bias, gout, saved=saved, **kw)
+    for a, r in zip(got, refs):
+        assert O.rel_err(a, r) < tol_b
+    n, first = host_faults(lib)
+    assert n == 0, f"LDS faults: {n} ({first})"
+    with pytest.raises(_lib.NdcError):   # both or neither
+        lib.backward(ops.make_geom_for(x, h, C, 1, sc, 1e-6, relu), x.data_ptr(), z.data_ptr(),
+                     t1.data_ptr(), saved[0].data_ptr(), None, h.data_ptr(), None,
+                     gout.data_ptr(), None, out.data_ptr(), None, None, None, 0, None)
 
 
 def test_fused_partial_outputs():
