@@ -114,28 +114,28 @@ class NdcLibrary:
         return self._dll.ndc_forward_workspace_bytes(ctypes.byref(g))
 
     def forward(self, g: Geom, x: int, z: int, h: int, bias: Optional[int], out: int,
-                t1: Optional[int], inv_den: Optional[int], ratio: Optional[int],
+                t1: Optional[int], s_over_den: Optional[int], ratio: Optional[int],
                 ws: Optional[int], ws_bytes: int, stream: Optional[int]) -> None:
-        self._check(self._dll.ndc_forward(ctypes.byref(g), x, z, h, bias, out, t1, inv_den, ratio,
+        self._check(self._dll.ndc_forward(ctypes.byref(g), x, z, h, bias, out, t1, s_over_den, ratio,
                                           ws, ws_bytes, stream), "ndc_forward")
 
     def backward_workspace_bytes(self, g: Geom, need_gx, need_gz, need_gh, need_gb) -> int:
         return self._dll.ndc_backward_workspace_bytes(
             ctypes.byref(g), int(need_gx), int(need_gz), int(need_gh), int(need_gb))
 
-    def backward(self, g: Geom, x, z, t1, inv_den, ratio, h, bias, gout, gx, gz, gh, gb, ws,
+    def backward(self, g: Geom, x, z, t1, s_over_den, ratio, h, bias, gout, gx, gz, gh, gb, ws,
                  ws_bytes, stream) -> None:
         self._check(
-            self._dll.ndc_backward(ctypes.byref(g), x, z, t1, inv_den, ratio, h, bias, gout, gx,
+            self._dll.ndc_backward(ctypes.byref(g), x, z, t1, s_over_den, ratio, h, bias, gout, gx,
                                    gz, gh, gb, ws, ws_bytes, stream),
             "ndc_backward")
 
-    def backward_profiled(self, g: Geom, x, z, t1, inv_den, ratio, h, bias, gout, gx, gz, gh, gb,
+    def backward_profiled(self, g: Geom, x, z, t1, s_over_den, ratio, h, bias, gout, gx, gz, gh, gb,
                           ws, ws_bytes, stream):
         """``backward`` plus the device time (ms) of pass 1, pass 2 and the reduction."""
         ms = (ctypes.c_float * 3)()
         self._check(
-            self._dll.ndc_backward_profiled(ctypes.byref(g), x, z, t1, inv_den, ratio, h, bias,
+            self._dll.ndc_backward_profiled(ctypes.byref(g), x, z, t1, s_over_den, ratio, h, bias,
                                             gout, gx, gz, gh, gb, ws, ws_bytes, stream, ms),
             "ndc_backward_profiled")
         return tuple(ms)

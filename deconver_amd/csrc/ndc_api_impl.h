@@ -64,7 +64,7 @@ static inline int choose_path(const ndc_geom *g, const KGeom &q)
 
 template <typename T>
 static int direct_forward(const KGeom &q, const T *x, const T *z, const float *h,
-                          const float *bias, T *out, T *t1, T *inv_den, T *ratio, void *stream)
+                          const float *bias, T *out, T *t1, T *s_over_den, T *ratio, void *stream)
 {
     // t1 = K(relu(z + b)) lands in the caller's t1; without one there is nowhere to put
     // it, so the direct path asks for it (the fused path does not need it)
@@ -75,7 +75,7 @@ static int direct_forward(const KGeom &q, const T *x, const T *z, const float *h
     });
     if (st) return st;
     return Backend::elementwise(n_s, stream, [=] NDC_LAMBDA(long long idx) {
-        direct::fwd<T>(idx, q, x, t1, z, h, bias, out, inv_den, ratio);
+        direct::fwd<T>(idx, q, x, t1, z, h, bias, out, s_over_den, ratio);
     });
 }
 
@@ -204,7 +204,7 @@ size_t ndc_forward_workspace_bytes(const ndc_geom *g)
 }
 
 int ndc_forward(const ndc_geom *g, const void *x, const void *z, const float *h,
-                const float *bias, void *out, void *t1, void *inv_den, void *ratio,
+                const float *bias, void *out, void *t1, void *s_over_den, void *ratio,
                 void *workspace, size_t workspace_bytes, void *stream)
 {
     using namespace ndc;
@@ -212,7 +212,7 @@ int ndc_forward(const ndc_geom *g, const void *x, const void *z, const float *h,
     int st = make_kgeom(g, q);
     if (st) return st;
     if (!x || !z || !h || !out) return NDC_ERR_NULL;
-    if ((inv_den == nullptr) != (ratio == nullptr)) return NDC_ERR_NULL;
+    if ((s_over_den == nullptr) != (ratio == nullptr)) return NDC_ERR_NULL;
     const int path = choose_path(g, q);
     if (path < 0) return path;
     if (path == NDC_PATH_FUSED) {
@@ -222,18 +222,18 @@ int ndc_forward(const ndc_geom *g, const void *x, const void *z, const float *h,
         void *ws = need ? workspace : nullptr;
         return g->dtype == NDC_F32
                    ? fused::forward<Backend, float>(q, (const float *)x, (const float *)z, h, bias,
-                                                    (float *)out, (float *)t1, (float *)inv_den,
+                                                    (float *)out, (float *)t1, (float *)s_over_den,
                                                     (float *)ratio, ws, stream)
                    : fused::forward<Backend, bf16_t>(q, (const bf16_t *)x, (const bf16_t *)z, h,
                                                      bias, (bf16_t *)out, (bf16_t *)t1,
-                                                     (bf16_t *)inv_den, (bf16_t *)ratio, ws, stream);
+                                                     (bf16_t *)s_over_den, (bf16_t *)ratio, ws, stream);
     }
     return g->dtype == NDC_F32
                ? direct_forward<float>(q, (const float *)x, (const float *)z, h, bias,
-                                       (float *)out, (float *)t1, (float *)inv_den,
+                                       (float *)out, (float *)t1, (float *)s_over_den,
                                        (float *)ratio, stream)
                : direct_forward<bf16_t>(q, (const bf16_t *)x, (const bf16_t *)z, h, bias,
-                                        (bf16_t *)out, (bf16_t *)t1, (bf16_t *)inv_den,
+                                        (bf16_t *)out, (bf16_t *)t1, (bf16_t *)s_over_den,
                                         (bf16_t *)ratio, stream);
 }
 
@@ -261,7 +261,7 @@ size_t ndc_backward_workspace_bytes(const ndc_geom *g, int need_gx, int need_gz,
 }
 
 static int backward_impl(const ndc_geom *g, const void *x, const void *z, const void *t1,
-                         const void *inv_den, const void *ratio, const float *h, const float *bias,
+                         const void *s_over_den, const void *ratio, const float *h, const float *bias,
                          const void *gout, void *gx, void *gz, float *gh, float *gb,
                          void *workspace, size_t workspace_bytes, void *stream, float *pass_ms)
 {
@@ -270,7 +270,7 @@ static int backward_impl(const ndc_geom *g, const void *x, const void *z, const 
     int st = make_kgeom(g, q);
     if (st) return st;
     if (!x || !z || !t1 || !h || !gout) return NDC_ERR_NULL;
-    if ((inv_den == nullptr) != (ratio == nullptr)) return NDC_ERR_NULL;
+    if ((s_over_den == nullptr) != (ratio == nullptr)) return NDC_ERR_NULL;
     if (!gx && !gz && !gh && !gb) return NDC_OK;
     const int path = choose_path(g, q);
     if (path < 0) return path;
@@ -281,12 +281,12 @@ static int backward_impl(const ndc_geom *g, const void *x, const void *z, const 
     if (path == NDC_PATH_FUSED) {
         return g->dtype == NDC_F32
                    ? fused::backward<Backend, float>(q, (const float *)x, (const float *)z,
-                                                     (const float *)t1, (const float *)inv_den,
+                                                     (const float *)t1, (const float *)s_over_den,
                                                      (const float *)ratio, h, bias,
                                                      (const float *)gout, (float *)gx,
                                                      (float *)gz, gh, gb, workspace, stream, pass_ms)
                    : fused::backward<Backend, bf16_t>(q, (const bf16_t *)x, (const bf16_t *)z,
-                                                      (const bf16_t *)t1, (const bf16_t *)inv_den,
+                                                      (const bf16_t *)t1, (const bf16_t *)s_over_den,
                                                       (const bf16_t *)ratio, h, bias,
                                                       (const bf16_t *)gout, (bf16_t *)gx,
                                                       (bf16_t *)gz, gh, gb, workspace, stream, pass_ms);
@@ -301,23 +301,23 @@ static int backward_impl(const ndc_geom *g, const void *x, const void *z, const 
 }
 
 int ndc_backward(const ndc_geom *g, const void *x, const void *z, const void *t1,
-                 const void *inv_den, const void *ratio, const float *h, const float *bias,
+                 const void *s_over_den, const void *ratio, const float *h, const float *bias,
                  const void *gout, void *gx, void *gz, float *gh, float *gb, void *workspace,
                  size_t workspace_bytes, void *stream)
 {
-    return backward_impl(g, x, z, t1, inv_den, ratio, h, bias, gout, gx, gz, gh, gb, workspace,
+    return backward_impl(g, x, z, t1, s_over_den, ratio, h, bias, gout, gx, gz, gh, gb, workspace,
                          workspace_bytes, stream, nullptr);
 }
 
 int ndc_backward_profiled(const ndc_geom *g, const void *x, const void *z, const void *t1,
-                          const void *inv_den, const void *ratio, const float *h,
+                          const void *s_over_den, const void *ratio, const float *h,
                           const float *bias, const void *gout, void *gx, void *gz, float *gh,
                           float *gb, void *workspace, size_t workspace_bytes, void *stream,
                           float *pass_ms)
 {
     if (!pass_ms) return NDC_ERR_NULL;
     pass_ms[0] = pass_ms[1] = pass_ms[2] = 0.f;
-    return backward_impl(g, x, z, t1, inv_den, ratio, h, bias, gout, gx, gz, gh, gb, workspace,
+    return backward_impl(g, x, z, t1, s_over_den, ratio, h, bias, gout, gx, gz, gh, gb, workspace,
                          workspace_bytes, stream, pass_ms);
 }
 

@@ -119,14 +119,14 @@ NDC_HD void num_den(const KGeom &q, const Pos &p, const T *x, const T *t1, const
 // out = s * (A(x)+eps) / (A(t1)+eps), idx over (B, G*sc, S)
 template <typename T>
 NDC_HD void fwd(long long idx, const KGeom &q, const T *x, const T *t1, const T *z,
-                const float *hf, const float *bias, T *out, T *inv_den, T *ratio)
+                const float *hf, const float *bias, T *out, T *s_over_den, T *ratio)
 {
     const Pos p = decode(idx, q, q.sc);
     float n, d;
     num_den<T>(q, p, x, t1, hf, n, d);
     const float s = source_at<T>(q, z, bias, idx, p.g * q.sc + p.ch);
     Elem<T>::store(out + idx, s * n / d);
-    if (inv_den) Elem<T>::store(inv_den + idx, 1.0f / d);
+    if (s_over_den) Elem<T>::store(s_over_den + idx, s / d);
     if (ratio) Elem<T>::store(ratio + idx, n / d);
 }
 

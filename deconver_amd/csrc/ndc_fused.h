@@ -120,7 +120,7 @@ template <typename T> struct FwdParams {
     const float *h, *bias;
     const float *wtab;   // packed bf16 tap tables (bf16 dot2 kernels only)
     T *out, *t1;
-    T *inv_den, *ratio;   // optional: 1/(A(t1)+eps) and (A(x)+eps)/(A(t1)+eps), shape of out
+    T *s_over_den, *ratio;   // optional: s/(A(t1)+eps) and (A(x)+eps)/(A(t1)+eps), shape of out
     int B, C, D, H, W;
     int relu;
     float eps;
@@ -129,7 +129,7 @@ template <typename T> struct FwdParams {
 
 template <typename T> struct BwdParams {
     const T *x, *z, *t1, *gout;
-    const T *inv_den, *ratio;   // optional: what the forward call saved (both or neither)
+    const T *s_over_den, *ratio;   // optional: what the forward call saved (both or neither)
     const float *h, *bias;
     const float *wtab;   // packed bf16 tap tables (bf16 dot2 kernels only)
     T *gx, *gz;
@@ -525,7 +525,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                     for (int i = 0; i < SC; ++i) copy_taps<KH * KW>(wn[i], wt[i]);
                 }
                 T *ok_ = og + (long long)j0 * plane;
-                T *dk_ = p.inv_den ? p.inv_den + (og - p.out) + (long long)j0 * plane : nullptr;
+                T *dk_ = p.s_over_den ? p.s_over_den + (og - p.out) + (long long)j0 * plane : nullptr;
                 T *rk_ = p.ratio ? p.ratio + (og - p.out) + (long long)j0 * plane : nullptr;
                 NDC_UNROLL
                 for (int r = 0; r < RH; ++r) {
@@ -535,8 +535,9 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                         float v[RW], rd[RW], rt[RW];
                         NDC_UNROLL
                         for (int c = 0; c < RW; ++c) {
-                            rd[c] = fast_rcp(acc[1][i][r][c] + eps);
-                            rt[c] = (acc[0][i][r][c] + eps) * rd[c];
+                            const float inv = fast_rcp(acc[1][i][r][c] + eps);
+                            rd[c] = sv[i][r][c] * inv;
+                            rt[c] = (acc[0][i][r][c] + eps) * inv;
                             v[c] = sv[i][r][c] * rt[c];
                         }
                         IO::store(ok_ + i * cplane + st.ooff[r], v);

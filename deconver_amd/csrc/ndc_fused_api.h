@@ -34,7 +34,7 @@ struct Variant {
 // Launch-shape choices that are not dictated by the geometry.  Defaults are the measured
 // best; the environment variables exist for tuning runs only.
 struct Tuning {
-    int rhf, rwf, rhb, rwb, threads_f, threads_b;
+    int rhf, rwf, rhb, rwb, threads_f, threads_b, threads_b2;
 };
 
 static inline int env_int(const char *name, int dflt)
@@ -52,6 +52,7 @@ static inline Tuning tuning()
     t.rwb = env_int("NDC_TUNE_RWB", 0);
     t.threads_f = env_int("NDC_TUNE_NTF", 256);
     t.threads_b = env_int("NDC_TUNE_NTB", 512);
+    t.threads_b2 = env_int("NDC_TUNE_NTB", 256);   // bf16 dot2 kernels
     return t;
 }
 
@@ -129,7 +130,7 @@ static inline bool make_plan(const KGeom &q, Plan &pl, bool pairs_ok = true, int
         pl.m.KH == 3 && pl.m.KW == 3 && env_int("NDC_TUNE_DOT2", 1)) {
         Tile tf, tb;
         if (make_tile(pl.m, kDot2RH, 2, tn.threads_f, tf) &&
-            make_tile(pl.m, kDot2RH, 2, tn.threads_b, tb)) {
+            make_tile(pl.m, kDot2RH, 2, tn.threads_b2, tb)) {
             const int lf = FwdKernelB<kDot2RH>::lds_floats(tf);
             const int l1 = Bwd1KernelB<kDot2RH>::lds_floats(tb);
             const int l2 = Bwd2KernelB<kDot2RH>::lds_floats(tb);
@@ -189,7 +190,7 @@ static inline size_t forward_ws(const KGeom &q, int dtype)
     return align256((size_t)q.G * kTabWords * 4);
 }
 
-// whether backward() reads the forward's 1/d and n/d for this geometry (aligned pointers
+// whether backward() reads the forward's s/d and n/d for this geometry (aligned pointers
 // assumed): only the bf16 dot2 kernels have that form
 static inline bool backward_uses_saved(const KGeom &q, int dtype)
 {
@@ -207,7 +208,7 @@ template <class BE> struct Dot2Launch<BE, bf16_t> {
     {
         return BE::template block_kernel<FwdKernelB<kDot2RH>>(p, pl.nblk_f, pl.tf.NT, pl.lds_f, stream);
     }
-    // saved: the call brought the forward's 1/d and n/d
+    // saved: the call brought the forward's s/d and n/d
     static int bwd1(const BwdParams<bf16_t> &p, const Plan &pl, void *stream, bool saved)
     {
         if (saved)
@@ -226,11 +227,11 @@ template <class BE> struct Dot2Launch<BE, bf16_t> {
 
 template <class BE, typename T>
 static int forward(const KGeom &q, const T *x, const T *z, const float *h, const float *bias,
-                   T *out, T *t1, T *inv_den, T *ratio, void *ws, void *stream)
+                   T *out, T *t1, T *s_over_den, T *ratio, void *ws, void *stream)
 {
     Plan pl;
     const bool pairs = pair_aligned<T>(x) && pair_aligned<T>(z) && pair_aligned<T>(out) &&
-                       pair_aligned<T>(t1) && pair_aligned<T>(inv_den) && pair_aligned<T>(ratio);
+                       pair_aligned<T>(t1) && pair_aligned<T>(s_over_den) && pair_aligned<T>(ratio);
     const int dtype = sizeof(T) == 2 ? NDC_BF16 : NDC_F32;
     if (!make_plan(q, pl, pairs, ws ? dtype : NDC_F32)) return NDC_ERR_GEOMETRY;
     FwdParams<T> p;
@@ -241,7 +242,7 @@ static int forward(const KGeom &q, const T *x, const T *z, const float *h, const
     p.bias = bias;
     p.out = out;
     p.t1 = t1;
-    p.inv_den = inv_den;
+    p.s_over_den = s_over_den;
     p.ratio = ratio;
     p.B = q.B;
     p.C = q.G;
@@ -269,7 +270,7 @@ static int forward(const KGeom &q, const T *x, const T *z, const float *h, const
 }
 
 template <class BE, typename T>
-static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const T *inv_den,
+static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const T *s_over_den,
                     const T *ratio, const float *h, const float *bias, const T *gout, T *gx,
                     T *gz, float *gh, float *gb, void *ws, void *stream, float *pass_ms = nullptr)
 {
@@ -279,8 +280,8 @@ static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const T
     Plan pl;
     const bool pairs = pair_aligned<T>(x) && pair_aligned<T>(z) && pair_aligned<T>(t1) &&
                        pair_aligned<T>(gout) && pair_aligned<T>(gx) && pair_aligned<T>(gz) &&
-                       pair_aligned<T>(inv_den) && pair_aligned<T>(ratio);
-    const bool saved = inv_den != nullptr && ratio != nullptr;
+                       pair_aligned<T>(s_over_den) && pair_aligned<T>(ratio);
+    const bool saved = s_over_den != nullptr && ratio != nullptr;
     const int dtype = sizeof(T) == 2 ? NDC_BF16 : NDC_F32;
     if (!make_plan(q, pl, pairs, dtype)) return NDC_ERR_GEOMETRY;
     const size_t n_x = (size_t)q.B * q.G * q.SP;
@@ -299,7 +300,7 @@ static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const T
     p.z = z;
     p.t1 = t1;
     p.gout = gout;
-    p.inv_den = inv_den;
+    p.s_over_den = s_over_den;
     p.ratio = ratio;
     p.h = h;
     p.bias = bias;

@@ -373,7 +373,7 @@ template <int RH_> struct FwdKernelB {
                     a_plane_d2<RH, RW, 2>(ex, base, P, wt, acc);
                 }
                 T *ok_ = og + (long long)j0 * plane;
-                T *dk_ = p.inv_den ? p.inv_den + (og - p.out) + (long long)j0 * plane : nullptr;
+                T *dk_ = p.s_over_den ? p.s_over_den + (og - p.out) + (long long)j0 * plane : nullptr;
                 T *rk_ = p.ratio ? p.ratio + (og - p.out) + (long long)j0 * plane : nullptr;
                 NDC_UNROLL
                 for (int r = 0; r < RH; ++r) {
@@ -385,8 +385,9 @@ template <int RH_> struct FwdKernelB {
                         for (int c = 0; c < RW; ++c) {
                             const uint32_t w = st.own[i >> 1][r][c];
                             const float s = (i & 1) ? bf_hi(w) : bf_lo(w);
-                            rd[c] = fast_rcp(acc[1][i][r][c]);
-                            rt[c] = acc[0][i][r][c] * rd[c];
+                            const float inv = fast_rcp(acc[1][i][r][c]);
+                            rd[c] = s * inv;
+                            rt[c] = acc[0][i][r][c] * inv;
                             v[c] = s * rt[c];
                         }
                         st_word(ok_ + i * cplane, st.ooff[r], pack_bf16x2(v[0], v[1]));
@@ -403,8 +404,9 @@ template <int RH_> struct FwdKernelB {
 
 // =================================================================== backward pass 1 (bf16, dot2)
 
-// SAVED: the call brings the forward's 1/d and n/d, so gn = g s (1/d), gd = -gn (n/d) are
-// elementwise and the plane-pair rings of x and t1 (for re-gathering n and d) are not kept.
+// SAVED: the call brings the forward's s/d and n/d, so gn = g (s/d), gd = -gn (n/d) are
+// elementwise (z is not read) and the plane-pair rings of x and t1 (for re-gathering n and d)
+// are not kept.
 template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
     static constexpr bool SAVED = SAVED_;
     static constexpr int KD = 3, KH = 3, KW = 3, SC = 4, RH = RH_, RW = 2;
@@ -448,7 +450,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
         const long long cbase = ((long long)id.b * p.C + id.c) * cplane;
         const T *xg = p.x + cbase, *t1g = p.t1 + cbase;
         const T *zg = p.z + cbase * SC, *gg = p.gout + cbase * SC;
-        const T *dg = SAVED ? p.inv_den + cbase * SC : nullptr;
+        const T *dg = SAVED ? p.s_over_den + cbase * SC : nullptr;
         const T *rg = SAVED ? p.ratio + cbase * SC : nullptr;
         T *gxg = p.gx ? p.gx + cbase : nullptr;
         T *gt1g = p.gt1 + cbase;
@@ -511,12 +513,13 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
                 const unsigned o = (unsigned)(clampi(row, 0, H - 1) * W + st.ln.c0) * 2u;
                 NDC_UNROLL
                 for (int i = 0; i < SC; ++i) {
-                    zw[i][r] = ld_word(zk + i * cplane, o);
                     gw[i][r] = ld_word(gk + i * cplane, o);
                     if (SAVED) {
+                        zw[i][r] = 0u;
                         dw[i][r] = ld_word(dg + (long long)j1 * plane + i * cplane, o);
                         rw[i][r] = ld_word(rg + (long long)j1 * plane + i * cplane, o);
                     } else {
+                        zw[i][r] = ld_word(zk + i * cplane, o);
                         dw[i][r] = rw[i][r] = 0u;
                     }
                 }
@@ -551,7 +554,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
                         const float sv = floor_f((c ? bf_hi(zw[i][r]) : bf_lo(zw[i][r])) + st.bv[i], floor_);
                         const float gv = ok[r] ? (c ? bf_hi(gw[i][r]) : bf_lo(gw[i][r])) : 0.f;
                         if (SAVED) {
-                            gn[i][c] = gv * sv * (c ? bf_hi(dw[i][r]) : bf_lo(dw[i][r]));
+                            gn[i][c] = gv * (c ? bf_hi(dw[i][r]) : bf_lo(dw[i][r]));
                             gd[i][c] = -(gn[i][c] * (c ? bf_hi(rw[i][r]) : bf_lo(rw[i][r])));
                         } else {
                             const float inv = fast_rcp(acc[1][i][r][c]);

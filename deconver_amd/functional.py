@@ -4,7 +4,7 @@ Mirrors ``deconver/deconvolution/functional.py:97-207`` of the reference
 (``DeconvUpdate`` / ``deconv_update``): same arguments, same returned gradients
 ``(gx, gz, gh, gb, None x5)``, same refusal of double backward.  It saves the reference's
 ``(x, z, t1, h, bias)`` plus, unless ``save_ratio(False)`` was called, the forward's
-``1/(A(t1)+eps)`` and ``(A(x)+eps)/(A(t1)+eps)``: two tensors of the size of the output
+``s/(A(t1)+eps)`` and ``(A(x)+eps)/(A(t1)+eps)``: two tensors of the size of the output
 kept until backward, which then does not gather ``A(x)`` and ``A(t1)`` a second time.
 The arithmetic is in ``libdeconver_ndc.so``; there is no PyTorch implementation behind
 this node.
@@ -83,9 +83,9 @@ class DeconvUpdate(torch.autograd.Function):
             res = ops.update_forward(lib, x, z, hc, bias, groups=groups, m=m, sc=sc, eps=eps,
                                      relu_input=relu_input, need_t1=need_t1, save_ratio=keep)
         out, t1 = res[0], res[1]
-        inv_den, ratio = res[2] if keep else (None, None)
+        s_over_den, ratio = res[2] if keep else (None, None)
         ctx.cfg = (groups, m, sc, eps, relu_input)
-        ctx.save_for_backward(x, z, t1, hc, bias, inv_den, ratio)
+        ctx.save_for_backward(x, z, t1, hc, bias, s_over_den, ratio)
         return out
 
     @staticmethod
@@ -97,7 +97,7 @@ class DeconvUpdate(torch.autograd.Function):
                 "double backward through the fused Deconv update is not supported; "
                 "construct the layer with a convolution keyword argument (e.g. stride=1) "
                 "to force the general path, which is plain PyTorch and doubly differentiable")
-        x, z, t1, h, bias, inv_den, ratio = ctx.saved_tensors
+        x, z, t1, h, bias, s_over_den, ratio = ctx.saved_tensors
         groups, m, sc, eps, relu_input = ctx.cfg
         need_x, need_z, need_h, need_b = ctx.needs_input_grad[:4]
         if t1 is None:
@@ -111,7 +111,7 @@ class DeconvUpdate(torch.autograd.Function):
                 lib, x, z, t1, h, bias, gout, groups=groups, m=m, sc=sc, eps=eps,
                 relu_input=relu_input, need_x=need_x, need_z=need_z, need_h=need_h,
                 need_b=need_b and bias is not None,
-                saved=None if inv_den is None else (inv_den, ratio))
+                saved=None if s_over_den is None else (s_over_den, ratio))
         return gx, gz, gh, gb, None, None, None, None, None
 
 

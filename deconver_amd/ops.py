@@ -70,7 +70,7 @@ def update_forward(lib: _lib.NdcLibrary, x: Tensor, z: Tensor, h: Tensor,
                    path: int = _lib.PATH_AUTO):
     """``out = s*(A(x)+eps)/(A(K(s))+eps)`` with ``s = relu?(z+bias)``.
 
-    Returns ``(out, t1)``, or ``(out, t1, (inv_den, ratio))`` with ``save_ratio``: the two
+    Returns ``(out, t1)``, or ``(out, t1, (s_over_den, ratio))`` with ``save_ratio``: the two
     extra tensors (shape of ``out``) that let :func:`update_backward` skip re-gathering
     ``A(x)`` and ``A(t1)``."""
     _check_common(x, z, h, bias, groups, m, sc)
@@ -83,12 +83,12 @@ def update_forward(lib: _lib.NdcLibrary, x: Tensor, z: Tensor, h: Tensor,
     if nbytes:
         ws = torch.empty(nbytes + 256, dtype=torch.uint8, device=x.device)
         ws_ptr = (ws.data_ptr() + 255) // 256 * 256
-    inv_den = torch.empty_like(z) if save_ratio else None
+    s_over_den = torch.empty_like(z) if save_ratio else None
     ratio = torch.empty_like(z) if save_ratio else None
-    lib.forward(g, _ptr(x), _ptr(z), _ptr(h), _ptr(bias), _ptr(out), _ptr(t1), _ptr(inv_den),
+    lib.forward(g, _ptr(x), _ptr(z), _ptr(h), _ptr(bias), _ptr(out), _ptr(t1), _ptr(s_over_den),
                 _ptr(ratio), ws_ptr, nbytes, _stream_of(x))
     if save_ratio:
-        return out, t1, (inv_den, ratio)
+        return out, t1, (s_over_den, ratio)
     return out, t1
 
 
@@ -100,7 +100,7 @@ def update_backward(lib: _lib.NdcLibrary, x: Tensor, z: Tensor, t1: Tensor, h: T
                     saved: Optional[Tuple[Tensor, Tensor]] = None):
     """Gradients ``(gx, gz, gh, gb)`` of the update; entries not asked for are ``None``.
 
-    ``saved``: the ``(inv_den, ratio)`` pair a ``save_ratio`` forward call returned for the
+    ``saved``: the ``(s_over_den, ratio)`` pair a ``save_ratio`` forward call returned for the
     same inputs.
 
     ``pass_times``: a list that, if given, receives the device milliseconds of the three
@@ -110,10 +110,10 @@ def update_backward(lib: _lib.NdcLibrary, x: Tensor, z: Tensor, t1: Tensor, h: T
         raise ValueError("gout must be contiguous with the shape and dtype of z")
     if t1.shape != x.shape or t1.dtype != x.dtype or not t1.is_contiguous():
         raise ValueError("t1 must be contiguous with the shape and dtype of x")
-    inv_den = ratio = None
+    s_over_den = ratio = None
     if saved is not None:
-        inv_den, ratio = saved
-        for t in (inv_den, ratio):
+        s_over_den, ratio = saved
+        for t in (s_over_den, ratio):
             if t.shape != z.shape or t.dtype != z.dtype or not t.is_contiguous():
                 raise ValueError("saved tensors must be contiguous with the shape and dtype of z")
     need_b = need_b and bias is not None
@@ -125,7 +125,7 @@ def update_backward(lib: _lib.NdcLibrary, x: Tensor, z: Tensor, t1: Tensor, h: T
     nbytes = lib.backward_workspace_bytes(g, need_x, need_z, need_h, need_b)
     ws = torch.empty(max(nbytes, 1) + 256, dtype=torch.uint8, device=x.device)
     ws_ptr = (ws.data_ptr() + 255) // 256 * 256
-    args = (g, _ptr(x), _ptr(z), _ptr(t1), _ptr(inv_den), _ptr(ratio), _ptr(h), _ptr(bias),
+    args = (g, _ptr(x), _ptr(z), _ptr(t1), _ptr(s_over_den), _ptr(ratio), _ptr(h), _ptr(bias),
             _ptr(gout), _ptr(gx),
             _ptr(gz), _ptr(gh), _ptr(gb), ws_ptr, nbytes, _stream_of(x))
     if pass_times is None:

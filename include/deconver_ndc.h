@@ -73,7 +73,7 @@ int ndc_fused_supported(const ndc_geom *g);
 /* 0 if some path covers `g` (then every entry point below accepts it), else a status. */
 int ndc_check_geometry(const ndc_geom *g);
 
-/* 1 if `ndc_backward` for `g` reads the forward's inv_den / ratio when they are passed (so
+/* 1 if `ndc_backward` for `g` reads the forward's s_over_den / ratio when they are passed (so
  * that keeping them pays), 0 if its kernels re-gather regardless.  No counterpart in the
  * reference. */
 int ndc_backward_uses_saved(const ndc_geom *g);
@@ -92,16 +92,16 @@ size_t ndc_forward_workspace_bytes(const ndc_geom *g);
  *   t1            optional output K(s), same shape/dtype as x: pass it when a backward
  *                 call will follow (it is what the reference saves for backward), null
  *                 for inference
- *   inv_den,      optional outputs 1/(A(t1)+eps) and (A(x)+eps)/(A(t1)+eps), same shape/dtype
+ *   s_over_den,   optional outputs s/(A(t1)+eps) and (A(x)+eps)/(A(t1)+eps), same shape/dtype
  *   ratio         as out; both or neither.  Handing them to ndc_backward lets it skip
  *                 re-gathering A(x) and A(t1): more memory kept between the two calls
- *                 (two tensors of the size of out) for fewer multiplications.  The
+ *                 (two tensors of the size of out) for fewer multiplications and no second read of z in pass 1.  The
  *                 reference has no counterpart (it re-gathers, kernels.py:791-838).
  *   workspace     >= ndc_forward_workspace_bytes(g) bytes, 256-byte aligned (may be null
  *                 when that is 0)
  */
 int ndc_forward(const ndc_geom *g, const void *x, const void *z, const float *h,
-                const float *bias, void *out, void *t1, void *inv_den, void *ratio,
+                const float *bias, void *out, void *t1, void *s_over_den, void *ratio,
                 void *workspace, size_t workspace_bytes, void *stream);
 
 /* Bytes of scratch `ndc_backward` needs for `g` with the requested outputs (each flag
@@ -114,7 +114,7 @@ size_t ndc_backward_workspace_bytes(const ndc_geom *g, int need_gx, int need_gz,
  * (deconver/deconvolution/functional.py:118-182), i.e. kernels.deconv_bwd, gconv x2,
  * wgrad x3, deconv_gz and the bias reduction (kernels.py:791-894).
  *   x, z, t1, h, bias   what the forward call saw / produced (bias may be null)
- *   inv_den, ratio      what the forward call wrote for the same inputs, or both null (then
+ *   s_over_den, ratio   what the forward call wrote for the same inputs, or both null (then
  *                       the kernels re-gather A(x) and A(t1)); results agree to rounding
  *   gout                upstream gradient, shape/dtype of out
  *   gx, gz, gh, gb      optional outputs (null = not needed); gh and gb are OVERWRITTEN,
@@ -123,7 +123,7 @@ size_t ndc_backward_workspace_bytes(const ndc_geom *g, int need_gx, int need_gz,
  *   workspace           >= ndc_backward_workspace_bytes(...) bytes, 256-byte aligned
  */
 int ndc_backward(const ndc_geom *g, const void *x, const void *z, const void *t1,
-                 const void *inv_den, const void *ratio, const float *h, const float *bias,
+                 const void *s_over_den, const void *ratio, const float *h, const float *bias,
                  const void *gout, void *gx, void *gz, float *gh, float *gb, void *workspace,
                  size_t workspace_bytes, void *stream);
 
@@ -136,7 +136,7 @@ int ndc_backward(const ndc_geom *g, const void *x, const void *z, const void *t1
  * The direct path is not instrumented and reports zeros.
  */
 int ndc_backward_profiled(const ndc_geom *g, const void *x, const void *z, const void *t1,
-                          const void *inv_den, const void *ratio, const float *h,
+                          const void *s_over_den, const void *ratio, const float *h,
                           const float *bias, const void *gout, void *gx, void *gz, float *gh,
                           float *gb, void *workspace, size_t workspace_bytes, void *stream,
                           float *pass_ms);

@@ -75,11 +75,11 @@ def _run_case(geom, dtype, path, relu=True, with_bias=True, saved=False):
     bad = {k: v for k, v in errs.items() if not v < tol}
     assert not bad, f"{geom} {dtype} path={path} saved={saved}: {bad} (all: {errs})"
     if saved:
-        # the kept tensors themselves: 1/(A(t1)+eps) and (A(x)+eps)/(A(t1)+eps)
+        # the kept tensors themselves: s/(A(t1)+eps) and (A(x)+eps)/(A(t1)+eps)
         d = [t.detach().cpu().double() for t in (x, z, h)]
         s = O.rectified_source(d[1], None if bias is None else bias.cpu().double(), relu)
         den = O.op_A(O.op_K(s, d[2], G, m, sc), d[2], G, m, sc) + 1e-16
-        assert O.rel_err(res[2][0].cpu(), 1.0 / den) < tol
+        assert O.rel_err(res[2][0].cpu(), s / den) < tol
         assert O.rel_err(res[2][1].cpu(), (O.op_A(d[0], d[2], G, m, sc) + 1e-16) / den) < tol
     return errs
 

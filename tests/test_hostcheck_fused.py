@@ -46,12 +46,12 @@ def test_fused_coverage_predicate():
 
 
 def _saved_refs(x, z, h, bias, C, sc, eps, relu):
-    """1/(A(t1)+eps) and (A(x)+eps)/(A(t1)+eps) from the oracle's operators, float64."""
+    """s/(A(t1)+eps) and (A(x)+eps)/(A(t1)+eps) from the oracle's operators, float64."""
     xd, zd, hd = x.double(), z.double(), h.double()
     s = O.rectified_source(zd, None if bias is None else bias.double(), relu)
     t1 = O.op_K(s, hd, C, 1, sc)
     den = O.op_A(t1, hd, C, 1, sc) + eps
-    return 1.0 / den, (O.op_A(xd, hd, C, 1, sc) + eps) / den
+    return s / den, (O.op_A(xd, hd, C, 1, sc) + eps) / den
 
 
 @pytest.mark.parametrize("geom", FUSED_GEOMS)
@@ -132,7 +132,7 @@ def test_fused_bf16_storage(geom):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("relu", [True, False])
 def test_fused_saved_denominator_and_ratio(geom, dtype, relu):
-    """The forward's optional 1/d and n/d outputs, and a backward that consumes them."""
+    """The forward's optional s/d and n/d outputs, and a backward that consumes them."""
     C, sc, ks, sp, B = geom
     tol_f, tol_b = (1e-5, 1e-4) if dtype == torch.float32 else (2e-2, 2e-2)
     lib = hostcheck_library()
