@@ -431,11 +431,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
             // ---- K-scatter: plane k of s feeds the KD pending planes of t1
             ex.each([&](State &st, int) NDC_LAMBDA {
                 if (!st.ln.active) return;
-#ifdef NDC_EXP_NOEXTRA
-                const bool extra = false;
-#else
                 const bool extra = XT && st.ln.strip < 2 * PH;
-#endif
                 const int jx = halo_row(st.ln.strip, PH, TH);
                 const int cb = PL + st.ln.c0 - PW;
                 if (k < D) {
@@ -476,9 +472,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                     }
                 }
             });
-#ifndef NDC_EXP_NOSYNC2
             ex.sync();
-#endif
 
             // ---- prefetch of the next plane, then A-gather + epilogue for plane k - 2*PD
             ex.each([&](State &st, int) NDC_LAMBDA {

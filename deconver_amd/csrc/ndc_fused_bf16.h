@@ -142,7 +142,7 @@ template <int RH_> struct FwdKernelB {
     static constexpr int KD = 3, KH = 3, KW = 3, SC = 4, RH = RH_, RW = 2;
     static constexpr int PD = 1, PH = 1, PW = 1, KT = 27;
     static constexpr int RHK = RH + 1, NZR = RH + 2, NXR = RH + 1;
-    static constexpr int NS = 3, NX = 3, NTP = 2;   // ring slots: source, x pairs, t1 pairs
+    static constexpr int NS = 3, NX = 2, NTP = 2;   // ring slots: source, x pairs, t1 pairs
     typedef bf16_t T;
     typedef FwdParams<T> Params;
     typedef VecIO<T, 2> IO;
@@ -208,8 +208,7 @@ template <int RH_> struct FwdKernelB {
             }
         };
 
-        // registers -> LDS: source plane k as channel-pair words into slot k % 3; x plane
-        // k - 1 completes the plane-pair word (x[k-2], x[k-1]) of slot (k - 2) % 3
+        // registers -> LDS: source plane k as channel-pair words into slot k % 3
         auto store_plane = [&](State &st, int k) NDC_LAMBDA {
             if (!st.ln.active) return;
             const int lb = PL + st.ln.c0;
@@ -233,6 +232,12 @@ template <int RH_> struct FwdKernelB {
                     ex.st_(sb + (RS + j) * P + lb + c, bits_to_float(pack_bf16x2(s[2][c], s[3][c])));
                 }
             }
+        };
+        // x plane k - 1 completes the plane-pair word (x[k-2], x[k-1]) of slot (k - 2) % 2.
+        // Runs in the scatter phase (a barrier after the gather that last read that slot), which
+        // is what lets two slots do.
+        auto store_x_pairs = [&](State &st, int k) NDC_LAMBDA {
+            const int lb = PL + st.ln.c0;
             const int xb = off_x + wrap((k - 2) % NX, NX) * RX * P;
             NDC_UNROLL
             for (int n = 0; n < NXR; ++n) {
@@ -292,6 +297,7 @@ template <int RH_> struct FwdKernelB {
             // ---- K-scatter of source plane k; own source words of plane k - 2; t1 plane k - 1
             ex.each([&](State &st, int) NDC_LAMBDA {
                 if (!st.ln.active) return;
+                store_x_pairs(st, k);
                 const bool extra = st.ln.strip < 2;
                 const int jx = halo_row(st.ln.strip, PH, TH);
                 const int cb = PL + st.ln.c0 - PW;
