@@ -2,6 +2,7 @@
 """Benchmark of the NDC update hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bf16|fp32] [--no-cpu]
+    python bench.py --workload train3d|model2d [--ndc hip|pytorch|both]   (model level, below)
 
 One step = one forward + one backward (input-, source-, filter- and bias-gradient) of the
 update node on config 3 of the baseline: batch 2, 128 depthwise channels, 64^3 voxels,
@@ -18,12 +19,23 @@ U = B*C*D*H*W channel-voxels and e bytes per element:
                           passes as pass 1 = 10 U e (x, z, gout in; gx out) and
                           pass 2 = 4 U e (gz out; its inputs are re-reads)
     whole step  23 U e
+
+Model-level workloads (not roofline-graded; same one-JSON-line output, `roofline` and
+`cpu_baseline` null):
+    train3d   config 4: Deconver 3-D (widths 64-512, 3x3x3, ratio 4, InstanceNorm3d), batch 2
+              of 128^3 two-channel ellipsoid phantoms, bf16 autocast, Dice+BCE, AdamW; one
+              step = forward + backward + optimiser update; metric = train steps/s
+    model2d   config 2: Deconver 2-D (widths 32-512, 5x5, ratio 4, InstanceNorm2d), batch 8 of
+              256^2 RGB-like images, float32, Dice+BCE; one step = forward + backward
+`--ndc hip` runs the NDC layers on the HIP kernels, `pytorch` on the layer's general PyTorch
+route (same GPU, same weights), `both` reports the two and their ratio.
 """
 
 from __future__ import annotations
 
 import argparse
 import json
+import math
 import os
 import statistics
 import sys
@@ -103,6 +115,100 @@ def cpu_baseline(torch, budget_channels=32):
     }
 
 
+MODEL_WORKLOADS = {
+    "train3d": dict(
+        net=dict(in_channels=2, out_channels=1, spatial_dims=3, encoder_depth=(1, 1, 1, 1),
+                 encoder_width=(64, 128, 256, 512), strides=(1, 2, 2, 2), decoder_depth=(1, 1, 1),
+                 kernel_size=(3, 3, 3), groups=-1, ratio=4),
+        batch=2, size=(128, 128, 128), autocast=True, optimizer=True,
+        metric="Deconver-3D train steps/s", unit="steps/s",
+        text="config 4: Deconver 3-D training step, batch 2 of 128^3 two-channel ellipsoid "
+             "phantoms, bf16 autocast, Dice+BCE, AdamW"),
+    "model2d": dict(
+        net=dict(in_channels=3, out_channels=1, spatial_dims=2, encoder_depth=(1, 1, 1, 1, 1),
+                 encoder_width=(32, 64, 128, 256, 512), strides=(1, 2, 2, 2, 2),
+                 decoder_depth=(1, 1, 1, 1), kernel_size=(5, 5), groups=-1, ratio=4),
+        batch=8, size=(256, 256), autocast=False, optimizer=False,
+        metric="Deconver-2D fwd+bwd steps/s", unit="steps/s",
+        text="config 2: Deconver 2-D forward + backward, batch 8 of 256^2 RGB-like images, "
+             "float32, Dice+BCE on smoothed-noise masks"),
+}
+
+
+def model_workload(args) -> int:
+    import torch
+    from torch import nn
+
+    import deconver_amd as dc
+    from deconver_amd import training as T
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    w = MODEL_WORKLOADS[args.workload]
+    dev = torch.device("cuda:0")
+    nd = len(w["size"])
+    norm = nn.InstanceNorm3d if nd == 3 else nn.InstanceNorm2d
+    if nd == 3:
+        images, targets = T.ellipsoid_phantoms(w["batch"], w["net"]["in_channels"], w["size"],
+                                               seed=0, device=dev)
+    else:
+        images, targets = T.smoothed_noise_masks(w["batch"], w["net"]["in_channels"], w["size"],
+                                                 seed=0, device=dev)
+
+    def run(route):
+        torch.manual_seed(0)
+        # a convolution keyword argument sends the NDC layers down their general PyTorch route
+        extra = {"stride": 1} if route == "pytorch" else {}
+        model = dc.Deconver(norm=norm, **w["net"], **extra).to(dev)
+        layers = [m for m in model.modules() if isinstance(m, dc.Deconv)]
+        on_hip = all(m.fast_path_applicable(torch.empty(1, m.channels, *([8] * nd), device=dev))
+                     for m in layers)
+        assert on_hip == (route == "hip"), f"route {route}: NDC layers on HIP kernels = {on_hip}"
+        opt = T.make_optimizer(model)
+        dtype = torch.bfloat16 if w["autocast"] else None
+
+        def step():
+            if w["optimizer"]:
+                return T.train_step(model, opt, images, targets, autocast_dtype=dtype)
+            model.zero_grad(set_to_none=True)
+            loss = T.dice_bce_loss(model(images), targets)
+            loss.backward()
+            return loss.detach()
+
+        for _ in range(args.warmup):
+            loss = step()
+        torch.cuda.synchronize()
+        torch.cuda.reset_peak_memory_stats()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            loss = step()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / args.steps
+        return dict(ms_per_step=dt * 1e3, steps_per_s=1.0 / dt, loss=float(loss),
+                    peak_mem_GB=torch.cuda.max_memory_allocated() / 1e9)
+
+    routes = ["hip", "pytorch"] if args.ndc == "both" else [args.ndc]
+    res = {r: run(r) for r in routes}
+    main_r = res[routes[0]]
+    vox = w["batch"] * math.prod(w["size"])
+    result = {
+        "metric": w["metric"], "value": main_r["steps_per_s"], "unit": w["unit"], "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": main_r["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if w["autocast"] else "f32", "data": "synthetic",
+        "config": {"workload": w["text"], "ndc": routes[0], "batch": w["batch"],
+                   "size": list(w["size"])},
+        "Gvoxel_per_s": vox / (main_r["ms_per_step"] * 1e-3) / 1e9,
+        "routes": res,
+        "roofline": None, "cpu_baseline": None,
+    }
+    if len(routes) == 2:
+        result["hip_over_pytorch"] = res["hip"]["steps_per_s"] / res["pytorch"]["steps_per_s"]
+    print(json.dumps(result))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -116,11 +222,18 @@ def main() -> int:
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
+    ap.add_argument("--workload", choices=("ndc", "train3d", "model2d"), default="ndc",
+                    help="ndc: the headline update node (default); the others are model level")
+    ap.add_argument("--ndc", choices=("hip", "pytorch", "both"), default="hip",
+                    help="model-level workloads: which route the NDC layers take")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures the one-GPU hot path only: this build has no multi-GPU code "
               "path (every box has one GPU); run with --gpus 1", file=sys.stderr)
         return 2
+
+    if args.workload != "ndc":
+        return model_workload(args)
 
     import torch
 
@@ -154,6 +267,20 @@ def main() -> int:
         dst.copy_(src)  # reads 1 GiB, writes 1 GiB
         torch.cuda.synchronize()
         del src, dst
+
+    # measured device-copy bandwidth (1 GiB read + 1 GiB written), for scale next to the
+    # published 8 TB/s the roofline is quoted on
+    src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+    dst = torch.empty_like(src)
+    dst.copy_(src)
+    c0, c1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    c0.record()
+    for _ in range(5):
+        dst.copy_(src)
+    c1.record()
+    torch.cuda.synchronize()
+    copy_gbs = 5 * 2 * src.numel() * 4 / (c0.elapsed_time(c1) * 1e-3) / 1e9
+    del src, dst
 
     for _ in range(args.warmup):
         step()
@@ -236,6 +363,7 @@ def main() -> int:
         "step_algorithmic_bytes": step_bytes,
         "step_hbm_frac": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "kernel_ms": k_ms,
+        "measured_copy_GBs": copy_gbs,
         "backward_reads_forward_ratio": bool(keep),
         "roofline": roofline,
     }
