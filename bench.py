@@ -159,7 +159,7 @@ def model_workload(args) -> int:
     def run(route):
         torch.manual_seed(0)
         # a convolution keyword argument sends the NDC layers down their general PyTorch route
-        extra = {"stride": 1} if route == "pytorch" else {}
+        extra = {"dilation": 1} if route == "pytorch" else {}
         model = dc.Deconver(norm=norm, **w["net"], **extra).to(dev)
         layers = [m for m in model.modules() if isinstance(m, dc.Deconv)]
         on_hip = all(m.fast_path_applicable(torch.empty(1, m.channels, *([8] * nd), device=dev))

@@ -24,25 +24,58 @@ def _ndc_layers(model):
     return [m for m in model.modules() if isinstance(m, dc.Deconv)]
 
 
+def _run_route(cfg, extra, state, x, g):
+    model = dc.Deconver(**cfg, **extra).cuda()
+    model.load_state_dict(state, strict=True)
+    y = model(x)
+    y.backward(g)
+    return model, y.detach(), {n: p.grad.detach() for n, p in model.named_parameters()}
+
+
 @pytest.mark.parametrize("cfg,spatial", [(NET_2D, (32, 24)), (NET_3D, (16, 12, 20))])
 def test_model_on_hip_matches_oracle(cfg, spatial):
-    """Tolerances of the reference's network test (tests/test_deconv_equivalence.py:314-329):
-    forward 1e-4, gradients 5e-3 of the largest reference entry."""
+    """Protocol of the reference's network test (tests/test_deconv_equivalence.py:332-379):
+    a float32 network sits 1e-3..1e-2 from a float64 evaluation of itself in its gradients
+    whatever runs the deconvolution, so both routes are compared with the float64 oracle and
+    the HIP route must be no further from it than the PyTorch route (x1.5, floor 1e-5).  The
+    forward output is also held to 1e-4 outright."""
     torch.manual_seed(0)
-    model = dc.Deconver(**cfg).cuda()
+    state = dc.Deconver(**cfg).state_dict()
     x = torch.rand(2, cfg["in_channels"], *spatial, device="cuda")
-    for layer in _ndc_layers(model):
+    g = torch.randn(2, cfg["out_channels"], *spatial, device="cuda")
+    hip, y_hip, g_hip = _run_route(cfg, {}, state, x, g)
+    for layer in _ndc_layers(hip):
         assert layer.fast_path_applicable(torch.empty(1, layer.channels, *spatial, device="cuda"))
-    y = model(x)
-    g = torch.randn_like(y)
-    y.backward(g)
-    state = {k: v.detach().cpu().double().requires_grad_(True)
-             for k, v in model.state_dict().items()}
-    yr = deconver_forward(state, x.cpu().double(), cfg)
+    pt, y_pt, g_pt = _run_route(cfg, {"dilation": 1}, state, x, g)
+    for layer in _ndc_layers(pt):
+        assert not layer.fast_path_applicable(torch.empty(1, layer.channels, *spatial, device="cuda"))
+    ref = {k: v.detach().cpu().double().requires_grad_(True) for k, v in state.items()}
+    yr = deconver_forward(ref, x.cpu().double(), cfg)
     yr.backward(g.cpu().double())
-    assert O.rel_err(y.cpu(), yr) < 1e-4
-    worst = max((O.rel_err(p.grad.cpu(), state[n].grad), n) for n, p in model.named_parameters())
-    assert worst[0] < 5e-3, worst
+    assert O.rel_err(y_hip.cpu(), yr) < 1e-4
+    assert O.rel_err(y_hip.cpu(), yr) <= 1.5 * max(O.rel_err(y_pt.cpu(), yr), 1e-5)
+    for name in g_hip:
+        e_hip = O.rel_err(g_hip[name].cpu(), ref[name].grad)
+        e_pt = O.rel_err(g_pt[name].cpu(), ref[name].grad)
+        assert e_hip <= 1.5 * max(e_pt, 1e-5), (name, e_hip, e_pt)
+
+
+def test_config2_model_at_full_width_matches_float64():
+    """The 2-D network of the baseline's config 2 (widths 32-512, 5x5, ratio 4) at 256^2,
+    batch 2: HIP route in float32 against the same network evaluated in float64 (which takes
+    the layers' PyTorch route).  Sizes the CPU oracle would need minutes for."""
+    import copy
+    net = dict(in_channels=3, out_channels=1, spatial_dims=2, encoder_depth=(1, 1, 1, 1, 1),
+               encoder_width=(32, 64, 128, 256, 512), strides=(1, 2, 2, 2, 2),
+               decoder_depth=(1, 1, 1, 1), kernel_size=(5, 5), groups=-1, ratio=4,
+               norm=nn.InstanceNorm2d)
+    torch.manual_seed(0)
+    model = dc.Deconver(**net).cuda()
+    images, _ = T.smoothed_noise_masks(2, 3, (256, 256), seed=0, device="cuda")
+    exact = copy.deepcopy(model).double()
+    with torch.no_grad():
+        y, ye = model(images), exact(images.double())
+    assert O.rel_err(y, ye) < 1e-4
 
 
 def test_training_step_reduces_loss_and_matches_pytorch_route():
@@ -50,7 +83,7 @@ def test_training_step_reduces_loss_and_matches_pytorch_route():
     same model trained on the layer's PyTorch route."""
     images, targets = T.ellipsoid_phantoms(2, 2, (32, 32, 32), seed=0, device="cuda")
     losses = {}
-    for route, extra in (("hip", {}), ("pytorch", {"stride": 1})):
+    for route, extra in (("hip", {}), ("pytorch", {"dilation": 1})):
         torch.manual_seed(0)
         model = dc.Deconver(**NET_3D, **extra).cuda()
         on_hip = all(m.fast_path_applicable(torch.empty(1, m.channels, 8, 8, 8, device="cuda"))
