@@ -151,4 +151,79 @@ template <class State> struct HostExec {
 
 #endif
 
+// A slice of a tensor in global memory, addressed as (slice base, wave-uniform byte offset,
+// per-lane byte offset), for 32-bit accesses.
+//   Device: a raw buffer resource of `bytes` bytes.  The memory unit adds the three parts
+//     (buffer_load_dword v, v_lane_off, s[resource], s_uniform_off offen), so no vector
+//     instruction is spent on 64-bit address arithmetic, and an access past `bytes` is
+//     dropped (loads return 0) instead of faulting.  A null base gives an empty slice.
+//   Host build: base pointer + size; an access outside the slice is reported as a fault.
+struct BufRef {
+#if NDC_DEVICE_BUILD && defined(__HIP_DEVICE_COMPILE__)
+    __amdgpu_buffer_rsrc_t r;
+#else
+    char *base;
+    size_t bytes;
+#endif
+};
+
+NDC_HD BufRef make_buf(const void *p, size_t bytes)
+{
+    BufRef b;
+#if NDC_DEVICE_BUILD && defined(__HIP_DEVICE_COMPILE__)
+    // the slice base is the same in every lane: say so, or each access is wrapped in a loop
+    // over the distinct resources of the wavefront
+    const unsigned long long a = (unsigned long long)p;
+    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)a);
+    const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(a >> 32));
+    void *up = (void *)(((unsigned long long)hi << 32) | lo);
+    const int n = __builtin_amdgcn_readfirstlane(p ? (int)(unsigned)bytes : 0);
+    // word 3 of the resource: 32-bit data format, raw (unstrided, unswizzled) addressing
+    b.r = __builtin_amdgcn_make_buffer_rsrc(up, 0, n, 0x00020000);
+#else
+    b.base = (char *)const_cast<void *>(p);
+    b.bytes = p ? bytes : 0;
+#endif
+    return b;
+}
+
+NDC_HD uint32_t buf_ld(const BufRef &b, unsigned lane_off, unsigned uniform_off)
+{
+#if NDC_DEVICE_BUILD && defined(__HIP_DEVICE_COMPILE__)
+    return __builtin_amdgcn_raw_buffer_load_b32(b.r, (int)lane_off, (int)uniform_off, 0);
+#elif NDC_DEVICE_BUILD
+    (void)b; (void)lane_off; (void)uniform_off;
+    return 0u;
+#else
+    const size_t o = (size_t)lane_off + uniform_off;
+    if (o + 4 > b.bytes) {
+        HostFaults &hf = host_faults();
+        ++hf.oob;
+        hf.note("out-of-bounds global read", (int)o, -1, -1);
+        return 0u;
+    }
+    uint32_t w;
+    memcpy(&w, b.base + o, 4);
+    return w;
+#endif
+}
+
+NDC_HD void buf_st(const BufRef &b, unsigned lane_off, unsigned uniform_off, uint32_t w)
+{
+#if NDC_DEVICE_BUILD && defined(__HIP_DEVICE_COMPILE__)
+    __builtin_amdgcn_raw_buffer_store_b32(w, b.r, (int)lane_off, (int)uniform_off, 0);
+#elif NDC_DEVICE_BUILD
+    (void)b; (void)lane_off; (void)uniform_off; (void)w;
+#else
+    const size_t o = (size_t)lane_off + uniform_off;
+    if (o + 4 > b.bytes) {
+        HostFaults &hf = host_faults();
+        ++hf.oob;
+        hf.note("out-of-bounds global write", (int)o, -1, -1);
+        return;
+    }
+    memcpy(b.base + o, &w, 4);
+#endif
+}
+
 }  // namespace ndc

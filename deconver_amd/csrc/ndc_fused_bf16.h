@@ -65,15 +65,6 @@ NDC_HD uint32_t zip_hi(uint32_t a, uint32_t b)
     return (a >> 16) | (b & 0xffff0000u);
 #endif
 }
-// one 32-bit global access at a uniform base plus a 32-bit byte offset
-template <typename T> NDC_HD uint32_t ld_word(const T *base, unsigned byte_off)
-{
-    return *reinterpret_cast<const uint32_t *>(reinterpret_cast<const char *>(base) + byte_off);
-}
-template <typename T> NDC_HD void st_word(T *base, unsigned byte_off, uint32_t w)
-{
-    *reinterpret_cast<uint32_t *>(reinterpret_cast<char *>(base) + byte_off) = w;
-}
 NDC_HD float bf_lo(uint32_t w) { return bits_to_float(w << 16); }
 NDC_HD float bf_hi(uint32_t w) { return bits_to_float(w & 0xffff0000u); }
 
@@ -176,10 +167,16 @@ template <int RH_> struct FwdKernelB {
         const int total = off_t + NTP * RX * P;
         const int plane = H * W;
         const long long cplane = (long long)D * plane;
-        const T *xg = p.x + ((long long)id.b * p.C + id.c) * cplane;
-        const T *zg = p.z + ((long long)id.b * p.C + id.c) * SC * cplane;
-        T *og = p.out + ((long long)id.b * p.C + id.c) * SC * cplane;
-        T *t1g = p.t1 ? p.t1 + ((long long)id.b * p.C + id.c) * cplane : nullptr;
+        // this workgroup's (sample, channel) slices; offsets inside them fit 32 bits
+        const long long cbase = ((long long)id.b * p.C + id.c) * cplane;
+        const size_t xbytes = (size_t)cplane * sizeof(T), sbytes = xbytes * SC;
+        const unsigned plane2 = (unsigned)plane * 2u, cplane2 = (unsigned)cplane * 2u;
+        const BufRef xb_ = make_buf(p.x + cbase, xbytes), zb_ = make_buf(p.z + cbase * SC, sbytes);
+        const BufRef ob_ = make_buf(p.out + cbase * SC, sbytes);
+        const BufRef tb_ = make_buf(p.t1 ? p.t1 + cbase : nullptr, xbytes);
+        const BufRef db_ = make_buf(p.s_over_den ? p.s_over_den + cbase * SC : nullptr, sbytes);
+        const BufRef rb_ = make_buf(p.ratio ? p.ratio + cbase * SC : nullptr, sbytes);
+        const bool have_t1 = p.t1 != nullptr, have_saved = p.s_over_den != nullptr;
         UniformF tab = as_uniform(p.wtab + (long long)id.c * kTabWords);
         const int r0 = id.r0;
         const int nthreads = ex.nthreads;
@@ -189,21 +186,20 @@ template <int RH_> struct FwdKernelB {
         auto load_plane = [&](State &st, int k) NDC_LAMBDA {
             if (!st.ln.active) return;
             if (k < D) {
-                const T *zk = zg + (long long)k * plane;
                 NDC_UNROLL
                 for (int n = 0; n < NZR; ++n)
                     NDC_UNROLL
                     for (int i = 0; i < SC; ++i)
-                        st.pz[i][n] = ld_word(zk + i * cplane, st.zoff[n]);
+                        st.pz[i][n] = buf_ld(zb_, st.zoff[n], (unsigned)k * plane2 + i * cplane2);
             }
             // planes outside the volume: load a clamped plane and select zero (a store in each
             // arm of a branch would push the staging registers into private memory)
             const int kx = k - PD;
             const bool xlive = kx >= 0 && kx < D;
-            const T *xk = xg + (long long)clampi(kx, 0, D - 1) * plane;
+            const unsigned xk = (unsigned)clampi(kx, 0, D - 1) * plane2;
             NDC_UNROLL
             for (int n = 0; n < NXR; ++n) {
-                const uint32_t v = ld_word(xk, st.xoff[n]);
+                const uint32_t v = buf_ld(xb_, st.xoff[n], xk);
                 st.px[n] = xlive ? v : 0u;
             }
         };
@@ -342,7 +338,8 @@ template <int RH_> struct FwdKernelB {
                         if (mine) ex.st_(tb + j * P + c, bits_to_float(pack_bf16x2(st.t1prev[r][c], v[c])));
                         st.t1prev[r][c] = v[c];
                     }
-                    if (r < RH && t1g && live) st_word(t1g + (long long)pf * plane, st.ooff[r < RH ? r : 0], pack_bf16x2(v[0], v[1]));
+                    if (r < RH && have_t1 && live)
+                        buf_st(tb_, st.ooff[r < RH ? r : 0], (unsigned)pf * plane2, pack_bf16x2(v[0], v[1]));
                     NDC_UNROLL
                     for (int c = 0; c < RW; ++c) {
                         st.t1acc[0][r][c] = st.t1acc[1][r][c];
@@ -378,9 +375,7 @@ template <int RH_> struct FwdKernelB {
                                          off_t + wrap(m % NTP, NTP) * RX * P + ob};
                     a_plane_d2<RH, RW, 2>(ex, base, P, wt, acc);
                 }
-                T *ok_ = og + (long long)j0 * plane;
-                T *dk_ = p.s_over_den ? p.s_over_den + (og - p.out) + (long long)j0 * plane : nullptr;
-                T *rk_ = p.ratio ? p.ratio + (og - p.out) + (long long)j0 * plane : nullptr;
+                const unsigned oj = (unsigned)j0 * plane2;
                 NDC_UNROLL
                 for (int r = 0; r < RH; ++r) {
                     if (!((st.ook >> r) & 1u)) continue;
@@ -396,10 +391,10 @@ template <int RH_> struct FwdKernelB {
                             rt[c] = acc[0][i][r][c] * inv;
                             v[c] = s * rt[c];
                         }
-                        st_word(ok_ + i * cplane, st.ooff[r], pack_bf16x2(v[0], v[1]));
-                        if (dk_) {
-                            st_word(dk_ + i * cplane, st.ooff[r], pack_bf16x2(rd[0], rd[1]));
-                            st_word(rk_ + i * cplane, st.ooff[r], pack_bf16x2(rt[0], rt[1]));
+                        buf_st(ob_, st.ooff[r], oj + i * cplane2, pack_bf16x2(v[0], v[1]));
+                        if (have_saved) {
+                            buf_st(db_, st.ooff[r], oj + i * cplane2, pack_bf16x2(rd[0], rd[1]));
+                            buf_st(rb_, st.ooff[r], oj + i * cplane2, pack_bf16x2(rt[0], rt[1]));
                         }
                     }
                 }
@@ -431,6 +426,10 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
         float gacc[SC][KT];
         float accx[KD][RH][RW], acct[KD][RH][RW];
         uint32_t px[NXR], pt[NXR], pxprev[NXR], ptprev[NXR];
+        // SAVED: gout, s/d, n/d words of the next plane, fetched one phase ahead (own rows,
+        // then the halo row of the first two strips)
+        uint32_t qg[SC][RH + 1], qd[SC][RH + 1], qr[SC][RH + 1];
+        unsigned hoff;
     };
 
     static NDC_HD int rows_x(int TH) { return TH + 4; }
@@ -454,12 +453,17 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
         const int plane = H * W;
         const long long cplane = (long long)D * plane;
         const long long cbase = ((long long)id.b * p.C + id.c) * cplane;
-        const T *xg = p.x + cbase, *t1g = p.t1 + cbase;
-        const T *zg = p.z + cbase * SC, *gg = p.gout + cbase * SC;
-        const T *dg = SAVED ? p.s_over_den + cbase * SC : nullptr;
-        const T *rg = SAVED ? p.ratio + cbase * SC : nullptr;
-        T *gxg = p.gx ? p.gx + cbase : nullptr;
-        T *gt1g = p.gt1 + cbase;
+        // this workgroup's (sample, channel) slices; offsets inside them fit 32 bits
+        const size_t xbytes = (size_t)cplane * sizeof(T), sbytes = xbytes * SC;
+        const unsigned plane2 = (unsigned)plane * 2u, cplane2 = (unsigned)cplane * 2u;
+        const BufRef xb_ = make_buf(p.x + cbase, xbytes), tb_ = make_buf(p.t1 + cbase, xbytes);
+        const BufRef zb_ = make_buf(SAVED ? nullptr : p.z + cbase * SC, sbytes);
+        const BufRef gb_ = make_buf(p.gout + cbase * SC, sbytes);
+        const BufRef db_ = make_buf(SAVED ? p.s_over_den + cbase * SC : nullptr, sbytes);
+        const BufRef rb_ = make_buf(SAVED ? p.ratio + cbase * SC : nullptr, sbytes);
+        const BufRef gxb_ = make_buf(p.gx ? p.gx + cbase : nullptr, xbytes);
+        const BufRef gtb_ = make_buf(p.gt1 + cbase, xbytes);
+        const bool have_gx = p.gx != nullptr;
         UniformF tab = as_uniform(p.wtab + (long long)id.c * kTabWords);
         const int r0 = id.r0;
         const int nthreads = ex.nthreads;
@@ -472,11 +476,11 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
             // planes past the end: load the last plane and select zero (a store in each arm of
             // a branch would push the staging registers into private memory)
             const bool live = k < D;
-            const long long ko = (long long)clampi(k, 0, D - 1) * plane;
+            const unsigned ko = (unsigned)clampi(k, 0, D - 1) * plane2;
             NDC_UNROLL
             for (int n = 0; n < NXR; ++n) {
-                const uint32_t vx = ld_word(xg + ko, st.xoff[n]);
-                const uint32_t vt = ld_word(t1g + ko, st.xoff[n]);
+                const uint32_t vx = buf_ld(xb_, st.xoff[n], ko);
+                const uint32_t vt = buf_ld(tb_, st.xoff[n], ko);
                 st.px[n] = live ? vx : 0u;
                 st.pt[n] = live ? vt : 0u;
             }
@@ -506,11 +510,29 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
 
         // gn, gd of NR rows from gn/gd tile row j (image row r0 - 1 + j): published to LDS as
         // channel-pair words; returned as operand pairs GG[i][r][c] = (gn_i, gd_i)
-        auto gn_gd_rows = [&](State &st, int j1, int j, auto nr_tag,
+        // SAVED: fetch plane jn of gout, s/d, n/d into the state, a phase before it is used
+        auto prefetch_g = [&](State &st, int jn) NDC_LAMBDA {
+            if (!SAVED || jn >= D) return;
+            const unsigned jo = (unsigned)jn * plane2;
+            NDC_UNROLL
+            for (int r = 0; r < RH + 1; ++r) {
+                if (r == RH && st.ln.strip >= 2) continue;
+                const unsigned o = r < RH ? st.ooff[r < RH ? r : 0] : st.hoff;
+                NDC_UNROLL
+                for (int i = 0; i < SC; ++i) {
+                    st.qg[i][r] = buf_ld(gb_, o, jo + i * cplane2);
+                    st.qd[i][r] = buf_ld(db_, o, jo + i * cplane2);
+                    st.qr[i][r] = buf_ld(rb_, o, jo + i * cplane2);
+                }
+            }
+        };
+
+        // roff: where the rows sit in the prefetched words (0: own rows, RH: halo row)
+        auto gn_gd_rows = [&](State &st, int j1, int j, auto nr_tag, int roff,
                               uint32_t (&gg_out)[SC][decltype(nr_tag)::value][RW]) NDC_LAMBDA {
             constexpr int NR = decltype(nr_tag)::value;
             uint32_t zw[SC][NR], gw[SC][NR], dw[SC][NR], rw[SC][NR];
-            const T *zk = zg + (long long)j1 * plane, *gk = gg + (long long)j1 * plane;
+            const unsigned jo = (unsigned)j1 * plane2;
             bool ok[NR];
             NDC_UNROLL
             for (int r = 0; r < NR; ++r) {
@@ -519,13 +541,14 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
                 const unsigned o = (unsigned)(clampi(row, 0, H - 1) * W + st.ln.c0) * 2u;
                 NDC_UNROLL
                 for (int i = 0; i < SC; ++i) {
-                    gw[i][r] = ld_word(gk + i * cplane, o);
                     if (SAVED) {
                         zw[i][r] = 0u;
-                        dw[i][r] = ld_word(dg + (long long)j1 * plane + i * cplane, o);
-                        rw[i][r] = ld_word(rg + (long long)j1 * plane + i * cplane, o);
+                        gw[i][r] = st.qg[i][roff + r];
+                        dw[i][r] = st.qd[i][roff + r];
+                        rw[i][r] = st.qr[i][roff + r];
                     } else {
-                        zw[i][r] = ld_word(zk + i * cplane, o);
+                        gw[i][r] = buf_ld(gb_, o, jo + i * cplane2);
+                        zw[i][r] = buf_ld(zb_, o, jo + i * cplane2);
                         dw[i][r] = rw[i][r] = 0u;
                     }
                 }
@@ -596,6 +619,14 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
                 if (row < H) st.ook |= 1u << r;
                 st.ooff[r] = (unsigned)(clampi(row, 0, H - 1) * W + st.ln.c0) * 2u;
             }
+            {
+                const int hrow = r0 - PH + halo_row(st.ln.strip, PH, TH);
+                st.hoff = (unsigned)(clampi(hrow, 0, H - 1) * W + st.ln.c0) * 2u;
+                NDC_UNROLL
+                for (int i = 0; i < SC; ++i)
+                    NDC_UNROLL
+                    for (int r = 0; r < RH + 1; ++r) st.qg[i][r] = st.qd[i][r] = st.qr[i][r] = 0u;
+            }
             NDC_UNROLL
             for (int i = 0; i < SC; ++i) {
                 st.bv[i] = p.bias ? p.bias[id.c * SC + i] : 0.f;
@@ -625,7 +656,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
                 {
                     uint32_t gg2[SC][RH][RW];
                     const int j = PH + st.ln.strip * RH;
-                    gn_gd_rows(st, j1, j, IntTag<RH>(), gg2);
+                    gn_gd_rows(st, j1, j, IntTag<RH>(), 0, gg2);
                     if (need_gh) {
                         // A-side filter-gradient terms: (gn_i, gd_i) . (x, t1)[neighbour]
                         NDC_UNROLL
@@ -657,7 +688,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
                 }
                 if (st.ln.strip < 2) {
                     uint32_t gg1[SC][1][RW];
-                    gn_gd_rows(st, j1, halo_row(st.ln.strip, PH, TH), IntTag<1>(), gg1);
+                    gn_gd_rows(st, j1, halo_row(st.ln.strip, PH, TH), IntTag<1>(), RH, gg1);
                 }
             });
             ex.sync();
@@ -665,6 +696,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
             ex.each([&](State &st, int) NDC_LAMBDA {
                 if (!st.ln.active) return;
                 load_plane(st, k + 1);
+                prefetch_g(st, k);
                 if (live1) {
                     const int gb_ = off_g + (st.ln.strip * RH) * P + PL + st.ln.c0 - PW;
                     float wp[KT], wn[KT];
@@ -681,10 +713,10 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
                 NDC_UNROLL
                 for (int r = 0; r < RH; ++r) {
                     if (pf >= 0 && ((st.ook >> r) & 1u)) {
-                        if (gxg) st_word(gxg + (long long)pf * plane, st.ooff[r],
-                                         pack_bf16x2(st.accx[0][r][0], st.accx[0][r][1]));
-                        st_word(gt1g + (long long)pf * plane, st.ooff[r],
-                                pack_bf16x2(st.acct[0][r][0], st.acct[0][r][1]));
+                        if (have_gx) buf_st(gxb_, st.ooff[r], (unsigned)pf * plane2,
+                                            pack_bf16x2(st.accx[0][r][0], st.accx[0][r][1]));
+                        buf_st(gtb_, st.ooff[r], (unsigned)pf * plane2,
+                               pack_bf16x2(st.acct[0][r][0], st.acct[0][r][1]));
                     }
                     NDC_UNROLL
                     for (int c = 0; c < RW; ++c) {
@@ -752,10 +784,16 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
         const int plane = H * W;
         const long long cplane = (long long)D * plane;
         const long long cbase = ((long long)id.b * p.C + id.c) * cplane;
-        const T *xg = p.x + cbase, *t1g = p.t1 + cbase, *gt1g = p.gt1 + cbase;
-        const T *zg = p.z + cbase * SC, *gg = p.gout + cbase * SC;
-        const T *rg = SAVED ? p.ratio + cbase * SC : nullptr;
-        T *gzg = p.gz ? p.gz + cbase * SC : nullptr;
+        // this workgroup's (sample, channel) slices; offsets inside them fit 32 bits
+        const size_t xbytes = (size_t)cplane * sizeof(T), sbytes = xbytes * SC;
+        const unsigned plane2 = (unsigned)plane * 2u, cplane2 = (unsigned)cplane * 2u;
+        const BufRef xb_ = make_buf(SAVED ? nullptr : p.x + cbase, xbytes);
+        const BufRef tb_ = make_buf(SAVED ? nullptr : p.t1 + cbase, xbytes);
+        const BufRef gtb_ = make_buf(p.gt1 + cbase, xbytes);
+        const BufRef zb_ = make_buf(p.z + cbase * SC, sbytes), gb_ = make_buf(p.gout + cbase * SC, sbytes);
+        const BufRef rb_ = make_buf(SAVED ? p.ratio + cbase * SC : nullptr, sbytes);
+        const BufRef gzb_ = make_buf(p.gz ? p.gz + cbase * SC : nullptr, sbytes);
+        const bool have_gz = p.gz != nullptr;
         UniformF tab = as_uniform(p.wtab + (long long)id.c * kTabWords);
         const int r0 = id.r0;
         const int nthreads = ex.nthreads;
@@ -768,12 +806,12 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
             // planes past the end: load the last plane and select zero (a store in each arm of
             // a branch would push the staging registers into private memory)
             const bool live = k < D;
-            const long long ko = (long long)clampi(k, 0, D - 1) * plane;
+            const unsigned ko = (unsigned)clampi(k, 0, D - 1) * plane2;
             NDC_UNROLL
             for (int n = 0; n < NXR; ++n) {
-                const uint32_t vx = SAVED ? 0u : ld_word(xg + ko, st.xoff[n]);
-                const uint32_t vt = SAVED ? 0u : ld_word(t1g + ko, st.xoff[n]);
-                const uint32_t vg = ld_word(gt1g + ko, st.xoff[n]);
+                const uint32_t vx = SAVED ? 0u : buf_ld(xb_, st.xoff[n], ko);
+                const uint32_t vt = SAVED ? 0u : buf_ld(tb_, st.xoff[n], ko);
+                const uint32_t vg = buf_ld(gtb_, st.xoff[n], ko);
                 st.px[n] = live ? vx : 0u;
                 st.pt[n] = live ? vt : 0u;
                 st.pg[n] = live ? vg : 0u;
@@ -855,14 +893,14 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
                         for (int c = 0; c < RW; ++c) sv[i][r][c] = 0.f;
                 if (j0 < D) {
                     uint32_t zw[SC][RH], gw[SC][RH], rw[SC][RH];
-                    const T *zk = zg + (long long)j0 * plane, *gk = gg + (long long)j0 * plane;
+                    const unsigned jo = (unsigned)j0 * plane2;
                     NDC_UNROLL
                     for (int r = 0; r < RH; ++r)
                         NDC_UNROLL
                         for (int i = 0; i < SC; ++i) {
-                            zw[i][r] = ld_word(zk + i * cplane, st.ooff[r]);
-                            gw[i][r] = ld_word(gk + i * cplane, st.ooff[r]);
-                            rw[i][r] = SAVED ? ld_word(rg + (long long)j0 * plane + i * cplane, st.ooff[r]) : 0u;
+                            zw[i][r] = buf_ld(zb_, st.ooff[r], jo + i * cplane2);
+                            gw[i][r] = buf_ld(gb_, st.ooff[r], jo + i * cplane2);
+                            rw[i][r] = SAVED ? buf_ld(rb_, st.ooff[r], jo + i * cplane2) : 0u;
                         }
                     float acc[NA][SC][RH][RW];
                     NDC_UNROLL
@@ -887,7 +925,6 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
                         }
                         a_plane_d2<RH, RW, NA>(ex, base, P, wt, acc);
                     }
-                    T *gzk = gzg ? gzg + (long long)j0 * plane : nullptr;
                     NDC_UNROLL
                     for (int r = 0; r < RH; ++r) {
                         const bool ok = (st.ook >> r) & 1u;
@@ -910,7 +947,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
                                 st.gbacc[i] += gzv;
                                 v[c] = gzv;
                             }
-                            if (gzk && ok) st_word(gzk + i * cplane, st.ooff[r], pack_bf16x2(v[0], v[1]));
+                            if (have_gz && ok) buf_st(gzb_, st.ooff[r], jo + i * cplane2, pack_bf16x2(v[0], v[1]));
                         }
                     }
                 }
