@@ -763,6 +763,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
         float gbacc[SC];
         float sprev[SC][RH][RW];   // own source values of the previous plane
         uint32_t px[NXR], pt[NXR], pg[NXR], pxprev[NXR], ptprev[NXR], pgprev[NXR];
+        uint32_t qz[SC][RH], qg[SC][RH], qr[SC][RH];   // SAVED: words fetched a step ahead
     };
 
     static NDC_HD int rows_x(int TH) { return TH + 2; }
@@ -866,6 +867,8 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
                 for (int r = 0; r < RH; ++r)
                     NDC_UNROLL
                     for (int c = 0; c < RW; ++c) st.sprev[i][r][c] = 0.f;
+                NDC_UNROLL
+                for (int r = 0; r < RH; ++r) st.qz[i][r] = st.qg[i][r] = st.qr[i][r] = 0u;
             }
             for (int i = tid; i < total; i += nthreads) ex.st_(i, 0.f);
             load_plane(st, 0);
@@ -883,6 +886,23 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
             ex.each([&](State &st, int) NDC_LAMBDA {
                 if (!st.ln.active) return;
                 load_plane(st, k + 1);
+                // SAVED: this plane's z, gout, n/d words were fetched a step ago; take them and
+                // start the fetch of the next plane's
+                uint32_t zw[SC][RH], gw[SC][RH], rw[SC][RH];
+                if (SAVED) {
+                    const unsigned jn = (unsigned)clampi(k, 0, D - 1) * plane2;
+                    NDC_UNROLL
+                    for (int r = 0; r < RH; ++r)
+                        NDC_UNROLL
+                        for (int i = 0; i < SC; ++i) {
+                            zw[i][r] = st.qz[i][r];
+                            gw[i][r] = st.qg[i][r];
+                            rw[i][r] = st.qr[i][r];
+                            st.qz[i][r] = buf_ld(zb_, st.ooff[r], jn + i * cplane2);
+                            st.qg[i][r] = buf_ld(gb_, st.ooff[r], jn + i * cplane2);
+                            st.qr[i][r] = buf_ld(rb_, st.ooff[r], jn + i * cplane2);
+                        }
+                }
                 if (j0 < 0) return;
                 float sv[SC][RH][RW];
                 NDC_UNROLL
@@ -892,16 +912,17 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
                         NDC_UNROLL
                         for (int c = 0; c < RW; ++c) sv[i][r][c] = 0.f;
                 if (j0 < D) {
-                    uint32_t zw[SC][RH], gw[SC][RH], rw[SC][RH];
                     const unsigned jo = (unsigned)j0 * plane2;
-                    NDC_UNROLL
-                    for (int r = 0; r < RH; ++r)
+                    if (!SAVED) {
                         NDC_UNROLL
-                        for (int i = 0; i < SC; ++i) {
-                            zw[i][r] = buf_ld(zb_, st.ooff[r], jo + i * cplane2);
-                            gw[i][r] = buf_ld(gb_, st.ooff[r], jo + i * cplane2);
-                            rw[i][r] = SAVED ? buf_ld(rb_, st.ooff[r], jo + i * cplane2) : 0u;
-                        }
+                        for (int r = 0; r < RH; ++r)
+                            NDC_UNROLL
+                            for (int i = 0; i < SC; ++i) {
+                                zw[i][r] = buf_ld(zb_, st.ooff[r], jo + i * cplane2);
+                                gw[i][r] = buf_ld(gb_, st.ooff[r], jo + i * cplane2);
+                                rw[i][r] = 0u;
+                            }
+                    }
                     float acc[NA][SC][RH][RW];
                     NDC_UNROLL
                     for (int a = 0; a < NA; ++a)
