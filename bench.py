@@ -2,6 +2,7 @@
 """Benchmark of the NDC update hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bf16|fp32] [--no-cpu]
+    python bench.py --workload sweep                                      (config 5, forward only)
     python bench.py --workload train3d|model2d [--ndc hip|pytorch|both]   (model level, below)
 
 One step = one forward + one backward (input-, source-, filter- and bias-gradient) of the
@@ -115,6 +116,56 @@ def cpu_baseline(torch, budget_channels=32):
     }
 
 
+SWEEP_SHAPES = [   # config 5: (channels, extent, batch), bottleneck to full resolution
+    (512, 16, 4), (256, 32, 2), (64, 128, 1), (32, 192, 1),
+]
+
+
+def sweep_workload(args) -> int:
+    """Config 5: forward-only (inference: no t1, nothing kept for backward) NDC update,
+    3x3x3, ratio 4, bf16, half-normal inputs; Gvoxel/s and HBM-roofline fraction (9 U e
+    algorithmic bytes) per shape.  `value` is the geometric mean over the shapes."""
+    import torch
+
+    from deconver_amd import _lib, ops
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    lib = _lib.get_library()
+    dev = torch.device("cuda:0")
+    rows = []
+    for C, n, B in SWEEP_SHAPES:
+        x, z, h, bias, _, sc = make_inputs(torch, torch.bfloat16, dev, B, C, (n, n, n), (3, 3, 3), 4)
+        kw = dict(groups=C, m=1, sc=sc, eps=1e-16, relu_input=True, need_t1=False)
+        for _ in range(args.warmup):
+            ops.update_forward(lib, x, z, h, bias, **kw)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            ops.update_forward(lib, x, z, h, bias, **kw)
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / args.steps
+        vox, U = B * n ** 3, B * C * n ** 3
+        rows.append({"channels": C, "extent": n, "batch": B, "ms": ms,
+                     "Gvoxel_per_s": vox / (ms * 1e-3) / 1e9,
+                     "channel_voxels_per_s": U / (ms * 1e-3),
+                     "hbm_frac": 9 * U * 2 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS})
+        del x, z
+    gmean = math.exp(sum(math.log(r["Gvoxel_per_s"]) for r in rows) / len(rows))
+    print(json.dumps({
+        "metric": "NDC mixer forward-only Gvoxel/s (geometric mean over the sweep)",
+        "value": gmean, "unit": "Gvoxel/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": sum(r["ms"] for r in rows),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "config 5: forward-only NDC update shape sweep, 3x3x3, ratio 4, "
+                               "bf16 storage / float32 accumulation, inference form"},
+        "shapes": rows, "roofline": None, "cpu_baseline": None}))
+    return 0
+
+
 MODEL_WORKLOADS = {
     "train3d": dict(
         net=dict(in_channels=2, out_channels=1, spatial_dims=3, encoder_depth=(1, 1, 1, 1),
@@ -222,7 +273,7 @@ def main() -> int:
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
-    ap.add_argument("--workload", choices=("ndc", "train3d", "model2d"), default="ndc",
+    ap.add_argument("--workload", choices=("ndc", "sweep", "train3d", "model2d"), default="ndc",
                     help="ndc: the headline update node (default); the others are model level")
     ap.add_argument("--ndc", choices=("hip", "pytorch", "both"), default="hip",
                     help="model-level workloads: which route the NDC layers take")
@@ -232,6 +283,8 @@ def main() -> int:
               "path (every box has one GPU); run with --gpus 1", file=sys.stderr)
         return 2
 
+    if args.workload == "sweep":
+        return sweep_workload(args)
     if args.workload != "ndc":
         return model_workload(args)
 

@@ -56,6 +56,8 @@ struct Tile {
     int P;       // LDS row pitch in words
     int PL;      // zero words to the left of column 0 in an LDS row (>= PW, multiple of RW)
     int CPW;     // column groups per row = W / RW
+    int nseg;    // segments of the marching axis per volume (each its own workgroup)
+    int SEG;     // planes per segment
 };
 
 // the marching view of a problem: 2-D inputs march along H
@@ -110,7 +112,27 @@ static inline bool make_tile(const March &m, int RH, int RW, int target_threads,
     t.ntile = (m.H + t.TH - 1) / t.TH;
     t.PL = round_up(PW, RW);
     t.P = round_up(t.PL + m.W + PW, RW);
+    t.nseg = 1;
+    t.SEG = m.D;
     return true;
+}
+
+// Split the marching axis so that a launch has enough wavefronts to fill the chip: a
+// workgroup that owns planes [d0, d1) marches over them plus 2*PD warm-up planes on each
+// side (whose outputs its neighbours own), so segments are kept >= 16*PD planes long.
+static inline void split_march(const March &m, long long blocks, Tile &t)
+{
+    const int PD = m.KD / 2;
+    const long long waves = blocks * (t.NT / 64);
+    const long long target = 4096;   // about four wavefronts per SIMD
+    const int min_seg = PD > 0 ? 16 * PD : m.D;
+    if (waves >= target || m.D < 2 * min_seg) return;
+    long long want = (target + waves - 1) / waves;
+    const int max_seg = m.D / min_seg;
+    if (want > max_seg) want = max_seg;
+    if (want < 2) return;
+    t.SEG = round_up((m.D + (int)want - 1) / (int)want, 2);
+    t.nseg = (m.D + t.SEG - 1) / t.SEG;
 }
 
 // ------------------------------------------------------------------ parameters
@@ -145,16 +167,22 @@ template <typename T> struct BwdParams {
 
 struct BlockId {
     int b, c, r0;
+    int d0, d1;   // planes [d0, d1) of the marching axis whose outputs this workgroup owns
 };
 
-NDC_HD BlockId decode_block(int block_id, int C, const Tile &t)
+// block_id = ((b * C + c) * nseg + segment) * ntile + row band
+NDC_HD BlockId decode_block(int block_id, int C, const Tile &t, int D)
 {
     BlockId id;
     const int tile = block_id % t.ntile;
-    const int bc = block_id / t.ntile;
+    const int rest = block_id / t.ntile;
+    const int seg = rest % t.nseg;
+    const int bc = rest / t.nseg;
     id.b = bc / C;
     id.c = bc % C;
     id.r0 = tile * t.TH;
+    id.d0 = seg * t.SEG;
+    id.d1 = id.d0 + t.SEG < D ? id.d0 + t.SEG : D;
     return id;
 }
 
@@ -302,7 +330,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
     template <class Exec> static NDC_D void run(Exec &ex, const Params &p, int block_id)
     {
         const Tile t = p.t;
-        const BlockId id = decode_block(block_id, p.C, t);
+        const BlockId id = decode_block(block_id, p.C, t, p.D);
         const int S = t.S, P = t.P, PL = t.PL, TH = t.TH, W = p.W, H = p.H, D = p.D;
         const int RS = rows_s(TH), RX = rows_x(TH);
         const int off_s = 0, off_x = SC * RS * P, off_t = off_x + XR * RX * P;
@@ -318,6 +346,10 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
         const int nthreads = ex.nthreads;
         const float floor_ = p.relu ? 0.f : -3.0e38f;   // max(s, floor_) rectifies or passes through
         const float eps = p.eps;
+        // owned output planes [d0, d1); the march starts 2*PD planes early so that t1 is
+        // complete from plane d0 - PD on, and runs 2*PD planes past the end
+        const int d0 = id.d0, d1 = id.d1;
+        const int k_first = d0 - 2 * PD > 0 ? d0 - 2 * PD : 0, k_end = d1 + 2 * PD;
 
         // global -> registers: plane k of s (bias / ReLU applied) and plane k - PD of x.
         // Rows outside the image read a clamped address and are zeroed by a select.
@@ -419,11 +451,11 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                     NDC_UNROLL
                     for (int c = 0; c < RW; ++c) st.t1acc[a][r][c] = 0.f;
             for (int i = tid; i < total; i += nthreads) ex.st_(i, 0.f);
-            load_plane(st, 0);
+            load_plane(st, k_first);
         });
         ex.sync();
 
-        for (int kk = 0; kk < D + 2 * PD; ++kk) {
+        for (int kk = k_first; kk < k_end; ++kk) {
             const int k = uniform_int(kk);   // the plane index stays on the scalar unit
             ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k); });
             ex.sync();
@@ -463,7 +495,8 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                         v[c] = live ? st.t1acc[0][r][c] : 0.f;
                         if (mine) ex.st_(tb + j * P + c, v[c]);
                     }
-                    if (r < RH && t1g && live) IO::store(t1g + (long long)pf * plane + st.ooff[r < RH ? r : 0], v);
+                    if (r < RH && t1g && live && pf >= d0 && pf < d1)
+                        IO::store(t1g + (long long)pf * plane + st.ooff[r < RH ? r : 0], v);
                     NDC_UNROLL
                     for (int c = 0; c < RW; ++c) {
                         NDC_UNROLL
@@ -479,7 +512,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                 if (!st.ln.active) return;
                 load_plane(st, k + 1);
                 const int j0 = k - 2 * PD;
-                if (j0 < 0) return;
+                if (j0 < d0) return;
                 // the thread's own source values: re-read from global (an L2 hit) rather
                 // than carried in registers across 2*PD planes
                 float sv[SC][RH][RW];
@@ -583,7 +616,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
     template <class Exec> static NDC_D void run(Exec &ex, const Params &p, int block_id)
     {
         const Tile t = p.t;
-        const BlockId id = decode_block(block_id, p.C, t);
+        const BlockId id = decode_block(block_id, p.C, t, p.D);
         const int S = t.S, P = t.P, PL = t.PL, TH = t.TH, W = p.W, H = p.H, D = p.D;
         const int RX = rows_x(TH), RG = rows_g(TH);
         const int off_x = 0, off_t = XR * RX * P, off_g = 2 * XR * RX * P;
@@ -601,6 +634,10 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
         const float floor_ = p.relu ? 0.f : -3.0e38f;   // max(s, floor_) rectifies or passes through
         const float eps = p.eps;
         const int need_gh = p.need_gh;
+        // owned output planes [d0, d1); gn / gd are needed PD planes beyond them on each side
+        // and the x / t1 rings another PD planes beyond that
+        const int d0 = id.d0, d1 = id.d1;
+        const int k_first = d0 - 2 * PD > 0 ? d0 - 2 * PD : 0, k_end = d1 + 2 * PD;
 
         auto load_plane = [&](State &st, int k) NDC_LAMBDA {
             if (!st.ln.active) return;
@@ -725,25 +762,26 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                     NDC_UNROLL
                     for (int c = 0; c < RW; ++c) st.accx[a][r][c] = st.acct[a][r][c] = 0.f;
             for (int i = tid; i < total; i += nthreads) ex.st_(i, 0.f);
-            load_plane(st, 0);
+            load_plane(st, k_first);
         });
         ex.sync();
 
-        for (int kk = 0; kk < D + 2 * PD; ++kk) {
+        for (int kk = k_first; kk < k_end; ++kk) {
             const int k = uniform_int(kk);   // the plane index stays on the scalar unit
             ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k); });
             ex.sync();
 
             // ---- gather: gn, gd of plane k - PD on the band plus PH halo rows each side
             const int j1 = k - PD;
-            const bool live1 = j1 >= 0 && j1 < D;
+            const bool live1 = j1 >= 0 && j1 < D && j1 >= d0 - PD;
+            const bool own1 = j1 >= d0 && j1 < d1;   // filter-gradient terms: owned planes only
             ex.each([&](State &st, int) NDC_LAMBDA {
                 if (!st.ln.active || !live1) return;
                 {
                     float acc[2][SC][RH][RW];
                     const int j = PH + st.ln.strip * RH;
                     gn_gd_rows(st, j1, j, IntTag<RH>(), acc);
-                    if (need_gh) {
+                    if (need_gh && own1) {
                         // own rows: A-side filter-gradient terms, re-reading the x / t1 windows
                         NDC_UNROLL
                         for (int td = 0; td < KD; ++td) {
@@ -801,7 +839,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                 const int pf = k - 2 * PD;
                 NDC_UNROLL
                 for (int r = 0; r < RH; ++r) {
-                    if (pf >= 0 && ((st.ook >> r) & 1u)) {
+                    if (pf >= d0 && ((st.ook >> r) & 1u)) {
                         const long long o = (long long)pf * plane + st.ooff[r];
                         if (gxg) IO::store(gxg + o, st.accx[0][r]);
                         IO::store(gt1g + o, st.acct[0][r]);
@@ -861,7 +899,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
     template <class Exec> static NDC_D void run(Exec &ex, const Params &p, int block_id)
     {
         const Tile t = p.t;
-        const BlockId id = decode_block(block_id, p.C, t);
+        const BlockId id = decode_block(block_id, p.C, t, p.D);
         const int S = t.S, P = t.P, PL = t.PL, TH = t.TH, W = p.W, H = p.H, D = p.D;
         const int RX = rows_x(TH);
         const int off_x = 0, off_t = XR * RX * P, off_g = 2 * XR * RX * P;
@@ -878,6 +916,9 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
         const float floor_ = p.relu ? 0.f : -3.0e38f;   // max(s, floor_) rectifies or passes through
         const float eps = p.eps;
         const int need_gh = p.need_gh;
+        // owned output planes [d0, d1); the rings need PD planes of lead-in and lead-out
+        const int d0 = id.d0, d1 = id.d1;
+        const int k_first = d0 - PD > 0 ? d0 - PD : 0, k_end = d1 + PD;
 
         auto load_plane = [&](State &st, int k) NDC_LAMBDA {
             if (!st.ln.active) return;
@@ -937,11 +978,11 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                 for (int a = 0; a < KT; ++a) st.gacc[i][a] = 0.f;
             }
             for (int i = tid; i < total; i += nthreads) ex.st_(i, 0.f);
-            load_plane(st, 0);
+            load_plane(st, k_first);
         });
         ex.sync();
 
-        for (int kk = 0; kk < D + PD; ++kk) {
+        for (int kk = k_first; kk < k_end; ++kk) {
             const int k = uniform_int(kk);   // the plane index stays on the scalar unit
             ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k); });
             ex.sync();
@@ -950,7 +991,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
             ex.each([&](State &st, int) NDC_LAMBDA {
                 if (!st.ln.active) return;
                 load_plane(st, k + 1);
-                if (j0 < 0) return;
+                if (j0 < d0) return;
                 float sv[SC][RH][RW], gv[SC][RH][RW];
                 const long long ko = (long long)j0 * plane;
                 NDC_UNROLL

@@ -121,6 +121,10 @@ static inline bool make_plan(const KGeom &q, Plan &pl, bool pairs_ok = true, int
     const Tuning tn = tuning();
     if (!make_tile(pl.m, pl.v.RHF, pl.v.RWF, tn.threads_f, pl.tf)) return false;
     if (!make_tile(pl.m, pl.v.RHB, pl.v.RWB, tn.threads_b, pl.tb)) return false;
+    if (env_int("NDC_TUNE_SPLIT", 1)) {
+        split_march(pl.m, (long long)q.B * q.G * pl.tf.ntile, pl.tf);
+        split_march(pl.m, (long long)q.B * q.G * pl.tb.ntile, pl.tb);
+    }
 #define X(kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_)                                        \
     if (NDC_IS_VARIANT(pl, kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_))                      \
         plan_lds<kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_>(pl);
@@ -148,9 +152,10 @@ static inline bool make_plan(const KGeom &q, Plan &pl, bool pairs_ok = true, int
     const int cap = kMaxLdsBytes / 4;
     if (pl.lds_f > cap || pl.lds_b1 > cap || pl.lds_b2 > cap) return false;
     const long long nbc = (long long)q.B * q.G;
-    if (nbc * pl.tf.ntile > 0x7fffffffLL || nbc * pl.tb.ntile > 0x7fffffffLL) return false;
-    pl.nblk_f = (int)(nbc * pl.tf.ntile);
-    pl.nblk_b = (int)(nbc * pl.tb.ntile);
+    const long long nf = nbc * pl.tf.ntile * pl.tf.nseg, nb = nbc * pl.tb.ntile * pl.tb.nseg;
+    if (nf > 0x7fffffffLL || nb > 0x7fffffffLL) return false;
+    pl.nblk_f = (int)nf;
+    pl.nblk_b = (int)nb;
     return true;
 }
 
@@ -360,7 +365,7 @@ static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const T
     tm.mark();
 
     // combine the per-workgroup partial sums: fixed order, so results are reproducible
-    const int C = q.G, SC = q.sc, ntile = pl.tb.ntile, B = q.B;
+    const int C = q.G, SC = q.sc, ntile = pl.tb.ntile * pl.tb.nseg, B = q.B;
     if (gh) {
         st = BE::elementwise((long long)C * kt, stream, [=] NDC_LAMBDA(long long idx) {
             const int c = (int)(idx / kt), r = (int)(idx % kt);

@@ -160,7 +160,7 @@ template <int RH_> struct FwdKernelB {
     template <class Exec> static NDC_D void run(Exec &ex, const Params &p, int block_id)
     {
         const Tile t = p.t;
-        const BlockId id = decode_block(block_id, p.C, t);
+        const BlockId id = decode_block(block_id, p.C, t, p.D);
         const int S = t.S, P = t.P, PL = t.PL, TH = t.TH, W = p.W, H = p.H, D = p.D;
         const int RS = rows_s(TH), RX = rows_x(TH);
         const int off_s = 0, off_x = NS * 2 * RS * P, off_t = off_x + NX * RX * P;
@@ -444,7 +444,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
     template <class Exec> static NDC_D void run(Exec &ex, const Params &p, int block_id)
     {
         const Tile t = p.t;
-        const BlockId id = decode_block(block_id, p.C, t);
+        const BlockId id = decode_block(block_id, p.C, t, p.D);
         const int S = t.S, P = t.P, PL = t.PL, TH = t.TH, W = p.W, H = p.H, D = p.D;
         const int RX = rows_x(TH), RG = rows_g(TH);
         const int off_xp = 0, off_tp = NP * RX * P, off_xt = SAVED ? 0 : 2 * NP * RX * P;
@@ -777,7 +777,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
     template <class Exec> static NDC_D void run(Exec &ex, const Params &p, int block_id)
     {
         const Tile t = p.t;
-        const BlockId id = decode_block(block_id, p.C, t);
+        const BlockId id = decode_block(block_id, p.C, t, p.D);
         const int S = t.S, P = t.P, PL = t.PL, TH = t.TH, W = p.W, H = p.H, D = p.D;
         const int RX = rows_x(TH);
         const int off_xp = 0, off_tp = NP * RX * P, off_gp = SAVED ? 0 : 2 * NP * RX * P;

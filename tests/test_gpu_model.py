@@ -37,10 +37,19 @@ def test_model_on_hip_matches_oracle(cfg, spatial):
     """Protocol of the reference's network test (tests/test_deconv_equivalence.py:332-379):
     a float32 network sits 1e-3..1e-2 from a float64 evaluation of itself in its gradients
     whatever runs the deconvolution, so both routes are compared with the float64 oracle and
-    the HIP route must be no further from it than the PyTorch route (x1.5, floor 1e-5).  The
-    forward output is also held to 1e-4 outright."""
+    the HIP route must be no further from it than the PyTorch route (x1.5; the floor is 1e-4, the
+    float32 parity tolerance of the update itself: below it the two routes differ by rounding
+    order only).  The forward output is also held to 1e-4 outright."""
     torch.manual_seed(0)
     state = dc.Deconver(**cfg).state_dict()
+    # Lift the projection biases (the reference's layer tests do the same,
+    # test_deconv_equivalence.py:44-46,64-65).  With the default biases some pre-activation z + b
+    # of the ~1e6 in the network lands within float32 rounding of zero; whether its ReLU is
+    # on then depends on the GEMM's summation order (it differs from box to box), and one
+    # flipped element moves a bias-gradient entry by tens of percent.
+    for k in state:
+        if k.endswith("deconv.init.linear.linear.bias"):
+            state[k] = state[k] + 1.0
     x = torch.rand(2, cfg["in_channels"], *spatial, device="cuda")
     g = torch.randn(2, cfg["out_channels"], *spatial, device="cuda")
     hip, y_hip, g_hip = _run_route(cfg, {}, state, x, g)
@@ -53,11 +62,12 @@ def test_model_on_hip_matches_oracle(cfg, spatial):
     yr = deconver_forward(ref, x.cpu().double(), cfg)
     yr.backward(g.cpu().double())
     assert O.rel_err(y_hip.cpu(), yr) < 1e-4
-    assert O.rel_err(y_hip.cpu(), yr) <= 1.5 * max(O.rel_err(y_pt.cpu(), yr), 1e-5)
+    assert O.rel_err(y_hip.cpu(), yr) <= 1.5 * max(O.rel_err(y_pt.cpu(), yr), 1e-4)
     for name in g_hip:
         e_hip = O.rel_err(g_hip[name].cpu(), ref[name].grad)
         e_pt = O.rel_err(g_pt[name].cpu(), ref[name].grad)
-        assert e_hip <= 1.5 * max(e_pt, 1e-5), (name, e_hip, e_pt)
+        assert e_hip <= 1.5 * max(e_pt, 1e-4), (name, e_hip, e_pt)
+        assert e_hip < 5e-3, (name, e_hip)   # 5x the reference's layer-level gradient tolerance (:64)
 
 
 def test_config2_model_at_full_width_matches_float64():

@@ -18,6 +18,9 @@ FUSED_GEOMS = [
     (3, 4, (5, 5), (9, 12), 2),           # 2-D 5x5 (marches along H)
     (2, 4, (5, 5), (3, 70), 1),
     (2, 4, (3, 3), (7, 9), 2),            # 2-D 3x3
+    (2, 4, (5, 5), (70, 12), 1),          # 2-D, long march: split into two segments
+    (1, 4, (5, 5), (101, 6), 2),          # 2-D, three segments, ragged last one
+    (1, 4, (3, 3, 3), (37, 4, 6), 1),     # 3-D, two segments
 ]
 
 
