@@ -581,7 +581,12 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
 
 // =================================================================== backward, pass 1
 
-template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> struct Bwd1Kernel {
+// SAVED: the call brings the forward's s/d and n/d, so gn = g (s/d), gd = -gn (n/d) are
+// elementwise (z is not read, n and d are not re-gathered); the x / t1 rings then serve the
+// filter-gradient terms only.
+template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T, bool SAVED_ = false>
+struct Bwd1Kernel {
+    static constexpr bool SAVED = SAVED_;
     static constexpr int KD = KD_, KH = KH_, KW = KW_, SC = SC_, RH = RH_, RW = RW_;
     static constexpr int PD = KD / 2, PH = KH / 2, PW = KW / 2, KT = KD * KH * KW;
     static constexpr int XT = PH > 0 ? 1 : 0;
@@ -626,6 +631,8 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
         const long long cbase = ((long long)id.b * p.C + id.c) * cplane;
         const T *xg = p.x + cbase, *t1g = p.t1 + cbase;
         const T *zg = p.z + cbase * SC, *gg = p.gout + cbase * SC;
+        const T *dg = SAVED ? p.s_over_den + cbase * SC : nullptr;
+        const T *rg = SAVED ? p.ratio + cbase * SC : nullptr;
         T *gxg = p.gx ? p.gx + cbase : nullptr;
         T *gt1g = p.gt1 + cbase;
         UniformF hw = as_uniform(p.h + (long long)id.c * SC * KT);
@@ -687,36 +694,46 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                 const int o = clampi(row, 0, H - 1) * W + st.ln.c0;
                 NDC_UNROLL
                 for (int i = 0; i < SC; ++i) {
-                    IO::load(zg + i * cplane + ko + o, sv[i][r]);
                     IO::load(gg + i * cplane + ko + o, gv[i][r]);
+                    if (SAVED) {
+                        // sv <- s/d, acc[0] <- n/d (as saved by the forward)
+                        IO::load(dg + i * cplane + ko + o, sv[i][r]);
+                        IO::load(rg + i * cplane + ko + o, acc[0][i][r]);
+                    } else {
+                        IO::load(zg + i * cplane + ko + o, sv[i][r]);
+                    }
                     NDC_UNROLL
                     for (int c = 0; c < RW; ++c) {
-                        float s = sv[i][r][c] + st.bv[i];
-                        s = floor_f(s, floor_);
-                        sv[i][r][c] = s;
+                        if (!SAVED) {
+                            float s = sv[i][r][c] + st.bv[i];
+                            s = floor_f(s, floor_);
+                            sv[i][r][c] = s;
+                        }
                         gv[i][r][c] = ok ? gv[i][r][c] : 0.f;
                     }
                 }
             }
-            NDC_UNROLL
-            for (int a = 0; a < 2; ++a)
+            if (!SAVED) {
                 NDC_UNROLL
-                for (int i = 0; i < SC; ++i)
+                for (int a = 0; a < 2; ++a)
                     NDC_UNROLL
-                    for (int r = 0; r < NR; ++r)
+                    for (int i = 0; i < SC; ++i)
                         NDC_UNROLL
-                        for (int c = 0; c < RW; ++c) acc[a][i][r][c] = 0.f;
-            float wt[SC][KH * KW], wn[SC][KH * KW];
-            load_plane_taps<SC, KT, KH * KW>(hw, wt);
-            NDC_ROLLED
-            for (int td = 0; td < KD; ++td) {
-                load_plane_taps<SC, KT, KH * KW>(hw + (td + 1 < KD ? td + 1 : 0) * KH * KW, wn);
-                const int slot = wrap((j1 + PD - td) % XR, XR);
-                const int ob = (slot * RX + j) * P + PL + st.ln.c0 - PW;
-                const int base[2] = {off_x + ob, off_t + ob};
-                a_plane<KH, KW, KT, SC, NR, RW, 2>(ex, base, P, wt, acc);
-                NDC_UNROLL
-                for (int i = 0; i < SC; ++i) copy_taps<KH * KW>(wn[i], wt[i]);
+                        for (int r = 0; r < NR; ++r)
+                            NDC_UNROLL
+                            for (int c = 0; c < RW; ++c) acc[a][i][r][c] = 0.f;
+                float wt[SC][KH * KW], wn[SC][KH * KW];
+                load_plane_taps<SC, KT, KH * KW>(hw, wt);
+                NDC_ROLLED
+                for (int td = 0; td < KD; ++td) {
+                    load_plane_taps<SC, KT, KH * KW>(hw + (td + 1 < KD ? td + 1 : 0) * KH * KW, wn);
+                    const int slot = wrap((j1 + PD - td) % XR, XR);
+                    const int ob = (slot * RX + j) * P + PL + st.ln.c0 - PW;
+                    const int base[2] = {off_x + ob, off_t + ob};
+                    a_plane<KH, KW, KT, SC, NR, RW, 2>(ex, base, P, wt, acc);
+                    NDC_UNROLL
+                    for (int i = 0; i < SC; ++i) copy_taps<KH * KW>(wn[i], wt[i]);
+                }
             }
             NDC_UNROLL
             for (int r = 0; r < NR; ++r)
@@ -724,9 +741,15 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                 for (int i = 0; i < SC; ++i)
                     NDC_UNROLL
                     for (int c = 0; c < RW; ++c) {
-                        const float inv = fast_rcp(acc[1][i][r][c] + eps);
-                        const float gn = gv[i][r][c] * sv[i][r][c] * inv;
-                        const float gd = -(gn * (acc[0][i][r][c] + eps)) * inv;
+                        float gn, gd;
+                        if (SAVED) {
+                            gn = gv[i][r][c] * sv[i][r][c];
+                            gd = -(gn * acc[0][i][r][c]);
+                        } else {
+                            const float inv = fast_rcp(acc[1][i][r][c] + eps);
+                            gn = gv[i][r][c] * sv[i][r][c] * inv;
+                            gd = -(gn * (acc[0][i][r][c] + eps)) * inv;
+                        }
                         ex.st_(off_g + (i * RG + j + r) * P + PL + st.ln.c0 + c, gn);
                         ex.st_(off_g + ((SC + i) * RG + j + r) * P + PL + st.ln.c0 + c, gd);
                         acc[0][i][r][c] = gn;
@@ -869,7 +892,11 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
 
 // =================================================================== backward, pass 2
 
-template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> struct Bwd2Kernel {
+// SAVED: gz = [s > 0] (g (n/d) + A(gt1)) with the forward's n/d: only the gt1 ring is kept.
+template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T, bool SAVED_ = false>
+struct Bwd2Kernel {
+    static constexpr bool SAVED = SAVED_;
+    static constexpr int NA = SAVED ? 1 : 3;   // gathered operands: (x, t1,) gt1
     static constexpr int KD = KD_, KH = KH_, KW = KW_, SC = SC_, RH = RH_, RW = RW_;
     static constexpr int PD = KD / 2, PH = KH / 2, PW = KW / 2, KT = KD * KH * KW;
     static constexpr int NXR = RH + (PH > 0 ? 1 : 0);
@@ -891,7 +918,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
     static NDC_HD int rows_x(int TH) { return TH + 2 * PH; }
     static NDC_HD int lds_floats(const Tile &t)
     {
-        const int main_ = 3 * XR * rows_x(t.TH) * t.P;
+        const int main_ = NA * XR * rows_x(t.TH) * t.P;
         const int red = (t.NT / 64) * NRED;
         return main_ > red ? main_ : red;
     }
@@ -902,13 +929,14 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
         const BlockId id = decode_block(block_id, p.C, t, p.D);
         const int S = t.S, P = t.P, PL = t.PL, TH = t.TH, W = p.W, H = p.H, D = p.D;
         const int RX = rows_x(TH);
-        const int off_x = 0, off_t = XR * RX * P, off_g = 2 * XR * RX * P;
-        const int total = 3 * XR * RX * P;
+        const int off_x = 0, off_t = XR * RX * P, off_g = SAVED ? 0 : 2 * XR * RX * P;
+        const int total = NA * XR * RX * P;
         const int plane = H * W;
         const long long cplane = (long long)D * plane;
         const long long cbase = ((long long)id.b * p.C + id.c) * cplane;
         const T *xg = p.x + cbase, *t1g = p.t1 + cbase, *gt1g = p.gt1 + cbase;
         const T *zg = p.z + cbase * SC, *gg = p.gout + cbase * SC;
+        const T *rg = SAVED ? p.ratio + cbase * SC : nullptr;
         T *gzg = p.gz ? p.gz + cbase * SC : nullptr;
         UniformF hw = as_uniform(p.h + (long long)id.c * SC * KT);
         const int r0 = id.r0;
@@ -926,8 +954,10 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                 const long long ko = (long long)k * plane;
                 NDC_UNROLL
                 for (int n = 0; n < NXR; ++n) {
-                    IO::load(xg + ko + st.xoff[n], st.px[n]);
-                    IO::load(t1g + ko + st.xoff[n], st.pt[n]);
+                    if (!SAVED) {
+                        IO::load(xg + ko + st.xoff[n], st.px[n]);
+                        IO::load(t1g + ko + st.xoff[n], st.pt[n]);
+                    }
                     IO::load(gt1g + ko + st.xoff[n], st.pg[n]);
                 }
             } else {
@@ -947,8 +977,10 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                     NDC_UNROLL
                     for (int c = 0; c < RW; ++c) {
                         const int o = (slot * RX + j) * P + PL + st.ln.c0 + c;
-                        ex.st_(off_x + o, st.px[n][c]);
-                        ex.st_(off_t + o, st.pt[n][c]);
+                        if (!SAVED) {
+                            ex.st_(off_x + o, st.px[n][c]);
+                            ex.st_(off_t + o, st.pt[n][c]);
+                        }
                         ex.st_(off_g + o, st.pg[n][c]);
                     }
                 }
@@ -992,7 +1024,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                 if (!st.ln.active) return;
                 load_plane(st, k + 1);
                 if (j0 < d0) return;
-                float sv[SC][RH][RW], gv[SC][RH][RW];
+                float sv[SC][RH][RW], gv[SC][RH][RW], rv[SC][RH][RW];
                 const long long ko = (long long)j0 * plane;
                 NDC_UNROLL
                 for (int r = 0; r < RH; ++r) {
@@ -1001,6 +1033,12 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                     for (int i = 0; i < SC; ++i) {
                         IO::load(zg + i * cplane + ko + st.ooff[r], sv[i][r]);
                         IO::load(gg + i * cplane + ko + st.ooff[r], gv[i][r]);
+                        if (SAVED) {
+                            IO::load(rg + i * cplane + ko + st.ooff[r], rv[i][r]);
+                        } else {
+                            NDC_UNROLL
+                            for (int c = 0; c < RW; ++c) rv[i][r][c] = 0.f;
+                        }
                         NDC_UNROLL
                         for (int c = 0; c < RW; ++c) {
                             // with the ReLU on, s <= 0 marks a masked element
@@ -1011,9 +1049,9 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                         }
                     }
                 }
-                float acc[3][SC][RH][RW];
+                float acc[NA][SC][RH][RW];
                 NDC_UNROLL
-                for (int a = 0; a < 3; ++a)
+                for (int a = 0; a < NA; ++a)
                     NDC_UNROLL
                     for (int i = 0; i < SC; ++i)
                         NDC_UNROLL
@@ -1027,8 +1065,13 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                     load_plane_taps<SC, KT, KH * KW>(hw + (td + 1 < KD ? td + 1 : 0) * KH * KW, wn);
                     const int slot = wrap((j0 + PD - td) % XR, XR);
                     const int ob = (slot * RX + st.ln.strip * RH) * P + PL + st.ln.c0 - PW;
-                    const int base[3] = {off_x + ob, off_t + ob, off_g + ob};
-                    a_plane<KH, KW, KT, SC, RH, RW, 3>(ex, base, P, wt, acc);
+                    int base[NA];
+                    base[NA - 1] = off_g + ob;
+                    if (!SAVED) {
+                        base[0] = off_x + ob;
+                        base[NA > 1 ? 1 : 0] = off_t + ob;
+                    }
+                    a_plane<KH, KW, KT, SC, RH, RW, NA>(ex, base, P, wt, acc);
                     NDC_UNROLL
                     for (int i = 0; i < SC; ++i) copy_taps<KH * KW>(wn[i], wt[i]);
                 }
@@ -1067,8 +1110,13 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                         float v[RW];
                         NDC_UNROLL
                         for (int c = 0; c < RW; ++c) {
-                            float gzv = gv[i][r][c] * (acc[0][i][r][c] + eps) * fast_rcp(acc[1][i][r][c] + eps) +
-                                        acc[2][i][r][c];
+                            float gzv;
+                            if (SAVED)
+                                gzv = gv[i][r][c] * rv[i][r][c] + acc[NA - 1][i][r][c];
+                            else
+                                gzv = gv[i][r][c] * (acc[0][i][r][c] + eps) *
+                                          fast_rcp(acc[NA > 1 ? 1 : 0][i][r][c] + eps) +
+                                      acc[NA - 1][i][r][c];
                             if (p.relu && !(sv[i][r][c] > 0.f)) gzv = 0.f;
                             st.gbacc[i] += gzv;
                             v[c] = gzv;

@@ -195,12 +195,12 @@ static inline size_t forward_ws(const KGeom &q, int dtype)
     return align256((size_t)q.G * kTabWords * 4);
 }
 
-// whether backward() reads the forward's s/d and n/d for this geometry (aligned pointers
-// assumed): only the bf16 dot2 kernels have that form
+// whether backward() reads the forward's s/d and n/d for this geometry: every fused kernel
+// family has that form
 static inline bool backward_uses_saved(const KGeom &q, int dtype)
 {
     Plan pl;
-    return make_plan(q, pl, true, dtype) && pl.dot2;
+    return make_plan(q, pl, true, dtype);
 }
 
 template <class BE, typename T> struct Dot2Launch {
@@ -335,9 +335,14 @@ static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const T
         st = Dot2Launch<BE, T>::bwd1(p, pl, stream, saved);
     } else {
 #define X(kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_)                                          \
-    if (NDC_IS_VARIANT(pl, kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_))                        \
-        st = BE::template block_kernel<Bwd1Kernel<kd_, kh_, kw_, sc_, rhb_, rwb_, T>>(         \
-            p, pl.nblk_b, pl.tb.NT, pl.lds_b1, stream);
+    if (NDC_IS_VARIANT(pl, kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_)) {                      \
+        if (saved)                                                                             \
+            st = BE::template block_kernel<Bwd1Kernel<kd_, kh_, kw_, sc_, rhb_, rwb_, T, true>>(\
+                p, pl.nblk_b, pl.tb.NT, pl.lds_b1, stream);                                    \
+        else                                                                                   \
+            st = BE::template block_kernel<Bwd1Kernel<kd_, kh_, kw_, sc_, rhb_, rwb_, T>>(     \
+                p, pl.nblk_b, pl.tb.NT, pl.lds_b1, stream);                                    \
+    }
         NDC_FUSED_VARIANTS(X)
 #undef X
     }
@@ -355,9 +360,15 @@ static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const T
         st = Dot2Launch<BE, T>::bwd2(p, pl, stream, saved);
     } else {
 #define X(kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_)                                          \
-    if (NDC_IS_VARIANT(pl, kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_))                        \
-        st = BE::template block_kernel<Bwd2Kernel<kd_, kh_, kw_, sc_, rhb_, rwb_, T>>(         \
-            p, pl.nblk_b, pl.tb.NT, pl.lds_b2, stream);
+    if (NDC_IS_VARIANT(pl, kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_)) {                      \
+        typedef Bwd2Kernel<kd_, kh_, kw_, sc_, rhb_, rwb_, T, true> KS;                        \
+        if (saved)                                                                             \
+            st = BE::template block_kernel<KS>(p, pl.nblk_b, pl.tb.NT, KS::lds_floats(pl.tb),  \
+                                               stream);                                        \
+        else                                                                                   \
+            st = BE::template block_kernel<Bwd2Kernel<kd_, kh_, kw_, sc_, rhb_, rwb_, T>>(     \
+                p, pl.nblk_b, pl.tb.NT, pl.lds_b2, stream);                                    \
+    }
         NDC_FUSED_VARIANTS(X)
 #undef X
     }

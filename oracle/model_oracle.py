@@ -59,7 +59,7 @@ def _block(state, prefix, x, cfg):
     ndc = OracleNDC(c, cfg["kernel_size"], ratio=cfg.get("ratio", 4), groups=cfg.get("groups", -1),
                     num_iters=cfg.get("num_iters", 1))
     u = _norm(state, prefix + ".norm1", x)
-    u = torch.relu(_pointwise(u, state[prefix + ".dcm.in_proj.linear.weight"]))
+    u = cfg.get("act_fn", torch.relu)(_pointwise(u, state[prefix + ".dcm.in_proj.linear.weight"]))
     u = ndc.forward(u, state[prefix + ".dcm.deconv.init.linear.linear.weight"].squeeze(-1),
                     state[prefix + ".dcm.deconv.init.linear.linear.bias"],
                     state[prefix + ".dcm.deconv.init.h0"])
@@ -79,7 +79,8 @@ def deconver_forward(state: Dict[str, torch.Tensor], x: torch.Tensor, cfg: dict)
     """Logits of the network with parameters ``state`` for input ``x``.
 
     ``cfg``: ``spatial_dims``, ``encoder_depth``, ``strides``, ``decoder_depth``,
-    ``kernel_size`` and optionally ``ratio``, ``groups``, ``num_iters``.
+    ``kernel_size`` and optionally ``ratio``, ``groups``, ``num_iters``, ``act_fn`` (the
+    mixer's activation as a function, default ``torch.relu``).
     """
     nd = cfg["spatial_dims"]
     enc_depth: Sequence[int] = cfg["encoder_depth"]

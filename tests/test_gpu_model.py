@@ -24,6 +24,41 @@ def _ndc_layers(model):
     return [m for m in model.modules() if isinstance(m, dc.Deconv)]
 
 
+def _smooth_case(cfg, spatial, margin=3e-6):
+    """Seeded weights and inputs whose gradients do not hinge on a ReLU sitting on its kink.
+
+    The network has ~1e6 ReLU inputs.  With random weights one of them usually lands within
+    float32 rounding of zero; whether that unit is on then depends on the GEMM's summation
+    order (it differs between routes and from box to box), and one flipped unit moves a
+    weight gradient by 1e-3..1e-2 of its largest entry -- a property of the test instance,
+    not of any implementation.  So the mixers use Softplus (smooth, positive, as the layer's
+    input must be), the NDC projections get the +1 bias of the reference's layer tests
+    (test_deconv_equivalence.py:44-46,64-65), and a float64 CPU probe confirms that no NDC
+    pre-activation z + b is within `margin` of zero (float32 rounding of these dot products
+    is ~2e-7)."""
+    cfg = {**cfg, "act": nn.Softplus}
+    for seed in range(20):
+        torch.manual_seed(seed)
+        state = dc.Deconver(**cfg).state_dict()
+        for k in state:
+            if k.endswith("deconv.init.linear.linear.bias"):
+                state[k] = state[k] + 1.0
+        x = torch.rand(2, cfg["in_channels"], *spatial)
+        g = torch.randn(2, cfg["out_channels"], *spatial)
+        probe = dc.Deconver(**cfg).double()
+        probe.load_state_dict({k: v.double() for k, v in state.items()})
+        smallest = []
+        for m in probe.modules():
+            if isinstance(m, dc.Deconv):
+                m.init.linear.register_forward_hook(
+                    lambda mod, i, o: smallest.append(float(o.abs().min())))
+        with torch.no_grad():
+            probe(x.double())
+        if min(smallest) > margin:
+            return cfg, state, x.cuda(), g.cuda()
+    raise RuntimeError("no instance without a near-zero NDC pre-activation among 20 seeds")
+
+
 def _run_route(cfg, extra, state, x, g):
     model = dc.Deconver(**cfg, **extra).cuda()
     model.load_state_dict(state, strict=True)
@@ -40,18 +75,7 @@ def test_model_on_hip_matches_oracle(cfg, spatial):
     the HIP route must be no further from it than the PyTorch route (x1.5; the floor is 1e-4, the
     float32 parity tolerance of the update itself: below it the two routes differ by rounding
     order only).  The forward output is also held to 1e-4 outright."""
-    torch.manual_seed(0)
-    state = dc.Deconver(**cfg).state_dict()
-    # Lift the projection biases (the reference's layer tests do the same,
-    # test_deconv_equivalence.py:44-46,64-65).  With the default biases some pre-activation z + b
-    # of the ~1e6 in the network lands within float32 rounding of zero; whether its ReLU is
-    # on then depends on the GEMM's summation order (it differs from box to box), and one
-    # flipped element moves a bias-gradient entry by tens of percent.
-    for k in state:
-        if k.endswith("deconv.init.linear.linear.bias"):
-            state[k] = state[k] + 1.0
-    x = torch.rand(2, cfg["in_channels"], *spatial, device="cuda")
-    g = torch.randn(2, cfg["out_channels"], *spatial, device="cuda")
+    cfg, state, x, g = _smooth_case(cfg, spatial)
     hip, y_hip, g_hip = _run_route(cfg, {}, state, x, g)
     for layer in _ndc_layers(hip):
         assert layer.fast_path_applicable(torch.empty(1, layer.channels, *spatial, device="cuda"))
@@ -59,7 +83,7 @@ def test_model_on_hip_matches_oracle(cfg, spatial):
     for layer in _ndc_layers(pt):
         assert not layer.fast_path_applicable(torch.empty(1, layer.channels, *spatial, device="cuda"))
     ref = {k: v.detach().cpu().double().requires_grad_(True) for k, v in state.items()}
-    yr = deconver_forward(ref, x.cpu().double(), cfg)
+    yr = deconver_forward(ref, x.cpu().double(), {**cfg, "act_fn": torch.nn.functional.softplus})
     yr.backward(g.cpu().double())
     assert O.rel_err(y_hip.cpu(), yr) < 1e-4
     assert O.rel_err(y_hip.cpu(), yr) <= 1.5 * max(O.rel_err(y_pt.cpu(), yr), 1e-4)

@@ -87,11 +87,11 @@ def test_fused_forward_backward_fp32(geom, relu, with_bias):
 
 def test_backward_uses_saved_predicate():
     lib = hostcheck_library()
-    mk = lambda dt, ks, sp: _lib.make_geom(2, 8, 1, 4, sp, ks, dt, True, 1e-16)
-    assert lib.backward_uses_saved(mk(_lib.NDC_BF16, (3, 3, 3), (8, 8, 8)))
-    assert not lib.backward_uses_saved(mk(_lib.NDC_F32, (3, 3, 3), (8, 8, 8)))
-    assert not lib.backward_uses_saved(mk(_lib.NDC_BF16, (5, 5), (8, 8)))
-    assert not lib.backward_uses_saved(mk(_lib.NDC_BF16, (3, 3, 3), (8, 8, 7)))   # odd width
+    mk = lambda dt, ks, sp, m=1, g=8: _lib.make_geom(2, g, m, 4, sp, ks, dt, True, 1e-16)
+    for g in (mk(_lib.NDC_BF16, (3, 3, 3), (8, 8, 8)), mk(_lib.NDC_F32, (3, 3, 3), (8, 8, 8)),
+              mk(_lib.NDC_BF16, (5, 5), (8, 8)), mk(_lib.NDC_BF16, (3, 3, 3), (8, 8, 7))):
+        assert lib.backward_uses_saved(g)               # every fused kernel family reads them
+    assert not lib.backward_uses_saved(mk(_lib.NDC_F32, (3, 3, 3), (8, 8, 8), m=2, g=4))  # direct path
 
 
 def test_fused_inference_needs_no_t1():
@@ -131,7 +131,7 @@ def test_fused_bf16_storage(geom):
     assert host_faults(lib)[0] == 0
 
 
-@pytest.mark.parametrize("geom", FUSED_GEOMS[:3] + FUSED_GEOMS[5:6])
+@pytest.mark.parametrize("geom", FUSED_GEOMS[:3] + FUSED_GEOMS[5:6] + FUSED_GEOMS[7:9] + FUSED_GEOMS[10:11])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("relu", [True, False])
 def test_fused_saved_denominator_and_ratio(geom, dtype, relu):
