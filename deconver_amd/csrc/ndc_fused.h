@@ -304,7 +304,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
     static constexpr int RHK = RH + XT;
     static constexpr int NZR = RH + (PH > 0 ? 2 : 0);    // rows of s a thread stages
     static constexpr int NXR = RH + (PH > 0 ? 1 : 0);    // rows of x a thread stages
-    static constexpr int XR = KD + 1;                    // x ring slots
+    static constexpr int XR = KD;                        // x ring slots (filled in the scatter phase)
     typedef FwdParams<T> Params;
     typedef VecIO<T, RW> IO;
 
@@ -407,6 +407,11 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                             ex.st_(off_s + (i * RS + j) * P + lb + c, st.pz[i][n][c]);
                 }
             }
+        };
+        // x plane k - PD into its ring slot.  Runs in the scatter phase: a barrier after the
+        // gather that last read that slot, which is what lets KD slots do.
+        auto store_x_plane = [&](State &st, int k) NDC_LAMBDA {
+            const int lb = PL + st.ln.c0;
             const int slot = wrap((k - PD) % XR, XR);
             NDC_UNROLL
             for (int n = 0; n < NXR; ++n) {
@@ -463,6 +468,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
             // ---- K-scatter: plane k of s feeds the KD pending planes of t1
             ex.each([&](State &st, int) NDC_LAMBDA {
                 if (!st.ln.active) return;
+                store_x_plane(st, k);
                 const bool extra = XT && st.ln.strip < 2 * PH;
                 const int jx = halo_row(st.ln.strip, PH, TH);
                 const int cb = PL + st.ln.c0 - PW;
