@@ -379,16 +379,17 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                         NDC_UNROLL
                         for (int c = 0; c < RW; ++c) st.pz[i][n][c] = 0.f;
             }
+            // planes outside the volume: load a clamped plane and select zero (a store in each
+            // arm of a branch would push the staging registers into private memory)
             const int kx = k - PD;
-            if (kx >= 0 && kx < D) {
-                const T *xk = xg + (long long)kx * plane;
+            const bool xlive = kx >= 0 && kx < D;
+            const T *xk = xg + (long long)clampi(kx, 0, D - 1) * plane;
+            NDC_UNROLL
+            for (int n = 0; n < NXR; ++n) {
+                float v[RW];
+                IO::load(xk + st.xoff[n], v);
                 NDC_UNROLL
-                for (int n = 0; n < NXR; ++n) IO::load(xk + st.xoff[n], st.px[n]);
-            } else {
-                NDC_UNROLL
-                for (int n = 0; n < NXR; ++n)
-                    NDC_UNROLL
-                    for (int c = 0; c < RW; ++c) st.px[n][c] = 0.f;
+                for (int c = 0; c < RW; ++c) st.px[n][c] = xlive ? v[c] : 0.f;
             }
         };
 
@@ -654,18 +655,20 @@ struct Bwd1Kernel {
 
         auto load_plane = [&](State &st, int k) NDC_LAMBDA {
             if (!st.ln.active) return;
-            if (k < D) {
-                const long long ko = (long long)k * plane;
+            // planes past the end: load the last plane and select zero (a store in each arm of
+            // a branch would push the staging registers into private memory)
+            const bool live = k < D;
+            const long long ko = (long long)clampi(k, 0, D - 1) * plane;
+            NDC_UNROLL
+            for (int n = 0; n < NXR; ++n) {
+                float vx[RW], vt[RW];
+                IO::load(xg + ko + st.xoff[n], vx);
+                IO::load(t1g + ko + st.xoff[n], vt);
                 NDC_UNROLL
-                for (int n = 0; n < NXR; ++n) {
-                    IO::load(xg + ko + st.xoff[n], st.px[n]);
-                    IO::load(t1g + ko + st.xoff[n], st.pt[n]);
+                for (int c = 0; c < RW; ++c) {
+                    st.px[n][c] = live ? vx[c] : 0.f;
+                    st.pt[n][c] = live ? vt[c] : 0.f;
                 }
-            } else {
-                NDC_UNROLL
-                for (int n = 0; n < NXR; ++n)
-                    NDC_UNROLL
-                    for (int c = 0; c < RW; ++c) st.px[n][c] = st.pt[n][c] = 0.f;
             }
         };
         auto store_plane = [&](State &st, int k) NDC_LAMBDA {
@@ -956,21 +959,24 @@ struct Bwd2Kernel {
 
         auto load_plane = [&](State &st, int k) NDC_LAMBDA {
             if (!st.ln.active) return;
-            if (k < D) {
-                const long long ko = (long long)k * plane;
-                NDC_UNROLL
-                for (int n = 0; n < NXR; ++n) {
-                    if (!SAVED) {
-                        IO::load(xg + ko + st.xoff[n], st.px[n]);
-                        IO::load(t1g + ko + st.xoff[n], st.pt[n]);
-                    }
-                    IO::load(gt1g + ko + st.xoff[n], st.pg[n]);
+            // planes past the end: load the last plane and select zero (a store in each arm of
+            // a branch would push the staging registers into private memory)
+            const bool live = k < D;
+            const long long ko = (long long)clampi(k, 0, D - 1) * plane;
+            NDC_UNROLL
+            for (int n = 0; n < NXR; ++n) {
+                float vx[RW], vt[RW], vg[RW];
+                if (!SAVED) {
+                    IO::load(xg + ko + st.xoff[n], vx);
+                    IO::load(t1g + ko + st.xoff[n], vt);
                 }
-            } else {
+                IO::load(gt1g + ko + st.xoff[n], vg);
                 NDC_UNROLL
-                for (int n = 0; n < NXR; ++n)
-                    NDC_UNROLL
-                    for (int c = 0; c < RW; ++c) st.px[n][c] = st.pt[n][c] = st.pg[n][c] = 0.f;
+                for (int c = 0; c < RW; ++c) {
+                    st.px[n][c] = (!SAVED && live) ? vx[c] : 0.f;
+                    st.pt[n][c] = (!SAVED && live) ? vt[c] : 0.f;
+                    st.pg[n][c] = live ? vg[c] : 0.f;
+                }
             }
         };
         auto store_plane = [&](State &st, int k) NDC_LAMBDA {
