@@ -3,6 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bf16|fp32] [--no-cpu]
     python bench.py --workload sweep                                      (config 5, forward only)
+    python bench.py --workload accuracy                                   (float32 error table)
     python bench.py --workload train3d|model2d [--ndc hip|pytorch|both]   (model level, below)
 
 One step = one forward + one backward (input-, source-, filter- and bias-gradient) of the
@@ -166,6 +167,77 @@ def sweep_workload(args) -> int:
     return 0
 
 
+ACCURACY_CASES = [   # the layer geometries of the reference's accuracy report (benchmarks/accuracy_report.py:36-50)
+    ("brats23 stage C=32", dict(channels=32, ratio=4, groups=-1, kernel_size=(3, 3, 3))),
+    ("brats23 stage C=64", dict(channels=64, ratio=4, groups=-1, kernel_size=(3, 3, 3))),
+    ("brats23 stage C=128", dict(channels=128, ratio=4, groups=-1, kernel_size=(3, 3, 3))),
+    ("brats23 stage C=256", dict(channels=256, ratio=4, groups=-1, kernel_size=(3, 3, 3))),
+    ("brats23 stage C=512", dict(channels=512, ratio=4, groups=-1, kernel_size=(3, 3, 3))),
+    ("fives/glas 2-D k=5", dict(channels=32, ratio=4, groups=-1, kernel_size=(5, 5))),
+    ("grouped C/G=4", dict(channels=12, ratio=2, groups=3, kernel_size=(3, 3, 3))),
+    ("dense groups=1", dict(channels=8, ratio=1, groups=1, kernel_size=(3, 3, 3))),
+    ("grouped C/G=4, small filter", dict(channels=8, ratio=1, groups=2, kernel_size=(3, 3, 3))),
+]
+
+
+def accuracy_workload(args) -> int:
+    """Float32 accuracy of the whole layer (projection + update, all gradients) on the HIP
+    route and on the layer's PyTorch route, both against the oracle evaluated in float64 on
+    the CPU from the same parameters; `max|d| / max|ref|` per case, worst tensor."""
+    import torch
+
+    import deconver_amd as dc
+    from oracle import ndc_oracle as O
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    dev = torch.device("cuda:0")
+    rows = []
+    for name, kw in ACCURACY_CASES:
+        nd = len(kw["kernel_size"])
+        spatial = (12,) * nd if nd == 3 else (48,) * nd
+        torch.manual_seed(0)
+        base = dc.Deconv(**kw)
+        with torch.no_grad():
+            base.init.linear.linear.bias.add_(1.0)
+        state = base.state_dict()
+        x0 = torch.rand(2, kw["channels"], *spatial)
+        g0 = torch.randn(2, base.groups * base.source_channels, *spatial)
+        oracle = O.OracleNDC(kw["channels"], kw["kernel_size"], ratio=kw["ratio"], groups=kw["groups"])
+        ref_p = [state["init.linear.linear.weight"].double().squeeze(-1).requires_grad_(True),
+                 state["init.linear.linear.bias"].double().requires_grad_(True),
+                 state["init.h0"].double().requires_grad_(True)]
+        xr = x0.double().requires_grad_(True)
+        yr = oracle.forward(xr, *ref_p)
+        yr.backward(g0.double())
+        ref = [yr.detach(), xr.grad, ref_p[0].grad.unsqueeze(-1), ref_p[1].grad, ref_p[2].grad]
+        errs = {}
+        for route, extra in (("hip", {}), ("pytorch", {"dilation": 1})):
+            layer = dc.Deconv(**kw, **extra)
+            layer.load_state_dict(state)
+            layer = layer.to(dev)
+            x = x0.to(dev).requires_grad_(True)
+            on_hip = layer.fast_path_applicable(x)
+            assert on_hip == (route == "hip")
+            y = layer(x)
+            y.backward(g0.to(dev))
+            got = [y.detach(), x.grad, layer.init.linear.linear.weight.grad,
+                   layer.init.linear.linear.bias.grad, layer.init.h0.grad]
+            e = [O.rel_err(a.cpu(), r) for a, r in zip(got, ref)]
+            errs[route] = {"forward": e[0], "worst_gradient": max(e[1:])}
+        rows.append({"case": name, "spatial": list(spatial), **errs})
+    worst = max(r["hip"]["worst_gradient"] for r in rows)
+    print(json.dumps({
+        "metric": "float32 layer accuracy vs float64 oracle (worst gradient, max|d|/max|ref|)",
+        "value": worst, "unit": "relative error", "n_gpus": 1, "steps": 1, "warmup": 0,
+        "ms_per_step": None, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "accuracy report over the reference's layer geometries, batch 2"},
+        "cases": rows, "roofline": None, "cpu_baseline": None}))
+    return 0
+
+
 MODEL_WORKLOADS = {
     "train3d": dict(
         net=dict(in_channels=2, out_channels=1, spatial_dims=3, encoder_depth=(1, 1, 1, 1),
@@ -273,7 +345,8 @@ def main() -> int:
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
-    ap.add_argument("--workload", choices=("ndc", "sweep", "train3d", "model2d"), default="ndc",
+    ap.add_argument("--workload", choices=("ndc", "sweep", "accuracy", "train3d", "model2d"),
+                    default="ndc",
                     help="ndc: the headline update node (default); the others are model level")
     ap.add_argument("--ndc", choices=("hip", "pytorch", "both"), default="hip",
                     help="model-level workloads: which route the NDC layers take")
@@ -285,6 +358,8 @@ def main() -> int:
 
     if args.workload == "sweep":
         return sweep_workload(args)
+    if args.workload == "accuracy":
+        return accuracy_workload(args)
     if args.workload != "ndc":
         return model_workload(args)
 
