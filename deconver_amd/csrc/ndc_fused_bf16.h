@@ -133,7 +133,9 @@ template <int RH_> struct FwdKernelB {
     static constexpr int KD = 3, KH = 3, KW = 3, SC = 4, RH = RH_, RW = 2;
     static constexpr int PD = 1, PH = 1, PW = 1, KT = 27;
     static constexpr int RHK = RH + 1, NZR = RH + 2, NXR = RH + 1;
-    static constexpr int NS = 3, NX = 2, NTP = 2;   // ring slots: source, x pairs, t1 pairs
+    // ring slots: source (one: it is only read in the scatter phase of the step that staged
+    // it), x pairs, t1 pairs
+    static constexpr int NS = 1, NX = 2, NTP = 2;
     typedef bf16_t T;
     typedef FwdParams<T> Params;
     typedef VecIO<T, 2> IO;
@@ -147,7 +149,6 @@ template <int RH_> struct FwdKernelB {
         float t1prev[RHK][RW];
         uint32_t pz[SC][NZR];       // staged source rows, raw (two bf16 columns per word)
         uint32_t px[NXR], pxprev[NXR];
-        uint32_t own[2][RH][RW];    // the thread's own source words of the plane being finished
     };
 
     static NDC_HD int rows_s(int TH) { return TH + 4; }
@@ -290,7 +291,7 @@ template <int RH_> struct FwdKernelB {
             ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k); });
             ex.sync();
 
-            // ---- K-scatter of source plane k; own source words of plane k - 2; t1 plane k - 1
+            // ---- K-scatter of source plane k; t1 plane k - 1
             ex.each([&](State &st, int) NDC_LAMBDA {
                 if (!st.ln.active) return;
                 store_x_pairs(st, k);
@@ -309,17 +310,6 @@ template <int RH_> struct FwdKernelB {
                         if (extra) k_rows_d2<1, RW, RHK>(ex, b0 + jx * P, P, wp, st.t1acc, RH);
                         copy_taps<KT>(wn, wp);
                     }
-                }
-                if (k >= 2) {
-                    const int ob = off_s + wrap((k - 2) % NS, NS) * 2 * RS * P + PL + st.ln.c0;
-                    NDC_UNROLL
-                    for (int pr = 0; pr < 2; ++pr)
-                        NDC_UNROLL
-                        for (int r = 0; r < RH; ++r)
-                            NDC_UNROLL
-                            for (int c = 0; c < RW; ++c)
-                                st.own[pr][r][c] = float_to_bits(
-                                    ex.ld(ob + (pr * RS + 2 * PH + st.ln.strip * RH + r) * P + c));
                 }
                 // t1 plane k - 1 is complete: word (t1[k-2], t1[k-1]) goes to pair slot (k - 2) % 2
                 const int pf = k - PD;
@@ -356,6 +346,14 @@ template <int RH_> struct FwdKernelB {
                 load_plane(st, k + 1);
                 const int j0 = k - 2;
                 if (j0 < 0) return;
+                // the thread's own source values of plane j0: z is read again (it was staged two
+                // steps ago, so this hits the L2) rather than kept in LDS or registers that long
+                uint32_t own[SC][RH];
+                NDC_UNROLL
+                for (int r = 0; r < RH; ++r)
+                    NDC_UNROLL
+                    for (int i = 0; i < SC; ++i)
+                        own[i][r] = buf_ld(zb_, st.ooff[r], (unsigned)j0 * plane2 + i * cplane2);
                 float acc[2][SC][RH][RW];
                 NDC_UNROLL
                 for (int a = 0; a < 2; ++a)
@@ -384,8 +382,10 @@ template <int RH_> struct FwdKernelB {
                         float v[RW], rd[RW], rt[RW];
                         NDC_UNROLL
                         for (int c = 0; c < RW; ++c) {
-                            const uint32_t w = st.own[i >> 1][r][c];
-                            const float s = (i & 1) ? bf_hi(w) : bf_lo(w);
+                            const uint32_t w = own[i][r];
+                            // same arithmetic as the staging, so s is the staged value before
+                            // its rounding to bf16
+                            const float s = floor_f((c ? bf_hi(w) : bf_lo(w)) + st.bv[i], floor_);
                             const float inv = fast_rcp(acc[1][i][r][c]);
                             rd[c] = s * inv;
                             rt[c] = acc[0][i][r][c] * inv;
