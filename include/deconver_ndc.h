@@ -79,7 +79,8 @@ int ndc_check_geometry(const ndc_geom *g);
 int ndc_backward_uses_saved(const ndc_geom *g);
 
 /* Bytes of scratch `ndc_forward` needs for `g` (0 for most geometries; the bfloat16 3x3x3
- * kernels keep their packed filter tables there). */
+ * kernels keep their packed filter tables there).  No counterpart in the reference, whose
+ * wrappers allocate their own temporaries (kernels.py:728-788). */
 size_t ndc_forward_workspace_bytes(const ndc_geom *g);
 
 /*
@@ -92,11 +93,11 @@ size_t ndc_forward_workspace_bytes(const ndc_geom *g);
  *   t1            optional output K(s), same shape/dtype as x: pass it when a backward
  *                 call will follow (it is what the reference saves for backward), null
  *                 for inference
- *   s_over_den,   optional outputs s/(A(t1)+eps) and (A(x)+eps)/(A(t1)+eps), same shape/dtype
- *   ratio         as out; both or neither.  Handing them to ndc_backward lets it skip
- *                 re-gathering A(x) and A(t1): more memory kept between the two calls
- *                 (two tensors of the size of out) for fewer multiplications and no second read of z in pass 1.  The
- *                 reference has no counterpart (it re-gathers, kernels.py:791-838).
+ *   s_over_den,   optional outputs s/(A(t1)+eps) and (A(x)+eps)/(A(t1)+eps), same
+ *   ratio         shape/dtype as out; both or neither.  Handing them to ndc_backward lets it
+ *                 skip re-gathering A(x) and A(t1): more memory kept between the two calls
+ *                 (two tensors of the size of out) for fewer multiplications.  The
+ *                 reference has no counterpart (it re-gathers, kernels.py:806-809).
  *   workspace     >= ndc_forward_workspace_bytes(g) bytes, 256-byte aligned (may be null
  *                 when that is 0)
  */
