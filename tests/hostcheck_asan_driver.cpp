@@ -71,6 +71,8 @@ int main()
 {
     const Case cases[] = {
         {2, 3, 1, 4, 5, 9, 8, 3, 3, 3, NDC_F32, NDC_PATH_FUSED},
+        {1, 1, 1, 4, 3, 16, 64, 3, 3, 3, NDC_BF16, NDC_PATH_FUSED},   // workgroups of four full wavefronts
+        {1, 2, 1, 4, 2, 32, 32, 3, 3, 3, NDC_BF16, NDC_PATH_FUSED},
         {1, 2, 1, 4, 3, 7, 13, 3, 3, 3, NDC_BF16, NDC_PATH_FUSED},
         {1, 2, 1, 4, 6, 3, 70, 3, 3, 3, NDC_F32, NDC_PATH_FUSED},
         {1, 2, 1, 4, 5, 9, 8, 3, 3, 3, NDC_BF16, NDC_PATH_FUSED},

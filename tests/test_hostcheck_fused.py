@@ -131,7 +131,17 @@ def test_fused_bf16_storage(geom):
     assert host_faults(lib)[0] == 0
 
 
-@pytest.mark.parametrize("geom", FUSED_GEOMS[:3] + FUSED_GEOMS[5:6] + FUSED_GEOMS[7:9] + FUSED_GEOMS[10:11])
+# workgroups of four full wavefronts (the shape of the large 3-D configurations)
+FULL_WG_GEOMS = [
+    (1, 4, (3, 3, 3), (3, 16, 64), 1),    # 32 lanes per row, 8 strips
+    (2, 4, (3, 3, 3), (2, 32, 32), 1),    # 16 lanes per row, 16 strips
+    (1, 4, (3, 3, 3), (4, 9, 128), 2),    # 64 lanes per row, 4 strips, ragged band
+    (1, 4, (3, 3, 3), (5, 40, 64), 1),    # several row bands
+]
+
+
+@pytest.mark.parametrize("geom", FUSED_GEOMS[:3] + FUSED_GEOMS[5:6] + FUSED_GEOMS[7:9] + FUSED_GEOMS[10:11]
+                         + FULL_WG_GEOMS)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("relu", [True, False])
 def test_fused_saved_denominator_and_ratio(geom, dtype, relu):
