@@ -4,6 +4,8 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bf16|fp32] [--no-cpu]
     python bench.py --workload sweep                                      (config 5, forward only)
     python bench.py --workload accuracy                                   (float32 error table)
+    python bench.py --workload grid                                       (ratio x groups x kernel grid)
+    python bench.py --workload valu                                       (instruction-issue ceiling probe)
     python bench.py --workload train3d|model2d [--ndc hip|pytorch|both]   (model level, below)
 
 One step = one forward + one backward (input-, source-, filter- and bias-gradient) of the
@@ -180,14 +182,27 @@ ACCURACY_CASES = [   # the layer geometries of the reference's accuracy report (
 ]
 
 
+def _rel_err(a, ref) -> float:
+    """max|a - ref| / max|ref| in float64."""
+    a, ref = a.detach().double().cpu(), ref.detach().double().cpu()
+    return float((a - ref).abs().max() / ref.abs().max().clamp_min(1e-30))
+
+
+def _layer_outputs(layer, x, g):
+    """Forward + backward of a Deconv layer: [y, dx, dW, db, dh0]."""
+    y = layer(x)
+    y.backward(g)
+    p = layer.init
+    return [y.detach(), x.grad, p.linear.linear.weight.grad, p.linear.linear.bias.grad, p.h0.grad]
+
+
 def accuracy_workload(args) -> int:
     """Float32 accuracy of the whole layer (projection + update, all gradients) on the HIP
-    route and on the layer's PyTorch route, both against the oracle evaluated in float64 on
-    the CPU from the same parameters; `max|d| / max|ref|` per case, worst tensor."""
+    route and on the layer's PyTorch route, both against the layer's PyTorch route evaluated
+    in float64 on the CPU from the same parameters; `max|d| / max|ref|` per case, worst tensor."""
     import torch
 
     import deconver_amd as dc
-    from oracle import ndc_oracle as O
 
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
@@ -204,14 +219,9 @@ def accuracy_workload(args) -> int:
         state = base.state_dict()
         x0 = torch.rand(2, kw["channels"], *spatial)
         g0 = torch.randn(2, base.groups * base.source_channels, *spatial)
-        oracle = O.OracleNDC(kw["channels"], kw["kernel_size"], ratio=kw["ratio"], groups=kw["groups"])
-        ref_p = [state["init.linear.linear.weight"].double().squeeze(-1).requires_grad_(True),
-                 state["init.linear.linear.bias"].double().requires_grad_(True),
-                 state["init.h0"].double().requires_grad_(True)]
-        xr = x0.double().requires_grad_(True)
-        yr = oracle.forward(xr, *ref_p)
-        yr.backward(g0.double())
-        ref = [yr.detach(), xr.grad, ref_p[0].grad.unsqueeze(-1), ref_p[1].grad, ref_p[2].grad]
+        truth = dc.Deconv(**kw, dilation=1)   # a convolution keyword selects the PyTorch route
+        truth.load_state_dict(state)
+        ref = _layer_outputs(truth.double(), x0.double().requires_grad_(True), g0.double())
         errs = {}
         for route, extra in (("hip", {}), ("pytorch", {"dilation": 1})):
             layer = dc.Deconv(**kw, **extra)
@@ -220,21 +230,167 @@ def accuracy_workload(args) -> int:
             x = x0.to(dev).requires_grad_(True)
             on_hip = layer.fast_path_applicable(x)
             assert on_hip == (route == "hip")
-            y = layer(x)
-            y.backward(g0.to(dev))
-            got = [y.detach(), x.grad, layer.init.linear.linear.weight.grad,
-                   layer.init.linear.linear.bias.grad, layer.init.h0.grad]
-            e = [O.rel_err(a.cpu(), r) for a, r in zip(got, ref)]
+            e = [_rel_err(a, r) for a, r in zip(_layer_outputs(layer, x, g0.to(dev)), ref)]
             errs[route] = {"forward": e[0], "worst_gradient": max(e[1:])}
         rows.append({"case": name, "spatial": list(spatial), **errs})
     worst = max(r["hip"]["worst_gradient"] for r in rows)
     print(json.dumps({
-        "metric": "float32 layer accuracy vs float64 oracle (worst gradient, max|d|/max|ref|)",
+        "metric": "float32 layer accuracy vs float64 (worst gradient, max|d|/max|ref|)",
         "value": worst, "unit": "relative error", "n_gpus": 1, "steps": 1, "warmup": 0,
         "ms_per_step": None, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "accuracy report over the reference's layer geometries, batch 2"},
         "cases": rows, "roofline": None, "cpu_baseline": None}))
+    return 0
+
+
+GRID_RATIOS = (1, 2, 4)
+GRID_GROUPS = (1, 2, 4, 8, -1)
+GRID_KERNELS = ((3, 3, 3), (5, 5, 5))
+
+
+def grid_workload(args) -> int:
+    """Correctness and efficiency of the layer over ratio x groups x kernel size, float32,
+    the grid of the reference's configuration sweep (benchmarks/sweep_configs.py:36-38,
+    16 channels, 24^3, batch 2): per configuration the route taken, the error of the HIP
+    route against the layer's PyTorch route on the same GPU, and PyTorch-route / HIP-route
+    ratios of forward, backward and forward+backward time and of peak memory.  `value` is
+    the geometric mean of the forward+backward speed-ups; `slower` lists configurations
+    where the default route loses more than 3 % in time or memory."""
+    import statistics
+
+    import torch
+
+    import deconver_amd as dc
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    dev = torch.device("cuda:0")
+    C, n, B = 16, 24, 2
+
+    def timed(fn):
+        for _ in range(args.warmup):
+            fn()
+        samples = []
+        for _ in range(args.steps):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            fn()
+            torch.cuda.synchronize()
+            samples.append((time.perf_counter() - t0) * 1e3)
+        return statistics.median(samples)
+
+    def measure(layer, x, g):
+        def reset():
+            layer.zero_grad(set_to_none=True)
+            x.grad = None
+
+        def fwd():
+            with torch.no_grad():
+                layer(x)
+
+        def fwd_bwd():
+            reset()
+            layer(x).backward(g)
+
+        t_f = timed(fwd)
+        t_fb = timed(fwd_bwd)
+        reset()
+        torch.cuda.synchronize()
+        torch.cuda.reset_peak_memory_stats()
+        fwd_bwd()
+        torch.cuda.synchronize()
+        mem = torch.cuda.max_memory_allocated() / 2 ** 20
+        reset()
+        return {"fwd_ms": t_f, "bwd_ms": max(t_fb - t_f, 0.0), "fwd_bwd_ms": t_fb, "peak_MiB": mem}
+
+    rows = []
+    for ratio in GRID_RATIOS:
+        for groups in GRID_GROUPS:
+            for kernel in GRID_KERNELS:
+                kw = dict(channels=C, ratio=ratio, groups=groups, kernel_size=kernel, num_iters=1)
+                torch.manual_seed(0)
+                general = dc.Deconv(**kw, dilation=1).to(dev)
+                with torch.no_grad():   # keeps the source away from zero (1/eps ratios)
+                    general.init.linear.linear.bias.add_(1.0)
+                default = dc.Deconv(**kw).to(dev)
+                default.load_state_dict(general.state_dict())
+                torch.manual_seed(1)
+                x0 = torch.rand(B, C, n, n, n, device=dev)
+                route = "hip" if default.fast_path_applicable(x0) else "general"
+                torch.manual_seed(2)
+                g = torch.randn(B, default.groups * default.source_channels, n, n, n, device=dev)
+                ref = _layer_outputs(general, x0.clone().requires_grad_(True), g)
+                got = _layer_outputs(default, x0.clone().requires_grad_(True), g)
+                e = [_rel_err(a, r) for a, r in zip(got, ref)]
+                x = x0.clone().requires_grad_(True)
+                pg, pd = measure(general, x, g), measure(default, x, g)
+                rows.append({"ratio": ratio, "groups": groups, "kernel": list(kernel),
+                             "m": default.filter_channels, "sc": default.source_channels,
+                             "route": route, "fwd_err": e[0], "grad_err": max(e[1:]),
+                             "pytorch_route": pg, "default_route": pd,
+                             "speedup": {k: pg[k] / pd[k] if pd[k] > 0 else None
+                                         for k in ("fwd_ms", "bwd_ms", "fwd_bwd_ms")},
+                             "memory_ratio": pd["peak_MiB"] / pg["peak_MiB"]})
+                del general, default, x, x0, g, ref, got
+                torch.cuda.empty_cache()
+    slower = [f"ratio={r['ratio']} groups={r['groups']} k={tuple(r['kernel'])} [{r['route']}]"
+              for r in rows if r["speedup"]["fwd_bwd_ms"] < 0.97 or r["memory_ratio"] > 1.03]
+    gmean = math.exp(sum(math.log(r["speedup"]["fwd_bwd_ms"]) for r in rows) / len(rows))
+    print(json.dumps({
+        "metric": "Deconv layer fwd+bwd speed-up over its PyTorch route (geometric mean over the grid)",
+        "value": gmean, "unit": "x", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": sum(r["default_route"]["fwd_bwd_ms"] for r in rows),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": f"configuration grid: ratio x groups x kernel, {C} channels, {n}^3, batch {B}"},
+        "worst_fwd_err": max(r["fwd_err"] for r in rows),
+        "worst_grad_err": max(r["grad_err"] for r in rows),
+        "slower": slower, "rows": rows, "roofline": None, "cpu_baseline": None}))
+    return 0
+
+
+DOT2_PER_CHANNEL_VOXEL = {"forward": 205, "backward_pass1": 216, "backward_pass2": 126}
+
+
+def valu_workload(args) -> int:
+    """Instruction-issue probe (deconver_amd/csrc/valu_probe.hip, built by
+    `python -m deconver_amd.build --probe`): clocks per wavefront instruction per SIMD for the
+    multiply-accumulate forms, and from the v_dot2c_f32_bf16 figure the least time the bf16
+    kernels' multiply-accumulates alone take on config 3.  `value` is that vector ceiling in
+    T multiply-accumulates per second."""
+    import subprocess
+
+    exe = os.path.join(ROOT, "deconver_amd", "valu_probe")
+    if not os.path.exists(exe):
+        print("bench.py --workload valu: deconver_amd/valu_probe is not built "
+              "(python -m deconver_amd.build --probe)", file=sys.stderr)
+        return 2
+    proc = subprocess.run([exe], stdout=subprocess.PIPE, text=True, timeout=300)
+    if proc.returncode != 0:
+        print("valu_probe failed", file=sys.stderr)
+        return 2
+    probe = json.loads(proc.stdout)
+    clk = {(r["op"], r["wavefronts_per_simd"]): r["clocks_per_instruction"] for r in probe["rows"]}
+    dot2 = clk[("v_dot2c_f32_bf16 (scalar multiplicand)", 4)]
+    lanes = probe["compute_units"] * 4 * 64
+    hz = probe["clock_GHz"] * 1e9
+    ceiling = lanes * 2 / dot2 * hz   # two multiply-accumulates per lane per instruction
+    U = 2 * 128 * 64 ** 3
+    least_ms = {k: U * n / lanes * dot2 / hz * 1e3 for k, n in DOT2_PER_CHANNEL_VOXEL.items()}
+    print(json.dumps({
+        "metric": "vector multiply-accumulate ceiling (v_dot2c_f32_bf16 issue rate)",
+        "value": ceiling / 1e12, "unit": "TMAC/s", "n_gpus": 1, "steps": 1, "warmup": 0,
+        "ms_per_step": None, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "instruction-issue probe, 256 threads per workgroup, registers only"},
+        "clocks_per_dot2c": dot2,
+        "fmac_scalar_operand_TMACs": lanes / clk[("v_fmac_f32 (scalar multiplicand)", 4)] * hz / 1e12,
+        "fmac_vector_operands_TMACs": lanes / clk[("v_fmac_f32 (vector operands)", 4)] * hz / 1e12,
+        "config3_dot2c_per_channel_voxel": DOT2_PER_CHANNEL_VOXEL,
+        "config3_least_ms_for_dot2c_alone": least_ms,
+        "probe": probe, "roofline": None, "cpu_baseline": None}))
     return 0
 
 
@@ -345,7 +501,7 @@ def main() -> int:
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
-    ap.add_argument("--workload", choices=("ndc", "sweep", "accuracy", "train3d", "model2d"),
+    ap.add_argument("--workload", choices=("ndc", "sweep", "accuracy", "grid", "valu", "train3d", "model2d"),
                     default="ndc",
                     help="ndc: the headline update node (default); the others are model level")
     ap.add_argument("--ndc", choices=("hip", "pytorch", "both"), default="hip",
@@ -360,6 +516,10 @@ def main() -> int:
         return sweep_workload(args)
     if args.workload == "accuracy":
         return accuracy_workload(args)
+    if args.workload == "grid":
+        return grid_workload(args)
+    if args.workload == "valu":
+        return valu_workload(args)
     if args.workload != "ndc":
         return model_workload(args)
 

@@ -90,6 +90,12 @@ def test_route_choice():
             return super().update_s(x, s, h)
 
     assert not Custom(**base).fast_path_applicable()
+    # dense geometries (many filter x source channels per group) go to the library convolutions
+    assert dc.Deconv(channels=16, ratio=4, groups=-1, kernel_size=(5, 5, 5)).fast_path_applicable()
+    assert dc.Deconv(channels=16, ratio=4, groups=1, kernel_size=(3, 3, 3)).fast_path_applicable()
+    assert not dc.Deconv(channels=16, ratio=2, groups=1, kernel_size=(5, 5, 5)).fast_path_applicable()
+    assert not dc.Deconv(channels=16, ratio=4, groups=2, kernel_size=(5, 5, 5)).fast_path_applicable()
+    assert not dc.Deconv(channels=16, ratio=1, groups=1, kernel_size=(5, 5, 5)).fast_path_applicable()
     layer = dc.Deconv(**base)
     assert not layer.fast_path_applicable(torch.rand(1, 8, 4, 4, 4))        # CPU tensor
     assert not layer.fast_path_applicable(torch.rand(1, 8, 4, 4, 4).double())
