@@ -216,6 +216,23 @@ def test_general_route_on_gpu_for_unsupported_regimes():
     assert O.rel_err(layer(x).cpu(), cpu(x.cpu())) < 1e-4
 
 
+def test_dense_geometries_choose_the_faster_route():
+    """Many source channels per group: HIP route when a backward may follow, library
+    convolutions for forward-only calls; the two agree.  Very dense filters never take the
+    HIP route."""
+    kwargs = dict(channels=16, ratio=4, groups=4, kernel_size=(3, 3, 3))   # m = 4, sc = 16
+    layer = _layer(kwargs)
+    x = torch.rand(2, 16, 6, 7, 8, device="cuda")
+    assert layer.fast_path_applicable(x)
+    y_hip = layer(x)
+    with torch.no_grad():
+        assert not layer.fast_path_applicable(x)
+        y_general = layer(x)
+    assert O.rel_err(y_hip.detach().cpu(), y_general.cpu()) < 1e-5
+    dense = _layer(dict(channels=16, ratio=4, groups=1, kernel_size=(5, 5, 5)))
+    assert not dense.fast_path_applicable(x)
+
+
 def test_config1_single_layer_2d_sum_of_squares():
     """Batch 1, 32 channels, 64x64, depthwise, ratio 4, 5x5, softplus-positive kernel."""
     torch.manual_seed(0)
