@@ -300,15 +300,14 @@ template <int RH_> struct FwdKernelB {
                 const int cb = PL + st.ln.c0 - PW;
                 if (k < D) {
                     const int sb = off_s + wrap(k % NS, NS) * 2 * RS * P + cb;
-                    float wp[KT], wn[KT];
-                    load_taps<KT>(tab, wp);
                     NDC_ROLLED
-                    for (int pr = 0; pr < 2; ++pr) {
-                        load_taps<KT>(tab + uniform_int((pr + 1) & 1) * KT, wn);
+                    for (int prr = 0; prr < 2; ++prr) {
+                        const int pr = uniform_int(prr);
+                        float wp[KT];
+                        load_taps<KT>(tab + pr * KT, wp);
                         const int b0 = sb + pr * RS * P;
                         k_rows_d2<RH, RW, RHK>(ex, b0 + (PH + st.ln.strip * RH) * P, P, wp, st.t1acc, 0);
                         if (extra) k_rows_d2<1, RW, RHK>(ex, b0 + jx * P, P, wp, st.t1acc, RH);
-                        copy_taps<KT>(wn, wp);
                     }
                 }
                 // t1 plane k - 1 is complete: word (t1[k-2], t1[k-1]) goes to pair slot (k - 2) % 2
@@ -699,14 +698,13 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
                 prefetch_g(st, k);
                 if (live1) {
                     const int gb_ = off_g + (st.ln.strip * RH) * P + PL + st.ln.c0 - PW;
-                    float wp[KT], wn[KT];
-                    load_taps<KT>(tab, wp);
                     NDC_ROLLED
-                    for (int pr = 0; pr < 2; ++pr) {
-                        load_taps<KT>(tab + uniform_int((pr + 1) & 1) * KT, wn);
+                    for (int prr = 0; prr < 2; ++prr) {
+                        const int pr = uniform_int(prr);
+                        float wp[KT];
+                        load_taps<KT>(tab + pr * KT, wp);
                         k_rows_d2<RH, RW, RH>(ex, gb_ + pr * RG * P, P, wp, st.accx, 0);
                         k_rows_d2<RH, RW, RH>(ex, gb_ + (2 + pr) * RG * P, P, wp, st.acct, 0);
-                        copy_taps<KT>(wn, wp);
                     }
                 }
                 const int pf = k - 2;
