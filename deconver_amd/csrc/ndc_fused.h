@@ -259,8 +259,9 @@ NDC_D void a_plane(Exec &ex, const int (&base)[NTEN], int P, const float (&wt)[S
     }
 }
 
-// Filter slices, fetched one loop iteration ahead so that the scalar loads of the next slice
-// overlap the multiply-adds of the current one.
+// Filter slices, fetched into scalar registers at the top of each tap-loop iteration (keeping
+// the next slice in flight as well costs more in scalar-register spills and copies than the
+// load latency it hides).
 template <int N> NDC_D void load_taps(UniformF src, float (&dst)[N])
 {
     NDC_UNROLL
@@ -273,12 +274,6 @@ template <int SC, int KT, int N> NDC_D void load_plane_taps(UniformF src, float 
     for (int i = 0; i < SC; ++i)
         NDC_UNROLL
         for (int a = 0; a < N; ++a) dst[i][a] = src[i * KT + a];
-}
-
-template <int N> NDC_D void copy_taps(const float (&src)[N], float (&dst)[N])
-{
-    NDC_UNROLL
-    for (int a = 0; a < N; ++a) dst[a] = src[a];
 }
 
 // thread coordinates shared by the three kernels
@@ -474,16 +469,15 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                 const int jx = halo_row(st.ln.strip, PH, TH);
                 const int cb = PL + st.ln.c0 - PW;
                 if (k < D) {
-                    float wi[KT], wn[KT];
-                    load_taps<KT>(hw, wi);
                     NDC_ROLLED
-                    for (int i = 0; i < SC; ++i) {
-                        load_taps<KT>(hw + (i + 1 < SC ? i + 1 : 0) * KT, wn);
+                    for (int ii = 0; ii < SC; ++ii) {
+                        const int i = uniform_int(ii);
+                        float wi[KT];
+                        load_taps<KT>(hw + i * KT, wi);
                         const int sb = off_s + i * RS * P + cb;
                         k_rows<KD, KH, KW, RH, RW, RHK>(ex, sb + (PH + st.ln.strip * RH) * P, P, wi,
                                                         st.t1acc, 0);
                         if (extra) k_rows<KD, KH, KW, 1, RW, RHK>(ex, sb + jx * P, P, wi, st.t1acc, RH);
-                        copy_taps<KT>(wn, wi);
                     }
                 }
                 // plane k - PD of t1 is complete: publish it (zero outside the volume)
@@ -545,18 +539,16 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                         for (int r = 0; r < RH; ++r)
                             NDC_UNROLL
                             for (int c = 0; c < RW; ++c) acc[a][i][r][c] = 0.f;
-                float wt[SC][KH * KW], wn[SC][KH * KW];
-                load_plane_taps<SC, KT, KH * KW>(hw, wt);
                 NDC_ROLLED
-                for (int td = 0; td < KD; ++td) {
-                    load_plane_taps<SC, KT, KH * KW>(hw + (td + 1 < KD ? td + 1 : 0) * KH * KW, wn);
+                for (int tdd = 0; tdd < KD; ++tdd) {
+                    const int td = uniform_int(tdd);
+                    float wt[SC][KH * KW];
+                    load_plane_taps<SC, KT, KH * KW>(hw + td * KH * KW, wt);
                     const int pl = j0 + PD - td;
                     const int ob = (st.ln.strip * RH) * P + PL + st.ln.c0 - PW;
                     const int base[2] = {off_x + wrap(pl % XR, XR) * RX * P + ob,
                                          off_t + wrap(pl % KD, KD) * RX * P + ob};
                     a_plane<KH, KW, KT, SC, RH, RW, 2>(ex, base, P, wt, acc);
-                    NDC_UNROLL
-                    for (int i = 0; i < SC; ++i) copy_taps<KH * KW>(wn[i], wt[i]);
                 }
                 T *ok_ = og + (long long)j0 * plane;
                 T *dk_ = p.s_over_den ? p.s_over_den + (og - p.out) + (long long)j0 * plane : nullptr;
@@ -731,17 +723,15 @@ struct Bwd1Kernel {
                         for (int r = 0; r < NR; ++r)
                             NDC_UNROLL
                             for (int c = 0; c < RW; ++c) acc[a][i][r][c] = 0.f;
-                float wt[SC][KH * KW], wn[SC][KH * KW];
-                load_plane_taps<SC, KT, KH * KW>(hw, wt);
                 NDC_ROLLED
-                for (int td = 0; td < KD; ++td) {
-                    load_plane_taps<SC, KT, KH * KW>(hw + (td + 1 < KD ? td + 1 : 0) * KH * KW, wn);
+                for (int tdd = 0; tdd < KD; ++tdd) {
+                    const int td = uniform_int(tdd);
+                    float wt[SC][KH * KW];
+                    load_plane_taps<SC, KT, KH * KW>(hw + td * KH * KW, wt);
                     const int slot = wrap((j1 + PD - td) % XR, XR);
                     const int ob = (slot * RX + j) * P + PL + st.ln.c0 - PW;
                     const int base[2] = {off_x + ob, off_t + ob};
                     a_plane<KH, KW, KT, SC, NR, RW, 2>(ex, base, P, wt, acc);
-                    NDC_UNROLL
-                    for (int i = 0; i < SC; ++i) copy_taps<KH * KW>(wn[i], wt[i]);
                 }
             }
             NDC_UNROLL
@@ -857,15 +847,14 @@ struct Bwd1Kernel {
                 if (!st.ln.active) return;
                 load_plane(st, k + 1);
                 if (live1) {
-                    float wi[KT], wn[KT];
-                    load_taps<KT>(hw, wi);
                     NDC_ROLLED
-                    for (int i = 0; i < SC; ++i) {
-                        load_taps<KT>(hw + (i + 1 < SC ? i + 1 : 0) * KT, wn);
+                    for (int ii = 0; ii < SC; ++ii) {
+                        const int i = uniform_int(ii);
+                        float wi[KT];
+                        load_taps<KT>(hw + i * KT, wi);
                         const int gb_ = off_g + (st.ln.strip * RH) * P + PL + st.ln.c0 - PW;
                         k_rows<KD, KH, KW, RH, RW, RH>(ex, gb_ + i * RG * P, P, wi, st.accx, 0);
                         k_rows<KD, KH, KW, RH, RW, RH>(ex, gb_ + (SC + i) * RG * P, P, wi, st.acct, 0);
-                        copy_taps<KT>(wn, wi);
                     }
                 }
                 const int pf = k - 2 * PD;
@@ -1070,11 +1059,11 @@ struct Bwd2Kernel {
                         for (int r = 0; r < RH; ++r)
                             NDC_UNROLL
                             for (int c = 0; c < RW; ++c) acc[a][i][r][c] = 0.f;
-                float wt[SC][KH * KW], wn[SC][KH * KW];
-                load_plane_taps<SC, KT, KH * KW>(hw, wt);
                 NDC_ROLLED
-                for (int td = 0; td < KD; ++td) {
-                    load_plane_taps<SC, KT, KH * KW>(hw + (td + 1 < KD ? td + 1 : 0) * KH * KW, wn);
+                for (int tdd = 0; tdd < KD; ++tdd) {
+                    const int td = uniform_int(tdd);
+                    float wt[SC][KH * KW];
+                    load_plane_taps<SC, KT, KH * KW>(hw + td * KH * KW, wt);
                     const int slot = wrap((j0 + PD - td) % XR, XR);
                     const int ob = (slot * RX + st.ln.strip * RH) * P + PL + st.ln.c0 - PW;
                     int base[NA];
@@ -1084,8 +1073,6 @@ struct Bwd2Kernel {
                         base[NA > 1 ? 1 : 0] = off_t + ob;
                     }
                     a_plane<KH, KW, KT, SC, RH, RW, NA>(ex, base, P, wt, acc);
-                    NDC_UNROLL
-                    for (int i = 0; i < SC; ++i) copy_taps<KH * KW>(wn[i], wt[i]);
                 }
                 if (need_gh) {
                     // K-side filter-gradient term: re-read the gt1 window
