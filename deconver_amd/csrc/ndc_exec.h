@@ -208,10 +208,13 @@ NDC_HD uint32_t buf_ld(const BufRef &b, unsigned lane_off, unsigned uniform_off)
 #endif
 }
 
+// STREAM: the word is not read again soon (a result tensor): stored with the non-temporal
+// hint, so that it does not push re-used lines out of the L2.
+template <bool STREAM = false>
 NDC_HD void buf_st(const BufRef &b, unsigned lane_off, unsigned uniform_off, uint32_t w)
 {
 #if NDC_DEVICE_BUILD && defined(__HIP_DEVICE_COMPILE__)
-    __builtin_amdgcn_raw_buffer_store_b32(w, b.r, (int)lane_off, (int)uniform_off, 0);
+    __builtin_amdgcn_raw_buffer_store_b32(w, b.r, (int)lane_off, (int)uniform_off, STREAM ? 2 : 0);
 #elif NDC_DEVICE_BUILD
     (void)b; (void)lane_off; (void)uniform_off; (void)w;
 #else

@@ -390,10 +390,10 @@ template <int RH_> struct FwdKernelB {
                             rt[c] = acc[0][i][r][c] * inv;
                             v[c] = s * rt[c];
                         }
-                        buf_st(ob_, st.ooff[r], oj + i * cplane2, pack_bf16x2(v[0], v[1]));
+                        buf_st<true>(ob_, st.ooff[r], oj + i * cplane2, pack_bf16x2(v[0], v[1]));
                         if (have_saved) {
-                            buf_st(db_, st.ooff[r], oj + i * cplane2, pack_bf16x2(rd[0], rd[1]));
-                            buf_st(rb_, st.ooff[r], oj + i * cplane2, pack_bf16x2(rt[0], rt[1]));
+                            buf_st<true>(db_, st.ooff[r], oj + i * cplane2, pack_bf16x2(rd[0], rd[1]));
+                            buf_st<true>(rb_, st.ooff[r], oj + i * cplane2, pack_bf16x2(rt[0], rt[1]));
                         }
                     }
                 }
@@ -711,7 +711,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
                 NDC_UNROLL
                 for (int r = 0; r < RH; ++r) {
                     if (pf >= 0 && ((st.ook >> r) & 1u)) {
-                        if (have_gx) buf_st(gxb_, st.ooff[r], (unsigned)pf * plane2,
+                        if (have_gx) buf_st<true>(gxb_, st.ooff[r], (unsigned)pf * plane2,
                                             pack_bf16x2(st.accx[0][r][0], st.accx[0][r][1]));
                         buf_st(gtb_, st.ooff[r], (unsigned)pf * plane2,
                                pack_bf16x2(st.acct[0][r][0], st.acct[0][r][1]));
@@ -966,7 +966,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
                                 st.gbacc[i] += gzv;
                                 v[c] = gzv;
                             }
-                            if (have_gz && ok) buf_st(gzb_, st.ooff[r], jo + i * cplane2, pack_bf16x2(v[0], v[1]));
+                            if (have_gz && ok) buf_st<true>(gzb_, st.ooff[r], jo + i * cplane2, pack_bf16x2(v[0], v[1]));
                         }
                     }
                 }
