@@ -187,10 +187,12 @@ NDC_HD BufRef make_buf(const void *p, size_t bytes)
     return b;
 }
 
+// STREAM: the word is read once (non-temporal hint, as for buf_st).
+template <bool STREAM = false>
 NDC_HD uint32_t buf_ld(const BufRef &b, unsigned lane_off, unsigned uniform_off)
 {
 #if NDC_DEVICE_BUILD && defined(__HIP_DEVICE_COMPILE__)
-    return __builtin_amdgcn_raw_buffer_load_b32(b.r, (int)lane_off, (int)uniform_off, 0);
+    return __builtin_amdgcn_raw_buffer_load_b32(b.r, (int)lane_off, (int)uniform_off, STREAM ? 2 : 0);
 #elif NDC_DEVICE_BUILD
     (void)b; (void)lane_off; (void)uniform_off;
     return 0u;

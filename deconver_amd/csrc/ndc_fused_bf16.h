@@ -519,9 +519,9 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
                 const unsigned o = r < RH ? st.ooff[r < RH ? r : 0] : st.hoff;
                 NDC_UNROLL
                 for (int i = 0; i < SC; ++i) {
-                    st.qg[i][r] = buf_ld(gb_, o, jo + i * cplane2);
-                    st.qd[i][r] = buf_ld(db_, o, jo + i * cplane2);
-                    st.qr[i][r] = buf_ld(rb_, o, jo + i * cplane2);
+                    st.qg[i][r] = buf_ld<true>(gb_, o, jo + i * cplane2);
+                    st.qd[i][r] = buf_ld<true>(db_, o, jo + i * cplane2);
+                    st.qr[i][r] = buf_ld<true>(rb_, o, jo + i * cplane2);
                 }
             }
         };
@@ -897,8 +897,8 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
                             gw[i][r] = st.qg[i][r];
                             rw[i][r] = st.qr[i][r];
                             st.qz[i][r] = buf_ld(zb_, st.ooff[r], jn + i * cplane2);
-                            st.qg[i][r] = buf_ld(gb_, st.ooff[r], jn + i * cplane2);
-                            st.qr[i][r] = buf_ld(rb_, st.ooff[r], jn + i * cplane2);
+                            st.qg[i][r] = buf_ld<true>(gb_, st.ooff[r], jn + i * cplane2);
+                            st.qr[i][r] = buf_ld<true>(rb_, st.ooff[r], jn + i * cplane2);
                         }
                 }
                 if (j0 < 0) return;
