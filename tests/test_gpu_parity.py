@@ -130,3 +130,76 @@ def test_fused_matches_direct_at_size():
     for name, a, b in zip(("out", "t1", "gx", "gz", "gh", "gb"), res[_lib.PATH_FUSED],
                           res[_lib.PATH_DIRECT]):
         assert O.rel_err(a, b) < 1e-4, name
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_full_size_scaling_laws(dtype):
+    """Config 3 at full size (batch 2, 128 channels, 64^3), where no oracle run is affordable:
+    what the update's algebra fixes exactly.  Doubling x doubles A(x) exactly in binary
+    floating point, so out(2x) = 2 out(x) up to the eps term; halving the filter halves K and
+    A, so out(h/2) = 2 out(h); the backward is linear in gout, so doubling gout doubles every
+    gradient exactly (gh and gb are summed in a fixed order)."""
+    C, sc, sp = 128, 4, (64, 64, 64)
+    gen = torch.Generator().manual_seed(0)
+    x = torch.randn(2, C, *sp, generator=gen).abs().to(dtype).cuda()
+    z = (torch.randn(2, C * sc, *sp, generator=gen) * 0.5).to(dtype).cuda()
+    h = torch.nn.functional.softplus(0.1 * torch.randn(C, sc, 3, 3, 3, generator=gen)).cuda()
+    bias = (0.1 * torch.randn(C * sc, generator=gen)).cuda()
+    gout = torch.randn(2, C * sc, *sp, generator=gen).to(dtype).cuda()
+    lib = _lib_gpu()
+    kw = dict(groups=C, m=1, sc=sc, eps=1e-16, relu_input=True, path=_lib.PATH_FUSED)
+
+    out, t1, saved = ops.update_forward(lib, x, z, h, bias, save_ratio=True, **kw)
+    out2 = ops.update_forward(lib, x * 2, z, h, bias, **kw)[0]
+    assert O.rel_err(out2.float(), out.float() * 2) < 1e-6
+    outh = ops.update_forward(lib, x, z, h * 0.5, bias, **kw)[0]
+    assert O.rel_err(outh.float(), out.float() * 2) < 1e-6
+    del out2, outh
+
+    g1 = ops.update_backward(lib, x, z, t1, h, bias, gout, saved=saved, **kw)
+    g2 = ops.update_backward(lib, x, z, t1, h, bias, gout * 2, saved=saved, **kw)
+    torch.cuda.synchronize()
+    for name, a, b in zip(("gx", "gz", "gh", "gb"), g1, g2):
+        assert torch.equal(b.float(), a.float() * 2), name
+    # and the saved-tensor backward agrees with the re-gathering one
+    g3 = ops.update_backward(lib, x, z, t1, h, bias, gout, **kw)
+    tol = TOL[dtype]
+    for name, a, b in zip(("gx", "gz", "gh", "gb"), g1, g3):
+        assert O.rel_err(a.float(), b.float()) < tol, name
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_graph_capture_replays_match_eager(dtype):
+    """The library neither allocates nor synchronises, so a forward + backward pair can be
+    captured in a HIP graph; every replay (with eager work and synchronisations between
+    them) must reproduce the eager results bit for bit."""
+    C, sc, sp = 16, 4, (12, 16, 32)
+    x, z, h, bias, gout = make_case(C, C, sc, (3, 3, 3), sp, B=2, dtype=dtype, bias_shift=0.3,
+                                    device="cuda")
+    lib = _lib_gpu()
+    kw = dict(groups=C, m=1, sc=sc, eps=1e-16, relu_input=True, path=_lib.PATH_FUSED)
+
+    def step():
+        out, t1, saved = ops.update_forward(lib, x, z, h, bias, save_ratio=True, **kw)
+        return (out,) + tuple(ops.update_backward(lib, x, z, t1, h, bias, gout, saved=saved, **kw))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()   # warm-up off the default stream, as graph capture asks
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = step()
+    gens = torch.Generator().manual_seed(7)
+    for replay in range(3):
+        x.copy_(torch.rand(x.shape, generator=gens).to(dtype))
+        gout.copy_(torch.randn(gout.shape, generator=gens).to(dtype))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in captured]
+        want = step()
+        torch.cuda.synchronize()
+        for name, a, b in zip(("out", "gx", "gz", "gh", "gb"), got, want):
+            assert torch.equal(a, b), f"replay {replay}: {name}"
