@@ -33,6 +33,9 @@ template <class State> struct DeviceExec {
     NDC_D void sync() { __syncthreads(); }
     NDC_D float ld(int i) const { return lds[i]; }
     NDC_D void st_(int i, float v) { lds[i] = v; }
+    // The instruction scheduler may not move anything across this point: used to keep the LDS
+    // reads of the next row ahead of the arithmetic on the current one.
+    NDC_D void fence() const { __builtin_amdgcn_sched_barrier(0); }
 
     // Sum N per-thread values over the workgroup: butterfly inside each wavefront, one LDS
     // row per wavefront, then thread i < N adds the rows in a fixed order and hands the sum
@@ -93,6 +96,7 @@ template <class State> struct HostExec {
         for (cur = 0; cur < nthreads; ++cur) f(states[cur], cur);
     }
     void sync() { ++epoch; }
+    void fence() const {}
 
     float ld(int i)
     {

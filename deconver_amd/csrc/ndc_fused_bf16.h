@@ -70,15 +70,35 @@ NDC_HD float bf_hi(uint32_t w) { return bits_to_float(w & 0xffff0000u); }
 
 // K-type pass over an NR x RW tile for ONE channel pair: words (s_2p, s_2p+1) staged at
 // `base` (first input row, first own column - 1); w = WK[p], 27 packed tap pairs.
-template <int NR, int RW, int STRIDE, class Exec>
+//
+// PIPE (here and below): the LDS words of a row are read one row ahead of the arithmetic
+// that uses them, and a scheduling fence keeps that order.  The backward kernels run two
+// wavefronts per SIMD, too few to hide the LDS latency otherwise (pass 1: 0.79 -> 0.75 ms);
+// the forward runs four and would lose one to the extra registers.
+template <int NR, int RW, int STRIDE, bool PIPE, class Exec>
 NDC_D void k_rows_d2(Exec &ex, int base, int P, const float (&w)[27], float (*acc)[STRIDE][RW],
                      int r_off)
 {
+    uint32_t vn[RW + 2];
+    if (PIPE) {
+        NDC_UNROLL
+        for (int u = 0; u < RW + 2; ++u) vn[u] = float_to_bits(ex.ld(base + u));
+    }
     NDC_UNROLL
     for (int q = 0; q < NR + 2; ++q) {
         uint32_t v[RW + 2];
-        NDC_UNROLL
-        for (int u = 0; u < RW + 2; ++u) v[u] = float_to_bits(ex.ld(base + q * P + u));
+        if (PIPE) {
+            NDC_UNROLL
+            for (int u = 0; u < RW + 2; ++u) v[u] = vn[u];
+            if (q + 1 < NR + 2) {
+                NDC_UNROLL
+                for (int u = 0; u < RW + 2; ++u) vn[u] = float_to_bits(ex.ld(base + (q + 1) * P + u));
+            }
+            ex.fence();
+        } else {
+            NDC_UNROLL
+            for (int u = 0; u < RW + 2; ++u) v[u] = float_to_bits(ex.ld(base + q * P + u));
+        }
         NDC_UNROLL
         for (int th = 0; th < 3; ++th) {
             const int rr = q - th;
@@ -97,17 +117,39 @@ NDC_D void k_rows_d2(Exec &ex, int base, int P, const float (&w)[27], float (*ac
 }
 
 // A-type pass over an NR x RW tile for one plane-pair slot of NTEN operands; wt = WA[s].
-template <int NR, int RW, int NTEN, class Exec>
+template <int NR, int RW, int NTEN, bool PIPE, class Exec>
 NDC_D void a_plane_d2(Exec &ex, const int (&base)[NTEN], int P, const float (&wt)[4][9],
                       float (&acc)[NTEN][4][NR][RW])
 {
-    NDC_UNROLL
-    for (int q = 0; q < NR + 2; ++q) {
-        uint32_t v[NTEN][RW + 2];
+    uint32_t vn[NTEN][RW + 2];
+    if (PIPE) {
         NDC_UNROLL
         for (int t = 0; t < NTEN; ++t)
             NDC_UNROLL
-            for (int u = 0; u < RW + 2; ++u) v[t][u] = float_to_bits(ex.ld(base[t] + q * P + u));
+            for (int u = 0; u < RW + 2; ++u) vn[t][u] = float_to_bits(ex.ld(base[t] + u));
+    }
+    NDC_UNROLL
+    for (int q = 0; q < NR + 2; ++q) {
+        uint32_t v[NTEN][RW + 2];
+        if (PIPE) {
+            NDC_UNROLL
+            for (int t = 0; t < NTEN; ++t)
+                NDC_UNROLL
+                for (int u = 0; u < RW + 2; ++u) v[t][u] = vn[t][u];
+            if (q + 1 < NR + 2) {
+                NDC_UNROLL
+                for (int t = 0; t < NTEN; ++t)
+                    NDC_UNROLL
+                    for (int u = 0; u < RW + 2; ++u)
+                        vn[t][u] = float_to_bits(ex.ld(base[t] + (q + 1) * P + u));
+            }
+            ex.fence();
+        } else {
+            NDC_UNROLL
+            for (int t = 0; t < NTEN; ++t)
+                NDC_UNROLL
+                for (int u = 0; u < RW + 2; ++u) v[t][u] = float_to_bits(ex.ld(base[t] + q * P + u));
+        }
         NDC_UNROLL
         for (int th = 0; th < 3; ++th) {
             const int rr = q - 2 + th;
@@ -124,6 +166,35 @@ NDC_D void a_plane_d2(Exec &ex, const int (&base)[NTEN], int P, const float (&wt
                             acc[t][i][rr][c] = dot2_bf16(v[t][c + 2 - tw], wv, acc[t][i][rr][c]);
                 }
         }
+    }
+}
+
+// NROWS rows of NW staged words each, row n at addr(n), handed to body(n, words) with the
+// reads running one row ahead (PIPE, see k_rows_d2).
+template <int NROWS, int NW, bool PIPE, class Exec, class Addr, class Body>
+NDC_D void stream_rows(Exec &ex, Addr addr, Body body)
+{
+    uint32_t vn[NW];
+    if (PIPE) {
+        NDC_UNROLL
+        for (int u = 0; u < NW; ++u) vn[u] = float_to_bits(ex.ld(addr(0) + u));
+    }
+    NDC_UNROLL
+    for (int n = 0; n < NROWS; ++n) {
+        uint32_t v[NW];
+        if (PIPE) {
+            NDC_UNROLL
+            for (int u = 0; u < NW; ++u) v[u] = vn[u];
+            if (n + 1 < NROWS) {
+                NDC_UNROLL
+                for (int u = 0; u < NW; ++u) vn[u] = float_to_bits(ex.ld(addr(n + 1) + u));
+            }
+            ex.fence();
+        } else {
+            NDC_UNROLL
+            for (int u = 0; u < NW; ++u) v[u] = float_to_bits(ex.ld(addr(n) + u));
+        }
+        body(n, v);
     }
 }
 
@@ -306,8 +377,8 @@ template <int RH_> struct FwdKernelB {
                         float wp[KT];
                         load_taps<KT>(tab + pr * KT, wp);
                         const int b0 = sb + pr * RS * P;
-                        k_rows_d2<RH, RW, RHK>(ex, b0 + (PH + st.ln.strip * RH) * P, P, wp, st.t1acc, 0);
-                        if (extra) k_rows_d2<1, RW, RHK>(ex, b0 + jx * P, P, wp, st.t1acc, RH);
+                        k_rows_d2<RH, RW, RHK, false>(ex, b0 + (PH + st.ln.strip * RH) * P, P, wp, st.t1acc, 0);
+                        if (extra) k_rows_d2<1, RW, RHK, false>(ex, b0 + jx * P, P, wp, st.t1acc, RH);
                     }
                 }
                 // t1 plane k - 1 is complete: word (t1[k-2], t1[k-1]) goes to pair slot (k - 2) % 2
@@ -370,7 +441,7 @@ template <int RH_> struct FwdKernelB {
                     const int ob = (st.ln.strip * RH) * P + PL + st.ln.c0 - PW;
                     const int base[2] = {off_x + wrap(m % NX, NX) * RX * P + ob,
                                          off_t + wrap(m % NTP, NTP) * RX * P + ob};
-                    a_plane_d2<RH, RW, 2>(ex, base, P, wt, acc);
+                    a_plane_d2<RH, RW, 2, false>(ex, base, P, wt, acc);
                 }
                 const unsigned oj = (unsigned)j0 * plane2;
                 NDC_UNROLL
@@ -569,7 +640,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
                     const int m = j1 - 1 + s;
                     const int ob = (wrap(m % NP, NP) * RX + j) * P + PL + st.ln.c0 - PW;
                     const int base[2] = {off_xp + ob, off_tp + ob};
-                    a_plane_d2<NR, RW, 2>(ex, base, P, wt, acc);
+                    a_plane_d2<NR, RW, 2, true>(ex, base, P, wt, acc);
                 }
             }
             NDC_UNROLL
@@ -658,31 +729,31 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
                     gn_gd_rows(st, j1, j, IntTag<RH>(), 0, gg2);
                     if (need_gh) {
                         // A-side filter-gradient terms: (gn_i, gd_i) . (x, t1)[neighbour]
-                        NDC_UNROLL
-                        for (int td = 0; td < KD; ++td) {
-                            const int ob = off_xt + (wrap((j1 + 1 - td) % NXT, NXT) * RX + j) * P + PL +
-                                           st.ln.c0 - PW;
-                            NDC_UNROLL
-                            for (int q = 0; q < RH + 2; ++q) {
-                                uint32_t v[RW + 2];
-                                NDC_UNROLL
-                                for (int u = 0; u < RW + 2; ++u) v[u] = float_to_bits(ex.ld(ob + q * P + u));
+                        const int cb = PL + st.ln.c0 - PW;
+                        stream_rows<KD * (RH + 2), RW + 2, true>(
+                            ex,
+                            [&](int n) NDC_LAMBDA {
+                                const int td = n / (RH + 2), q = n % (RH + 2);
+                                return off_xt + (wrap((j1 + 1 - td) % NXT, NXT) * RX + j + q) * P + cb;
+                            },
+                            [&](int n, const uint32_t (&v)[RW + 2]) NDC_LAMBDA {
+                                const int td = n / (RH + 2), q = n % (RH + 2);
                                 NDC_UNROLL
                                 for (int th = 0; th < KH; ++th) {
                                     const int rr = q - 2 + th;
-                                    if (rr < 0 || rr >= RH) continue;
-                                    NDC_UNROLL
-                                    for (int tw = 0; tw < KW; ++tw)
+                                    if (rr >= 0 && rr < RH) {
                                         NDC_UNROLL
-                                        for (int i = 0; i < SC; ++i)
+                                        for (int tw = 0; tw < KW; ++tw)
                                             NDC_UNROLL
-                                            for (int c = 0; c < RW; ++c)
-                                                st.gacc[i][(td * KH + th) * KW + tw] = dot2_bf16(
-                                                    v[c + 2 - tw], gg2[i][rr][c],
-                                                    st.gacc[i][(td * KH + th) * KW + tw]);
+                                            for (int i = 0; i < SC; ++i)
+                                                NDC_UNROLL
+                                                for (int c = 0; c < RW; ++c)
+                                                    st.gacc[i][(td * KH + th) * KW + tw] = dot2_bf16(
+                                                        v[c + 2 - tw], gg2[i][rr][c],
+                                                        st.gacc[i][(td * KH + th) * KW + tw]);
+                                    }
                                 }
-                            }
-                        }
+                            });
                     }
                 }
                 if (st.ln.strip < 2) {
@@ -703,8 +774,8 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
                         const int pr = uniform_int(prr);
                         float wp[KT];
                         load_taps<KT>(tab + pr * KT, wp);
-                        k_rows_d2<RH, RW, RH>(ex, gb_ + pr * RG * P, P, wp, st.accx, 0);
-                        k_rows_d2<RH, RW, RH>(ex, gb_ + (2 + pr) * RG * P, P, wp, st.acct, 0);
+                        k_rows_d2<RH, RW, RH, true>(ex, gb_ + pr * RG * P, P, wp, st.accx, 0);
+                        k_rows_d2<RH, RW, RH, true>(ex, gb_ + (2 + pr) * RG * P, P, wp, st.acct, 0);
                     }
                 }
                 const int pf = k - 2;
@@ -942,7 +1013,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
                             base[0] = off_xp + wrap(m % NP, NP) * RX * P + ob;
                             base[NA > 1 ? 1 : 0] = off_tp + wrap(m % NP, NP) * RX * P + ob;
                         }
-                        a_plane_d2<RH, RW, NA>(ex, base, P, wt, acc);
+                        a_plane_d2<RH, RW, NA, SAVED>(ex, base, P, wt, acc);
                     }
                     NDC_UNROLL
                     for (int r = 0; r < RH; ++r) {
@@ -980,31 +1051,31 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
                         for (int r = 0; r < RH; ++r)
                             NDC_UNROLL
                             for (int c = 0; c < RW; ++c) ss[i][r][c] = pack_bf16x2(st.sprev[i][r][c], sv[i][r][c]);
-                    NDC_UNROLL
-                    for (int td = 0; td < KD; ++td) {
-                        const int ob = off_gp + (wrap((j0 - td) % NG, NG) * RX + st.ln.strip * RH) * P + PL +
-                                       st.ln.c0 - PW;
-                        NDC_UNROLL
-                        for (int q = 0; q < RH + 2; ++q) {
-                            uint32_t v[RW + 2];
-                            NDC_UNROLL
-                            for (int u = 0; u < RW + 2; ++u) v[u] = float_to_bits(ex.ld(ob + q * P + u));
+                    const int cb = PL + st.ln.c0 - PW;
+                    stream_rows<KD * (RH + 2), RW + 2, SAVED>(
+                        ex,
+                        [&](int n) NDC_LAMBDA {
+                            const int td = n / (RH + 2), q = n % (RH + 2);
+                            return off_gp + (wrap((j0 - td) % NG, NG) * RX + st.ln.strip * RH + q) * P + cb;
+                        },
+                        [&](int n, const uint32_t (&v)[RW + 2]) NDC_LAMBDA {
+                            const int td = n / (RH + 2), q = n % (RH + 2);
                             NDC_UNROLL
                             for (int th = 0; th < KH; ++th) {
                                 const int rr = q - 2 + th;
-                                if (rr < 0 || rr >= RH) continue;
-                                NDC_UNROLL
-                                for (int tw = 0; tw < KW; ++tw)
+                                if (rr >= 0 && rr < RH) {
                                     NDC_UNROLL
-                                    for (int i = 0; i < SC; ++i)
+                                    for (int tw = 0; tw < KW; ++tw)
                                         NDC_UNROLL
-                                        for (int c = 0; c < RW; ++c)
-                                            st.gacc[i][(td * KH + th) * KW + tw] = dot2_bf16(
-                                                v[c + 2 - tw], ss[i][rr][c],
-                                                st.gacc[i][(td * KH + th) * KW + tw]);
+                                        for (int i = 0; i < SC; ++i)
+                                            NDC_UNROLL
+                                            for (int c = 0; c < RW; ++c)
+                                                st.gacc[i][(td * KH + th) * KW + tw] = dot2_bf16(
+                                                    v[c + 2 - tw], ss[i][rr][c],
+                                                    st.gacc[i][(td * KH + th) * KW + tw]);
+                                }
                             }
-                        }
-                    }
+                        });
                 }
                 NDC_UNROLL
                 for (int i = 0; i < SC; ++i)
