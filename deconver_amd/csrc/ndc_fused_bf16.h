@@ -70,6 +70,27 @@ NDC_HD float bf_hi(uint32_t w) { return bits_to_float(w & 0xffff0000u); }
 
 // K-type pass over an NR x RW tile for ONE channel pair: words (s_2p, s_2p+1) staged at
 // `base` (first input row, first own column - 1); w = WK[p], 27 packed tap pairs.
+template <int NR, int RW, int STRIDE>
+NDC_D void k_row_d2(int q, const uint32_t (&v)[RW + 2], const float (&w)[27],
+                    float (*acc)[STRIDE][RW], int r_off)
+{
+    NDC_UNROLL
+    for (int th = 0; th < 3; ++th) {
+        const int rr = q - th;
+        if (rr >= 0 && rr < NR) {
+            NDC_UNROLL
+            for (int tw = 0; tw < 3; ++tw)
+                NDC_UNROLL
+                for (int jd = 0; jd < 3; ++jd) {
+                    const uint32_t wv = float_to_bits(w[((2 - jd) * 3 + th) * 3 + tw]);
+                    NDC_UNROLL
+                    for (int c = 0; c < RW; ++c)
+                        acc[jd][r_off + rr][c] = dot2_bf16(v[c + tw], wv, acc[jd][r_off + rr][c]);
+                }
+        }
+    }
+}
+
 //
 // PIPE (here and below): the LDS words of a row are read one row ahead of the arithmetic
 // that uses them, and a scheduling fence keeps that order.  The backward kernels run two
@@ -99,20 +120,7 @@ NDC_D void k_rows_d2(Exec &ex, int base, int P, const float (&w)[27], float (*ac
             NDC_UNROLL
             for (int u = 0; u < RW + 2; ++u) v[u] = float_to_bits(ex.ld(base + q * P + u));
         }
-        NDC_UNROLL
-        for (int th = 0; th < 3; ++th) {
-            const int rr = q - th;
-            if (rr < 0 || rr >= NR) continue;
-            NDC_UNROLL
-            for (int tw = 0; tw < 3; ++tw)
-                NDC_UNROLL
-                for (int jd = 0; jd < 3; ++jd) {
-                    const uint32_t wv = float_to_bits(w[((2 - jd) * 3 + th) * 3 + tw]);
-                    NDC_UNROLL
-                    for (int c = 0; c < RW; ++c)
-                        acc[jd][r_off + rr][c] = dot2_bf16(v[c + tw], wv, acc[jd][r_off + rr][c]);
-                }
-        }
+        k_row_d2<NR, RW, STRIDE>(q, v, w, acc, r_off);
     }
 }
 
@@ -774,8 +782,18 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
                         const int pr = uniform_int(prr);
                         float wp[KT];
                         load_taps<KT>(tab + pr * KT, wp);
-                        k_rows_d2<RH, RW, RH, true>(ex, gb_ + pr * RG * P, P, wp, st.accx, 0);
-                        k_rows_d2<RH, RW, RH, true>(ex, gb_ + (2 + pr) * RG * P, P, wp, st.acct, 0);
+                        // gn rows of this channel pair feed gx, then its gd rows feed gt1
+                        stream_rows<2 * (RH + 2), RW + 2, true>(
+                            ex,
+                            [&](int n) NDC_LAMBDA {
+                                return gb_ + ((n / (RH + 2)) * 2 + pr) * RG * P + (n % (RH + 2)) * P;
+                            },
+                            [&](int n, const uint32_t (&v)[RW + 2]) NDC_LAMBDA {
+                                if (n < RH + 2)
+                                    k_row_d2<RH, RW, RH>(n, v, wp, st.accx, 0);
+                                else
+                                    k_row_d2<RH, RW, RH>(n - (RH + 2), v, wp, st.acct, 0);
+                            });
                     }
                 }
                 const int pf = k - 2;
