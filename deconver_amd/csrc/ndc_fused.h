@@ -201,15 +201,35 @@ NDC_HD int halo_row(int s, int PH, int TH) { return s < PH ? s : TH + s; }
 // plane of ONE source channel, the word (first input row, first own column - PW); input
 // rows base .. base + NR + KH - 2 feed the NR output rows and every tap plane jd of the KD
 // pending output planes.  w = taps of that source channel in (KD, KH, KW) order.
-template <int KD, int KH, int KW, int NR, int RW, int STRIDE, class Exec>
+//
+// PIPE (here and in a_plane): the LDS words of a row are read one row ahead of the arithmetic
+// that uses them, and a scheduling fence keeps that order; for kernels that run too few
+// wavefronts per SIMD to hide the LDS latency otherwise and have the registers to spare.
+template <int KD, int KH, int KW, int NR, int RW, int STRIDE, bool PIPE = false, class Exec>
 NDC_D void k_rows(Exec &ex, int base, int P, const float (&w)[KD * KH * KW],
                   float (*acc)[STRIDE][RW], int r_off)
 {
-    NDC_UNROLL
-    for (int q = 0; q < NR + KH - 1; ++q) {
-        float v[RW + KW - 1];
+    constexpr int NW = RW + KW - 1, NROW = NR + KH - 1;
+    float vn[NW];
+    if (PIPE) {
         NDC_UNROLL
-        for (int u = 0; u < RW + KW - 1; ++u) v[u] = ex.ld(base + q * P + u);
+        for (int u = 0; u < NW; ++u) vn[u] = ex.ld(base + u);
+    }
+    NDC_UNROLL
+    for (int q = 0; q < NROW; ++q) {
+        float v[NW];
+        if (PIPE) {
+            NDC_UNROLL
+            for (int u = 0; u < NW; ++u) v[u] = vn[u];
+            if (q + 1 < NROW) {
+                NDC_UNROLL
+                for (int u = 0; u < NW; ++u) vn[u] = ex.ld(base + (q + 1) * P + u);
+            }
+            ex.fence();
+        } else {
+            NDC_UNROLL
+            for (int u = 0; u < NW; ++u) v[u] = ex.ld(base + q * P + u);
+        }
         NDC_UNROLL
         for (int th = 0; th < KH; ++th) {
             const int rr = q - th;
@@ -229,18 +249,39 @@ NDC_D void k_rows(Exec &ex, int base, int P, const float (&w)[KD * KH * KW],
 // One tap plane of an A-type gather for NT tensors at once over an NR x RW register tile:
 // base[t] addresses, in plane-slot form, the word (first input row, first own column - PW)
 // of tensor t; wt = taps of tap plane td, indexed wt[i][th*KW + tw].
-template <int KH, int KW, int KT, int SC, int NR, int RW, int NTEN, class Exec>
+template <int KH, int KW, int KT, int SC, int NR, int RW, int NTEN, bool PIPE = false, class Exec>
 NDC_D void a_plane(Exec &ex, const int (&base)[NTEN], int P, const float (&wt)[SC][KH * KW],
                    float (&acc)[NTEN][SC][NR][RW])
 {
-    constexpr int PH = KH / 2;
-    NDC_UNROLL
-    for (int q = 0; q < NR + 2 * PH; ++q) {
-        float v[NTEN][RW + KW - 1];
+    constexpr int PH = KH / 2, NW = RW + KW - 1, NROW = NR + 2 * PH;
+    float vn[NTEN][NW];
+    if (PIPE) {
         NDC_UNROLL
         for (int t = 0; t < NTEN; ++t)
             NDC_UNROLL
-            for (int u = 0; u < RW + KW - 1; ++u) v[t][u] = ex.ld(base[t] + q * P + u);
+            for (int u = 0; u < NW; ++u) vn[t][u] = ex.ld(base[t] + u);
+    }
+    NDC_UNROLL
+    for (int q = 0; q < NROW; ++q) {
+        float v[NTEN][NW];
+        if (PIPE) {
+            NDC_UNROLL
+            for (int t = 0; t < NTEN; ++t)
+                NDC_UNROLL
+                for (int u = 0; u < NW; ++u) v[t][u] = vn[t][u];
+            if (q + 1 < NROW) {
+                NDC_UNROLL
+                for (int t = 0; t < NTEN; ++t)
+                    NDC_UNROLL
+                    for (int u = 0; u < NW; ++u) vn[t][u] = ex.ld(base[t] + (q + 1) * P + u);
+            }
+            ex.fence();
+        } else {
+            NDC_UNROLL
+            for (int t = 0; t < NTEN; ++t)
+                NDC_UNROLL
+                for (int u = 0; u < NW; ++u) v[t][u] = ex.ld(base[t] + q * P + u);
+        }
         NDC_UNROLL
         for (int th = 0; th < KH; ++th) {
             const int rr = q - 2 * PH + th;
@@ -853,8 +894,8 @@ struct Bwd1Kernel {
                         float wi[KT];
                         load_taps<KT>(hw + i * KT, wi);
                         const int gb_ = off_g + (st.ln.strip * RH) * P + PL + st.ln.c0 - PW;
-                        k_rows<KD, KH, KW, RH, RW, RH>(ex, gb_ + i * RG * P, P, wi, st.accx, 0);
-                        k_rows<KD, KH, KW, RH, RW, RH>(ex, gb_ + (SC + i) * RG * P, P, wi, st.acct, 0);
+                        k_rows<KD, KH, KW, RH, RW, RH, (KH > 1 && SAVED)>(ex, gb_ + i * RG * P, P, wi, st.accx, 0);
+                        k_rows<KD, KH, KW, RH, RW, RH, (KH > 1 && SAVED)>(ex, gb_ + (SC + i) * RG * P, P, wi, st.acct, 0);
                     }
                 }
                 const int pf = k - 2 * PD;
@@ -1072,7 +1113,7 @@ struct Bwd2Kernel {
                         base[0] = off_x + ob;
                         base[NA > 1 ? 1 : 0] = off_t + ob;
                     }
-                    a_plane<KH, KW, KT, SC, RH, RW, NA>(ex, base, P, wt, acc);
+                    a_plane<KH, KW, KT, SC, RH, RW, NA, (KH > 1 && SAVED)>(ex, base, P, wt, acc);
                 }
                 if (need_gh) {
                     // K-side filter-gradient term: re-read the gt1 window
