@@ -179,13 +179,24 @@ NDC_D void a_plane_d2(Exec &ex, const int (&base)[NTEN], int P, const float (&wt
 
 // NROWS rows of NW staged words each, row n at addr(n), handed to body(n, words) with the
 // reads running one row ahead (PIPE, see k_rows_d2).
+template <int NW, class Exec> NDC_D void read_row(Exec &ex, int at, uint32_t (&v)[NW])
+{
+    NDC_UNROLL
+    for (int u = 0; u < NW; ++u) v[u] = float_to_bits(ex.ld(at + u));
+}
+
+// `first`: row 0 already read by the caller (ahead of other work), or null.
 template <int NROWS, int NW, bool PIPE, class Exec, class Addr, class Body>
-NDC_D void stream_rows(Exec &ex, Addr addr, Body body)
+NDC_D void stream_rows(Exec &ex, Addr addr, Body body, const uint32_t (*first)[NW] = nullptr)
 {
     uint32_t vn[NW];
     if (PIPE) {
-        NDC_UNROLL
-        for (int u = 0; u < NW; ++u) vn[u] = float_to_bits(ex.ld(addr(0) + u));
+        if (first) {
+            NDC_UNROLL
+            for (int u = 0; u < NW; ++u) vn[u] = (*first)[u];
+        } else {
+            read_row<NW>(ex, addr(0), vn);
+        }
     }
     NDC_UNROLL
     for (int n = 0; n < NROWS; ++n) {
@@ -734,16 +745,21 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
                 {
                     uint32_t gg2[SC][RH][RW];
                     const int j = PH + st.ln.strip * RH;
+                    const int cb = PL + st.ln.c0 - PW;
+                    auto xt_row = [&](int n) NDC_LAMBDA {
+                        const int td = n / (RH + 2), q = n % (RH + 2);
+                        return off_xt + (wrap((j1 + 1 - td) % NXT, NXT) * RX + j + q) * P + cb;
+                    };
+                    // the first (x, t1) row of the filter-gradient stream is requested before
+                    // the elementwise work, so that it has arrived when that is done
+                    uint32_t row0[RW + 2];
+                    read_row<RW + 2>(ex, xt_row(0), row0);
+                    ex.fence();
                     gn_gd_rows(st, j1, j, IntTag<RH>(), 0, gg2);
                     if (need_gh) {
                         // A-side filter-gradient terms: (gn_i, gd_i) . (x, t1)[neighbour]
-                        const int cb = PL + st.ln.c0 - PW;
                         stream_rows<KD * (RH + 2), RW + 2, true>(
-                            ex,
-                            [&](int n) NDC_LAMBDA {
-                                const int td = n / (RH + 2), q = n % (RH + 2);
-                                return off_xt + (wrap((j1 + 1 - td) % NXT, NXT) * RX + j + q) * P + cb;
-                            },
+                            ex, xt_row,
                             [&](int n, const uint32_t (&v)[RW + 2]) NDC_LAMBDA {
                                 const int td = n / (RH + 2), q = n % (RH + 2);
                                 NDC_UNROLL
@@ -761,7 +777,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
                                                         st.gacc[i][(td * KH + th) * KW + tw]);
                                     }
                                 }
-                            });
+                            }, &row0);
                     }
                 }
                 if (st.ln.strip < 2) {
