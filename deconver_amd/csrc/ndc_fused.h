@@ -300,6 +300,43 @@ NDC_D void a_plane(Exec &ex, const int (&base)[NTEN], int P, const float (&wt)[S
     }
 }
 
+// NROWS rows of NW staged words of each of NOP operands (row n of operand t at addr(n, t)),
+// handed to body(n, words); PIPE: read one row ahead of the arithmetic (see k_rows).
+template <int NROWS, int NW, int NOP, bool PIPE, class Exec, class Addr, class Body>
+NDC_D void stream_rows(Exec &ex, Addr addr, Body body)
+{
+    float vn[NOP][NW];
+    if (PIPE) {
+        NDC_UNROLL
+        for (int t = 0; t < NOP; ++t)
+            NDC_UNROLL
+            for (int u = 0; u < NW; ++u) vn[t][u] = ex.ld(addr(0, t) + u);
+    }
+    NDC_UNROLL
+    for (int n = 0; n < NROWS; ++n) {
+        float v[NOP][NW];
+        if (PIPE) {
+            NDC_UNROLL
+            for (int t = 0; t < NOP; ++t)
+                NDC_UNROLL
+                for (int u = 0; u < NW; ++u) v[t][u] = vn[t][u];
+            if (n + 1 < NROWS) {
+                NDC_UNROLL
+                for (int t = 0; t < NOP; ++t)
+                    NDC_UNROLL
+                    for (int u = 0; u < NW; ++u) vn[t][u] = ex.ld(addr(n + 1, t) + u);
+            }
+            ex.fence();
+        } else {
+            NDC_UNROLL
+            for (int t = 0; t < NOP; ++t)
+                NDC_UNROLL
+                for (int u = 0; u < NW; ++u) v[t][u] = ex.ld(addr(n, t) + u);
+        }
+        body(n, v);
+    }
+}
+
 // Filter slices, fetched into scalar registers at the top of each tap-loop iteration (keeping
 // the next slice in flight as well costs more in scalar-register spills and copies than the
 // load latency it hides).
@@ -846,34 +883,35 @@ struct Bwd1Kernel {
                     gn_gd_rows(st, j1, j, IntTag<RH>(), acc);
                     if (need_gh && own1) {
                         // own rows: A-side filter-gradient terms, re-reading the x / t1 windows
-                        NDC_UNROLL
-                        for (int td = 0; td < KD; ++td) {
-                            const int slot = wrap((j1 + PD - td) % XR, XR);
-                            const int ob = (slot * RX + j) * P + PL + st.ln.c0 - PW;
-                            NDC_UNROLL
-                            for (int q = 0; q < RH + 2 * PH; ++q) {
-                                float vx[RW + KW - 1], vt[RW + KW - 1];
-                                NDC_UNROLL
-                                for (int u = 0; u < RW + KW - 1; ++u) {
-                                    vx[u] = ex.ld(off_x + ob + q * P + u);
-                                    vt[u] = ex.ld(off_t + ob + q * P + u);
-                                }
+                        // (read ahead: for the 2x2 float32 tile this costs two spilled registers
+                        // and is still 3 % faster)
+                        constexpr int NQ = RH + 2 * PH;
+                        const int cb = PL + st.ln.c0 - PW;
+                        stream_rows<KD * NQ, RW + KW - 1, 2, (KH > 1 && SAVED)>(
+                            ex,
+                            [&](int n, int t) NDC_LAMBDA {
+                                const int td = n / NQ, q = n % NQ;
+                                const int slot = wrap((j1 + PD - td) % XR, XR);
+                                return (t ? off_t : off_x) + (slot * RX + j + q) * P + cb;
+                            },
+                            [&](int n, const float (&v)[2][RW + KW - 1]) NDC_LAMBDA {
+                                const int td = n / NQ, q = n % NQ;
                                 NDC_UNROLL
                                 for (int th = 0; th < KH; ++th) {
                                     const int rr = q - 2 * PH + th;
-                                    if (rr < 0 || rr >= RH) continue;
-                                    NDC_UNROLL
-                                    for (int tw = 0; tw < KW; ++tw)
+                                    if (rr >= 0 && rr < RH) {
                                         NDC_UNROLL
-                                        for (int i = 0; i < SC; ++i)
+                                        for (int tw = 0; tw < KW; ++tw)
                                             NDC_UNROLL
-                                            for (int c = 0; c < RW; ++c)
-                                                st.gacc[i][(td * KH + th) * KW + tw] +=
-                                                    acc[0][i][rr][c] * vx[c + KW - 1 - tw] +
-                                                    acc[1][i][rr][c] * vt[c + KW - 1 - tw];
+                                            for (int i = 0; i < SC; ++i)
+                                                NDC_UNROLL
+                                                for (int c = 0; c < RW; ++c)
+                                                    st.gacc[i][(td * KH + th) * KW + tw] +=
+                                                        acc[0][i][rr][c] * v[0][c + KW - 1 - tw] +
+                                                        acc[1][i][rr][c] * v[1][c + KW - 1 - tw];
+                                    }
                                 }
-                            }
-                        }
+                            });
                     }
                 }
                 if (XT && st.ln.strip < 2 * PH) {
@@ -1117,30 +1155,32 @@ struct Bwd2Kernel {
                 }
                 if (need_gh) {
                     // K-side filter-gradient term: re-read the gt1 window
-                    NDC_UNROLL
-                    for (int td = 0; td < KD; ++td) {
-                        const int slot = wrap((j0 + PD - td) % XR, XR);
-                        const int ob = (slot * RX + st.ln.strip * RH) * P + PL + st.ln.c0 - PW;
-                        NDC_UNROLL
-                        for (int q = 0; q < RH + 2 * PH; ++q) {
-                            float vg[RW + KW - 1];
-                            NDC_UNROLL
-                            for (int u = 0; u < RW + KW - 1; ++u) vg[u] = ex.ld(off_g + ob + q * P + u);
+                    constexpr int NQ = RH + 2 * PH;
+                    const int cb = PL + st.ln.c0 - PW;
+                    stream_rows<KD * NQ, RW + KW - 1, 1, (KH > 1 && SAVED)>(
+                        ex,
+                        [&](int n, int) NDC_LAMBDA {
+                            const int td = n / NQ, q = n % NQ;
+                            const int slot = wrap((j0 + PD - td) % XR, XR);
+                            return off_g + (slot * RX + st.ln.strip * RH + q) * P + cb;
+                        },
+                        [&](int n, const float (&v)[1][RW + KW - 1]) NDC_LAMBDA {
+                            const int td = n / NQ, q = n % NQ;
                             NDC_UNROLL
                             for (int th = 0; th < KH; ++th) {
                                 const int rr = q - 2 * PH + th;
-                                if (rr < 0 || rr >= RH) continue;
-                                NDC_UNROLL
-                                for (int tw = 0; tw < KW; ++tw)
+                                if (rr >= 0 && rr < RH) {
                                     NDC_UNROLL
-                                    for (int i = 0; i < SC; ++i)
+                                    for (int tw = 0; tw < KW; ++tw)
                                         NDC_UNROLL
-                                        for (int c = 0; c < RW; ++c)
-                                            st.gacc[i][(td * KH + th) * KW + tw] +=
-                                                sv[i][rr][c] * vg[c + KW - 1 - tw];
+                                        for (int i = 0; i < SC; ++i)
+                                            NDC_UNROLL
+                                            for (int c = 0; c < RW; ++c)
+                                                st.gacc[i][(td * KH + th) * KW + tw] +=
+                                                    sv[i][rr][c] * v[0][c + KW - 1 - tw];
+                                }
                             }
-                        }
-                    }
+                        });
                 }
                 NDC_UNROLL
                 for (int r = 0; r < RH; ++r) {
