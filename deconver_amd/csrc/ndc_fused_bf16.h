@@ -1,6 +1,6 @@
 // bfloat16 variants of the fused kernels for the 3x3x3, SC = 4 depthwise geometry, built on
 // v_dot2c_f32_bf16 (two bf16 MACs per lane-instruction, float32 accumulate, same issue
-// rate as an fp32 FMA).  Same work decomposition, rings and march as ndc_fused.h; what
+// rate as an fp32 FMA that takes its tap from a scalar register).  Same work decomposition, rings and march as ndc_fused.h; what
 // changes is the LDS word format and the tap loops:
 //
 //   K-type applications (4 -> 1 channels) pair CHANNELS: the staged source is kept as two
