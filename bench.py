@@ -11,7 +11,9 @@
 One step = one forward + one backward (input-, source-, filter- and bias-gradient) of the
 update node on config 3 of the baseline: batch 2, 128 depthwise channels, 64^3 voxels,
 3x3x3 filter, ratio 4, bfloat16 storage with float32 accumulation; inputs resident in HBM.
-Prints ONE JSON line: whole-step throughput in Gvoxel/s, plus a ``roofline`` object for the
+Prints ONE JSON line: whole-step throughput in Gvoxel/s, a ``vector_ceiling`` object (bf16:
+time the kernels' v_dot2c_f32_bf16 alone would take at the measured issue rate, over the
+measured time), plus a ``roofline`` object for the
 slowest kernel (device time from events on the launch stream, algorithmic bytes as stated
 below) and a ``cpu_baseline`` object (the oracle timed on the host cores on a bounded
 sample of the same workload).
@@ -352,6 +354,7 @@ def grid_workload(args) -> int:
 
 
 DOT2_PER_CHANNEL_VOXEL = {"forward": 205, "backward_pass1": 216, "backward_pass2": 126}
+CLOCKS_PER_DOT2C = 4.52   # per SIMD, four wavefronts resident: measured by `--workload valu`
 
 
 def valu_workload(args) -> int:
@@ -658,6 +661,19 @@ def main() -> int:
         "backward_reads_forward_ratio": bool(keep),
         "roofline": roofline,
     }
+    if dtype == torch.bfloat16 and keep:
+        # the path is bound by vector issue, not by HBM: the least time the kernels'
+        # v_dot2c_f32_bf16 alone take, at the issue rate `--workload valu` measured
+        props = torch.cuda.get_device_properties(dev)
+        lanes = props.multi_processor_count * 4 * 64
+        hz = getattr(props, "clock_rate", 2400000) * 1e3   # kHz; MI355X peak engine clock 2.4 GHz
+        least = {k: U * n / lanes * CLOCKS_PER_DOT2C / hz * 1e3 for k, n in DOT2_PER_CHANNEL_VOXEL.items()}
+        result["vector_ceiling"] = {
+            "dot2c_per_channel_voxel": DOT2_PER_CHANNEL_VOXEL, "clocks_per_dot2c": CLOCKS_PER_DOT2C,
+            "least_ms": least,
+            "frac": {k: least[k] / k_ms[k] for k in least},
+            "step_frac": sum(least.values()) / sum(k_ms[k] for k in least),
+        }
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(torch)
     print(json.dumps(result))
