@@ -1,0 +1,129 @@
+"""The benchmark configurations at their full sizes on a real MI355X, through the C ABI.
+
+Depthwise channels are independent end to end, so any channel slice of a full-size result
+must equal the oracle evaluated on that slice alone -- which the CPU does in seconds.  This
+covers what no small case reaches: the row-band / column-strip shapes the launch planner
+picks for 128- and 192-column rows, volumes beyond 2^31 elements, the inference form of the
+forward call (no t1, nothing kept) and the kept-ratio backward kernels the benchmark times.
+Tolerances: ``max|d| / max|ref|`` <= 2e-2 for bfloat16 storage, <= 1e-4 for float32.
+"""
+
+import pytest
+import torch
+
+from deconver_amd import _lib, ops
+from oracle import ndc_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+SC = 4
+KS = (3, 3, 3)
+EPS = 1e-16
+
+
+def _inputs(B, C, sp, dtype, seed=0, with_gout=True):
+    """Half-normal x, signed z, softplus filter, small bias (config 3 / 5 construction),
+    drawn on the GPU (the CPU generator needs tens of seconds for 2^30 normals); the oracle
+    gets the channel slices it needs copied back."""
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    rn = lambda *s: torch.randn(*s, generator=gen, device="cuda")
+    h = torch.nn.functional.softplus(0.1 * rn(C, SC, *KS))
+    x = rn(B, C, *sp).abs_().to(dtype)
+    z = rn(B, C * SC, *sp).mul_(0.5).to(dtype)
+    bias = 0.1 * rn(C * SC)
+    gout = rn(B, C * SC, *sp).to(dtype) if with_gout else None
+    return x, z, h, bias, gout
+
+
+def _slice(c, x, z, h, bias, gout=None):
+    cs = slice(c * SC, (c + 1) * SC)
+    out = [x[:, c:c + 1].cpu().double(), z[:, cs].cpu().double(), h[c:c + 1].cpu().double(),
+           bias[cs].cpu().double()]
+    if gout is not None:
+        out.append(gout[:, cs].cpu().double())
+    return cs, out
+
+
+# config 5: (channels, extent, batch), bottleneck to full resolution
+SWEEP = [(512, 16, 4), (256, 32, 2), (64, 128, 1), (32, 192, 1)]
+
+
+@pytest.mark.parametrize("C,n,B", SWEEP)
+def test_config5_inference_form_channel_slices(C, n, B):
+    """Forward only, bfloat16, t1 = null, nothing kept: the call `bench.py --workload sweep`
+    times, at each of its four shapes."""
+    print("case config5", C, n, B, flush=True)
+    sp = (n, n, n)
+    x, z, h, bias, _ = _inputs(B, C, sp, torch.bfloat16, with_gout=False)
+    lib = _lib.get_library()
+    dev = [x, z, h, bias]
+    g = ops.make_geom_for(dev[0], dev[2], C, 1, SC, EPS, True)
+    assert lib.fused_supported(g), "the fused kernels must cover every config-5 shape"
+    out, t1 = ops.update_forward(lib, *dev, groups=C, m=1, sc=SC, eps=EPS, relu_input=True,
+                                 need_t1=False)
+    assert t1 is None
+    torch.cuda.synchronize()
+    for c in (0, C // 3, C - 1):
+        cs, d = _slice(c, x, z, h, bias)
+        ro, _ = O.update_grouped(d[0], d[1], d[2], d[3], 1, 1, SC, EPS, True)
+        e = O.rel_err(out[:, cs].cpu(), ro)
+        assert e < 2e-2, f"out channel {c}: {e:.3e}"
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.bfloat16, 2e-2), (torch.float32, 1e-4)])
+def test_config3_kept_ratio_backward_channel_slices(dtype, tol):
+    """Config 3 at full size with the forward's s/d and n/d kept: the kernels the headline
+    benchmark times (forward with four outputs, both kept-ratio backward passes), including
+    the two kept tensors themselves."""
+    B, C, sp = 2, 128, (64, 64, 64)
+    x, z, h, bias, gout = _inputs(B, C, sp, dtype)
+    lib = _lib.get_library()
+    dev = [x, z, h, bias, gout]
+    kw = dict(groups=C, m=1, sc=SC, eps=EPS, relu_input=True)
+    out, t1, saved = ops.update_forward(lib, *dev[:4], save_ratio=True, **kw)
+    gx, gz, gh, gb = ops.update_backward(lib, dev[0], dev[1], t1, dev[2], dev[3], dev[4],
+                                         saved=saved, **kw)
+    torch.cuda.synchronize()
+    kept = saved
+    for c in (1, 64, 126):
+        cs, d = _slice(c, x, z, h, bias, gout)
+        ro, rt1 = O.update_grouped(d[0], d[1], d[2], d[3], 1, 1, SC, EPS, True)
+        rgx, rgz, rgh, rgb = O.update_backward(d[0], d[1], d[2], d[3], d[4], 1, 1, SC, EPS, True)
+        s = O.rectified_source(d[1], d[3], True)
+        den = O.op_A(rt1, d[2], 1, 1, SC) + EPS
+        num = O.op_A(d[0], d[2], 1, 1, SC) + EPS
+        errs = dict(out=O.rel_err(out[:, cs].cpu(), ro), t1=O.rel_err(t1[:, c:c + 1].cpu(), rt1),
+                    s_over_den=O.rel_err(kept[0][:, cs].cpu(), s / den),
+                    ratio=O.rel_err(kept[1][:, cs].cpu(), num / den),
+                    gx=O.rel_err(gx[:, c:c + 1].cpu(), rgx), gz=O.rel_err(gz[:, cs].cpu(), rgz),
+                    gh=O.rel_err(gh[c:c + 1].cpu(), rgh), gb=O.rel_err(gb[cs].cpu(), rgb))
+        bad = {k: v for k, v in errs.items() if not v < tol}
+        assert not bad, f"channel {c}: {bad} (all: {errs})"
+
+
+def test_config4_stage0_layer_channel_slices():
+    """Config 4's full-resolution layer: batch 2, 64 channels, 128^3, bfloat16.  The source
+    tensors hold 2^30 elements (2 GiB) each, so tensor bases need 64-bit arithmetic; rows of
+    128 columns take the widest column strip.  Forward and the kept-ratio backward."""
+    B, C, sp = 2, 64, (128, 128, 128)
+    dtype = torch.bfloat16
+    x, z, h, bias, gout = _inputs(B, C, sp, dtype, seed=4)
+    assert z.numel() == 2 ** 30
+    lib = _lib.get_library()
+    dev = [x, z, h, bias, gout]
+    kw = dict(groups=C, m=1, sc=SC, eps=EPS, relu_input=True)
+    out, t1, saved = ops.update_forward(lib, *dev[:4], save_ratio=True, **kw)
+    gx, gz, gh, gb = ops.update_backward(lib, dev[0], dev[1], t1, dev[2], dev[3], dev[4],
+                                         saved=saved, **kw)
+    torch.cuda.synchronize()
+    del saved
+    # the last channel of the last sample sits past the 2^31-byte and 2^31-element marks
+    for c in (0, C - 1):
+        cs, d = _slice(c, x, z, h, bias, gout)
+        ro, _ = O.update_grouped(d[0], d[1], d[2], d[3], 1, 1, SC, EPS, True)
+        rgx, rgz, rgh, rgb = O.update_backward(d[0], d[1], d[2], d[3], d[4], 1, 1, SC, EPS, True)
+        errs = dict(out=O.rel_err(out[:, cs].cpu(), ro), gx=O.rel_err(gx[:, c:c + 1].cpu(), rgx),
+                    gz=O.rel_err(gz[:, cs].cpu(), rgz), gh=O.rel_err(gh[c:c + 1].cpu(), rgh),
+                    gb=O.rel_err(gb[cs].cpu(), rgb))
+        bad = {k: v for k, v in errs.items() if not v < 2e-2}
+        assert not bad, f"channel {c}: {bad} (all: {errs})"

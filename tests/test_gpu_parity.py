@@ -105,6 +105,28 @@ def test_fused_kernels_with_saved_ratio(geom, dtype):
     _run_case(geom, dtype, _lib.PATH_FUSED, saved=True)
 
 
+@pytest.mark.parametrize("geom", DIRECT_GEOMS + FUSED_GEOMS[:2] + FUSED_GEOMS[8:9])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gconv_matches_oracle(geom, dtype):
+    """ndc_gconv, the counterpart of kernels.gconv (kernels.py:728-759): K and A on their own,
+    plain and with the forward's on-load bias + ReLU of the input."""
+    C, G, sc, ks, sp, B = geom
+    m = C // G
+    x, z, h, bias, _ = make_case(C, G, sc, ks, sp, B=B, dtype=dtype, bias_shift=0.1, device="cuda")
+    lib = _lib_gpu()
+    tol = TOL[dtype]
+    hd, zd, xd = h.cpu().double(), z.cpu().double(), x.cpu().double()
+    k_plain = ops.gconv(lib, z, h, groups=G, m=m, sc=sc, adjoint=False)
+    k_rect = ops.gconv(lib, z, h, groups=G, m=m, sc=sc, adjoint=False, bias=bias, relu_input=True)
+    a_plain = ops.gconv(lib, x, h, groups=G, m=m, sc=sc, adjoint=True)
+    torch.cuda.synchronize()
+    assert k_plain.dtype == dtype and k_plain.shape == x.shape and a_plain.shape == z.shape
+    assert O.rel_err(k_plain.cpu(), O.op_K(zd, hd, G, m, sc)) < tol
+    s = O.rectified_source(zd, bias.cpu().double(), True)
+    assert O.rel_err(k_rect.cpu(), O.op_K(s, hd, G, m, sc)) < tol
+    assert O.rel_err(a_plain.cpu(), O.op_A(xd, hd, G, m, sc)) < tol
+
+
 def test_saved_ratio_later_iteration_form():
     _run_case(FUSED_GEOMS[0], torch.bfloat16, _lib.PATH_FUSED, relu=False, with_bias=False,
               saved=True)

@@ -187,3 +187,38 @@ def test_fused_partial_outputs():
             assert (a is None) == (not want)
             if want:
                 assert torch.equal(a, b)
+
+
+# rows as wide as the large 3-D configurations use (128^3, 192^3 and the widest the 3-D
+# kernels accept, 256 columns): the launch planner picks other strip counts and LDS pitches there
+WIDE_GEOMS = [
+    (1, 4, (3, 3, 3), (3, 10, 128), 1),
+    (1, 4, (3, 3, 3), (2, 9, 192), 1),
+    (1, 4, (3, 3, 3), (2, 6, 256), 2),
+    (1, 4, (3, 3, 3), (2, 5, 250), 1),
+]
+
+
+@pytest.mark.parametrize("geom", WIDE_GEOMS)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_fused_wide_rows(geom, dtype):
+    """Wide rows through the bounds/race checker: the inference form of the forward (no t1,
+    nothing kept), the training form with the kept ratio, and both backward forms."""
+    C, sc, ks, sp, B = geom
+    tol_f, tol_b = (1e-5, 1e-4) if dtype == torch.float32 else (2e-2, 2e-2)
+    lib = hostcheck_library()
+    x, z, h, bias, gout = make_case(C, C, sc, ks, sp, B=B, dtype=dtype, bias_shift=0.3)
+    kw = dict(groups=C, m=1, sc=sc, eps=1e-16, relu_input=True, path=_lib.PATH_FUSED)
+    host_faults(lib)
+    out_inf, none = ops.update_forward(lib, x, z, h, bias, need_t1=False, **kw)
+    assert none is None
+    out, t1, saved = ops.update_forward(lib, x, z, h, bias, save_ratio=True, **kw)
+    assert torch.equal(out, out_inf)
+    ro, rt1, refs = _oracle(x, z, h, bias, gout, C, sc, 1e-16, True)
+    assert O.rel_err(out, ro) < tol_f and O.rel_err(t1, rt1) < tol_f
+    for sv in (saved, None):
+        got = ops.update_backward(lib, x, z, t1, h, bias, gout, saved=sv, **kw)
+        for a, r in zip(got, refs):
+            assert O.rel_err(a, r) < tol_b
+    n, first = host_faults(lib)
+    assert n == 0, f"LDS faults: {n} ({first})"
