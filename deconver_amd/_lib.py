@@ -26,6 +26,7 @@ EXPORTS = (
     "ndc_backward_uses_saved",
     "ndc_forward",
     "ndc_forward_workspace_bytes",
+    "ndc_forward_noalloc",
     "ndc_backward_workspace_bytes",
     "ndc_backward",
     "ndc_backward_profiled",
@@ -84,6 +85,8 @@ class NdcLibrary:
         d.ndc_check_geometry.argtypes = [gp]
         d.ndc_backward_uses_saved.argtypes = [gp]
         d.ndc_forward.argtypes = [gp, vp, vp, fp, fp, vp, vp, vp, vp, vp, ctypes.c_size_t, vp]
+        if hasattr(d, "ndc_forward_noalloc"):   # HIP build only
+            d.ndc_forward_noalloc.argtypes = [gp, vp, vp, fp, fp, vp, vp, vp, vp, vp]
         d.ndc_forward_workspace_bytes.restype = ctypes.c_size_t
         d.ndc_forward_workspace_bytes.argtypes = [gp]
         d.ndc_backward_workspace_bytes.restype = ctypes.c_size_t
@@ -118,6 +121,13 @@ class NdcLibrary:
                 ws: Optional[int], ws_bytes: int, stream: Optional[int]) -> None:
         self._check(self._dll.ndc_forward(ctypes.byref(g), x, z, h, bias, out, t1, s_over_den, ratio,
                                           ws, ws_bytes, stream), "ndc_forward")
+
+    def forward_noalloc(self, g: Geom, x: int, z: int, h: int, bias: Optional[int], out: int,
+                        t1: Optional[int], s_over_den: Optional[int], ratio: Optional[int],
+                        stream: Optional[int]) -> None:
+        """``forward`` with the scratch in the library's own device array (no workspace)."""
+        self._check(self._dll.ndc_forward_noalloc(ctypes.byref(g), x, z, h, bias, out, t1,
+                                                  s_over_den, ratio, stream), "ndc_forward_noalloc")
 
     def backward_workspace_bytes(self, g: Geom, need_gx, need_gz, need_gh, need_gb) -> int:
         return self._dll.ndc_backward_workspace_bytes(

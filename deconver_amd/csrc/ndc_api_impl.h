@@ -173,6 +173,8 @@ const char *ndc_status_string(int status)
     case NDC_ERR_DTYPE: return "unknown dtype tag";
     case NDC_ERR_WORKSPACE: return "workspace too small or misaligned";
     case NDC_ERR_LAUNCH: return "kernel launch failed";
+    case NDC_ERR_SCRATCH_LIMIT:
+        return "geometry needs more scratch than the no-allocation entry point's device array holds";
     default: return "unknown status";
     }
 }

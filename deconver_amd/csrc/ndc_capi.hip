@@ -123,3 +123,61 @@ struct Backend {
 }  // namespace ndc
 
 #include "ndc_api_impl.h"
+
+// ============================================================================ no-allocation forward
+//
+// ndc_forward for callers that cannot hand over a workspace they allocated (code under graph
+// capture that was set up without one, serving loops and harnesses that forbid hipMalloc):
+// the forward's scratch -- the packed filter tables of the bfloat16 3x3x3 kernels -- lives in
+// a file-scope device array instead.  Every GPU the library runs on holds its own copy of the
+// array, at its own address, until the process ends.
+
+#include <mutex>
+
+namespace {
+
+static __device__ __align__(256) unsigned char scratch[NDC_NOALLOC_SCRATCH_BYTES];
+
+// In host code the name `scratch` is only a handle for hipGetSymbolAddress; the device
+// address is looked up once per device (with that device current) and kept here.  Kernels,
+// copies and memsets are always given this pointer, never the array's name.
+const int kMaxDevices = 64;
+void *scratch_dev_ptr[kMaxDevices] = {nullptr};
+std::mutex scratch_mutex;
+
+int scratch_address(void **out)
+{
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return NDC_ERR_LAUNCH;
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (!scratch_dev_ptr[dev]) {
+        void *ptr = nullptr;
+        if (hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr)
+            return NDC_ERR_LAUNCH;
+        scratch_dev_ptr[dev] = ptr;
+    }
+    *out = scratch_dev_ptr[dev];
+    return NDC_OK;
+}
+
+}  // namespace
+
+extern "C" int ndc_forward_noalloc(const ndc_geom *g, const void *x, const void *z, const float *h,
+                                   const float *bias, void *out, void *t1, void *s_over_den,
+                                   void *ratio, void *stream)
+{
+    ndc::KGeom q;
+    const int st = ndc::make_kgeom(g, q);
+    if (st) return st;
+    const size_t need = ndc_forward_workspace_bytes(g);
+    if (need > (size_t)NDC_NOALLOC_SCRATCH_BYTES) return NDC_ERR_SCRATCH_LIMIT;
+    void *ptr = nullptr;
+    if (need) {
+        const int sa = scratch_address(&ptr);
+        if (sa) return sa;
+    }
+    // the tables are rewritten in full by every call (nothing has to start at zero); the
+    // launches that fill and read them are ordered on `stream`
+    return ndc_forward(g, x, z, h, bias, out, t1, s_over_den, ratio, ptr,
+                       need ? (size_t)NDC_NOALLOC_SCRATCH_BYTES : 0, stream);
+}

@@ -39,7 +39,9 @@ enum ndc_status {
     NDC_ERR_GEOMETRY = -2,    /* extents/kernel/groups outside what the kernels cover */
     NDC_ERR_DTYPE = -3,       /* unknown dtype tag */
     NDC_ERR_WORKSPACE = -4,   /* workspace too small or misaligned */
-    NDC_ERR_LAUNCH = -5       /* hipGetLastError() reported a failure after a launch */
+    NDC_ERR_LAUNCH = -5,      /* hipGetLastError() reported a failure after a launch */
+    NDC_ERR_SCRATCH_LIMIT = -6 /* ndc_forward_noalloc: the geometry needs more scratch than
+                                  NDC_NOALLOC_SCRATCH_BYTES */
 };
 
 /* Which implementation a call may use.  AUTO picks the fused LDS-tiled kernels when the
@@ -104,6 +106,25 @@ size_t ndc_forward_workspace_bytes(const ndc_geom *g);
 int ndc_forward(const ndc_geom *g, const void *x, const void *z, const float *h,
                 const float *bias, void *out, void *t1, void *s_over_den, void *ratio,
                 void *workspace, size_t workspace_bytes, void *stream);
+
+/* Size of the device array behind ndc_forward_noalloc: room for the packed filter tables of
+ * 2080 depthwise channels (504 bytes per channel). */
+#define NDC_NOALLOC_SCRATCH_BYTES (1u << 20)
+
+/*
+ * ndc_forward without a workspace argument and without any allocation: same inputs, outputs
+ * and results as ndc_forward, with the forward's scratch in a device array that is part of
+ * the library image (each GPU the library runs on holds NDC_NOALLOC_SCRATCH_BYTES of it
+ * until the process ends).  It has no counterpart in the reference; it is for callers that
+ * cannot allocate: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  A geometry whose ndc_forward_workspace_bytes() exceeds the array is refused
+ * with NDC_ERR_SCRATCH_LIMIT before anything is launched.  All calls on one GPU share the one
+ * array: calls that may overlap on a GPU (different streams, different threads) race on it
+ * and must be serialised by the caller, or use ndc_forward with a workspace of their own.
+ */
+int ndc_forward_noalloc(const ndc_geom *g, const void *x, const void *z, const float *h,
+                        const float *bias, void *out, void *t1, void *s_over_den, void *ratio,
+                        void *stream);
 
 /* Bytes of scratch `ndc_backward` needs for `g` with the requested outputs (each flag
  * nonzero when the matching output pointer will be non-null). */
