@@ -1,0 +1,186 @@
+"""Numbers of the reference's ORIGINAL layer against the oracle, the package and the HIP route.
+
+``tests/golden/reference_vectors.json`` holds outputs and every gradient of the reference's
+``ReferenceDeconv`` (float64, CPU) on the case list of its own equivalence tests
+(``tests/test_deconv_equivalence.py:29-35,112-169``) and of the small network of
+``:311-379``, written by ``tests/golden/make_reference_vectors.py`` from the reference
+package.  Each tensor is stored as shape, three global checksums and evenly strided entries.
+The same weights and inputs are rebuilt here from the seeds (``test_golden_state.py`` checks
+that the package's constructors draw from the generator as the reference's do) and
+
+* ``oracle/ndc_oracle.py`` and ``oracle/model_oracle.py`` (float64) must reproduce the
+  stored numbers to 1e-9: this pins the oracles to the reference itself, not only to
+  mathematics;
+* the package's general route (float64, CPU) likewise;
+* on a GPU, the HIP route in float32 must be within north_star's 1e-4 of them.
+"""
+
+import json
+import os
+
+import pytest
+import torch
+from torch import nn
+
+import deconver_amd as dc
+from oracle import model_oracle as MO
+from oracle import ndc_oracle as O
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+with open(os.path.join(HERE, "golden", "reference_vectors.json")) as fh:
+    GOLDEN = json.load(fh)
+NPROBE = GOLDEN["nprobe"]
+PARAMS = {"w": "init.linear.linear.weight", "b": "init.linear.linear.bias", "h": "init.h0"}
+
+
+def _probe_idx(n):
+    k = min(n, NPROBE)
+    return [(i * (n - 1)) // max(k - 1, 1) for i in range(k)]
+
+
+def _mismatch(t, ref):
+    """Largest deviation of a tensor from its stored description, relative to the stored
+    tensor's largest magnitude (the reference tests' metric, test_deconv_equivalence.py:51-59)."""
+    assert list(t.shape) == ref["shape"]
+    v = t.detach().double().cpu().reshape(-1)
+    n = v.numel()
+    scale = max(ref["absmax"], 1e-30)
+    w = torch.cos(torch.arange(n, dtype=torch.float64) * 0.7390851332151607 + 0.25)
+    probes = (v[_probe_idx(n)] - torch.tensor(ref["probe"], dtype=torch.float64)).abs().max().item()
+    # checksums are sums over n entries of magnitude <= scale
+    sums = max(abs(float(v.sum()) - ref["sum"]), abs(float((v * w).sum()) - ref["cosdot"])) / n ** 0.5
+    sq = abs(float((v * v).sum()) - ref["sumsq"]) / max(ref["sumsq"], 1e-300) * scale
+    return max(probes, sums, sq) / scale
+
+
+def _case_inputs(name, seed=0):
+    spec = GOLDEN["specs"][name]
+    kwargs = {k: (tuple(v) if isinstance(v, list) else v) for k, v in spec["kwargs"].items()}
+    torch.manual_seed(seed)
+    layer = dc.Deconv(**kwargs)
+    if spec["bias"]:
+        with torch.no_grad():
+            layer.init.linear.linear.bias.add_(spec["bias"])
+    torch.manual_seed(seed + 1)
+    x0 = torch.rand(spec["batch"], kwargs["channels"], *spec["spatial"])
+    torch.manual_seed(seed + 2)
+    g0 = torch.randn(spec["batch"], layer.init.linear.linear.weight.shape[0], *spec["spatial"])
+    stored = GOLDEN["layer_cases"][name]
+    assert _mismatch(x0, stored["x"]) < 1e-12 and _mismatch(g0, stored["g"]) < 1e-12
+    return kwargs, layer, x0, g0, stored
+
+
+LAYER_CASES = sorted(GOLDEN["layer_cases"])
+
+
+@pytest.mark.parametrize("name", LAYER_CASES)
+def test_oracle_reproduces_the_reference_layer(name):
+    kwargs, layer, x0, g0, stored = _case_inputs(name)
+    oracle = O.OracleNDC(kwargs["channels"], kwargs["kernel_size"], ratio=kwargs.get("ratio", 1),
+                         groups=kwargs.get("groups", -1), num_iters=kwargs.get("num_iters", 1),
+                         num_grad_iters=kwargs.get("num_grad_iters"))
+    w = layer.init.linear.linear.weight.detach().double().squeeze(-1).requires_grad_(True)
+    b = layer.init.linear.linear.bias.detach().double().requires_grad_(True)
+    h0 = layer.init.h0.detach().double().requires_grad_(True)
+    x = x0.double().requires_grad_(True)
+    y = oracle.forward(x, w, b, h0)
+    y.backward(g0.double())
+    assert _mismatch(y, stored["y"]) < 1e-9
+    assert _mismatch(x.grad, stored["grad_x"]) < 1e-9
+    for got, key in ((w.grad, "w"), (b.grad, "b"), (h0.grad, "h")):
+        ref = stored["grad_" + PARAMS[key]]
+        # truncated back-propagation leaves the projection without a gradient on both sides
+        assert (got is None) == (ref is None), key
+        if ref is not None:
+            assert _mismatch(got.reshape(ref["shape"]), ref) < 1e-9, key
+
+
+@pytest.mark.parametrize("name", LAYER_CASES)
+def test_general_route_reproduces_the_reference_layer(name):
+    kwargs, layer, x0, g0, stored = _case_inputs(name)
+    layer = layer.double()
+    x = x0.double().requires_grad_(True)
+    assert not layer.fast_path_applicable(x)   # CPU tensors take the general route
+    y = layer(x)
+    y.backward(g0.double())
+    assert _mismatch(y, stored["y"]) < 1e-9
+    assert _mismatch(x.grad, stored["grad_x"]) < 1e-9
+    for pname, p in layer.named_parameters():
+        ref = stored["grad_" + pname]
+        assert (p.grad is None) == (ref is None), pname
+        if ref is not None:
+            assert _mismatch(p.grad, ref) < 1e-9, pname
+
+
+def _network():
+    spec = dict(GOLDEN["network_spec"])
+    cfg = {k: (tuple(v) if isinstance(v, list) else v) for k, v in spec.items()}
+    kwargs = dict(cfg, norm=getattr(nn, cfg["norm"]), act=getattr(nn, cfg["act"]))
+    torch.manual_seed(0)
+    net = dc.Deconver(**kwargs).eval()
+    torch.manual_seed(1)
+    x0 = torch.rand(2, 4, 16, 16, 16)
+    g0 = torch.randn(2, 3, 16, 16, 16)
+    return cfg, net, x0, g0
+
+
+def test_network_parameters_match_the_reference():
+    _, net, x0, g0 = _network()
+    stored = GOLDEN["network"]
+    assert sorted(n for n, _ in net.named_parameters()) == sorted(stored["params"])
+    for name, p in net.named_parameters():
+        assert _mismatch(p, stored["params"][name]["value"]) < 1e-12, name
+    assert _mismatch(x0, stored["x"]) < 1e-12 and _mismatch(g0, stored["g"]) < 1e-12
+
+
+def test_model_oracle_reproduces_the_reference_network():
+    cfg, net, x0, g0 = _network()
+    stored = GOLDEN["network"]
+    state = {k: v.detach().double().requires_grad_(True) for k, v in net.state_dict().items()}
+    x = x0.double().requires_grad_(True)
+    y = MO.deconver_forward(state, x, cfg)
+    y.backward(g0.double())
+    assert _mismatch(y, stored["y"]) < 1e-9
+    assert _mismatch(x.grad, stored["grad_x"]) < 1e-9
+    for name, ref in stored["params"].items():
+        assert _mismatch(state[name].grad, ref["grad"]) < 1e-9, name
+
+
+def test_package_network_general_route_reproduces_the_reference_network():
+    cfg, net, x0, g0 = _network()
+    stored = GOLDEN["network"]
+    net = net.double()
+    x = x0.double().requires_grad_(True)
+    y = net(x)
+    y.backward(g0.double())
+    assert _mismatch(y, stored["y"]) < 1e-9
+    assert _mismatch(x.grad, stored["grad_x"]) < 1e-9
+    for name, p in net.named_parameters():
+        assert _mismatch(p.grad, stored["params"][name]["grad"]) < 1e-9, name
+
+
+# ------------------------------------------------------------------ HIP route (MI355X)
+
+# the well-conditioned regime the reference's own comparisons run in (bias +1.0,
+# test_deconv_equivalence.py:69-76)
+HIP_CASES = [n for n in LAYER_CASES if GOLDEN["specs"][n]["bias"]]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", HIP_CASES)
+def test_hip_route_matches_the_reference_layer(name):
+    kwargs, layer, x0, g0, stored = _case_inputs(name)
+    layer = layer.cuda()
+    x = x0.cuda().requires_grad_(True)
+    assert layer.fast_path_applicable(x), "expected the HIP route"
+    y = layer(x)
+    y.backward(g0.cuda())
+    tol = 5e-4 if kwargs.get("num_iters", 1) > 1 else 1e-4
+    assert _mismatch(y, stored["y"]) < tol
+    assert _mismatch(x.grad, stored["grad_x"]) < tol
+    for pname, p in layer.named_parameters():
+        ref = stored["grad_" + pname]
+        if ref is None:
+            assert p.grad is None, pname
+            continue
+        assert _mismatch(p.grad, ref) < tol, pname

@@ -100,38 +100,93 @@ class _GeneralRoute(dc.Deconv):
         return super().update_s(x, s, h)
 
 
-def test_bf16_autocast_layer_no_further_from_exact_than_pytorch():
-    """Whole layer under bfloat16 autocast (which the reference's fused path declines).  The
-    bf16 projection feeds a rounded z into the update, so neither route is within 2e-2 of a
-    float64 evaluation of the unrounded layer; as in the reference's own network test
-    (test_deconv_equivalence.py:332-379) the HIP route must be no further from exact than
-    the PyTorch route is (x2, with a 3e-2 floor: both routes sit at the 1e-2 level here)."""
+def _bf16_layer_case(cls):
     kwargs = dict(channels=16, ratio=4, groups=-1, kernel_size=(3, 3, 3))
     torch.manual_seed(1)
     x0 = torch.rand(2, 16, 9, 8, 10)
     g0 = torch.randn(2, 64, 9, 8, 10)
+    torch.manual_seed(0)
+    layer = cls(**kwargs)
+    with torch.no_grad():
+        layer.init.linear.linear.bias.add_(1.0)
+    return kwargs, layer.cuda(), x0, g0
+
+
+def _layer_errors(layer, x, y, yr, gr):
+    return dict(out=O.rel_err(y.detach().float().cpu(), yr),
+                x=O.rel_err(x.grad.cpu(), gr["x"]),
+                h=O.rel_err(layer.init.h0.grad.cpu(), gr["h"]),
+                b=O.rel_err(layer.init.linear.linear.bias.grad.cpu(), gr["b"]),
+                w=O.rel_err(layer.init.linear.linear.weight.grad.cpu().squeeze(-1), gr["w"]))
+
+
+def test_bf16_autocast_layer_within_2e_2_of_float64():
+    """Whole layer under bfloat16 autocast (which the reference's fused path declines): output
+    and every gradient within 2e-2 of a float64 evaluation of the unrounded layer.
+
+    One thing has to be taken out of that comparison.  The bf16 projection hands the update a
+    rounded z, so a source unit whose exact pre-activation z + b lies within that rounding of
+    zero may come out switched (on instead of off or the reverse), and one switched unit moves
+    dx by a finite amount -- in any bf16 implementation, the PyTorch route included; which
+    units switch is a matter of rounding luck (on this seed 4 of 92 160 do, and they alone put
+    dx 3e-2 from float64).  The float64 oracle is therefore evaluated on the on/off pattern
+    the route computed, and the switched units are checked to be exactly such borderline
+    units and few."""
+    kwargs, layer, x0, g0 = _bf16_layer_case(dc.Deconv)
+    x = x0.cuda().requires_grad_(True)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        assert layer.fast_path_applicable(x)
+        y = layer(x)
+    assert y.dtype == torch.bfloat16
+    y.backward(g0.cuda().to(y.dtype))
+    assert x.grad.dtype == torch.float32 and layer.init.h0.grad.dtype == torch.float32
+    # the pattern the route computed: sign of (bf16 projection, float32 bias added on load)
+    proj = layer.init.linear.linear
+    with torch.no_grad():
+        z_route = torch.nn.functional.conv1d(x0.cuda().bfloat16().flatten(2), proj.weight.bfloat16())
+        gate = (z_route.float() + proj.bias.float().view(1, -1, 1) > 0).view(2, 64, 9, 8, 10).cpu()
+        z_exact = torch.nn.functional.conv1d(x0.double().flatten(2), proj.weight.double().cpu(),
+                                             proj.bias.double().cpu()).view(2, 64, 9, 8, 10)
+    switched = gate != (z_exact > 0)
+    assert switched.sum().item() <= 1e-3 * gate.numel()
+    if switched.any():   # only units within bf16 rounding (of z, x and the weights) of zero
+        assert z_exact[switched].abs().max().item() < 2e-2
+    oracle = O.OracleNDC(16, (3, 3, 3), ratio=4)
+    w = proj.weight.detach().cpu().double().squeeze(-1).requires_grad_(True)
+    b = proj.bias.detach().cpu().double().requires_grad_(True)
+    h0 = layer.init.h0.detach().cpu().double().requires_grad_(True)
+    xr = x0.double().requires_grad_(True)
+    yr = oracle.forward(xr, w, b, h0, gate=gate)
+    yr.backward(g0.double())
+    errs = _layer_errors(layer, x, y, yr.detach(), dict(x=xr.grad, w=w.grad, b=b.grad, h=h0.grad))
+    bad = {k: v for k, v in errs.items() if not v < 2e-2}
+    assert not bad, (bad, errs)
+
+
+def test_bf16_autocast_layer_no_further_from_exact_than_pytorch():
+    """The reference's own criterion for a low-precision network (test_deconv_equivalence.py:
+    332-379): no further from the float64 evaluation than the PyTorch route is (x1.5), with
+    the 2e-2 bf16 bound as the floor.  Units switched by rounding are a property of the
+    operands, not of a route (see the test above), so both routes are measured on a case
+    where a float64 screen finds no pre-activation within bf16 rounding of zero: the bias is
+    raised until every z + b is clear of it."""
     errs = {}
     for name, cls in (("hip", dc.Deconv), ("torch", _GeneralRoute)):
-        torch.manual_seed(0)
-        layer = cls(**kwargs)
+        kwargs, layer, x0, g0 = _bf16_layer_case(cls)
+        proj = layer.init.linear.linear
         with torch.no_grad():
-            layer.init.linear.linear.bias.add_(1.0)
-        layer = layer.cuda()
+            z = torch.nn.functional.conv1d(x0.double().flatten(2), proj.weight.double().cpu(),
+                                           proj.bias.double().cpu())
+            proj.bias.add_(float(-z.min()) + 0.05)   # smallest pre-activation becomes 0.05
         x = x0.cuda().requires_grad_(True)
         with torch.autocast("cuda", dtype=torch.bfloat16):
             assert layer.fast_path_applicable(x) == (name == "hip")
             y = layer(x)
-        assert y.dtype == torch.bfloat16
         y.backward(g0.cuda().to(y.dtype))
-        assert x.grad.dtype == torch.float32 and layer.init.h0.grad.dtype == torch.float32
         yr, gr = _oracle_run(layer, kwargs, x0, g0)
-        errs[name] = dict(out=O.rel_err(y.detach().float().cpu(), yr),
-                          x=O.rel_err(x.grad.cpu(), gr["x"]),
-                          h=O.rel_err(layer.init.h0.grad.cpu(), gr["h"]),
-                          b=O.rel_err(layer.init.linear.linear.bias.grad.cpu(), gr["b"]),
-                          w=O.rel_err(layer.init.linear.linear.weight.grad.cpu().squeeze(-1), gr["w"]))
+        errs[name] = _layer_errors(layer, x, y, yr, gr)
     for k, e in errs["hip"].items():
-        assert e <= max(2.0 * errs["torch"][k], 3e-2), (k, errs)
+        assert e <= max(1.5 * errs["torch"][k], 2e-2), (k, errs)
 
 
 def test_bf16_update_node_autograd():
