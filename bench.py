@@ -7,6 +7,7 @@
     python bench.py --workload grid                                       (ratio x groups x kernel grid)
     python bench.py --workload valu                                       (instruction-issue ceiling probe)
     python bench.py --workload train3d|model2d [--ndc hip|pytorch|both]   (model level, below)
+    python bench.py --workload mixer [--dtype bf16|fp32]                  (one DeconvMixer, fwd+bwd)
 
 One step = one forward + one backward (input-, source-, filter- and bias-gradient) of the
 update node on config 3 of the baseline: batch 2, 128 depthwise channels, 64^3 voxels,
@@ -491,6 +492,56 @@ def model_workload(args) -> int:
     return 0
 
 
+def mixer_workload(args) -> int:
+    """One DeconvMixer (in_proj -> ReLU -> NDC layer -> out_proj, the caller of the hot path,
+    deconver/deconver.py:22-46) at config 3's shape: batch 2, 128 channels, 64^3, 3x3x3,
+    ratio 4; bf16 autocast or float32; one step = forward + backward.  Exists so that a
+    rocprofv3 kernel trace of it shows what the projections around the update cost next to
+    the update itself (bytes of z and of the update's output written by one GEMM and read
+    by the next kernel)."""
+    import torch
+
+    import deconver_amd as dc
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    w = WORKLOAD
+    dev = torch.device("cuda:0")
+    C = w["channels"]
+    torch.manual_seed(0)
+    mixer = dc.DeconvMixer(C, C, kernel_size=w["kernel"], ratio=w["ratio"], groups=-1).to(dev)
+    x = torch.randn(w["batch"], C, *w["spatial"], device=dev).requires_grad_(True)
+    g = torch.randn(w["batch"], C, *w["spatial"], device=dev)
+    dtype = torch.bfloat16 if args.dtype == "bf16" else None
+
+    def step():
+        mixer.zero_grad(set_to_none=True)
+        x.grad = None
+        with torch.autocast("cuda", dtype=torch.bfloat16, enabled=dtype is not None):
+            y = mixer(x)
+        y.backward(g.to(y.dtype))
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    vox = w["batch"] * math.prod(w["spatial"])
+    print(json.dumps({
+        "metric": "DeconvMixer fwd+bwd Gvoxel/s", "value": vox / (ms * 1e-3) / 1e9,
+        "unit": "Gvoxel/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype if args.dtype == "bf16" else "f32", "data": "synthetic",
+        "config": {"workload": "one DeconvMixer at config 3's shape (batch 2, 128 channels, "
+                               "64^3, 3x3x3, ratio 4), forward + backward"},
+        "roofline": None, "cpu_baseline": None}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -504,7 +555,7 @@ def main() -> int:
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
-    ap.add_argument("--workload", choices=("ndc", "sweep", "accuracy", "grid", "valu", "train3d", "model2d"),
+    ap.add_argument("--workload", choices=("ndc", "sweep", "accuracy", "grid", "valu", "train3d", "model2d", "mixer"),
                     default="ndc",
                     help="ndc: the headline update node (default); the others are model level")
     ap.add_argument("--ndc", choices=("hip", "pytorch", "both"), default="hip",
@@ -523,6 +574,8 @@ def main() -> int:
         return grid_workload(args)
     if args.workload == "valu":
         return valu_workload(args)
+    if args.workload == "mixer":
+        return mixer_workload(args)
     if args.workload != "ndc":
         return model_workload(args)
 

@@ -160,13 +160,23 @@ NDC_HD float relu_f(float v)
 #endif
 }
 
-// max(v, lo): one v_max_f32
+// max(v, lo) that hands a NaN in v on (as torch.relu does; fmaxf would return lo): one
+// v_maximum3_f32.  With lo = kPassThrough it is the identity for every v, -inf included.
 NDC_HD float floor_f(float v, float lo)
 {
 #if NDC_DEVICE_BUILD && defined(__HIP_DEVICE_COMPILE__)
-    return __builtin_fmaxf(v, lo);
+    return __builtin_elementwise_maximum(v, lo);
 #else
-    return v > lo ? v : lo;
+    return v != v ? v : (v > lo ? v : lo);
+#endif
+}
+
+NDC_HD float pass_through_floor()
+{
+#if NDC_DEVICE_BUILD && defined(__HIP_DEVICE_COMPILE__)
+    return -__builtin_huge_valf();
+#else
+    return -__builtin_huge_valf();
 #endif
 }
 

@@ -49,7 +49,7 @@ NDC_HD float source_at(const KGeom &q, const T *z, const float *bias, long long 
 {
     float v = Elem<T>::load(z + off);
     if (bias) v += bias[chan];
-    if (q.relu) v = v > 0.f ? v : 0.f;
+    if (q.relu) v = v < 0.f ? 0.f : v;   // a NaN stays a NaN, as in torch.relu
     return v;
 }
 
@@ -80,7 +80,7 @@ NDC_HD void gconv(long long idx, const KGeom &q, const TI *in, const float *hf, 
                     if (rectify) {
                         v = Elem<TI>::load(in + off);
                         if (bias) v += bias[p.g * cin + ci];
-                        if (q.relu) v = v > 0.f ? v : 0.f;
+                        if (q.relu) v = v < 0.f ? 0.f : v;   // a NaN stays a NaN, as in torch.relu
                     } else {
                         v = Elem<TI>::load(in + off);
                     }
@@ -173,7 +173,7 @@ NDC_HD void bwd_gz(long long idx, const KGeom &q, const T *x, const T *t1, const
     if (q.relu) {
         float pre = Elem<T>::load(z + idx);
         if (bias) pre += bias[p.g * q.sc + p.ch];
-        if (!(pre > 0.f)) r = 0.f;
+        if (pre <= 0.f) r = 0.f;   // a NaN passes, as through torch.relu's backward
     }
     Elem<T>::store(gz + idx, r);
 }

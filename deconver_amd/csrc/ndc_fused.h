@@ -417,7 +417,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
         UniformF hw = as_uniform(p.h + (long long)id.c * SC * KT);
         const int r0 = id.r0;
         const int nthreads = ex.nthreads;
-        const float floor_ = p.relu ? 0.f : -3.0e38f;   // max(s, floor_) rectifies or passes through
+        const float floor_ = p.relu ? 0.f : pass_through_floor();   // floor_f(s, floor_) rectifies or passes through
         const float eps = p.eps;
         // owned output planes [d0, d1); the march starts 2*PD planes early so that t1 is
         // complete from plane d0 - PD on, and runs 2*PD planes past the end
@@ -715,7 +715,7 @@ struct Bwd1Kernel {
         UniformF hw = as_uniform(p.h + (long long)id.c * SC * KT);
         const int r0 = id.r0;
         const int nthreads = ex.nthreads;
-        const float floor_ = p.relu ? 0.f : -3.0e38f;   // max(s, floor_) rectifies or passes through
+        const float floor_ = p.relu ? 0.f : pass_through_floor();   // floor_f(s, floor_) rectifies or passes through
         const float eps = p.eps;
         const int need_gh = p.need_gh;
         // owned output planes [d0, d1); gn / gd are needed PD planes beyond them on each side
@@ -1018,7 +1018,7 @@ struct Bwd2Kernel {
         UniformF hw = as_uniform(p.h + (long long)id.c * SC * KT);
         const int r0 = id.r0;
         const int nthreads = ex.nthreads;
-        const float floor_ = p.relu ? 0.f : -3.0e38f;   // max(s, floor_) rectifies or passes through
+        const float floor_ = p.relu ? 0.f : pass_through_floor();   // floor_f(s, floor_) rectifies or passes through
         const float eps = p.eps;
         const int need_gh = p.need_gh;
         // owned output planes [d0, d1); the rings need PD planes of lead-in and lead-out
@@ -1197,7 +1197,7 @@ struct Bwd2Kernel {
                                 gzv = gv[i][r][c] * (acc[0][i][r][c] + eps) *
                                           fast_rcp(acc[NA > 1 ? 1 : 0][i][r][c] + eps) +
                                       acc[NA - 1][i][r][c];
-                            if (p.relu && !(sv[i][r][c] > 0.f)) gzv = 0.f;
+                            if (p.relu && sv[i][r][c] <= 0.f) gzv = 0.f;   // a NaN passes
                             st.gbacc[i] += gzv;
                             v[c] = gzv;
                         }

@@ -271,7 +271,7 @@ template <int RH_> struct FwdKernelB {
         UniformF tab = as_uniform(p.wtab + (long long)id.c * kTabWords);
         const int r0 = id.r0;
         const int nthreads = ex.nthreads;
-        const float floor_ = p.relu ? 0.f : -3.0e38f;   // max(s, floor_) rectifies or passes through
+        const float floor_ = p.relu ? 0.f : pass_through_floor();   // floor_f(s, floor_) rectifies or passes through
         const float eps = p.eps;
 
         auto load_plane = [&](State &st, int k) NDC_LAMBDA {
@@ -556,7 +556,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
         UniformF tab = as_uniform(p.wtab + (long long)id.c * kTabWords);
         const int r0 = id.r0;
         const int nthreads = ex.nthreads;
-        const float floor_ = p.relu ? 0.f : -3.0e38f;
+        const float floor_ = p.relu ? 0.f : pass_through_floor();   // floor_f(s, floor_) rectifies or passes through
         const float eps = p.eps;
         const int need_gh = p.need_gh;
 
@@ -901,7 +901,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
         UniformF tab = as_uniform(p.wtab + (long long)id.c * kTabWords);
         const int r0 = id.r0;
         const int nthreads = ex.nthreads;
-        const float floor_ = p.relu ? 0.f : -3.0e38f;
+        const float floor_ = p.relu ? 0.f : pass_through_floor();   // floor_f(s, floor_) rectifies or passes through
         const float eps = p.eps;
         const int need_gh = p.need_gh;
 
@@ -1065,7 +1065,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
                                 else
                                     gzv = g * acc[0][i][r][c] * fast_rcp(acc[NA > 1 ? 1 : 0][i][r][c]) +
                                           acc[NA - 1][i][r][c];
-                                if (p.relu && !(s > 0.f)) gzv = 0.f;
+                                if (p.relu && s <= 0.f) gzv = 0.f;   // a NaN passes
                                 if (!ok) gzv = 0.f;
                                 sv[i][r][c] = ok ? s : 0.f;
                                 st.gbacc[i] += gzv;

@@ -235,7 +235,8 @@ def update_backward(x, z, h, bias, gout, groups, m, sc, eps, relu_input):
     gz = gout * n / d + op_A(gt1, h, groups, m, sc)
     if relu_input:
         pre = z if bias is None else z + bias.view(1, -1, *([1] * (z.dim() - 2)))
-        gz = torch.where(pre > 0, gz, torch.zeros_like(gz))
+        # as autograd of torch.relu: zero where the pre-activation is <= 0, so a NaN passes
+        gz = torch.where(pre <= 0, torch.zeros_like(gz), gz)
     gb = gz.sum(dim=[0] + list(range(2, gz.dim())))
     # filter gradient: (G, sc, m, *k) products, then swap to (G, m, sc, *k)
     gh_a = _shifted_products(gn, x, ks, groups, sc, m) + _shifted_products(gd, t1, ks, groups, sc, m)

@@ -222,3 +222,35 @@ def test_fused_wide_rows(geom, dtype):
             assert O.rel_err(a, r) < tol_b
     n, first = host_faults(lib)
     assert n == 0, f"LDS faults: {n} ({first})"
+
+
+@pytest.mark.parametrize("dtype,path,relu", [
+    (torch.float32, _lib.PATH_FUSED, True), (torch.float32, _lib.PATH_FUSED, False),
+    (torch.bfloat16, _lib.PATH_FUSED, True), (torch.bfloat16, _lib.PATH_FUSED, False),
+    (torch.float32, _lib.PATH_DIRECT, True), (torch.float32, _lib.PATH_DIRECT, False),
+])
+def test_nan_in_source_propagates_like_torch(dtype, path, relu):
+    """A NaN in z is handed on exactly where the reference's PyTorch arithmetic hands it on
+    (torch.relu and a plain load both propagate it; reference.py:113-118,169-173): the set of
+    non-finite entries of out, t1 and of every gradient equals the oracle's."""
+    C, sc, ks, sp = 2, 4, (3, 3, 3), (4, 16, 16)
+    lib = hostcheck_library()
+    x, z, h, bias, gout = make_case(C, C, sc, ks, sp, B=1, dtype=dtype, bias_shift=0.3,
+                                    positive_z=not relu)
+    if not relu:
+        bias = None
+    z[0, 5, 2, 7, 9] = float("nan")
+    z[0, 2, 0, 0, 0] = float("-inf") if relu else float("nan")
+    out, t1 = ops.update_forward(lib, x, z, h, bias, groups=C, m=1, sc=sc, eps=1e-16,
+                                 relu_input=relu, path=path)
+    ro, rt1, (rgx, rgz, rgh, rgb) = _oracle(x, z, h, bias, gout, C, sc, 1e-16, relu)
+    assert torch.equal(torch.isfinite(out), torch.isfinite(ro))
+    assert torch.equal(torch.isfinite(t1), torch.isfinite(rt1))
+    assert not torch.isfinite(ro).all() and torch.isfinite(ro).any()
+    gx, gz, gh, gb = ops.update_backward(lib, x, z, t1, h, bias, gout, groups=C, m=1, sc=sc,
+                                         eps=1e-16, relu_input=relu, path=path)
+    for got, ref in ((gx, rgx), (gz, rgz), (gh, rgh)):
+        assert torch.equal(torch.isfinite(got), torch.isfinite(ref))
+    fin = torch.isfinite(ro)
+    tol = 2e-2 if dtype == torch.bfloat16 else 1e-5
+    assert ((out.double() - ro)[fin].abs().max() / ro[fin].abs().max()) < tol
