@@ -358,18 +358,35 @@ DOT2_PER_CHANNEL_VOXEL = {"forward": 205, "backward_pass1": 216, "backward_pass2
 CLOCKS_PER_DOT2C = 4.52   # per SIMD, four wavefronts resident: measured by `--workload valu`
 
 
+def build_valu_probe() -> str:
+    """Compile bench_valu_probe.hip (beside this file) for gfx950 into ./bench_valu_probe; no GPU
+    needed.  Same device flags as the library (deconver_amd/build.py)."""
+    import subprocess
+
+    from deconver_amd import build as ndc_build
+
+    exe = os.path.join(ROOT, "bench_valu_probe")
+    flags = [f for f in ndc_build.HIPCC_FLAGS if f not in ("-shared", "-fPIC")]
+    subprocess.check_call([os.environ.get("HIPCC", "/opt/rocm/bin/hipcc"), *flags, "-o", exe,
+                           os.path.join(ROOT, "bench_valu_probe.hip")], stderr=subprocess.DEVNULL)
+    return exe
+
+
 def valu_workload(args) -> int:
-    """Instruction-issue probe (deconver_amd/csrc/valu_probe.hip, built by
-    `python -m deconver_amd.build --probe`): clocks per wavefront instruction per SIMD for the
+    """Instruction-issue probe (bench_valu_probe.hip, built by `python bench.py --workload valu
+    --build-probe`): clocks per wavefront instruction per SIMD for the
     multiply-accumulate forms, and from the v_dot2c_f32_bf16 figure the least time the bf16
     kernels' multiply-accumulates alone take on config 3.  `value` is that vector ceiling in
     T multiply-accumulates per second."""
     import subprocess
 
-    exe = os.path.join(ROOT, "deconver_amd", "valu_probe")
+    if args.build_probe:
+        print(build_valu_probe())
+        return 0
+    exe = os.path.join(ROOT, "bench_valu_probe")
     if not os.path.exists(exe):
-        print("bench.py --workload valu: deconver_amd/valu_probe is not built "
-              "(python -m deconver_amd.build --probe)", file=sys.stderr)
+        print("bench.py --workload valu: ./bench_valu_probe is not built "
+              "(python bench.py --workload valu --build-probe)", file=sys.stderr)
         return 2
     proc = subprocess.run([exe], stdout=subprocess.PIPE, text=True, timeout=300)
     if proc.returncode != 0:
@@ -555,6 +572,8 @@ def main() -> int:
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
+    ap.add_argument("--build-probe", action="store_true",
+                    help="with --workload valu: compile the probe (no GPU needed) and exit")
     ap.add_argument("--workload", choices=("ndc", "sweep", "accuracy", "grid", "valu", "train3d", "model2d", "mixer"),
                     default="ndc",
                     help="ndc: the headline update node (default); the others are model level")

@@ -27,6 +27,10 @@ EXPORTS = (
     "ndc_forward",
     "ndc_forward_workspace_bytes",
     "ndc_forward_noalloc",
+    "ndc_taps_bytes",
+    "ndc_prepare_taps",
+    "ndc_forward_taps",
+    "ndc_backward_taps",
     "ndc_backward_workspace_bytes",
     "ndc_backward",
     "ndc_backward_profiled",
@@ -95,6 +99,30 @@ class NdcLibrary:
                                    ctypes.c_size_t, vp]
         d.ndc_backward_profiled.argtypes = d.ndc_backward.argtypes + [ctypes.POINTER(ctypes.c_float)]
         d.ndc_gconv.argtypes = [gp, vp, fp, fp, ctypes.c_int, vp, vp]
+        d.ndc_taps_bytes.restype = ctypes.c_size_t
+        d.ndc_taps_bytes.argtypes = [gp]
+        d.ndc_prepare_taps.argtypes = [gp, fp, vp, ctypes.c_size_t, vp]
+        d.ndc_forward_taps.argtypes = [gp, vp, vp, fp, vp, fp, vp, vp, vp, vp, vp]
+        d.ndc_backward_taps.argtypes = [gp, vp, vp, vp, vp, vp, fp, vp, fp, vp, vp, vp, fp, fp, vp,
+                                        ctypes.c_size_t, vp]
+        # answers of the geometry queries, per geometry: they depend on nothing else, and a
+        # layer asks the same few questions on every call
+        self._answers = {}
+
+    @staticmethod
+    def _key(g: Geom) -> tuple:
+        return (g.batch, g.groups, g.m, g.sc, tuple(g.size), tuple(g.kernel), g.dtype,
+                g.relu_input, g.path)
+
+    def _cached(self, what: str, g: Geom, extra, ask):
+        key = (what, self._key(g), extra)
+        try:
+            return self._answers[key]
+        except KeyError:
+            if len(self._answers) > 4096:
+                self._answers.clear()
+            val = self._answers[key] = ask()
+            return val
 
     def _check(self, status: int, what: str) -> None:
         if status != 0:
@@ -105,16 +133,39 @@ class NdcLibrary:
         return self._dll.ndc_version()
 
     def fused_supported(self, g: Geom) -> bool:
-        return bool(self._dll.ndc_fused_supported(ctypes.byref(g)))
+        return self._cached("fused", g, None,
+                            lambda: bool(self._dll.ndc_fused_supported(ctypes.byref(g))))
 
     def check_geometry(self, g: Geom) -> int:
-        return self._dll.ndc_check_geometry(ctypes.byref(g))
+        return self._cached("check", g, None, lambda: self._dll.ndc_check_geometry(ctypes.byref(g)))
 
     def backward_uses_saved(self, g: Geom) -> bool:
-        return bool(self._dll.ndc_backward_uses_saved(ctypes.byref(g)))
+        return self._cached("saved", g, None,
+                            lambda: bool(self._dll.ndc_backward_uses_saved(ctypes.byref(g))))
 
     def forward_workspace_bytes(self, g: Geom) -> int:
-        return self._dll.ndc_forward_workspace_bytes(ctypes.byref(g))
+        return self._cached("fws", g, None,
+                            lambda: self._dll.ndc_forward_workspace_bytes(ctypes.byref(g)))
+
+    def taps_bytes(self, g: Geom) -> int:
+        """Bytes of a prepared filter table for ``g`` (0: its kernels read the filter itself)."""
+        return self._cached("taps", g, None, lambda: self._dll.ndc_taps_bytes(ctypes.byref(g)))
+
+    def prepare_taps(self, g: Geom, h: int, taps: int, taps_bytes: int, stream) -> None:
+        self._check(self._dll.ndc_prepare_taps(ctypes.byref(g), h, taps, taps_bytes, stream),
+                    "ndc_prepare_taps")
+
+    def forward_taps(self, g: Geom, x, z, h, taps, bias, out, t1, s_over_den, ratio, stream) -> None:
+        """``forward`` with a filter table prepared by ``prepare_taps``: no workspace."""
+        self._check(self._dll.ndc_forward_taps(ctypes.byref(g), x, z, h, taps, bias, out, t1,
+                                               s_over_den, ratio, stream), "ndc_forward_taps")
+
+    def backward_taps(self, g: Geom, x, z, t1, s_over_den, ratio, h, taps, bias, gout, gx, gz, gh,
+                      gb, ws, ws_bytes, stream) -> None:
+        self._check(
+            self._dll.ndc_backward_taps(ctypes.byref(g), x, z, t1, s_over_den, ratio, h, taps, bias,
+                                        gout, gx, gz, gh, gb, ws, ws_bytes, stream),
+            "ndc_backward_taps")
 
     def forward(self, g: Geom, x: int, z: int, h: int, bias: Optional[int], out: int,
                 t1: Optional[int], s_over_den: Optional[int], ratio: Optional[int],
@@ -130,8 +181,9 @@ class NdcLibrary:
                                                   s_over_den, ratio, stream), "ndc_forward_noalloc")
 
     def backward_workspace_bytes(self, g: Geom, need_gx, need_gz, need_gh, need_gb) -> int:
-        return self._dll.ndc_backward_workspace_bytes(
-            ctypes.byref(g), int(need_gx), int(need_gz), int(need_gh), int(need_gb))
+        flags = (int(need_gx), int(need_gz), int(need_gh), int(need_gb))
+        return self._cached("bws", g, flags, lambda: self._dll.ndc_backward_workspace_bytes(
+            ctypes.byref(g), *flags))
 
     def backward(self, g: Geom, x, z, t1, s_over_den, ratio, h, bias, gout, gx, gz, gh, gb, ws,
                  ws_bytes, stream) -> None:

@@ -2,7 +2,6 @@
 
     python -m deconver_amd.build            # libdeconver_ndc.so for gfx950
     python -m deconver_amd.build --hostcheck  # + libndc_hostcheck.so (CPU test-suite)
-    python -m deconver_amd.build --probe      # + valu_probe (instruction-issue probe, bench.py --workload valu)
 """
 
 from __future__ import annotations
@@ -43,15 +42,6 @@ def build_hip(extra_flags=()) -> str:
     return out
 
 
-def build_probe() -> str:
-    """The instruction-issue probe, a stand-alone executable."""
-    out = os.path.join(_HERE, "valu_probe")
-    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    flags = [f for f in HIPCC_FLAGS if f not in ("-shared", "-fPIC")]
-    _run([hipcc, *flags, "-o", out, os.path.join(CSRC, "valu_probe.hip")])
-    return out
-
-
 def build_hostcheck(sanitize: bool = False) -> str:
     out = os.path.join(_HERE, "libndc_hostcheck.so")
     flags = ["-O1", "-g", "-fsanitize=address,undefined"] if sanitize else ["-O2"]
@@ -64,14 +54,11 @@ def main(argv=None) -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--hostcheck", action="store_true")
     ap.add_argument("--no-hip", action="store_true")
-    ap.add_argument("--probe", action="store_true")
     args = ap.parse_args(argv)
     if not args.no_hip:
         print(build_hip())
     if args.hostcheck:
         print(build_hostcheck())
-    if args.probe:
-        print(build_probe())
 
 
 if __name__ == "__main__":

@@ -205,9 +205,24 @@ size_t ndc_forward_workspace_bytes(const ndc_geom *g)
     return fused::forward_ws(q, g->dtype);
 }
 
-int ndc_forward(const ndc_geom *g, const void *x, const void *z, const float *h,
-                const float *bias, void *out, void *t1, void *s_over_den, void *ratio,
-                void *workspace, size_t workspace_bytes, void *stream)
+size_t ndc_taps_bytes(const ndc_geom *g) { return ndc_forward_workspace_bytes(g); }
+
+int ndc_prepare_taps(const ndc_geom *g, const float *h, void *taps, size_t taps_bytes, void *stream)
+{
+    using namespace ndc;
+    KGeom q;
+    const int st = make_kgeom(g, q);
+    if (st) return st;
+    const size_t need = ndc_taps_bytes(g);
+    if (!need) return NDC_OK;
+    if (!h) return NDC_ERR_NULL;
+    if (!taps || taps_bytes < need || ((uintptr_t)taps & 255u)) return NDC_ERR_WORKSPACE;
+    return fused::prepare_taps<Backend>(q, h, (float *)taps, stream);
+}
+
+static int forward_impl(const ndc_geom *g, const void *x, const void *z, const float *h,
+                        const float *bias, void *out, void *t1, void *s_over_den, void *ratio,
+                        const void *taps, void *workspace, size_t workspace_bytes, void *stream)
 {
     using namespace ndc;
     KGeom q;
@@ -218,17 +233,19 @@ int ndc_forward(const ndc_geom *g, const void *x, const void *z, const float *h,
     const int path = choose_path(g, q);
     if (path < 0) return path;
     if (path == NDC_PATH_FUSED) {
-        const size_t need = fused::forward_ws(q, g->dtype);
+        const size_t need = taps ? 0 : fused::forward_ws(q, g->dtype);
         if (need && (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255u)))
             return NDC_ERR_WORKSPACE;
         void *ws = need ? workspace : nullptr;
+        const float *tp = fused::forward_ws(q, g->dtype) ? (const float *)taps : nullptr;
         return g->dtype == NDC_F32
                    ? fused::forward<Backend, float>(q, (const float *)x, (const float *)z, h, bias,
                                                     (float *)out, (float *)t1, (float *)s_over_den,
-                                                    (float *)ratio, ws, stream)
+                                                    (float *)ratio, tp, ws, stream)
                    : fused::forward<Backend, bf16_t>(q, (const bf16_t *)x, (const bf16_t *)z, h,
                                                      bias, (bf16_t *)out, (bf16_t *)t1,
-                                                     (bf16_t *)s_over_den, (bf16_t *)ratio, ws, stream);
+                                                     (bf16_t *)s_over_den, (bf16_t *)ratio, tp, ws,
+                                                     stream);
     }
     return g->dtype == NDC_F32
                ? direct_forward<float>(q, (const float *)x, (const float *)z, h, bias,
@@ -237,6 +254,22 @@ int ndc_forward(const ndc_geom *g, const void *x, const void *z, const float *h,
                : direct_forward<bf16_t>(q, (const bf16_t *)x, (const bf16_t *)z, h, bias,
                                         (bf16_t *)out, (bf16_t *)t1, (bf16_t *)s_over_den,
                                         (bf16_t *)ratio, stream);
+}
+
+int ndc_forward(const ndc_geom *g, const void *x, const void *z, const float *h,
+                const float *bias, void *out, void *t1, void *s_over_den, void *ratio,
+                void *workspace, size_t workspace_bytes, void *stream)
+{
+    return forward_impl(g, x, z, h, bias, out, t1, s_over_den, ratio, nullptr, workspace,
+                        workspace_bytes, stream);
+}
+
+int ndc_forward_taps(const ndc_geom *g, const void *x, const void *z, const float *h,
+                     const void *taps, const float *bias, void *out, void *t1, void *s_over_den,
+                     void *ratio, void *stream)
+{
+    if (ndc_taps_bytes(g) && (!taps || ((uintptr_t)taps & 255u))) return NDC_ERR_WORKSPACE;
+    return forward_impl(g, x, z, h, bias, out, t1, s_over_den, ratio, taps, nullptr, 0, stream);
 }
 
 int ndc_backward_uses_saved(const ndc_geom *g)
@@ -264,7 +297,7 @@ size_t ndc_backward_workspace_bytes(const ndc_geom *g, int need_gx, int need_gz,
 
 static int backward_impl(const ndc_geom *g, const void *x, const void *z, const void *t1,
                          const void *s_over_den, const void *ratio, const float *h, const float *bias,
-                         const void *gout, void *gx, void *gz, float *gh, float *gb,
+                         const void *gout, void *gx, void *gz, float *gh, float *gb, const void *taps,
                          void *workspace, size_t workspace_bytes, void *stream, float *pass_ms)
 {
     using namespace ndc;
@@ -281,17 +314,19 @@ static int backward_impl(const ndc_geom *g, const void *x, const void *z, const 
     if (need && (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255u)))
         return NDC_ERR_WORKSPACE;
     if (path == NDC_PATH_FUSED) {
+        const float *tp = fused::forward_ws(q, g->dtype) ? (const float *)taps : nullptr;
         return g->dtype == NDC_F32
                    ? fused::backward<Backend, float>(q, (const float *)x, (const float *)z,
                                                      (const float *)t1, (const float *)s_over_den,
                                                      (const float *)ratio, h, bias,
                                                      (const float *)gout, (float *)gx,
-                                                     (float *)gz, gh, gb, workspace, stream, pass_ms)
+                                                     (float *)gz, gh, gb, tp, workspace, stream, pass_ms)
                    : fused::backward<Backend, bf16_t>(q, (const bf16_t *)x, (const bf16_t *)z,
                                                       (const bf16_t *)t1, (const bf16_t *)s_over_den,
                                                       (const bf16_t *)ratio, h, bias,
                                                       (const bf16_t *)gout, (bf16_t *)gx,
-                                                      (bf16_t *)gz, gh, gb, workspace, stream, pass_ms);
+                                                      (bf16_t *)gz, gh, gb, tp, workspace, stream,
+                                                      pass_ms);
     }
     return g->dtype == NDC_F32
                ? direct_backward<float>(q, (const float *)x, (const float *)z, (const float *)t1,
@@ -307,8 +342,18 @@ int ndc_backward(const ndc_geom *g, const void *x, const void *z, const void *t1
                  const void *gout, void *gx, void *gz, float *gh, float *gb, void *workspace,
                  size_t workspace_bytes, void *stream)
 {
-    return backward_impl(g, x, z, t1, s_over_den, ratio, h, bias, gout, gx, gz, gh, gb, workspace,
-                         workspace_bytes, stream, nullptr);
+    return backward_impl(g, x, z, t1, s_over_den, ratio, h, bias, gout, gx, gz, gh, gb, nullptr,
+                         workspace, workspace_bytes, stream, nullptr);
+}
+
+int ndc_backward_taps(const ndc_geom *g, const void *x, const void *z, const void *t1,
+                      const void *s_over_den, const void *ratio, const float *h, const void *taps,
+                      const float *bias, const void *gout, void *gx, void *gz, float *gh, float *gb,
+                      void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (ndc_taps_bytes(g) && (!taps || ((uintptr_t)taps & 255u))) return NDC_ERR_WORKSPACE;
+    return backward_impl(g, x, z, t1, s_over_den, ratio, h, bias, gout, gx, gz, gh, gb, taps,
+                         workspace, workspace_bytes, stream, nullptr);
 }
 
 int ndc_backward_profiled(const ndc_geom *g, const void *x, const void *z, const void *t1,
@@ -319,8 +364,8 @@ int ndc_backward_profiled(const ndc_geom *g, const void *x, const void *z, const
 {
     if (!pass_ms) return NDC_ERR_NULL;
     pass_ms[0] = pass_ms[1] = pass_ms[2] = 0.f;
-    return backward_impl(g, x, z, t1, s_over_den, ratio, h, bias, gout, gx, gz, gh, gb, workspace,
-                         workspace_bytes, stream, pass_ms);
+    return backward_impl(g, x, z, t1, s_over_den, ratio, h, bias, gout, gx, gz, gh, gb, nullptr,
+                         workspace, workspace_bytes, stream, pass_ms);
 }
 
 int ndc_gconv(const ndc_geom *g, const void *in, const float *h, const float *bias, int adjoint,

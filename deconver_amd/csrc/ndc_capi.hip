@@ -42,6 +42,28 @@ __global__ void __launch_bounds__(512) block_kernel_entry(typename Kernel::Param
     Kernel::run(ex, p, (int)blockIdx.x);
 }
 
+// The same for a kernel that declares `kWavesPerSimd = 4`: its LDS footprint lets four
+// workgroups share a CU, so the register allocator is held to the 128 VGPRs that four
+// wavefronts per SIMD leave each lane.
+template <class Kernel>
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4)))
+block_kernel_entry_w4(typename Kernel::Params p)
+{
+    extern __shared__ float ndc_lds[];
+    DeviceExec<typename Kernel::State> ex;
+    ex.lds = ndc_lds;
+    ex.tid = threadIdx.x;
+    ex.nthreads = blockDim.x;
+    Kernel::run(ex, p, (int)blockIdx.x);
+}
+
+template <class K, class = void> struct WavesWanted {
+    static constexpr int value = 0;
+};
+template <class K> struct WavesWanted<K, decltype((void)K::kWavesPerSimd)> {
+    static constexpr int value = K::kWavesPerSimd;
+};
+
 // Event stopwatch on one stream: mark() after each stage, finish() synchronises and
 // reports the stage durations in milliseconds.
 struct HipTimer {
@@ -84,15 +106,16 @@ struct Backend {
     {
         if (nblocks <= 0) return 0;
         const size_t bytes = (size_t)lds_floats * sizeof(float);
+        void (*entry)(typename Kernel::Params) = block_kernel_entry<Kernel>;
+        if constexpr (WavesWanted<Kernel>::value == 4) entry = block_kernel_entry_w4<Kernel>;
         if (bytes > 64 * 1024) {
             // more dynamic LDS than the default cap: raise it for this kernel (idempotent)
-            if (hipFuncSetAttribute((const void *)block_kernel_entry<Kernel>,
-                                    hipFuncAttributeMaxDynamicSharedMemorySize,
+            if (hipFuncSetAttribute((const void *)entry, hipFuncAttributeMaxDynamicSharedMemorySize,
                                     (int)bytes) != hipSuccess)
                 return -5;
         }
-        hipLaunchKernelGGL(block_kernel_entry<Kernel>, dim3((unsigned)nblocks),
-                           dim3((unsigned)nthreads), bytes, (hipStream_t)stream, p);
+        hipLaunchKernelGGL(entry, dim3((unsigned)nblocks), dim3((unsigned)nthreads), bytes,
+                           (hipStream_t)stream, p);
         return check();
     }
 

@@ -93,13 +93,15 @@ static const int kMaxLdsBytes = 160 * 1024;
 
 // S strips of RH rows, RW columns per thread; S >= 2*PH so that the halo rows fit the
 // fixed per-thread bounds
-static inline bool make_tile(const March &m, int RH, int RW, int target_threads, Tile &t)
+static inline bool make_tile(const March &m, int RH, int RW, int target_threads, Tile &t,
+                             int min_strips = 0)
 {
     const int PH = m.KH / 2, PW = m.KW / 2;
     if (m.W % RW) return false;
     const int cpw = m.W / RW;
     if (cpw > kMaxThreads) return false;
     int smin = PH > 0 ? 2 * PH : 1;
+    if (smin < min_strips) smin = min_strips;
     int s = target_threads / cpw;
     const int srows = (m.H + RH - 1) / RH;
     if (s > srows) s = srows;

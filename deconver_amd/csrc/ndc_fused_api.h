@@ -31,30 +31,34 @@ struct Variant {
     int KD, KH, KW, SC, RHF, RWF, RHB, RWB;
 };
 
-// Launch-shape choices that are not dictated by the geometry.  Defaults are the measured
-// best; the environment variables exist for tuning runs only.
+// Launch-shape choices that are not dictated by the geometry: the measured best, fixed at
+// compile time.  A tuning build (-DNDC_TUNING, never the shipped library) reads them from
+// NDC_TUNE_* environment variables once, at the first call.
 struct Tuning {
-    int rhf, rwf, rhb, rwb, threads_f, threads_b, threads_b2;
+    int rhf, rwf, rhb, rwb;      // forced register tiles (0: the table's order of preference)
+    int threads_f, threads_b;    // workgroup sizes of the FMA kernels, forward / backward
+    int threads_f2, threads_b2;  // ... of the bf16 dot2 kernels
+    int split, dot2;             // march segments on / bf16 dot2 kernels on
 };
 
+#ifdef NDC_TUNING
 static inline int env_int(const char *name, int dflt)
 {
     const char *v = getenv(name);
     return v && *v ? atoi(v) : dflt;
 }
-
-static inline Tuning tuning()
+static inline const Tuning &tuning()
 {
-    Tuning t;
-    t.rhf = env_int("NDC_TUNE_RHF", 0);
-    t.rwf = env_int("NDC_TUNE_RWF", 0);
-    t.rhb = env_int("NDC_TUNE_RHB", 0);
-    t.rwb = env_int("NDC_TUNE_RWB", 0);
-    t.threads_f = env_int("NDC_TUNE_NTF", 256);
-    t.threads_b = env_int("NDC_TUNE_NTB", 512);
-    t.threads_b2 = env_int("NDC_TUNE_NTB", 256);   // bf16 dot2 kernels
+    static const Tuning t = {env_int("NDC_TUNE_RHF", 0),  env_int("NDC_TUNE_RWF", 0),
+                             env_int("NDC_TUNE_RHB", 0),  env_int("NDC_TUNE_RWB", 0),
+                             env_int("NDC_TUNE_NTF", 256), env_int("NDC_TUNE_NTB", 512),
+                             env_int("NDC_TUNE_NTF2", 256), env_int("NDC_TUNE_NTB2", 256),
+                             env_int("NDC_TUNE_SPLIT", 1), env_int("NDC_TUNE_DOT2", 1)};
     return t;
 }
+#else
+static inline Tuning tuning() { return Tuning{0, 0, 0, 0, 256, 512, 256, 256, 1, 1}; }
+#endif
 
 // first listed row of this filter geometry that the width / alignment allow (and, in a
 // tuning run, that matches the requested register tiles)
@@ -125,7 +129,7 @@ static inline bool make_plan(const KGeom &q, Plan &pl, bool pairs_ok = true, int
     const Tuning tn = tuning();
     if (!make_tile(pl.m, pl.v.RHF, pl.v.RWF, tn.threads_f, pl.tf)) return false;
     if (!make_tile(pl.m, pl.v.RHB, pl.v.RWB, tn.threads_b, pl.tb)) return false;
-    if (env_int("NDC_TUNE_SPLIT", 1)) {
+    if (tn.split) {
         split_march(pl.m, (long long)q.B * q.G * pl.tf.ntile, pl.tf);
         split_march(pl.m, (long long)q.B * q.G * pl.tb.ntile, pl.tb);
     }
@@ -135,9 +139,9 @@ static inline bool make_plan(const KGeom &q, Plan &pl, bool pairs_ok = true, int
     NDC_FUSED_VARIANTS(X)
 #undef X
     if (dtype == NDC_BF16 && pairs_ok && pl.m.W % 2 == 0 && q.sc == 4 && pl.m.KD == 3 &&
-        pl.m.KH == 3 && pl.m.KW == 3 && env_int("NDC_TUNE_DOT2", 1)) {
+        pl.m.KH == 3 && pl.m.KW == 3 && tn.dot2) {
         Tile tf, tb;
-        if (make_tile(pl.m, kDot2RH, 2, tn.threads_f, tf) &&
+        if (make_tile(pl.m, kDot2RH, 2, tn.threads_f2, tf, FwdKernelB<kDot2RH>::kMinStrips) &&
             make_tile(pl.m, kDot2RH, 2, tn.threads_b2, tb)) {
             const int lf = FwdKernelB<kDot2RH>::lds_floats(tf);
             const int l1 = Bwd1KernelB<kDot2RH>::lds_floats(tb);
@@ -234,15 +238,25 @@ template <class BE> struct Dot2Launch<BE, bf16_t> {
     }
 };
 
+// the packed filter tables of the bf16 dot2 kernels: G * kTabWords words from h
+template <class BE> static int prepare_taps(const KGeom &q, const float *h, float *tab, void *stream)
+{
+    return BE::elementwise((long long)q.G * kTabWords, stream,
+                           [=] NDC_LAMBDA(long long idx) { prep_tables(idx, h, tab); });
+}
+
 template <class BE, typename T>
 static int forward(const KGeom &q, const T *x, const T *z, const float *h, const float *bias,
-                   T *out, T *t1, T *s_over_den, T *ratio, void *ws, void *stream)
+                   T *out, T *t1, T *s_over_den, T *ratio, const float *taps, void *ws,
+                   void *stream)
 {
+    // taps: packed filter tables prepared earlier for this h (prepare_taps), or null: then
+    // they are packed into ws by a small launch ahead of the kernel
     Plan pl;
     const bool pairs = pair_aligned<T>(x) && pair_aligned<T>(z) && pair_aligned<T>(out) &&
                        pair_aligned<T>(t1) && pair_aligned<T>(s_over_den) && pair_aligned<T>(ratio);
     const int dtype = sizeof(T) == 2 ? NDC_BF16 : NDC_F32;
-    if (!make_plan(q, pl, pairs, ws ? dtype : NDC_F32)) return NDC_ERR_GEOMETRY;
+    if (!make_plan(q, pl, pairs, (ws || taps) ? dtype : NDC_F32)) return NDC_ERR_GEOMETRY;
     FwdParams<T> p;
     p.wtab = nullptr;
     p.x = x;
@@ -262,11 +276,14 @@ static int forward(const KGeom &q, const T *x, const T *z, const float *h, const
     p.eps = q.eps;
     p.t = pl.tf;
     if (pl.dot2) {
-        float *tab = (float *)ws;
-        const int st = BE::elementwise((long long)q.G * kTabWords, stream,
-                                       [=] NDC_LAMBDA(long long idx) { prep_tables(idx, h, tab); });
-        if (st) return st;
-        p.wtab = tab;
+        if (taps) {
+            p.wtab = taps;
+        } else {
+            float *tab = (float *)ws;
+            const int st = prepare_taps<BE>(q, h, tab, stream);
+            if (st) return st;
+            p.wtab = tab;
+        }
         return Dot2Launch<BE, T>::fwd(p, pl, stream);
     }
 #define X(kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_)                                          \
@@ -281,7 +298,8 @@ static int forward(const KGeom &q, const T *x, const T *z, const float *h, const
 template <class BE, typename T>
 static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const T *s_over_den,
                     const T *ratio, const float *h, const float *bias, const T *gout, T *gx,
-                    T *gz, float *gh, float *gb, void *ws, void *stream, float *pass_ms = nullptr)
+                    T *gz, float *gh, float *gb, const float *taps, void *ws, void *stream,
+                    float *pass_ms = nullptr)
 {
     // pass_ms (optional, 3 floats): device time of pass 1, pass 2 and the partial-sum
     // reduction, taken with events on `stream`; makes the call synchronous
@@ -332,10 +350,13 @@ static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const T
     p.part = part1;
     p.part_stride = kt;
     if (pl.dot2) {
-        st = BE::elementwise((long long)q.G * kTabWords, stream,
-                             [=] NDC_LAMBDA(long long idx) { prep_tables(idx, h, tab); });
-        if (st) return st;
-        p.wtab = tab;
+        if (taps) {
+            p.wtab = taps;
+        } else {
+            st = prepare_taps<BE>(q, h, tab, stream);
+            if (st) return st;
+            p.wtab = tab;
+        }
         st = Dot2Launch<BE, T>::bwd1(p, pl, stream, saved);
     } else {
 #define X(kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_)                                          \

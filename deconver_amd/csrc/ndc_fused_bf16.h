@@ -12,6 +12,13 @@
 //                               + P[j]   . (0,           h[i,0,th,tw])
 //     : 2 dot2 per (th, tw) instead of 3 FMAs.  The producer of plane m+1 completes word m
 //     from the value of plane m it kept in a register.
+//     The forward and the kept-ratio pass 2 replace the half-empty second term by COLUMN
+//     pairs of plane j+1, which arrive from global memory (or leave for it) in that form:
+//     with Q[c] = (v[2c], v[2c+1]) of plane j+1, per input row
+//       column 2c  :  Q[c] . (h1, h0) + Q[c-1] . (0,  h2)        h_tw = h[i,0,th,tw]
+//       column 2c+1:  Q[c] . (h2, h1) + Q[c+1] . (h0, 0)
+//     : 4 dot2 per column pair for the 6 products of a tap row, 15 instead of 18 dot2 per
+//     output voxel and source channel.
 //   The filter-gradient terms pair OPERANDS: (gn_i, gd_i) . (x, t1)[neighbour] in pass 1,
 //     and (s_i[j-1], s_i[j]) . (gt1[m], gt1[m+1])[neighbour] every second plane in pass 2.
 //
@@ -22,6 +29,8 @@
 //   WK[p][tau]        = (h[2p][tau], h[2p+1][tau])            p = 0, 1       54 words
 //   WA[s][i][th][tw]  = s = 0: (h[i][2][th][tw], h[i][1][th][tw])
 //                       s = 1: (0,               h[i][0][th][tw])             72 words
+//   WQ[th][i][n]      = n = 0: (h1, h0)  1: (0, h2)  2: (h2, h1)  3: (h0, 0),
+//                       h_tw = h[i][0][th][tw]                                  48 words
 #pragma once
 
 #include "ndc_fused.h"
@@ -29,7 +38,8 @@
 namespace ndc {
 namespace fused {
 
-static const int kTabWords = 126;   // packed tap words per channel (54 WK + 72 WA)
+static const int kTabWK = 0, kTabWA = 54, kTabWQ = 126;
+static const int kTabWords = 174;   // packed tap words per channel (54 WK + 72 WA + 48 WQ)
 
 // idx over C * kTabWords
 NDC_HD void prep_tables(long long idx, const float *h, float *tab)
@@ -40,10 +50,15 @@ NDC_HD void prep_tables(long long idx, const float *h, float *tab)
     if (e < 54) {
         const int p = e / 27, tau = e % 27;
         w = pack_bf16x2(hc[(2 * p) * 27 + tau], hc[(2 * p + 1) * 27 + tau]);
-    } else {
+    } else if (e < kTabWQ) {
         const int r = e - 54, s = r / 36, i = (r % 36) / 9, t9 = r % 9;
         w = s == 0 ? pack_bf16x2(hc[i * 27 + 2 * 9 + t9], hc[i * 27 + 1 * 9 + t9])
                    : pack_bf16x2(0.f, hc[i * 27 + t9]);
+    } else {
+        const int r = e - kTabWQ, th = r / 16, i = (r % 16) / 4, n = r % 4;
+        const float *ht = hc + i * 27 + th * 3;   // the tap row h[i][0][th][0..2]
+        w = n == 0 ? pack_bf16x2(ht[1], ht[0]) : n == 1 ? pack_bf16x2(0.f, ht[2])
+          : n == 2 ? pack_bf16x2(ht[2], ht[1]) : pack_bf16x2(ht[0], 0.f);
     }
     tab[idx] = bits_to_float(w);
 }
@@ -177,6 +192,77 @@ NDC_D void a_plane_d2(Exec &ex, const int (&base)[NTEN], int P, const float (&wt
     }
 }
 
+// The depth tap td = 0 of an A-type application (input plane j + 1) from column-pair words:
+// base[t] = word (first output row - 1, own column pair - 1) of operand t's plane, staged
+// with row pitch PQ; wq = WQ of the channel.  Rolled over the tap rows: 16 packed taps in
+// scalar registers per iteration, NR rows of three words read for each.
+template <int NR, int NTEN, class Exec>
+NDC_D void a_plane_q(Exec &ex, const int (&base)[NTEN], int PQ, UniformF wq,
+                     float (&acc)[NTEN][4][NR][2])
+{
+#ifndef NDC_AQ_MODE
+#define NDC_AQ_MODE 0
+#endif
+#if NDC_AQ_MODE == 0
+    NDC_ROLLED
+    for (int thh = 0; thh < 3; ++thh) {
+        const int th = uniform_int(thh);
+        float w[16];
+        load_taps<16>(wq + th * 16, w);
+        NDC_UNROLL
+        for (int r = 0; r < NR; ++r) {
+            const int at = (r + 2 - th) * PQ;
+            uint32_t v[NTEN][3];
+            NDC_UNROLL
+            for (int t = 0; t < NTEN; ++t)
+                NDC_UNROLL
+                for (int u = 0; u < 3; ++u) v[t][u] = float_to_bits(ex.ld(base[t] + at + u));
+            NDC_UNROLL
+            for (int i = 0; i < 4; ++i)
+                NDC_UNROLL
+                for (int t = 0; t < NTEN; ++t) {
+                    float a0 = acc[t][i][r][0], a1 = acc[t][i][r][1];
+                    a0 = dot2_bf16(v[t][1], float_to_bits(w[i * 4 + 0]), a0);
+                    a1 = dot2_bf16(v[t][1], float_to_bits(w[i * 4 + 2]), a1);
+                    a0 = dot2_bf16(v[t][0], float_to_bits(w[i * 4 + 1]), a0);
+                    a1 = dot2_bf16(v[t][2], float_to_bits(w[i * 4 + 3]), a1);
+                    acc[t][i][r][0] = a0;
+                    acc[t][i][r][1] = a1;
+                }
+        }
+    }
+#else
+    // input rows in order, each read once; all 48 packed taps in scalar registers
+    float w[48];
+    load_taps<48>(wq, w);
+    NDC_UNROLL
+    for (int q = 0; q < NR + 2; ++q) {
+        uint32_t v[NTEN][3];
+        NDC_UNROLL
+        for (int t = 0; t < NTEN; ++t)
+            NDC_UNROLL
+            for (int u = 0; u < 3; ++u) v[t][u] = float_to_bits(ex.ld(base[t] + q * PQ + u));
+        NDC_UNROLL
+        for (int th = 0; th < 3; ++th) {
+            const int r = q - 2 + th;
+            if (r < 0 || r >= NR) continue;
+            NDC_UNROLL
+            for (int i = 0; i < 4; ++i)
+                NDC_UNROLL
+                for (int t = 0; t < NTEN; ++t) {
+                    float a0 = acc[t][i][r][0], a1 = acc[t][i][r][1];
+                    a0 = dot2_bf16(v[t][1], float_to_bits(w[th * 16 + i * 4 + 0]), a0);
+                    a1 = dot2_bf16(v[t][1], float_to_bits(w[th * 16 + i * 4 + 2]), a1);
+                    a0 = dot2_bf16(v[t][0], float_to_bits(w[th * 16 + i * 4 + 1]), a0);
+                    a1 = dot2_bf16(v[t][2], float_to_bits(w[th * 16 + i * 4 + 3]), a1);
+                    acc[t][i][r][0] = a0;
+                    acc[t][i][r][1] = a1;
+                }
+        }
+    }
+#endif
+}
+
 // NROWS rows of NW staged words each, row n at addr(n), handed to body(n, words) with the
 // reads running one row ahead (PIPE, see k_rows_d2).
 template <int NW, class Exec> NDC_D void read_row(Exec &ex, int at, uint32_t (&v)[NW])
@@ -222,10 +308,15 @@ NDC_D void stream_rows(Exec &ex, Addr addr, Body body, const uint32_t (*first)[N
 template <int RH_> struct FwdKernelB {
     static constexpr int KD = 3, KH = 3, KW = 3, SC = 4, RH = RH_, RW = 2;
     static constexpr int PD = 1, PH = 1, PW = 1, KT = 27;
-    static constexpr int RHK = RH + 1, NZR = RH + 2, NXR = RH + 1;
+    // staging slots per thread: thread (strip, lane) stages rows strip, strip + S, ... of the
+    // TH + 4 source rows and TH + 2 x rows; with S >= kMinStrips strips, RH + 1 slots cover both
+    static constexpr int kMinStrips = 4;
+    static constexpr int RHK = RH + 1, NZR = RH + 1, NXR = RH + 1;
     // ring slots: source (one: it is only read in the scatter phase of the step that staged
-    // it), x pairs, t1 pairs
+    // it), x pairs, t1 pairs; plus one plane each of x and t1 as column-pair words (written
+    // in the scatter phase, read in the gather phase of the same step)
     static constexpr int NS = 1, NX = 2, NTP = 2;
+    static constexpr int kWavesPerSimd = 4;   // LDS leaves room for four workgroups per CU
     typedef bf16_t T;
     typedef FwdParams<T> Params;
     typedef VecIO<T, 2> IO;
@@ -236,16 +327,18 @@ template <int RH_> struct FwdKernelB {
         unsigned zok, xok, ook;
         float bv[SC];
         float t1acc[KD][RHK][RW];
-        float t1prev[RHK][RW];
+        uint32_t t1prev[RHK];       // previous t1 plane of the own rows, as column pairs
         uint32_t pz[SC][NZR];       // staged source rows, raw (two bf16 columns per word)
         uint32_t px[NXR], pxprev[NXR];
     };
 
     static NDC_HD int rows_s(int TH) { return TH + 4; }
     static NDC_HD int rows_x(int TH) { return TH + 2; }
+    // row pitch of a column-pair plane: W/2 words and a zero word on either side
+    static NDC_HD int pitch_q(const Tile &t) { return t.CPW + 2; }
     static NDC_HD int lds_floats(const Tile &t)
     {
-        return (NS * 2 * rows_s(t.TH) + (NX + NTP) * rows_x(t.TH)) * t.P;
+        return (NS * 2 * rows_s(t.TH) + (NX + NTP) * rows_x(t.TH)) * t.P + 2 * rows_x(t.TH) * pitch_q(t);
     }
 
     template <class Exec> static NDC_D void run(Exec &ex, const Params &p, int block_id)
@@ -255,7 +348,9 @@ template <int RH_> struct FwdKernelB {
         const int S = t.S, P = t.P, PL = t.PL, TH = t.TH, W = p.W, H = p.H, D = p.D;
         const int RS = rows_s(TH), RX = rows_x(TH);
         const int off_s = 0, off_x = NS * 2 * RS * P, off_t = off_x + NX * RX * P;
-        const int total = off_t + NTP * RX * P;
+        const int PQ = pitch_q(t);
+        const int off_qx = off_t + NTP * RX * P, off_qt = off_qx + RX * PQ;
+        const int total = off_qt + RX * PQ;
         const int plane = H * W;
         const long long cplane = (long long)D * plane;
         // this workgroup's (sample, channel) slices; offsets inside them fit 32 bits
@@ -320,7 +415,8 @@ template <int RH_> struct FwdKernelB {
                 }
             }
         };
-        // x plane k - 1 completes the plane-pair word (x[k-2], x[k-1]) of slot (k - 2) % 2.
+        // x plane k - 1 completes the plane-pair word (x[k-2], x[k-1]) of slot (k - 2) % 2 and
+        // is kept as column pairs for the gather of plane k - 2.
         // Runs in the scatter phase (a barrier after the gather that last read that slot), which
         // is what lets two slots do.
         auto store_x_pairs = [&](State &st, int k) NDC_LAMBDA {
@@ -332,6 +428,8 @@ template <int RH_> struct FwdKernelB {
                     const int j = st.ln.strip + n * S;
                     ex.st_(xb + j * P + lb, bits_to_float(zip_lo(st.pxprev[n], st.px[n])));
                     ex.st_(xb + j * P + lb + 1, bits_to_float(zip_hi(st.pxprev[n], st.px[n])));
+                    // plane k - 1 as it came from memory: the column-pair word of this lane
+                    ex.st_(off_qx + j * PQ + 1 + (st.ln.c0 >> 1), bits_to_float(st.px[n]));
                 }
                 st.pxprev[n] = st.px[n];
             }
@@ -364,13 +462,13 @@ template <int RH_> struct FwdKernelB {
             NDC_UNROLL
             for (int i = 0; i < SC; ++i) st.bv[i] = p.bias ? p.bias[id.c * SC + i] : 0.f;
             NDC_UNROLL
-            for (int r = 0; r < RHK; ++r)
+            for (int r = 0; r < RHK; ++r) {
+                st.t1prev[r] = 0u;
                 NDC_UNROLL
-                for (int c = 0; c < RW; ++c) {
-                    st.t1prev[r][c] = 0.f;
+                for (int c = 0; c < RW; ++c)
                     NDC_UNROLL
                     for (int a = 0; a < KD; ++a) st.t1acc[a][r][c] = 0.f;
-                }
+            }
             for (int i = tid; i < total; i += nthreads) ex.st_(i, 0.f);
             load_plane(st, 0);
         });
@@ -410,15 +508,17 @@ template <int RH_> struct FwdKernelB {
                     const int j = r < RH ? PH + st.ln.strip * RH + r : jx;
                     const int row = r0 - PH + j;
                     const bool live = inplane && row >= 0 && row < H;
-                    float v[RW];
-                    NDC_UNROLL
-                    for (int c = 0; c < RW; ++c) {
-                        v[c] = live ? st.t1acc[0][r][c] : 0.f;
-                        if (mine) ex.st_(tb + j * P + c, bits_to_float(pack_bf16x2(st.t1prev[r][c], v[c])));
-                        st.t1prev[r][c] = v[c];
+                    // the plane as column pairs: kept for the gather of plane k - 2, zipped with
+                    // the previous plane's into the plane-pair words, and stored as t1
+                    const uint32_t vq = live ? pack_bf16x2(st.t1acc[0][r][0], st.t1acc[0][r][1]) : 0u;
+                    if (mine) {
+                        ex.st_(tb + j * P, bits_to_float(zip_lo(st.t1prev[r], vq)));
+                        ex.st_(tb + j * P + 1, bits_to_float(zip_hi(st.t1prev[r], vq)));
+                        ex.st_(off_qt + j * PQ + 1 + (st.ln.c0 >> 1), bits_to_float(vq));
                     }
+                    st.t1prev[r] = vq;
                     if (r < RH && have_t1 && live)
-                        buf_st(tb_, st.ooff[r < RH ? r : 0], (unsigned)pf * plane2, pack_bf16x2(v[0], v[1]));
+                        buf_st(tb_, st.ooff[r < RH ? r : 0], (unsigned)pf * plane2, vq);
                     NDC_UNROLL
                     for (int c = 0; c < RW; ++c) {
                         st.t1acc[0][r][c] = st.t1acc[1][r][c];
@@ -452,15 +552,21 @@ template <int RH_> struct FwdKernelB {
                         for (int r = 0; r < RH; ++r)
                             NDC_UNROLL
                             for (int c = 0; c < RW; ++c) acc[a][i][r][c] = eps;   // n, d start at eps
-                NDC_ROLLED
-                for (int s = 0; s < 2; ++s) {
+                {
+                    // depth taps 2 and 1 from the plane-pair words (x, t1)[j0-1 .. j0]
                     float wt[SC][9];
-                    load_plane_taps<SC, 9, 9>(tab + 54 + s * 36, wt);
-                    const int m = j0 - 1 + s;
+                    load_plane_taps<SC, 9, 9>(tab + kTabWA, wt);
+                    const int m = j0 - 1;
                     const int ob = (st.ln.strip * RH) * P + PL + st.ln.c0 - PW;
                     const int base[2] = {off_x + wrap(m % NX, NX) * RX * P + ob,
                                          off_t + wrap(m % NTP, NTP) * RX * P + ob};
                     a_plane_d2<RH, RW, 2, false>(ex, base, P, wt, acc);
+                }
+                {
+                    // depth tap 0 from the column-pair words of plane j0 + 1
+                    const int oq = (st.ln.strip * RH) * PQ + (st.ln.c0 >> 1);
+                    const int base[2] = {off_qx + oq, off_qt + oq};
+                    a_plane_q<RH, 2>(ex, base, PQ, tab + kTabWQ, acc);
                 }
                 const unsigned oj = (unsigned)j0 * plane2;
                 NDC_UNROLL

@@ -65,7 +65,7 @@ class DeconvUpdate(torch.autograd.Function):
     """``out = relu(z + b) * (A(x) + eps) / (A(K(relu(z + b))) + eps)``."""
 
     @staticmethod
-    def forward(ctx, x, z, h, bias, groups, m, sc, eps, relu_input):
+    def forward(ctx, x, z, h, bias, groups, m, sc, eps, relu_input, taps=None):
         if not x.is_cuda:
             raise RuntimeError("deconv_update runs on the GPU only (HIP kernels); "
                                "CPU tensors take the layer's general PyTorch path")
@@ -80,11 +80,16 @@ class DeconvUpdate(torch.autograd.Function):
             keep = lib.backward_uses_saved(
                 ops.make_geom_for(x, hc, groups, m, sc, eps, relu_input))
         with torch.cuda.device(x.device):
+            if taps is None:
+                # packed once here, used by the forward kernel and again by the backward's
+                taps = ops.prepare_taps(lib, x, hc, groups=groups, m=m, sc=sc)
             res = ops.update_forward(lib, x, z, hc, bias, groups=groups, m=m, sc=sc, eps=eps,
-                                     relu_input=relu_input, need_t1=need_t1, save_ratio=keep)
+                                     relu_input=relu_input, need_t1=need_t1, save_ratio=keep,
+                                     taps=taps)
         out, t1 = res[0], res[1]
         s_over_den, ratio = res[2] if keep else (None, None)
         ctx.cfg = (groups, m, sc, eps, relu_input)
+        ctx.taps = taps if need_t1 else None   # a function of h alone; h is saved below
         ctx.save_for_backward(x, z, t1, hc, bias, s_over_den, ratio)
         return out
 
@@ -111,12 +116,13 @@ class DeconvUpdate(torch.autograd.Function):
                 lib, x, z, t1, h, bias, gout, groups=groups, m=m, sc=sc, eps=eps,
                 relu_input=relu_input, need_x=need_x, need_z=need_z, need_h=need_h,
                 need_b=need_b and bias is not None,
-                saved=None if s_over_den is None else (s_over_den, ratio))
-        return gx, gz, gh, gb, None, None, None, None, None
+                saved=None if s_over_den is None else (s_over_den, ratio), taps=ctx.taps)
+        return gx, gz, gh, gb, None, None, None, None, None, None
 
 
 def deconv_update(x: Tensor, z: Tensor, h: Tensor, bias: Optional[Tensor], *, groups: int,
-                  m: int, sc: int, eps: float, relu_input: bool) -> Tensor:
+                  m: int, sc: int, eps: float, relu_input: bool,
+                  taps: Optional[Tensor] = None) -> Tensor:
     """One multiplicative source update.
 
     Args:
@@ -126,5 +132,7 @@ def deconv_update(x: Tensor, z: Tensor, h: Tensor, bias: Optional[Tensor], *, gr
         h: rectified filter ``(C, sc, *k)``, float32.
         bias: the projection's bias (float32) or ``None``.
         eps: stabiliser added to numerator and denominator.
+        taps: optional (not in the reference): the table ``ops.prepare_taps`` made for this
+            ``h``, for callers that run several updates with one filter; made here otherwise.
     """
-    return DeconvUpdate.apply(x, z, h, bias, groups, m, sc, eps, relu_input)
+    return DeconvUpdate.apply(x, z, h, bias, groups, m, sc, eps, relu_input, taps)

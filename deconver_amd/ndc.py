@@ -35,6 +35,8 @@ import torch.nn.functional as F
 from torch import Tensor, nn
 
 from . import operations as ops_general
+from . import ops
+from ._lib import get_library
 from .functional import deconv_update, hip_kernels_apply
 from .layers import Linear
 
@@ -185,10 +187,15 @@ class Deconv(nn.Module):
         s = F.conv1d(x.flatten(2), proj.weight.to(dtype), None).view(x.shape[0], -1, *x.shape[2:])
         first = dict(bias=None if proj.bias is None else proj.bias.float(), relu_input=True)
         later = dict(bias=None, relu_input=False)
+        taps = None
+        if self.num_iters > 1:   # one filter table for all iterations (a single one makes its own)
+            with torch.no_grad(), torch.cuda.device(x.device):
+                taps = ops.prepare_taps(get_library(), x, h.detach().contiguous(), groups=self.groups,
+                                        m=self.filter_channels, sc=self.source_channels)
         for it in range(1, self.num_iters + 1):
             with self.context(it):
                 s = deconv_update(x, s, h, groups=self.groups, m=self.filter_channels,
-                                  sc=self.source_channels, eps=self.eps,
+                                  sc=self.source_channels, eps=self.eps, taps=taps,
                                   **(first if it == 1 else later))
         return s, h
 

@@ -64,10 +64,27 @@ def make_geom_for(x: Tensor, h: Tensor, groups: int, m: int, sc: int, eps: float
                           dtype_tag(x.dtype), relu_input, eps, path)
 
 
+def prepare_taps(lib: _lib.NdcLibrary, x: Tensor, h: Tensor, *, groups: int, m: int,
+                 sc: int) -> Optional[Tensor]:
+    """The filter table the kernels for this geometry read instead of ``h`` (today: the packed
+    bfloat16 tap pairs of the 3x3x3 dot2 kernels), or ``None`` if they read ``h`` itself.  One
+    small launch; valid for every update with this ``h`` on tensors of ``x``'s shape and
+    dtype, forward and backward, until ``h`` changes."""
+    g = make_geom_for(x, h, groups, m, sc, 0.0, True)
+    nbytes = lib.taps_bytes(g)
+    if not nbytes:
+        return None
+    buf = torch.empty(nbytes + 256, dtype=torch.uint8, device=x.device)
+    off = -buf.data_ptr() % 256
+    taps = buf[off:off + nbytes]   # 256-byte aligned view
+    lib.prepare_taps(g, _ptr(h), _ptr(taps), nbytes, _stream_of(x))
+    return taps
+
+
 def update_forward(lib: _lib.NdcLibrary, x: Tensor, z: Tensor, h: Tensor,
                    bias: Optional[Tensor], *, groups: int, m: int, sc: int, eps: float,
                    relu_input: bool, need_t1: bool = True, save_ratio: bool = False,
-                   path: int = _lib.PATH_AUTO):
+                   path: int = _lib.PATH_AUTO, taps: Optional[Tensor] = None):
     """``out = s*(A(x)+eps)/(A(K(s))+eps)`` with ``s = relu?(z+bias)``.
 
     Returns ``(out, t1)``, or ``(out, t1, (s_over_den, ratio))`` with ``save_ratio``: the two
@@ -78,15 +95,19 @@ def update_forward(lib: _lib.NdcLibrary, x: Tensor, z: Tensor, h: Tensor,
     out = torch.empty_like(z)
     want_t1 = need_t1 or not lib.fused_supported(g) or path == _lib.PATH_DIRECT
     t1 = torch.empty_like(x) if want_t1 else None
-    nbytes = lib.forward_workspace_bytes(g)
-    ws_ptr = None
-    if nbytes:
-        ws = torch.empty(nbytes + 256, dtype=torch.uint8, device=x.device)
-        ws_ptr = (ws.data_ptr() + 255) // 256 * 256
     s_over_den = torch.empty_like(z) if save_ratio else None
     ratio = torch.empty_like(z) if save_ratio else None
-    lib.forward(g, _ptr(x), _ptr(z), _ptr(h), _ptr(bias), _ptr(out), _ptr(t1), _ptr(s_over_den),
-                _ptr(ratio), ws_ptr, nbytes, _stream_of(x))
+    if taps is not None:
+        lib.forward_taps(g, _ptr(x), _ptr(z), _ptr(h), _ptr(taps), _ptr(bias), _ptr(out), _ptr(t1),
+                         _ptr(s_over_den), _ptr(ratio), _stream_of(x))
+    else:
+        nbytes = lib.forward_workspace_bytes(g)
+        ws_ptr = None
+        if nbytes:
+            ws = torch.empty(nbytes + 256, dtype=torch.uint8, device=x.device)
+            ws_ptr = (ws.data_ptr() + 255) // 256 * 256
+        lib.forward(g, _ptr(x), _ptr(z), _ptr(h), _ptr(bias), _ptr(out), _ptr(t1),
+                    _ptr(s_over_den), _ptr(ratio), ws_ptr, nbytes, _stream_of(x))
     if save_ratio:
         return out, t1, (s_over_den, ratio)
     return out, t1
@@ -97,11 +118,14 @@ def update_backward(lib: _lib.NdcLibrary, x: Tensor, z: Tensor, t1: Tensor, h: T
                     eps: float, relu_input: bool, need_x: bool = True, need_z: bool = True,
                     need_h: bool = True, need_b: bool = True,
                     path: int = _lib.PATH_AUTO, pass_times: Optional[list] = None,
-                    saved: Optional[Tuple[Tensor, Tensor]] = None):
+                    saved: Optional[Tuple[Tensor, Tensor]] = None,
+                    taps: Optional[Tensor] = None):
     """Gradients ``(gx, gz, gh, gb)`` of the update; entries not asked for are ``None``.
 
     ``saved``: the ``(s_over_den, ratio)`` pair a ``save_ratio`` forward call returned for the
     same inputs.
+
+    ``taps``: the table :func:`prepare_taps` made for this ``h`` (skips packing it again).
 
     ``pass_times``: a list that, if given, receives the device milliseconds of the three
     backward stages (the call then synchronises)."""
@@ -128,7 +152,9 @@ def update_backward(lib: _lib.NdcLibrary, x: Tensor, z: Tensor, t1: Tensor, h: T
     args = (g, _ptr(x), _ptr(z), _ptr(t1), _ptr(s_over_den), _ptr(ratio), _ptr(h), _ptr(bias),
             _ptr(gout), _ptr(gx),
             _ptr(gz), _ptr(gh), _ptr(gb), ws_ptr, nbytes, _stream_of(x))
-    if pass_times is None:
+    if taps is not None and pass_times is None:
+        lib.backward_taps(*args[:7], _ptr(taps), *args[7:])
+    elif pass_times is None:
         lib.backward(*args)
     else:
         pass_times[:] = lib.backward_profiled(*args)

@@ -126,6 +126,32 @@ int ndc_forward_noalloc(const ndc_geom *g, const void *x, const void *z, const f
                         const float *bias, void *out, void *t1, void *s_over_den, void *ratio,
                         void *stream);
 
+/*
+ * Prepared filter tables.  Some kernel families read the filter from a packed table instead
+ * of `h` (today: the bfloat16 3x3x3 kernels, 504 bytes per channel).  ndc_forward and
+ * ndc_backward pack it into their workspace on every call; a caller that runs several calls
+ * with one filter (forward and backward of one step, several iterations of one layer) can
+ * pack it once with ndc_prepare_taps and hand it to ndc_forward_taps / ndc_backward_taps,
+ * which then launch nothing but the update kernels.  The table is a function of `h` and of
+ * the filter geometry, channel count and dtype in `g` only (not of batch, extents, eps,
+ * relu_input).  The reference keeps no such table (its kernels read h, kernels.py:728-894).
+ *   ndc_taps_bytes     bytes of the table for `g`; 0 when the kernels for `g` read `h`
+ *                      (then `taps` is ignored everywhere and may be null)
+ *   ndc_prepare_taps   fills `taps` (256-byte aligned, >= ndc_taps_bytes(g)) from `h`
+ *   ndc_forward_taps   ndc_forward with the table in place of the workspace
+ *   ndc_backward_taps  ndc_backward with the table; workspace as for ndc_backward
+ */
+size_t ndc_taps_bytes(const ndc_geom *g);
+int ndc_prepare_taps(const ndc_geom *g, const float *h, void *taps, size_t taps_bytes,
+                     void *stream);
+int ndc_forward_taps(const ndc_geom *g, const void *x, const void *z, const float *h,
+                     const void *taps, const float *bias, void *out, void *t1, void *s_over_den,
+                     void *ratio, void *stream);
+int ndc_backward_taps(const ndc_geom *g, const void *x, const void *z, const void *t1,
+                      const void *s_over_den, const void *ratio, const float *h, const void *taps,
+                      const float *bias, const void *gout, void *gx, void *gz, float *gh, float *gb,
+                      void *workspace, size_t workspace_bytes, void *stream);
+
 /* Bytes of scratch `ndc_backward` needs for `g` with the requested outputs (each flag
  * nonzero when the matching output pointer will be non-null). */
 size_t ndc_backward_workspace_bytes(const ndc_geom *g, int need_gx, int need_gz, int need_gh,
