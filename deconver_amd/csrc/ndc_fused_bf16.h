@@ -200,10 +200,6 @@ template <int NR, int NTEN, class Exec>
 NDC_D void a_plane_q(Exec &ex, const int (&base)[NTEN], int PQ, UniformF wq,
                      float (&acc)[NTEN][4][NR][2])
 {
-#ifndef NDC_AQ_MODE
-#define NDC_AQ_MODE 0
-#endif
-#if NDC_AQ_MODE == 0
     NDC_ROLLED
     for (int thh = 0; thh < 3; ++thh) {
         const int th = uniform_int(thh);
@@ -231,36 +227,6 @@ NDC_D void a_plane_q(Exec &ex, const int (&base)[NTEN], int PQ, UniformF wq,
                 }
         }
     }
-#else
-    // input rows in order, each read once; all 48 packed taps in scalar registers
-    float w[48];
-    load_taps<48>(wq, w);
-    NDC_UNROLL
-    for (int q = 0; q < NR + 2; ++q) {
-        uint32_t v[NTEN][3];
-        NDC_UNROLL
-        for (int t = 0; t < NTEN; ++t)
-            NDC_UNROLL
-            for (int u = 0; u < 3; ++u) v[t][u] = float_to_bits(ex.ld(base[t] + q * PQ + u));
-        NDC_UNROLL
-        for (int th = 0; th < 3; ++th) {
-            const int r = q - 2 + th;
-            if (r < 0 || r >= NR) continue;
-            NDC_UNROLL
-            for (int i = 0; i < 4; ++i)
-                NDC_UNROLL
-                for (int t = 0; t < NTEN; ++t) {
-                    float a0 = acc[t][i][r][0], a1 = acc[t][i][r][1];
-                    a0 = dot2_bf16(v[t][1], float_to_bits(w[th * 16 + i * 4 + 0]), a0);
-                    a1 = dot2_bf16(v[t][1], float_to_bits(w[th * 16 + i * 4 + 2]), a1);
-                    a0 = dot2_bf16(v[t][0], float_to_bits(w[th * 16 + i * 4 + 1]), a0);
-                    a1 = dot2_bf16(v[t][2], float_to_bits(w[th * 16 + i * 4 + 3]), a1);
-                    acc[t][i][r][0] = a0;
-                    acc[t][i][r][1] = a1;
-                }
-        }
-    }
-#endif
 }
 
 // NROWS rows of NW staged words each, row n at addr(n), handed to body(n, words) with the
