@@ -354,7 +354,7 @@ def grid_workload(args) -> int:
     return 0
 
 
-DOT2_PER_CHANNEL_VOXEL = {"forward": 205, "backward_pass1": 216, "backward_pass2": 126}
+DOT2_PER_CHANNEL_VOXEL = {"forward": 181, "backward_pass1": 216, "backward_pass2": 126}
 CLOCKS_PER_DOT2C = 4.52   # per SIMD, four wavefronts resident: measured by `--workload valu`
 
 
@@ -435,17 +435,17 @@ MODEL_WORKLOADS = {
 }
 
 
-def model_workload(args) -> int:
+def run_model_routes(workload: str, routes, warmup: int, steps: int) -> dict:
+    """One model-level workload (MODEL_WORKLOADS) on each of `routes` ("hip": the NDC layers on
+    the HIP kernels; "pytorch": the same network with the layers on their general PyTorch
+    route): ms per step, steps per second, last loss, peak memory."""
     import torch
     from torch import nn
 
     import deconver_amd as dc
     from deconver_amd import training as T
 
-    if not torch.cuda.is_available():
-        print("bench.py needs a GPU", file=sys.stderr)
-        return 2
-    w = MODEL_WORKLOADS[args.workload]
+    w = MODEL_WORKLOADS[workload]
     dev = torch.device("cuda:0")
     nd = len(w["size"])
     norm = nn.InstanceNorm3d if nd == 3 else nn.InstanceNorm2d
@@ -476,20 +476,33 @@ def model_workload(args) -> int:
             loss.backward()
             return loss.detach()
 
-        for _ in range(args.warmup):
+        for _ in range(warmup):
             loss = step()
         torch.cuda.synchronize()
         torch.cuda.reset_peak_memory_stats()
         t0 = time.perf_counter()
-        for _ in range(args.steps):
+        for _ in range(steps):
             loss = step()
         torch.cuda.synchronize()
-        dt = (time.perf_counter() - t0) / args.steps
-        return dict(ms_per_step=dt * 1e3, steps_per_s=1.0 / dt, loss=float(loss),
-                    peak_mem_GB=torch.cuda.max_memory_allocated() / 1e9)
+        dt = (time.perf_counter() - t0) / steps
+        out = dict(ms_per_step=dt * 1e3, steps_per_s=1.0 / dt, loss=float(loss), steps=steps,
+                   warmup=warmup, peak_mem_GB=torch.cuda.max_memory_allocated() / 1e9)
+        del model, opt
+        torch.cuda.empty_cache()
+        return out
 
+    return {r: run(r) for r in routes}
+
+
+def model_workload(args) -> int:
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    w = MODEL_WORKLOADS[args.workload]
     routes = ["hip", "pytorch"] if args.ndc == "both" else [args.ndc]
-    res = {r: run(r) for r in routes}
+    res = run_model_routes(args.workload, routes, args.warmup, args.steps)
     main_r = res[routes[0]]
     vox = w["batch"] * math.prod(w["size"])
     result = {
@@ -566,6 +579,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--dtype", choices=("bf16", "fp32"), default="bf16")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-train", action="store_true",
+                    help="skip the Deconver-3D train-step leg that follows the timed region")
     ap.add_argument("--recompute", action="store_true",
                     help="backward re-gathers the denominator and ratio (as the reference does) "
                          "instead of reading the forward's copies")
@@ -685,11 +700,16 @@ def main() -> int:
     alg = {"forward": 9 * U * esz, "backward_pass1": 10 * U * esz, "backward_pass2": 4 * U * esz}
     dominant = max(alg, key=lambda k: k_ms[k])
     achieved = alg[dominant] / (k_ms[dominant] * 1e-3) / 1e9
-    traffic = None
+    # HBM bytes per launch from rocprofv3's FETCH_SIZE / WRITE_SIZE counters: they cannot be
+    # read from inside this process, so the figure is the one recorded in profiles/traffic.json
+    # by the profiling runs described there, stamped with the commit it was measured at
+    traffic = traffic_at = None
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(tpath):
         try:
-            traffic = json.load(open(tpath)).get(args.dtype, {}).get(dominant)
+            rec = json.load(open(tpath))
+            traffic = rec.get(args.dtype, {}).get(dominant)
+            traffic_at = rec.get("measured_at_commit")
         except (ValueError, OSError):
             traffic = None
     roofline = {
@@ -700,6 +720,7 @@ def main() -> int:
         "unit": "GB/s",
         "frac": achieved / HBM_PEAK_GBS,
         "traffic": traffic,
+        "traffic_measured_at_commit": traffic_at,
         "algorithmic_bytes": alg[dominant],
         "avg_launch_ms": k_ms[dominant],
     }
@@ -748,6 +769,18 @@ def main() -> int:
         }
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(torch)
+    if not args.no_train:
+        # the second half of the metric, outside the timed region above: Deconver-3D train
+        # steps per second (config 4) with the NDC layers on the HIP kernels and, for
+        # reference, on the layers' PyTorch route on the same GPU
+        del x, z, g
+        torch.cuda.empty_cache()
+        t3 = run_model_routes("train3d", ["hip"], warmup=2, steps=5)
+        t3.update(run_model_routes("train3d", ["pytorch"], warmup=1, steps=2))
+        result["train3d_steps_per_s"] = t3["hip"]["steps_per_s"]
+        result["train3d_steps_per_s_pytorch_route"] = t3["pytorch"]["steps_per_s"]
+        result["train3d"] = {"workload": MODEL_WORKLOADS["train3d"]["text"], "routes": t3,
+                             "hip_over_pytorch": t3["hip"]["steps_per_s"] / t3["pytorch"]["steps_per_s"]}
     print(json.dumps(result))
     return 0
 

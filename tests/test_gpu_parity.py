@@ -225,3 +225,29 @@ def test_graph_capture_replays_match_eager(dtype):
         torch.cuda.synchronize()
         for name, a, b in zip(("out", "gx", "gz", "gh", "gb"), got, want):
             assert torch.equal(a, b), f"replay {replay}: {name}"
+
+
+@pytest.mark.parametrize("geom", [FUSED_GEOMS[2], FUSED_GEOMS[7], (24, 24, 4, (3, 3, 3), (9, 16, 192), 1)])
+def test_prepared_taps_bit_equal_on_gpu(geom):
+    """ndc_prepare_taps once, then ndc_forward_taps / ndc_backward_taps: the same bits as the
+    entry points that pack the filter table on every call (bf16 3x3x3 kernels; the last case
+    is a 192-column row, i.e. six wavefronts per workgroup in the forward)."""
+    C, G, sc, ks, sp, B = geom
+    lib = _lib_gpu()
+    x, z, h, bias, gout = make_case(C, G, sc, ks, sp, B=B, dtype=torch.bfloat16, bias_shift=0.3,
+                                    device="cuda")
+    kw = dict(groups=G, m=1, sc=sc, eps=1e-16, relu_input=True)
+    taps = ops.prepare_taps(lib, x, h, groups=G, m=1, sc=sc)
+    assert taps is not None and taps.data_ptr() % 256 == 0
+    out0, t0, saved0 = ops.update_forward(lib, x, z, h, bias, save_ratio=True, **kw)
+    out1, t1, saved1 = ops.update_forward(lib, x, z, h, bias, save_ratio=True, taps=taps, **kw)
+    assert torch.equal(out0, out1) and torch.equal(t0, t1)
+    assert torch.equal(saved0[0], saved1[0]) and torch.equal(saved0[1], saved1[1])
+    g0 = ops.update_backward(lib, x, z, t0, h, bias, gout, saved=saved0, **kw)
+    g1 = ops.update_backward(lib, x, z, t0, h, bias, gout, saved=saved0, taps=taps, **kw)
+    for a, b in zip(g0, g1):
+        assert torch.equal(a, b)
+    ro, _, (rgx, rgz, rgh, rgb) = _oracle(x, z, h, bias, gout, G, 1, sc, 1e-16, True)
+    assert O.rel_err(out1.float().cpu(), ro) < 2e-2
+    for got, ref in zip(g1, (rgx, rgz, rgh, rgb)):
+        assert O.rel_err(got.float().cpu(), ref) < 2e-2
