@@ -865,9 +865,13 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
                 prefetch_g(st, k);
                 if (live1) {
                     const int gb_ = off_g + (st.ln.strip * RH) * P + PL + st.ln.c0 - PW;
-                    NDC_ROLLED
-                    for (int prr = 0; prr < 2; ++prr) {
-                        const int pr = uniform_int(prr);
+                    // the two channel pairs one after the other in straight-line code (as a
+                    // rolled loop the accumulators it carries were permuted by register copies
+                    // on every trip); the fence keeps the second pair's tap loads behind the
+                    // first pair's arithmetic
+                    NDC_UNROLL
+                    for (int pr = 0; pr < 2; ++pr) {
+                        ex.fence();
                         float wp[KT];
                         load_taps<KT>(tab + pr * KT, wp);
                         // gn rows of this channel pair feed gx, then its gd rows feed gt1
