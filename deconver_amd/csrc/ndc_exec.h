@@ -162,6 +162,11 @@ template <class State> struct HostExec {
 //     instruction is spent on 64-bit address arithmetic, and an access past `bytes` is
 //     dropped (loads return 0) instead of faulting.  A null base gives an empty slice.
 //   Host build: base pointer + size; an access outside the slice is reported as a fault.
+// A per-lane offset that lies outside every slice (slices addressed this way are kept below
+// 2^31 bytes): a lane that has nothing to read or write at some row uses it instead of a
+// branch or a select, and gets 0 from a load and no effect from a store.
+static const unsigned kNoAccess = 0x80000000u;
+
 struct BufRef {
 #if NDC_DEVICE_BUILD && defined(__HIP_DEVICE_COMPILE__)
     __amdgpu_buffer_rsrc_t r;
@@ -201,6 +206,7 @@ NDC_HD uint32_t buf_ld(const BufRef &b, unsigned lane_off, unsigned uniform_off)
     (void)b; (void)lane_off; (void)uniform_off;
     return 0u;
 #else
+    if (lane_off >= kNoAccess) return 0u;
     const size_t o = (size_t)lane_off + uniform_off;
     if (o + 4 > b.bytes) {
         HostFaults &hf = host_faults();
@@ -224,6 +230,7 @@ NDC_HD void buf_st(const BufRef &b, unsigned lane_off, unsigned uniform_off, uin
 #elif NDC_DEVICE_BUILD
     (void)b; (void)lane_off; (void)uniform_off; (void)w;
 #else
+    if (lane_off >= kNoAccess) return;
     const size_t o = (size_t)lane_off + uniform_off;
     if (o + 4 > b.bytes) {
         HostFaults &hf = host_faults();

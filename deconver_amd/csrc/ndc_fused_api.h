@@ -138,7 +138,9 @@ static inline bool make_plan(const KGeom &q, Plan &pl, bool pairs_ok = true, int
         plan_lds<kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_>(pl);
     NDC_FUSED_VARIANTS(X)
 #undef X
+    // (their buffer addressing wants every (sample, channel group) slice below 2^31 bytes)
     if (dtype == NDC_BF16 && pairs_ok && pl.m.W % 2 == 0 && q.sc == 4 && pl.m.KD == 3 &&
+        (long long)q.sc * q.SP * 2 < (1LL << 31) &&
         pl.m.KH == 3 && pl.m.KW == 3 && tn.dot2) {
         Tile tf, tb;
         if (make_tile(pl.m, kDot2RH, 2, tn.threads_f2, tf, FwdKernelB<kDot2RH>::kMinStrips) &&

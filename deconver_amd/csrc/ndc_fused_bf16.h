@@ -581,8 +581,9 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
 
     struct State {
         Lane ln;
-        unsigned xoff[NXR], ooff[RH];   // byte offsets inside one plane
-        unsigned xok, ook;
+        // byte offsets inside one plane; ooff / hoff: kNoAccess for a row outside the image
+        unsigned xoff[NXR], ooff[RH];
+        unsigned xok;
         float bv[SC];
         float gacc[SC][KT];
         float accx[KD][RH][RW], acct[KD][RH][RW];
@@ -742,7 +743,9 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
                     NDC_UNROLL
                     for (int c = 0; c < RW; ++c) {
                         const float sv = floor_f((c ? bf_hi(zw[i][r]) : bf_lo(zw[i][r])) + st.bv[i], floor_);
-                        const float gv = ok[r] ? (c ? bf_hi(gw[i][r]) : bf_lo(gw[i][r])) : 0.f;
+                        // SAVED: the words of a row outside the image were read as zeros
+                        const float g_ = c ? bf_hi(gw[i][r]) : bf_lo(gw[i][r]);
+                        const float gv = SAVED || ok[r] ? g_ : 0.f;
                         if (SAVED) {
                             gn[i][c] = gv * (c ? bf_hi(dw[i][r]) : bf_lo(dw[i][r]));
                             gd[i][c] = -(gn[i][c] * (c ? bf_hi(rw[i][r]) : bf_lo(rw[i][r])));
@@ -766,7 +769,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
 
         ex.each([&](State &st, int tid) NDC_LAMBDA {
             st.ln = make_lane(tid, t, RW);
-            st.xok = st.ook = 0u;
+            st.xok = 0u;
             NDC_UNROLL
             for (int n = 0; n < NXR; ++n) {
                 const int j = st.ln.strip + n * S, row = r0 - 2 * PH + j;
@@ -777,12 +780,11 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
             NDC_UNROLL
             for (int r = 0; r < RH; ++r) {
                 const int row = r0 + st.ln.strip * RH + r;
-                if (row < H) st.ook |= 1u << r;
-                st.ooff[r] = (unsigned)(clampi(row, 0, H - 1) * W + st.ln.c0) * 2u;
+                st.ooff[r] = row < H ? (unsigned)(row * W + st.ln.c0) * 2u : kNoAccess;
             }
             {
                 const int hrow = r0 - PH + halo_row(st.ln.strip, PH, TH);
-                st.hoff = (unsigned)(clampi(hrow, 0, H - 1) * W + st.ln.c0) * 2u;
+                st.hoff = hrow >= 0 && hrow < H ? (unsigned)(hrow * W + st.ln.c0) * 2u : kNoAccess;
                 NDC_UNROLL
                 for (int i = 0; i < SC; ++i)
                     NDC_UNROLL
@@ -891,7 +893,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
                 const int pf = k - 2;
                 NDC_UNROLL
                 for (int r = 0; r < RH; ++r) {
-                    if (pf >= 0 && ((st.ook >> r) & 1u)) {
+                    if (pf >= 0) {   // rows outside the image: the stores go nowhere
                         if (have_gx) buf_st<true>(gxb_, st.ooff[r], (unsigned)pf * plane2,
                                             pack_bf16x2(st.accx[0][r][0], st.accx[0][r][1]));
                         buf_st(gtb_, st.ooff[r], (unsigned)pf * plane2,
