@@ -289,8 +289,9 @@ template <int RH_> struct FwdKernelB {
 
     struct State {
         Lane ln;
-        unsigned zoff[NZR], xoff[NXR], ooff[RH];   // BYTE offsets inside one plane (rows clamped)
-        unsigned zok, xok, ook;
+        // BYTE offsets inside one plane (rows clamped; ooff: kNoAccess for a row outside the image)
+        unsigned zoff[NZR], xoff[NXR], ooff[RH];
+        unsigned zok, xok;
         float bv[SC];
         float t1acc[KD][RHK][RW];
         uint32_t t1prev[RHK];       // previous t1 plane of the own rows, as column pairs
@@ -403,7 +404,7 @@ template <int RH_> struct FwdKernelB {
 
         ex.each([&](State &st, int tid) NDC_LAMBDA {
             st.ln = make_lane(tid, t, RW);
-            st.zok = st.xok = st.ook = 0u;
+            st.zok = st.xok = 0u;
             NDC_UNROLL
             for (int n = 0; n < NZR; ++n) {
                 const int j = st.ln.strip + n * S, row = r0 - 2 * PH + j;
@@ -422,8 +423,7 @@ template <int RH_> struct FwdKernelB {
             NDC_UNROLL
             for (int r = 0; r < RH; ++r) {
                 const int row = r0 + st.ln.strip * RH + r;
-                if (row < H) st.ook |= 1u << r;
-                st.ooff[r] = (unsigned)(clampi(row, 0, H - 1) * W + st.ln.c0) * 2u;
+                st.ooff[r] = row < H ? (unsigned)(row * W + st.ln.c0) * 2u : kNoAccess;
             }
             NDC_UNROLL
             for (int i = 0; i < SC; ++i) st.bv[i] = p.bias ? p.bias[id.c * SC + i] : 0.f;
@@ -537,7 +537,7 @@ template <int RH_> struct FwdKernelB {
                 const unsigned oj = (unsigned)j0 * plane2;
                 NDC_UNROLL
                 for (int r = 0; r < RH; ++r) {
-                    if (!((st.ook >> r) & 1u)) continue;
+                    // (a row outside the image: its stores go nowhere)
                     NDC_UNROLL
                     for (int i = 0; i < SC; ++i) {
                         float v[RW], rd[RW], rt[RW];
