@@ -38,7 +38,7 @@ from . import operations as ops_general
 from . import ops
 from ._lib import get_library
 from .functional import deconv_update, hip_kernels_apply
-from .layers import Linear
+from .layers import Linear, pointwise_linear
 
 __all__ = ["Initializer", "Deconv", "NDC"]
 
@@ -184,7 +184,7 @@ class Deconv(nn.Module):
         h = F.relu(self.init.h0).float()
         # bias-free projection; bias and ReLU are folded into the first update's loads, so
         # neither relu(Linear(x)) nor the biased projection ever exists in memory
-        s = F.conv1d(x.flatten(2), proj.weight.to(dtype), None).view(x.shape[0], -1, *x.shape[2:])
+        s = pointwise_linear(x.flatten(2), proj.weight.to(dtype)).view(x.shape[0], -1, *x.shape[2:])
         first = dict(bias=None if proj.bias is None else proj.bias.float(), relu_input=True)
         later = dict(bias=None, relu_input=False)
         taps = None

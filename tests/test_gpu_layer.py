@@ -5,6 +5,7 @@ import pytest
 import torch
 
 import deconver_amd as dc
+from deconver_amd.layers import pointwise_linear
 from oracle import ndc_oracle as O
 
 pytestmark = pytest.mark.gpu
@@ -143,7 +144,8 @@ def test_bf16_autocast_layer_within_2e_2_of_float64():
     # the pattern the route computed: sign of (bf16 projection, float32 bias added on load)
     proj = layer.init.linear.linear
     with torch.no_grad():
-        z_route = torch.nn.functional.conv1d(x0.cuda().bfloat16().flatten(2), proj.weight.bfloat16())
+        # (the route's own projection routine: its bf16 sums decide the borderline units)
+        z_route = pointwise_linear(x0.cuda().bfloat16().flatten(2), proj.weight.bfloat16())
         gate = (z_route.float() + proj.bias.float().view(1, -1, 1) > 0).view(2, 64, 9, 8, 10).cpu()
         z_exact = torch.nn.functional.conv1d(x0.double().flatten(2), proj.weight.double().cpu(),
                                              proj.bias.double().cpu()).view(2, 64, 9, 8, 10)
