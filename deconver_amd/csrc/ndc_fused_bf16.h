@@ -1036,7 +1036,8 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
             for (int r = 0; r < RH; ++r) {
                 const int row = r0 + st.ln.strip * RH + r;
                 if (row < H) st.ook |= 1u << r;
-                st.ooff[r] = (unsigned)(clampi(row, 0, H - 1) * W + st.ln.c0) * 2u;
+                // a row outside the image: its loads give 0 and its stores go nowhere
+                st.ooff[r] = row < H ? (unsigned)(row * W + st.ln.c0) * 2u : kNoAccess;
             }
             NDC_UNROLL
             for (int i = 0; i < SC; ++i) {
@@ -1149,7 +1150,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
                                 st.gbacc[i] += gzv;
                                 v[c] = gzv;
                             }
-                            if (have_gz && ok) buf_st<true>(gzb_, st.ooff[r], jo + i * cplane2, pack_bf16x2(v[0], v[1]));
+                            if (have_gz) buf_st<true>(gzb_, st.ooff[r], jo + i * cplane2, pack_bf16x2(v[0], v[1]));
                         }
                     }
                 }
