@@ -127,3 +127,35 @@ def test_config4_stage0_layer_channel_slices():
                     gb=O.rel_err(gb[cs].cpu(), rgb))
         bad = {k: v for k, v in errs.items() if not v < 2e-2}
         assert not bad, f"channel {c}: {bad} (all: {errs})"
+
+
+def test_config4_full_size_train_steps_on_both_routes():
+    """Config 4 at full size (Deconver 3-D, widths 64-512, batch 2 of 128^3, bf16 autocast,
+    Dice+BCE, AdamW): two training steps from the same weights with the NDC layers on the HIP
+    kernels and on the layers' PyTorch route; the losses of both steps agree to 3e-2 (bf16
+    arithmetic on either side), and the step lowers the loss on both."""
+    from torch import nn
+
+    import deconver_amd as dc
+    from deconver_amd import training as T
+
+    net = dict(in_channels=2, out_channels=1, spatial_dims=3, encoder_depth=(1, 1, 1, 1),
+               encoder_width=(64, 128, 256, 512), strides=(1, 2, 2, 2), decoder_depth=(1, 1, 1),
+               kernel_size=(3, 3, 3), groups=-1, ratio=4, norm=nn.InstanceNorm3d)
+    images, targets = T.ellipsoid_phantoms(2, 2, (128, 128, 128), seed=0, device="cuda")
+    losses = {}
+    for route, extra in (("hip", {}), ("pytorch", {"dilation": 1})):
+        torch.manual_seed(0)
+        model = dc.Deconver(**net, **extra).cuda()
+        layers = [m for m in model.modules() if isinstance(m, dc.Deconv)]
+        on_hip = all(m.fast_path_applicable(torch.empty(1, m.channels, 8, 8, 8, device="cuda"))
+                     for m in layers)
+        assert on_hip == (route == "hip") and len(layers) == 7
+        opt = T.make_optimizer(model)
+        losses[route] = [float(T.train_step(model, opt, images, targets,
+                                            autocast_dtype=torch.bfloat16)) for _ in range(2)]
+        del model, opt
+        torch.cuda.empty_cache()
+    for a, b in zip(losses["hip"], losses["pytorch"]):
+        assert abs(a - b) < 3e-2 * abs(b), losses
+    assert losses["hip"][1] < losses["hip"][0] and losses["pytorch"][1] < losses["pytorch"][0], losses
