@@ -17,6 +17,7 @@
 
 #if !NDC_DEVICE_BUILD
 #include <cstdio>
+#include <cstring>
 #include <vector>
 #endif
 
@@ -33,6 +34,18 @@ template <class State> struct DeviceExec {
     NDC_D void sync() { __syncthreads(); }
     NDC_D float ld(int i) const { return lds[i]; }
     NDC_D void st_(int i, float v) { lds[i] = v; }
+    // four consecutive words from an EVEN word index, as two 8-byte reads (one ds_read2_b64
+    // where the compiler pairs them) instead of four 4-byte ones
+    NDC_D void ld4(int i, uint32_t (&v)[4]) const
+    {
+        typedef __attribute__((ext_vector_type(2))) uint32_t u2_t;
+        const u2_t a = *reinterpret_cast<const u2_t *>(lds + i);
+        const u2_t b = *reinterpret_cast<const u2_t *>(lds + i + 2);
+        v[0] = a.x;
+        v[1] = a.y;
+        v[2] = b.x;
+        v[3] = b.y;
+    }
     // The instruction scheduler may not move anything across this point: used to keep the LDS
     // reads of the next row ahead of the arithmetic on the current one.
     NDC_D void fence() const { __builtin_amdgcn_sched_barrier(0); }
@@ -120,6 +133,18 @@ template <class State> struct HostExec {
             r_tid[i] = -2;
         }
         return mem[i];
+    }
+    void ld4(int i, uint32_t (&v)[4])
+    {
+        if (i & 1) {
+            HostFaults &hf = host_faults();
+            ++hf.oob;
+            hf.note("misaligned four-word read", i, cur, -1);
+        }
+        for (int u = 0; u < 4; ++u) {
+            const float f = ld(i + u);
+            memcpy(&v[u], &f, 4);
+        }
     }
     void st_(int i, float v)
     {

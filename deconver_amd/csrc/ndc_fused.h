@@ -54,7 +54,7 @@ struct Tile {
     int TH;      // output rows per workgroup
     int ntile;   // row bands per volume
     int P;       // LDS row pitch in words
-    int PL;      // zero words to the left of column 0 in an LDS row (>= PW, multiple of RW)
+    int PL;      // zero words to the left of column 0 in an LDS row (>= PW)
     int CPW;     // column groups per row = W / RW
     int nseg;    // segments of the marching axis per volume (each its own workgroup)
     int SEG;     // planes per segment
@@ -93,8 +93,9 @@ static const int kMaxLdsBytes = 160 * 1024;
 
 // S strips of RH rows, RW columns per thread; S >= 2*PH so that the halo rows fit the
 // fixed per-thread bounds
+// left_pad: zero words left of column 0 in an LDS row; 0 = the default, PW rounded up to RW
 static inline bool make_tile(const March &m, int RH, int RW, int target_threads, Tile &t,
-                             int min_strips = 0)
+                             int min_strips = 0, int left_pad = 0)
 {
     const int PH = m.KH / 2, PW = m.KW / 2;
     if (m.W % RW) return false;
@@ -112,7 +113,7 @@ static inline bool make_tile(const March &m, int RH, int RW, int target_threads,
     t.NT = round_up(s * cpw, 64);
     t.TH = s * RH;
     t.ntile = (m.H + t.TH - 1) / t.TH;
-    t.PL = round_up(PW, RW);
+    t.PL = left_pad ? left_pad : round_up(PW, RW);
     t.P = round_up(t.PL + m.W + PW, RW);
     t.nseg = 1;
     t.SEG = m.D;

@@ -83,6 +83,19 @@ NDC_HD uint32_t zip_hi(uint32_t a, uint32_t b)
 NDC_HD float bf_lo(uint32_t w) { return bits_to_float(w << 16); }
 NDC_HD float bf_hi(uint32_t w) { return bits_to_float(w & 0xffff0000u); }
 
+// NW staged words from `at`; four at a time where NW = 4 (the word index of every such read
+// is even: the tiles of these kernels put one zero word left of column 0, so a thread's
+// window starts at its own even column)
+template <int NW, class Exec> NDC_D void read_words(Exec &ex, int at, uint32_t (&v)[NW])
+{
+    if constexpr (NW == 4) {
+        ex.ld4(at, v);
+    } else {
+        NDC_UNROLL
+        for (int u = 0; u < NW; ++u) v[u] = float_to_bits(ex.ld(at + u));
+    }
+}
+
 // K-type pass over an NR x RW tile for ONE channel pair: words (s_2p, s_2p+1) staged at
 // `base` (first input row, first own column - 1); w = WK[p], 27 packed tap pairs.
 template <int NR, int RW, int STRIDE>
@@ -116,24 +129,17 @@ NDC_D void k_rows_d2(Exec &ex, int base, int P, const float (&w)[27], float (*ac
                      int r_off)
 {
     uint32_t vn[RW + 2];
-    if (PIPE) {
-        NDC_UNROLL
-        for (int u = 0; u < RW + 2; ++u) vn[u] = float_to_bits(ex.ld(base + u));
-    }
+    if (PIPE) read_words<RW + 2>(ex, base, vn);
     NDC_UNROLL
     for (int q = 0; q < NR + 2; ++q) {
         uint32_t v[RW + 2];
         if (PIPE) {
             NDC_UNROLL
             for (int u = 0; u < RW + 2; ++u) v[u] = vn[u];
-            if (q + 1 < NR + 2) {
-                NDC_UNROLL
-                for (int u = 0; u < RW + 2; ++u) vn[u] = float_to_bits(ex.ld(base + (q + 1) * P + u));
-            }
+            if (q + 1 < NR + 2) read_words<RW + 2>(ex, base + (q + 1) * P, vn);
             ex.fence();
         } else {
-            NDC_UNROLL
-            for (int u = 0; u < RW + 2; ++u) v[u] = float_to_bits(ex.ld(base + q * P + u));
+            read_words<RW + 2>(ex, base + q * P, v);
         }
         k_row_d2<NR, RW, STRIDE>(q, v, w, acc, r_off);
     }
@@ -147,9 +153,7 @@ NDC_D void a_plane_d2(Exec &ex, const int (&base)[NTEN], int P, const float (&wt
     uint32_t vn[NTEN][RW + 2];
     if (PIPE) {
         NDC_UNROLL
-        for (int t = 0; t < NTEN; ++t)
-            NDC_UNROLL
-            for (int u = 0; u < RW + 2; ++u) vn[t][u] = float_to_bits(ex.ld(base[t] + u));
+        for (int t = 0; t < NTEN; ++t) read_words<RW + 2>(ex, base[t], vn[t]);
     }
     NDC_UNROLL
     for (int q = 0; q < NR + 2; ++q) {
@@ -161,17 +165,12 @@ NDC_D void a_plane_d2(Exec &ex, const int (&base)[NTEN], int P, const float (&wt
                 for (int u = 0; u < RW + 2; ++u) v[t][u] = vn[t][u];
             if (q + 1 < NR + 2) {
                 NDC_UNROLL
-                for (int t = 0; t < NTEN; ++t)
-                    NDC_UNROLL
-                    for (int u = 0; u < RW + 2; ++u)
-                        vn[t][u] = float_to_bits(ex.ld(base[t] + (q + 1) * P + u));
+                for (int t = 0; t < NTEN; ++t) read_words<RW + 2>(ex, base[t] + (q + 1) * P, vn[t]);
             }
             ex.fence();
         } else {
             NDC_UNROLL
-            for (int t = 0; t < NTEN; ++t)
-                NDC_UNROLL
-                for (int u = 0; u < RW + 2; ++u) v[t][u] = float_to_bits(ex.ld(base[t] + q * P + u));
+            for (int t = 0; t < NTEN; ++t) read_words<RW + 2>(ex, base[t] + q * P, v[t]);
         }
         NDC_UNROLL
         for (int th = 0; th < 3; ++th) {
@@ -233,8 +232,7 @@ NDC_D void a_plane_q(Exec &ex, const int (&base)[NTEN], int PQ, UniformF wq,
 // reads running one row ahead (PIPE, see k_rows_d2).
 template <int NW, class Exec> NDC_D void read_row(Exec &ex, int at, uint32_t (&v)[NW])
 {
-    NDC_UNROLL
-    for (int u = 0; u < NW; ++u) v[u] = float_to_bits(ex.ld(at + u));
+    read_words<NW>(ex, at, v);
 }
 
 // `first`: row 0 already read by the caller (ahead of other work), or null.
@@ -256,14 +254,10 @@ NDC_D void stream_rows(Exec &ex, Addr addr, Body body, const uint32_t (*first)[N
         if (PIPE) {
             NDC_UNROLL
             for (int u = 0; u < NW; ++u) v[u] = vn[u];
-            if (n + 1 < NROWS) {
-                NDC_UNROLL
-                for (int u = 0; u < NW; ++u) vn[u] = float_to_bits(ex.ld(addr(n + 1) + u));
-            }
+            if (n + 1 < NROWS) read_words<NW>(ex, addr(n + 1), vn);
             ex.fence();
         } else {
-            NDC_UNROLL
-            for (int u = 0; u < NW; ++u) v[u] = float_to_bits(ex.ld(addr(n) + u));
+            read_words<NW>(ex, addr(n), v);
         }
         body(n, v);
     }
