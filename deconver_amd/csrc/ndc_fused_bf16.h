@@ -369,11 +369,14 @@ template <int RH_> struct FwdKernelB {
                     s[i][0] = floor_f(s[i][0], floor_);
                     s[i][1] = floor_f(s[i][1], floor_);
                 }
+                // the two columns of a channel pair one after the other: adjacent words, one
+                // ds_write2_b32
                 NDC_UNROLL
-                for (int c = 0; c < RW; ++c) {
-                    ex.st_(sb + j * P + lb + c, bits_to_float(pack_bf16x2(s[0][c], s[1][c])));
-                    ex.st_(sb + (RS + j) * P + lb + c, bits_to_float(pack_bf16x2(s[2][c], s[3][c])));
-                }
+                for (int pr = 0; pr < 2; ++pr)
+                    NDC_UNROLL
+                    for (int c = 0; c < RW; ++c)
+                        ex.st_(sb + (pr * RS + j) * P + lb + c,
+                               bits_to_float(pack_bf16x2(s[2 * pr][c], s[2 * pr + 1][c])));
             }
         };
         // x plane k - 1 completes the plane-pair word (x[k-2], x[k-1]) of slot (k - 2) % 2 and
@@ -750,14 +753,19 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
                         }
                         gg_out[i][r][c] = pack_bf16x2(gn[i][c], gd[i][c]);
                     }
+                // (the two columns of each word plane one after the other: adjacent words, one
+                // ds_write2_b32)
+                const int o = off_g + (j + r) * P + PL + st.ln.c0;
                 NDC_UNROLL
-                for (int c = 0; c < RW; ++c) {
-                    const int o = off_g + (j + r) * P + PL + st.ln.c0 + c;
-                    ex.st_(o, bits_to_float(pack_bf16x2(gn[0][c], gn[1][c])));
-                    ex.st_(o + RG * P, bits_to_float(pack_bf16x2(gn[2][c], gn[3][c])));
-                    ex.st_(o + 2 * RG * P, bits_to_float(pack_bf16x2(gd[0][c], gd[1][c])));
-                    ex.st_(o + 3 * RG * P, bits_to_float(pack_bf16x2(gd[2][c], gd[3][c])));
-                }
+                for (int pr = 0; pr < 2; ++pr)
+                    NDC_UNROLL
+                    for (int c = 0; c < RW; ++c)
+                        ex.st_(o + pr * RG * P + c, bits_to_float(pack_bf16x2(gn[2 * pr][c], gn[2 * pr + 1][c])));
+                NDC_UNROLL
+                for (int pr = 0; pr < 2; ++pr)
+                    NDC_UNROLL
+                    for (int c = 0; c < RW; ++c)
+                        ex.st_(o + (2 + pr) * RG * P + c, bits_to_float(pack_bf16x2(gd[2 * pr][c], gd[2 * pr + 1][c])));
             }
         };
 
