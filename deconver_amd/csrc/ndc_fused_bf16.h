@@ -940,8 +940,12 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
     struct State {
         Lane ln;
         unsigned xoff[NXR], ooff[RH];
-        unsigned xok, ook;
-        float bv[SC];
+        unsigned xok;
+        // bias per own row: the channel's bias; for a row outside the image (whose z, gout,
+        // n/d words read as zeros) -1 when the source is rectified and 0 when it is not, so
+        // that its source values and rectified gradients come out as zeros without a select
+        float bvr[SC][RH];
+        float okf[RH];   // 1 for a row inside the image, 0 outside: weight of its gz in gb
         float gacc[SC][KT];
         float gbacc[SC];
         float sprev[SC][RH][RW];   // own source values of the previous plane
@@ -1026,7 +1030,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
 
         ex.each([&](State &st, int tid) NDC_LAMBDA {
             st.ln = make_lane(tid, t, RW);
-            st.xok = st.ook = 0u;
+            st.xok = 0u;
             NDC_UNROLL
             for (int n = 0; n < NXR; ++n) {
                 const int j = st.ln.strip + n * S, row = r0 - PH + j;
@@ -1037,13 +1041,15 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
             NDC_UNROLL
             for (int r = 0; r < RH; ++r) {
                 const int row = r0 + st.ln.strip * RH + r;
-                if (row < H) st.ook |= 1u << r;
                 // a row outside the image: its loads give 0 and its stores go nowhere
                 st.ooff[r] = row < H ? (unsigned)(row * W + st.ln.c0) * 2u : kNoAccess;
+                st.okf[r] = row < H ? 1.f : 0.f;
+                NDC_UNROLL
+                for (int i = 0; i < SC; ++i)
+                    st.bvr[i][r] = row < H ? (p.bias ? p.bias[id.c * SC + i] : 0.f) : (p.relu ? -1.f : 0.f);
             }
             NDC_UNROLL
             for (int i = 0; i < SC; ++i) {
-                st.bv[i] = p.bias ? p.bias[id.c * SC + i] : 0.f;
                 st.gbacc[i] = 0.f;
                 NDC_UNROLL
                 for (int a = 0; a < KT; ++a) st.gacc[i][a] = 0.f;
@@ -1132,13 +1138,12 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
                     }
                     NDC_UNROLL
                     for (int r = 0; r < RH; ++r) {
-                        const bool ok = (st.ook >> r) & 1u;
                         NDC_UNROLL
                         for (int i = 0; i < SC; ++i) {
                             float v[RW];
                             NDC_UNROLL
                             for (int c = 0; c < RW; ++c) {
-                                const float s = floor_f((c ? bf_hi(zw[i][r]) : bf_lo(zw[i][r])) + st.bv[i], floor_);
+                                const float s = floor_f((c ? bf_hi(zw[i][r]) : bf_lo(zw[i][r])) + st.bvr[i][r], floor_);
                                 const float g = c ? bf_hi(gw[i][r]) : bf_lo(gw[i][r]);
                                 float gzv;
                                 if (SAVED)
@@ -1147,9 +1152,8 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
                                     gzv = g * acc[0][i][r][c] * fast_rcp(acc[NA > 1 ? 1 : 0][i][r][c]) +
                                           acc[NA - 1][i][r][c];
                                 if (p.relu && s <= 0.f) gzv = 0.f;   // a NaN passes
-                                if (!ok) gzv = 0.f;
-                                sv[i][r][c] = ok ? s : 0.f;
-                                st.gbacc[i] += gzv;
+                                sv[i][r][c] = s;
+                                st.gbacc[i] += gzv * st.okf[r];
                                 v[c] = gzv;
                             }
                             if (have_gz) buf_st<true>(gzb_, st.ooff[r], jo + i * cplane2, pack_bf16x2(v[0], v[1]));
