@@ -435,6 +435,11 @@ MODEL_WORKLOADS = {
 }
 
 
+def _progress(msg: str) -> None:
+    """A line on stderr (stdout carries the one JSON line): long legs report as they go."""
+    print(f"[bench] {msg}", file=sys.stderr, flush=True)
+
+
 def run_model_routes(workload: str, routes, warmup: int, steps: int) -> dict:
     """One model-level workload (MODEL_WORKLOADS) on each of `routes` ("hip": the NDC layers on
     the HIP kernels; "pytorch": the same network with the layers on their general PyTorch
@@ -476,15 +481,17 @@ def run_model_routes(workload: str, routes, warmup: int, steps: int) -> dict:
             loss.backward()
             return loss.detach()
 
-        for _ in range(warmup):
+        for i in range(warmup):
             loss = step()
-        torch.cuda.synchronize()
+            torch.cuda.synchronize()
+            _progress(f"{workload} on the {route} route: warm-up step {i + 1} of {warmup} done")
         torch.cuda.reset_peak_memory_stats()
         t0 = time.perf_counter()
         for _ in range(steps):
             loss = step()
         torch.cuda.synchronize()
         dt = (time.perf_counter() - t0) / steps
+        _progress(f"{workload} on the {route} route: {steps} timed steps, {dt * 1e3:.1f} ms each")
         out = dict(ms_per_step=dt * 1e3, steps_per_s=1.0 / dt, loss=float(loss), steps=steps,
                    warmup=warmup, peak_mem_GB=torch.cuda.max_memory_allocated() / 1e9)
         del model, opt
@@ -767,20 +774,25 @@ def main() -> int:
             "frac": {k: least[k] / k_ms[k] for k in least},
             "step_frac": sum(least.values()) / sum(k_ms[k] for k in least),
         }
+    _progress(f"update node: {ms_per_step:.3f} ms per step")
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(torch)
+        _progress("CPU baseline done")
     if not args.no_train:
         # the second half of the metric, outside the timed region above: Deconver-3D train
         # steps per second (config 4) with the NDC layers on the HIP kernels and, for
         # reference, on the layers' PyTorch route on the same GPU
         del x, z, g
         torch.cuda.empty_cache()
-        t3 = run_model_routes("train3d", ["hip"], warmup=2, steps=5)
-        t3.update(run_model_routes("train3d", ["pytorch"], warmup=1, steps=2))
-        result["train3d_steps_per_s"] = t3["hip"]["steps_per_s"]
-        result["train3d_steps_per_s_pytorch_route"] = t3["pytorch"]["steps_per_s"]
-        result["train3d"] = {"workload": MODEL_WORKLOADS["train3d"]["text"], "routes": t3,
-                             "hip_over_pytorch": t3["hip"]["steps_per_s"] / t3["pytorch"]["steps_per_s"]}
+        try:
+            t3 = run_model_routes("train3d", ["hip"], warmup=2, steps=5)
+            t3.update(run_model_routes("train3d", ["pytorch"], warmup=1, steps=2))
+            result["train3d_steps_per_s"] = t3["hip"]["steps_per_s"]
+            result["train3d_steps_per_s_pytorch_route"] = t3["pytorch"]["steps_per_s"]
+            result["train3d"] = {"workload": MODEL_WORKLOADS["train3d"]["text"], "routes": t3,
+                                 "hip_over_pytorch": t3["hip"]["steps_per_s"] / t3["pytorch"]["steps_per_s"]}
+        except Exception as exc:   # the headline line above is complete without this leg
+            result["train3d_error"] = f"{type(exc).__name__}: {exc}"
     print(json.dumps(result))
     return 0
 
