@@ -8,6 +8,8 @@ forward call (no t1, nothing kept) and the kept-ratio backward kernels the bench
 Tolerances: ``max|d| / max|ref|`` <= 2e-2 for bfloat16 storage, <= 1e-4 for float32.
 """
 
+import sys
+
 import pytest
 import torch
 
@@ -152,8 +154,14 @@ def test_config4_full_size_train_steps_on_both_routes():
                      for m in layers)
         assert on_hip == (route == "hip") and len(layers) == 7
         opt = T.make_optimizer(model)
-        losses[route] = [float(T.train_step(model, opt, images, targets,
-                                            autocast_dtype=torch.bfloat16)) for _ in range(2)]
+        losses[route] = []
+        for step in range(2):
+            losses[route].append(float(T.train_step(model, opt, images, targets,
+                                                    autocast_dtype=torch.bfloat16)))
+            # straight to the process's stderr (past pytest's capture): this test runs for a
+            # minute or two, most of it the library's kernel selection on the PyTorch route
+            sys.__stderr__.write(f"[config 4, {route} route] step {step + 1}: loss {losses[route][-1]:.4f}\n")
+            sys.__stderr__.flush()
         del model, opt
         torch.cuda.empty_cache()
     for a, b in zip(losses["hip"], losses["pytorch"]):
