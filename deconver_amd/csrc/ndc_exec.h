@@ -34,6 +34,14 @@ template <class State> struct DeviceExec {
     NDC_D void sync() { __syncthreads(); }
     NDC_D float ld(int i) const { return lds[i]; }
     NDC_D void st_(int i, float v) { lds[i] = v; }
+    // two consecutive words from an EVEN word index: one 8-byte read
+    NDC_D void ld2(int i, float (&v)[2]) const
+    {
+        typedef __attribute__((ext_vector_type(2))) float f2_t;
+        const f2_t a = *reinterpret_cast<const f2_t *>(lds + i);
+        v[0] = a.x;
+        v[1] = a.y;
+    }
     // four consecutive words from an EVEN word index, as two 8-byte reads (one ds_read2_b64
     // where the compiler pairs them) instead of four 4-byte ones
     NDC_D void ld4(int i, uint32_t (&v)[4]) const
@@ -133,6 +141,16 @@ template <class State> struct HostExec {
             r_tid[i] = -2;
         }
         return mem[i];
+    }
+    void ld2(int i, float (&v)[2])
+    {
+        if (i & 1) {
+            HostFaults &hf = host_faults();
+            ++hf.oob;
+            hf.note("misaligned two-word read", i, cur, -1);
+        }
+        v[0] = ld(i);
+        v[1] = ld(i + 1);
     }
     void ld4(int i, uint32_t (&v)[4])
     {

@@ -93,9 +93,8 @@ static const int kMaxLdsBytes = 160 * 1024;
 
 // S strips of RH rows, RW columns per thread; S >= 2*PH so that the halo rows fit the
 // fixed per-thread bounds
-// left_pad: zero words left of column 0 in an LDS row; 0 = the default, PW rounded up to RW
 static inline bool make_tile(const March &m, int RH, int RW, int target_threads, Tile &t,
-                             int min_strips = 0, int left_pad = 0)
+                             int min_strips = 0)
 {
     const int PH = m.KH / 2, PW = m.KW / 2;
     if (m.W % RW) return false;
@@ -113,7 +112,9 @@ static inline bool make_tile(const March &m, int RH, int RW, int target_threads,
     t.NT = round_up(s * cpw, 64);
     t.TH = s * RH;
     t.ntile = (m.H + t.TH - 1) / t.TH;
-    t.PL = left_pad ? left_pad : round_up(PW, RW);
+    // PW zero words left of column 0: a thread's window (its RW columns and PW either side)
+    // then starts at its own first column, an even word when RW = 2
+    t.PL = PW;
     t.P = round_up(t.PL + m.W + PW, RW);
     t.nseg = 1;
     t.SEG = m.D;
@@ -200,6 +201,24 @@ NDC_HD int clampi(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? hi : v
 // is image row r0 - PH + j: the PH rows above the band, then the PH rows below it.
 NDC_HD int halo_row(int s, int PH, int TH) { return s < PH ? s : TH + s; }
 
+// NW staged words from `at`.  RW = 2: the window starts at an even word (see make_tile) and
+// is read two words at a time.
+template <int NW, int RW, class Exec> NDC_D void read_window(Exec &ex, int at, float (&v)[NW])
+{
+    if constexpr (RW == 2 && NW % 2 == 0) {
+        NDC_UNROLL
+        for (int u = 0; u < NW; u += 2) {
+            float pair[2];
+            ex.ld2(at + u, pair);
+            v[u] = pair[0];
+            v[u + 1] = pair[1];
+        }
+    } else {
+        NDC_UNROLL
+        for (int u = 0; u < NW; ++u) v[u] = ex.ld(at + u);
+    }
+}
+
 // One K-type pass over an NR x RW register tile of outputs.  `base` addresses, in a staged
 // plane of ONE source channel, the word (first input row, first own column - PW); input
 // rows base .. base + NR + KH - 2 feed the NR output rows and every tap plane jd of the KD
@@ -214,24 +233,17 @@ NDC_D void k_rows(Exec &ex, int base, int P, const float (&w)[KD * KH * KW],
 {
     constexpr int NW = RW + KW - 1, NROW = NR + KH - 1;
     float vn[NW];
-    if (PIPE) {
-        NDC_UNROLL
-        for (int u = 0; u < NW; ++u) vn[u] = ex.ld(base + u);
-    }
+    if (PIPE) read_window<NW, RW>(ex, base, vn);
     NDC_UNROLL
     for (int q = 0; q < NROW; ++q) {
         float v[NW];
         if (PIPE) {
             NDC_UNROLL
             for (int u = 0; u < NW; ++u) v[u] = vn[u];
-            if (q + 1 < NROW) {
-                NDC_UNROLL
-                for (int u = 0; u < NW; ++u) vn[u] = ex.ld(base + (q + 1) * P + u);
-            }
+            if (q + 1 < NROW) read_window<NW, RW>(ex, base + (q + 1) * P, vn);
             ex.fence();
         } else {
-            NDC_UNROLL
-            for (int u = 0; u < NW; ++u) v[u] = ex.ld(base + q * P + u);
+            read_window<NW, RW>(ex, base + q * P, v);
         }
         NDC_UNROLL
         for (int th = 0; th < KH; ++th) {
@@ -260,9 +272,7 @@ NDC_D void a_plane(Exec &ex, const int (&base)[NTEN], int P, const float (&wt)[S
     float vn[NTEN][NW];
     if (PIPE) {
         NDC_UNROLL
-        for (int t = 0; t < NTEN; ++t)
-            NDC_UNROLL
-            for (int u = 0; u < NW; ++u) vn[t][u] = ex.ld(base[t] + u);
+        for (int t = 0; t < NTEN; ++t) read_window<NW, RW>(ex, base[t], vn[t]);
     }
     NDC_UNROLL
     for (int q = 0; q < NROW; ++q) {
@@ -274,16 +284,12 @@ NDC_D void a_plane(Exec &ex, const int (&base)[NTEN], int P, const float (&wt)[S
                 for (int u = 0; u < NW; ++u) v[t][u] = vn[t][u];
             if (q + 1 < NROW) {
                 NDC_UNROLL
-                for (int t = 0; t < NTEN; ++t)
-                    NDC_UNROLL
-                    for (int u = 0; u < NW; ++u) vn[t][u] = ex.ld(base[t] + (q + 1) * P + u);
+                for (int t = 0; t < NTEN; ++t) read_window<NW, RW>(ex, base[t] + (q + 1) * P, vn[t]);
             }
             ex.fence();
         } else {
             NDC_UNROLL
-            for (int t = 0; t < NTEN; ++t)
-                NDC_UNROLL
-                for (int u = 0; u < NW; ++u) v[t][u] = ex.ld(base[t] + q * P + u);
+            for (int t = 0; t < NTEN; ++t) read_window<NW, RW>(ex, base[t] + q * P, v[t]);
         }
         NDC_UNROLL
         for (int th = 0; th < KH; ++th) {
@@ -305,15 +311,13 @@ NDC_D void a_plane(Exec &ex, const int (&base)[NTEN], int P, const float (&wt)[S
 
 // NROWS rows of NW staged words of each of NOP operands (row n of operand t at addr(n, t)),
 // handed to body(n, words); PIPE: read one row ahead of the arithmetic (see k_rows).
-template <int NROWS, int NW, int NOP, bool PIPE, class Exec, class Addr, class Body>
+template <int NROWS, int NW, int NOP, bool PIPE, int RW, class Exec, class Addr, class Body>
 NDC_D void stream_rows(Exec &ex, Addr addr, Body body)
 {
     float vn[NOP][NW];
     if (PIPE) {
         NDC_UNROLL
-        for (int t = 0; t < NOP; ++t)
-            NDC_UNROLL
-            for (int u = 0; u < NW; ++u) vn[t][u] = ex.ld(addr(0, t) + u);
+        for (int t = 0; t < NOP; ++t) read_window<NW, RW>(ex, addr(0, t), vn[t]);
     }
     NDC_UNROLL
     for (int n = 0; n < NROWS; ++n) {
@@ -325,16 +329,12 @@ NDC_D void stream_rows(Exec &ex, Addr addr, Body body)
                 for (int u = 0; u < NW; ++u) v[t][u] = vn[t][u];
             if (n + 1 < NROWS) {
                 NDC_UNROLL
-                for (int t = 0; t < NOP; ++t)
-                    NDC_UNROLL
-                    for (int u = 0; u < NW; ++u) vn[t][u] = ex.ld(addr(n + 1, t) + u);
+                for (int t = 0; t < NOP; ++t) read_window<NW, RW>(ex, addr(n + 1, t), vn[t]);
             }
             ex.fence();
         } else {
             NDC_UNROLL
-            for (int t = 0; t < NOP; ++t)
-                NDC_UNROLL
-                for (int u = 0; u < NW; ++u) v[t][u] = ex.ld(addr(n, t) + u);
+            for (int t = 0; t < NOP; ++t) read_window<NW, RW>(ex, addr(n, t), v[t]);
         }
         body(n, v);
     }
@@ -890,7 +890,7 @@ struct Bwd1Kernel {
                         // and is still 3 % faster)
                         constexpr int NQ = RH + 2 * PH;
                         const int cb = PL + st.ln.c0 - PW;
-                        stream_rows<KD * NQ, RW + KW - 1, 2, (KH > 1 && SAVED)>(
+                        stream_rows<KD * NQ, RW + KW - 1, 2, (KH > 1 && SAVED), RW>(
                             ex,
                             [&](int n, int t) NDC_LAMBDA {
                                 const int td = n / NQ, q = n % NQ;
@@ -1160,7 +1160,7 @@ struct Bwd2Kernel {
                     // K-side filter-gradient term: re-read the gt1 window
                     constexpr int NQ = RH + 2 * PH;
                     const int cb = PL + st.ln.c0 - PW;
-                    stream_rows<KD * NQ, RW + KW - 1, 1, (KH > 1 && SAVED)>(
+                    stream_rows<KD * NQ, RW + KW - 1, 1, (KH > 1 && SAVED), RW>(
                         ex,
                         [&](int n, int) NDC_LAMBDA {
                             const int td = n / NQ, q = n % NQ;

@@ -143,10 +143,8 @@ static inline bool make_plan(const KGeom &q, Plan &pl, bool pairs_ok = true, int
         (long long)q.sc * q.SP * 2 < (1LL << 31) &&
         pl.m.KH == 3 && pl.m.KW == 3 && tn.dot2) {
         Tile tf, tb;
-        // one zero word left of column 0: every thread's four-word window (its column pair
-        // and one column either side) then starts at an even word, i.e. 8-byte aligned
-        if (make_tile(pl.m, kDot2RH, 2, tn.threads_f2, tf, FwdKernelB<kDot2RH>::kMinStrips, 1) &&
-            make_tile(pl.m, kDot2RH, 2, tn.threads_b2, tb, 0, 1)) {
+        if (make_tile(pl.m, kDot2RH, 2, tn.threads_f2, tf, FwdKernelB<kDot2RH>::kMinStrips) &&
+            make_tile(pl.m, kDot2RH, 2, tn.threads_b2, tb)) {
             const int lf = FwdKernelB<kDot2RH>::lds_floats(tf);
             const int l1 = Bwd1KernelB<kDot2RH>::lds_floats(tb);
             const int l2 = Bwd2KernelB<kDot2RH>::lds_floats(tb);

@@ -84,8 +84,7 @@ NDC_HD float bf_lo(uint32_t w) { return bits_to_float(w << 16); }
 NDC_HD float bf_hi(uint32_t w) { return bits_to_float(w & 0xffff0000u); }
 
 // NW staged words from `at`; four at a time where NW = 4 (the word index of every such read
-// is even: the tiles of these kernels put one zero word left of column 0, so a thread's
-// window starts at its own even column)
+// is even: a thread's window starts at its own first column, see make_tile)
 template <int NW, class Exec> NDC_D void read_words(Exec &ex, int at, uint32_t (&v)[NW])
 {
     if constexpr (NW == 4) {
