@@ -949,7 +949,10 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
         float gbacc[SC];
         float sprev[SC][RH][RW];   // own source values of the previous plane
         uint32_t px[NXR], pt[NXR], pg[NXR], pxprev[NXR], ptprev[NXR], pgprev[NXR];
-        uint32_t qz[SC][RH], qg[SC][RH], qr[SC][RH];   // SAVED: words fetched a step ahead
+        // SAVED: the z, gout, n/d words of two planes: the step of plane parity P works on set P
+        // and fetches the next plane's into set 1 - P (the plane loop is unrolled twice, so
+        // the sets are fixed registers and nothing is copied from step to step)
+        uint32_t qz[2][SC][RH], qg[2][SC][RH], qr[2][SC][RH];
     };
 
     static NDC_HD int rows_x(int TH) { return TH + 2; }
@@ -1057,7 +1060,9 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
                     NDC_UNROLL
                     for (int c = 0; c < RW; ++c) st.sprev[i][r][c] = 0.f;
                 NDC_UNROLL
-                for (int r = 0; r < RH; ++r) st.qz[i][r] = st.qg[i][r] = st.qr[i][r] = 0u;
+                for (int r = 0; r < RH; ++r)
+                    NDC_UNROLL
+                    for (int a = 0; a < 2; ++a) st.qz[a][i][r] = st.qg[a][i][r] = st.qr[a][i][r] = 0u;
             }
             for (int i = tid; i < total; i += nthreads) ex.st_(i, 0.f);
             load_plane(st, 0);
@@ -1066,13 +1071,10 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
 
         // one step past the usual end so that an unpaired last plane still gets its
         // filter-gradient contribution (paired with a zero plane)
-        for (int kk = 0; kk < D + 2; ++kk) {
-            const int k = uniform_int(kk);   // the plane index stays on the scalar unit
-            ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k); });
-            ex.sync();
-
-            const int j0 = k - 1;
-            ex.each([&](State &st, int) NDC_LAMBDA {
+        // one plane step; PAR = k % 2, known at compile time (the loop below is unrolled twice)
+        auto compute = [&](State &st, int k, auto par_tag) NDC_LAMBDA {
+                constexpr int PAR = decltype(par_tag)::value;
+                const int j0 = k - 1;
                 if (!st.ln.active) return;
                 load_plane(st, k + 1);
                 // SAVED: this plane's z, gout, n/d words were fetched a step ago; take them and
@@ -1084,12 +1086,12 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
                     for (int r = 0; r < RH; ++r)
                         NDC_UNROLL
                         for (int i = 0; i < SC; ++i) {
-                            zw[i][r] = st.qz[i][r];
-                            gw[i][r] = st.qg[i][r];
-                            rw[i][r] = st.qr[i][r];
-                            st.qz[i][r] = buf_ld(zb_, st.ooff[r], jn + i * cplane2);
-                            st.qg[i][r] = buf_ld<true>(gb_, st.ooff[r], jn + i * cplane2);
-                            st.qr[i][r] = buf_ld<true>(rb_, st.ooff[r], jn + i * cplane2);
+                            zw[i][r] = st.qz[PAR][i][r];
+                            gw[i][r] = st.qg[PAR][i][r];
+                            rw[i][r] = st.qr[PAR][i][r];
+                            st.qz[1 - PAR][i][r] = buf_ld(zb_, st.ooff[r], jn + i * cplane2);
+                            st.qg[1 - PAR][i][r] = buf_ld<true>(gb_, st.ooff[r], jn + i * cplane2);
+                            st.qr[1 - PAR][i][r] = buf_ld<true>(rb_, st.ooff[r], jn + i * cplane2);
                         }
                 }
                 if (j0 < 0) return;
@@ -1159,7 +1161,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
                         }
                     }
                 }
-                if (need_gh && (j0 & 1) && j0 <= D) {
+                if (PAR == 0 && need_gh && j0 <= D) {   // j0 odd
                     // K-side filter-gradient term for the plane pair (j0 - 1, j0):
                     // (s_i[j0-1], s_i[j0]) . (gt1[m], gt1[m+1])[neighbour], m = j0 - td
                     uint32_t ss[SC][RH][RW];
@@ -1195,13 +1197,28 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
                             }
                         });
                 }
-                NDC_UNROLL
-                for (int i = 0; i < SC; ++i)
+                if (PAR == 1) {   // j0 even: the next step pairs this plane's source values with its own
                     NDC_UNROLL
-                    for (int r = 0; r < RH; ++r)
+                    for (int i = 0; i < SC; ++i)
                         NDC_UNROLL
-                        for (int c = 0; c < RW; ++c) st.sprev[i][r][c] = sv[i][r][c];
-            });
+                        for (int r = 0; r < RH; ++r)
+                            NDC_UNROLL
+                            for (int c = 0; c < RW; ++c) st.sprev[i][r][c] = sv[i][r][c];
+                }
+        };
+        for (int kk = 0; kk < D + 2; kk += 2) {
+            {
+                const int k = uniform_int(kk);   // the plane index stays on the scalar unit
+                ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k); });
+                ex.sync();
+                ex.each([&](State &st, int) NDC_LAMBDA { compute(st, k, IntTag<0>()); });
+            }
+            if (kk + 1 < D + 2) {
+                const int k = uniform_int(kk + 1);
+                ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k); });
+                ex.sync();
+                ex.each([&](State &st, int) NDC_LAMBDA { compute(st, k, IntTag<1>()); });
+            }
         }
 
         if (p.need_gh || p.need_gb) {
