@@ -112,6 +112,21 @@ NDC_HD float dot2_bf16(uint32_t a, uint32_t b, float acc)
 #endif
 }
 
+// init + a.lo*b.lo + a.hi*b.hi with `b` a wave-uniform word: the three-operand
+// v_dot2_f32_bf16, for the FIRST term of an accumulation.  The two-operand form the compiler
+// selects for dot2_bf16 accumulates in place, so starting a sum from a value held elsewhere
+// costs it a register copy per accumulator first; this form reads `init` where it lies.
+NDC_HD float dot2_bf16_from(uint32_t a, uint32_t b_uniform, float init)
+{
+#if NDC_DEVICE_BUILD && defined(__HIP_DEVICE_COMPILE__)
+    float r;
+    asm("v_dot2_f32_bf16 %0, %1, %2, %3" : "=v"(r) : "s"(b_uniform), "v"(a), "v"(init));
+    return r;
+#else
+    return dot2_bf16(a, b_uniform, init);
+#endif
+}
+
 // N consecutive elements <-> N floats with one memory access (N = 1 or 2; the address must
 // be aligned to N elements)
 template <typename T, int N> struct VecIO;

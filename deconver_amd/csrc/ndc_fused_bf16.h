@@ -145,9 +145,10 @@ NDC_D void k_rows_d2(Exec &ex, int base, int P, const float (&w)[27], float (*ac
 }
 
 // A-type pass over an NR x RW tile for one plane-pair slot of NTEN operands; wt = WA[s].
-template <int NR, int RW, int NTEN, bool PIPE, class Exec>
+// FRESH: the sums start here, from `init` (what `acc` holds on entry is not read).
+template <int NR, int RW, int NTEN, bool PIPE, bool FRESH = false, class Exec>
 NDC_D void a_plane_d2(Exec &ex, const int (&base)[NTEN], int P, const float (&wt)[4][9],
-                      float (&acc)[NTEN][4][NR][RW])
+                      float (&acc)[NTEN][4][NR][RW], float init = 0.f)
 {
     uint32_t vn[NTEN][RW + 2];
     if (PIPE) {
@@ -180,11 +181,15 @@ NDC_D void a_plane_d2(Exec &ex, const int (&base)[NTEN], int P, const float (&wt
                 NDC_UNROLL
                 for (int i = 0; i < 4; ++i) {
                     const uint32_t wv = float_to_bits(wt[i][th * 3 + tw]);
+                    // an output row's first term comes from its first input row (q = rr: th = 2)
+                    // and first column tap
+                    const bool first = FRESH && th == 2 && tw == 0;
                     NDC_UNROLL
                     for (int t = 0; t < NTEN; ++t)
                         NDC_UNROLL
                         for (int c = 0; c < RW; ++c)
-                            acc[t][i][rr][c] = dot2_bf16(v[t][c + 2 - tw], wv, acc[t][i][rr][c]);
+                            acc[t][i][rr][c] = first ? dot2_bf16_from(v[t][c + 2 - tw], wv, init)
+                                                     : dot2_bf16(v[t][c + 2 - tw], wv, acc[t][i][rr][c]);
                 }
         }
     }
@@ -505,15 +510,7 @@ template <int RH_> struct FwdKernelB {
                     NDC_UNROLL
                     for (int i = 0; i < SC; ++i)
                         own[i][r] = buf_ld(zb_, st.ooff[r], (unsigned)j0 * plane2 + i * cplane2);
-                float acc[2][SC][RH][RW];
-                NDC_UNROLL
-                for (int a = 0; a < 2; ++a)
-                    NDC_UNROLL
-                    for (int i = 0; i < SC; ++i)
-                        NDC_UNROLL
-                        for (int r = 0; r < RH; ++r)
-                            NDC_UNROLL
-                            for (int c = 0; c < RW; ++c) acc[a][i][r][c] = eps;   // n, d start at eps
+                float acc[2][SC][RH][RW];   // n, d: their sums start at eps (first pass below)
                 {
                     // depth taps 2 and 1 from the plane-pair words (x, t1)[j0-1 .. j0]
                     float wt[SC][9];
@@ -522,7 +519,7 @@ template <int RH_> struct FwdKernelB {
                     const int ob = (st.ln.strip * RH) * P + PL + st.ln.c0 - PW;
                     const int base[2] = {off_x + wrap(m % NX, NX) * RX * P + ob,
                                          off_t + wrap(m % NTP, NTP) * RX * P + ob};
-                    a_plane_d2<RH, RW, 2, false>(ex, base, P, wt, acc);
+                    a_plane_d2<RH, RW, 2, false, true>(ex, base, P, wt, acc, eps);
                 }
                 {
                     // depth tap 0 from the column-pair words of plane j0 + 1
