@@ -249,7 +249,7 @@ NDC_HD uint32_t buf_ld(const BufRef &b, unsigned lane_off, unsigned uniform_off)
     (void)b; (void)lane_off; (void)uniform_off;
     return 0u;
 #else
-    if (lane_off >= kNoAccess) return 0u;
+    if (lane_off >= kNoAccess || b.base == nullptr) return 0u;   // by design: nothing there
     const size_t o = (size_t)lane_off + uniform_off;
     if (o + 4 > b.bytes) {
         HostFaults &hf = host_faults();
@@ -273,7 +273,7 @@ NDC_HD void buf_st(const BufRef &b, unsigned lane_off, unsigned uniform_off, uin
 #elif NDC_DEVICE_BUILD
     (void)b; (void)lane_off; (void)uniform_off; (void)w;
 #else
-    if (lane_off >= kNoAccess) return;
+    if (lane_off >= kNoAccess || b.base == nullptr) return;   // by design: goes nowhere
     const size_t o = (size_t)lane_off + uniform_off;
     if (o + 4 > b.bytes) {
         HostFaults &hf = host_faults();

@@ -980,7 +980,6 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
         const BufRef zb_ = make_buf(p.z + cbase * SC, sbytes), gb_ = make_buf(p.gout + cbase * SC, sbytes);
         const BufRef rb_ = make_buf(SAVED ? p.ratio + cbase * SC : nullptr, sbytes);
         const BufRef gzb_ = make_buf(p.gz ? p.gz + cbase * SC : nullptr, sbytes);
-        const bool have_gz = p.gz != nullptr;
         UniformF tab = as_uniform(p.wtab + (long long)id.c * kTabWords);
         const int r0 = id.r0;
         const int nthreads = ex.nthreads;
@@ -1154,7 +1153,8 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
                                 st.gbacc[i] += gzv * st.okf[r];
                                 v[c] = gzv;
                             }
-                            if (have_gz) buf_st<true>(gzb_, st.ooff[r], jo + i * cplane2, pack_bf16x2(v[0], v[1]));
+                            // (no gz asked for: gzb_ is an empty slice and the store goes nowhere)
+                            buf_st<true>(gzb_, st.ooff[r], jo + i * cplane2, pack_bf16x2(v[0], v[1]));
                         }
                     }
                 }
