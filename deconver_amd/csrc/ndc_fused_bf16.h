@@ -440,11 +440,13 @@ template <int RH_> struct FwdKernelB {
             load_plane(st, 0);
         });
         ex.sync();
+        ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, 0); });
+        ex.sync();
 
+        // Two barriers per plane step: the source plane of the NEXT step is staged at the end of
+        // the gather phase (nothing reads the source slot there), not in a phase of its own.
         for (int kk = 0; kk < D + 2; ++kk) {
             const int k = uniform_int(kk);   // the plane index stays on the scalar unit
-            ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k); });
-            ex.sync();
 
             // ---- K-scatter of source plane k; t1 plane k - 1
             ex.each([&](State &st, int) NDC_LAMBDA {
@@ -496,12 +498,15 @@ template <int RH_> struct FwdKernelB {
             });
             ex.sync();
 
-            // ---- prefetch, then A-gather + epilogue of plane k - 2
+            // ---- prefetch, then A-gather + epilogue of plane k - 2, then staging of plane k + 1
             ex.each([&](State &st, int) NDC_LAMBDA {
                 if (!st.ln.active) return;
                 load_plane(st, k + 1);
                 const int j0 = k - 2;
-                if (j0 < 0) return;
+                if (j0 < 0) {
+                    store_plane(st, k + 1);
+                    return;
+                }
                 // the thread's own source values of plane j0: z is read again (it was staged two
                 // steps ago, so this hits the L2) rather than kept in LDS or registers that long
                 uint32_t own[SC][RH];
@@ -552,7 +557,9 @@ template <int RH_> struct FwdKernelB {
                         }
                     }
                 }
+                store_plane(st, k + 1);
             });
+            ex.sync();
         }
     }
 };
@@ -804,11 +811,13 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
             load_plane(st, 0);
         });
         ex.sync();
+        ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, 0); });
+        ex.sync();
 
+        // Two barriers per plane step: the (x, t1) plane of the NEXT step is staged at the end
+        // of the scatter phase (the ring slots it overwrites were last read in the phase before).
         for (int kk = 0; kk < D + 2; ++kk) {
             const int k = uniform_int(kk);   // the plane index stays on the scalar unit
-            ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k); });
-            ex.sync();
 
             const int j1 = k - 1;
             const bool live1 = j1 >= 0 && j1 < D;
@@ -907,7 +916,9 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
                         st.acct[2][r][c] = 0.f;
                     }
                 }
+                store_plane(st, k + 1);
             });
+            ex.sync();
         }
 
         if (need_gh) {
