@@ -536,11 +536,13 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
             load_plane(st, k_first);
         });
         ex.sync();
+        ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k_first); });
+        ex.sync();
 
+        // Two barriers per plane step: the source plane of the NEXT step is staged at the end of
+        // the gather phase (which does not read the source area), not in a phase of its own.
         for (int kk = k_first; kk < k_end; ++kk) {
             const int k = uniform_int(kk);   // the plane index stays on the scalar unit
-            ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k); });
-            ex.sync();
 
             // ---- K-scatter: plane k of s feeds the KD pending planes of t1
             ex.each([&](State &st, int) NDC_LAMBDA {
@@ -594,7 +596,10 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                 if (!st.ln.active) return;
                 load_plane(st, k + 1);
                 const int j0 = k - 2 * PD;
-                if (j0 < d0) return;
+                if (j0 < d0) {
+                    store_plane(st, k + 1);
+                    return;
+                }
                 // the thread's own source values: re-read from global (an L2 hit) rather
                 // than carried in registers across 2*PD planes
                 float sv[SC][RH][RW];
@@ -654,7 +659,9 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                         }
                     }
                 }
+                store_plane(st, k + 1);
             });
+            ex.sync();
         }
     }
 };
@@ -868,11 +875,13 @@ struct Bwd1Kernel {
             load_plane(st, k_first);
         });
         ex.sync();
+        ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k_first); });
+        ex.sync();
 
+        // Two barriers per plane step: the (x, t1) plane of the NEXT step is staged at the end
+        // of the scatter phase, into the ring slot that no phase of this step reads.
         for (int kk = k_first; kk < k_end; ++kk) {
             const int k = uniform_int(kk);   // the plane index stays on the scalar unit
-            ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k); });
-            ex.sync();
 
             // ---- gather: gn, gd of plane k - PD on the band plus PH halo rows each side
             const int j1 = k - PD;
@@ -958,7 +967,9 @@ struct Bwd1Kernel {
                         st.acct[KD - 1][r][c] = 0.f;
                     }
                 }
+                store_plane(st, k + 1);
             });
+            ex.sync();
         }
 
         if (need_gh) {
