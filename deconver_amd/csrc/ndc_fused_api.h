@@ -119,7 +119,7 @@ static inline void plan_lds(Plan &pl)
 // pairs_ok: every activation pointer of the call is aligned to two elements
 static const int kDot2RH = 2;   // rows per thread of the bf16 dot2 kernels (columns: 2)
 
-static inline bool make_plan(const KGeom &q, Plan &pl, bool pairs_ok = true, int dtype = NDC_F32)
+static inline bool make_plan_for(const KGeom &q, Plan &pl, bool pairs_ok, int dtype)
 {
     pl.m = march_of(q);
     pl.dot2 = false;
@@ -167,6 +167,15 @@ static inline bool make_plan(const KGeom &q, Plan &pl, bool pairs_ok = true, int
     pl.nblk_f = (int)nf;
     pl.nblk_b = (int)nb;
     return true;
+}
+
+// The column-pair variants hold more of a row per workgroup: where their LDS need exceeds a
+// workgroup's share (wide rows of a tall image) the one-column variants may still fit, and
+// those are what supported() answers for.
+static inline bool make_plan(const KGeom &q, Plan &pl, bool pairs_ok = true, int dtype = NDC_F32)
+{
+    if (make_plan_for(q, pl, pairs_ok, dtype)) return true;
+    return pairs_ok && make_plan_for(q, pl, false, dtype);
 }
 
 static inline bool supported(const KGeom &q)

@@ -37,6 +37,9 @@ FUSED_GEOMS = [
     (32, 32, 4, (5, 5), (64, 64), 1),
     (8, 8, 4, (5, 5), (40, 100), 2),
     (16, 16, 4, (3, 3), (17, 15), 2),
+    # widest row of the bf16 dot2 kernels (512 threads, > 64 KiB of LDS); in float32 the
+    # column-pair kernels' LDS does not fit and the plan falls back to the one-column ones
+    (4, 4, 4, (3, 3, 3), (6, 10, 256), 1),
 ]
 
 

@@ -21,6 +21,8 @@ FUSED_GEOMS = [
     (2, 4, (5, 5), (70, 12), 1),          # 2-D, long march: split into two segments
     (1, 4, (5, 5), (101, 6), 2),          # 2-D, three segments, ragged last one
     (1, 4, (3, 3, 3), (37, 4, 6), 1),     # 3-D, two segments
+    (2, 4, (3, 3, 3), (3, 10, 256), 1),   # wide rows of a tall plane: the column-pair variant's
+                                          # LDS does not fit, the plan falls back to one column
 ]
 
 
@@ -112,6 +114,7 @@ BF16_GEOMS = [
     (1, 4, (3, 3, 3), (1, 4, 6), 1),      # dot2: single plane
     (2, 4, (3, 3, 3), (6, 3, 70), 1),     # dot2: two wavefronts per row
     (2, 4, (3, 3, 3), (3, 7, 13), 2),     # odd width: unpaired FMA kernels
+    (2, 4, (3, 3, 3), (3, 10, 256), 1),   # dot2: widest row (512 threads, > 64 KiB of LDS)
 ]
 
 
