@@ -34,7 +34,7 @@ __global__ void __launch_bounds__(256) block_reduce_kernel(float *out, F partial
 template <class Kernel>
 __global__ void __launch_bounds__(512) block_kernel_entry(typename Kernel::Params p)
 {
-    extern __shared__ float ndc_lds[];
+    extern __shared__ __attribute__((aligned(16))) float ndc_lds[];
     DeviceExec<typename Kernel::State> ex;
     ex.lds = ndc_lds;
     ex.tid = threadIdx.x;
@@ -49,7 +49,7 @@ template <class Kernel>
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4)))
 block_kernel_entry_w4(typename Kernel::Params p)
 {
-    extern __shared__ float ndc_lds[];
+    extern __shared__ __attribute__((aligned(16))) float ndc_lds[];
     DeviceExec<typename Kernel::State> ex;
     ex.lds = ndc_lds;
     ex.tid = threadIdx.x;

@@ -54,6 +54,24 @@ template <class State> struct DeviceExec {
         v[2] = b.x;
         v[3] = b.y;
     }
+    // four consecutive words from a word index that is a multiple of 4: one 16-byte read
+    NDC_D void ld4a(int i, uint32_t (&v)[4]) const
+    {
+        typedef __attribute__((ext_vector_type(4))) uint32_t u4_t;
+        const u4_t a = *reinterpret_cast<const u4_t *>(lds + i);
+        v[0] = a.x;
+        v[1] = a.y;
+        v[2] = a.z;
+        v[3] = a.w;
+    }
+    // two words to an EVEN word index: one 8-byte write
+    NDC_D void st2(int i, uint32_t a, uint32_t b)
+    {
+        typedef __attribute__((ext_vector_type(2))) uint32_t u2_t;
+        const u2_t v = {a, b};
+        *reinterpret_cast<u2_t *>(lds + i) = v;
+    }
+    NDC_D void stw(int i, uint32_t a) { lds[i] = __uint_as_float(a); }
     // The instruction scheduler may not move anything across this point: used to keep the LDS
     // reads of the next row ahead of the arithmetic on the current one.
     NDC_D void fence() const { __builtin_amdgcn_sched_barrier(0); }
@@ -163,6 +181,34 @@ template <class State> struct HostExec {
             const float f = ld(i + u);
             memcpy(&v[u], &f, 4);
         }
+    }
+    void ld4a(int i, uint32_t (&v)[4])
+    {
+        if (i & 3) {
+            HostFaults &hf = host_faults();
+            ++hf.oob;
+            hf.note("misaligned 16-byte read", i, cur, -1);
+        }
+        for (int u = 0; u < 4; ++u) {
+            const float f = ld(i + u);
+            memcpy(&v[u], &f, 4);
+        }
+    }
+    void stw(int i, uint32_t a)
+    {
+        float f;
+        memcpy(&f, &a, 4);
+        st_(i, f);
+    }
+    void st2(int i, uint32_t a, uint32_t b)
+    {
+        if (i & 1) {
+            HostFaults &hf = host_faults();
+            ++hf.oob;
+            hf.note("misaligned 8-byte write", i, cur, -1);
+        }
+        stw(i, a);
+        stw(i + 1, b);
     }
     void st_(int i, float v)
     {

@@ -7,7 +7,7 @@
 #include <stdlib.h>
 
 #include "ndc_fused.h"
-#include "ndc_fused_bf16.h"
+#include "ndc_fused_mfma.h"
 
 namespace ndc {
 namespace fused {
@@ -39,6 +39,7 @@ struct Tuning {
     int threads_f, threads_b;    // workgroup sizes of the FMA kernels, forward / backward
     int threads_f2, threads_b2;  // ... of the bf16 dot2 kernels
     int split, dot2;             // march segments on / bf16 dot2 kernels on
+    int mfma;                    // bf16 matrix-instruction kernels on (where they cover the geometry)
 };
 
 #ifdef NDC_TUNING
@@ -53,11 +54,12 @@ static inline const Tuning &tuning()
                              env_int("NDC_TUNE_RHB", 0),  env_int("NDC_TUNE_RWB", 0),
                              env_int("NDC_TUNE_NTF", 256), env_int("NDC_TUNE_NTB", 512),
                              env_int("NDC_TUNE_NTF2", 256), env_int("NDC_TUNE_NTB2", 256),
-                             env_int("NDC_TUNE_SPLIT", 1), env_int("NDC_TUNE_DOT2", 1)};
+                             env_int("NDC_TUNE_SPLIT", 1), env_int("NDC_TUNE_DOT2", 1),
+                             env_int("NDC_TUNE_MFMA", 1)};
     return t;
 }
 #else
-static inline Tuning tuning() { return Tuning{0, 0, 0, 0, 256, 512, 256, 256, 1, 1}; }
+static inline Tuning tuning() { return Tuning{0, 0, 0, 0, 256, 512, 256, 256, 1, 1, 1}; }
 #endif
 
 // first listed row of this filter geometry that the width / alignment allow (and, in a
@@ -99,6 +101,7 @@ struct Plan {
     Variant v;
     March m;
     bool dot2;            // bf16 dot2 kernels (3x3x3, SC = 4, even W, aligned pairs)
+    bool mfma1;           // ... with pass 1 on the matrix instruction when it reads the forward's ratios
     Tile tf, tb;          // forward / backward launch shapes
     int lds_f, lds_b1, lds_b2;
     int nblk_f, nblk_b;
@@ -123,6 +126,7 @@ static inline bool make_plan_for(const KGeom &q, Plan &pl, bool pairs_ok, int dt
 {
     pl.m = march_of(q);
     pl.dot2 = false;
+    pl.mfma1 = false;
     // 32-bit offsets inside one (sample, channel) volume
     if ((long long)q.sc * q.SP >= (1LL << 31)) return false;
     if (!find_variant(q, pl.m, pairs_ok, pl.v)) return false;
@@ -156,6 +160,8 @@ static inline bool make_plan_for(const KGeom &q, Plan &pl, bool pairs_ok, int dt
                 pl.lds_f = lf;
                 pl.lds_b1 = l1;
                 pl.lds_b2 = l2;
+                pl.mfma1 = tn.mfma && Bwd1KernelM<kDot2RH>::covers(pl.m.W) &&
+                           Bwd1KernelM<kDot2RH>::lds_floats(tb) <= cap2;
             }
         }
     }
@@ -235,6 +241,9 @@ template <class BE> struct Dot2Launch<BE, bf16_t> {
     // saved: the call brought the forward's s/d and n/d
     static int bwd1(const BwdParams<bf16_t> &p, const Plan &pl, void *stream, bool saved)
     {
+        if (saved && pl.mfma1)
+            return BE::template block_kernel<Bwd1KernelM<kDot2RH>>(
+                p, pl.nblk_b, pl.tb.NT, Bwd1KernelM<kDot2RH>::lds_floats(pl.tb), stream);
         if (saved)
             return BE::template block_kernel<Bwd1KernelB<kDot2RH, true>>(
                 p, pl.nblk_b, pl.tb.NT, Bwd1KernelB<kDot2RH, true>::lds_floats(pl.tb), stream);

@@ -31,6 +31,9 @@
 //                       s = 1: (0,               h[i][0][th][tw])             72 words
 //   WQ[th][i][n]      = n = 0: (h1, h0)  1: (0, h2)  2: (h2, h1)  3: (h0, 0),
 //                       h_tw = h[i][0][th][tw]                                  48 words
+//   WM[m][th][tw]     = rows of the 4x4 tap matrices of the matrix-instruction kernels
+//                       (ndc_fused_mfma.h): the four source channels' taps of tap plane
+//                       2 - m, (h[0], h[1]) then (h[2], h[3]); m = 3: zeros        72 words
 #pragma once
 
 #include "ndc_fused.h"
@@ -38,8 +41,8 @@
 namespace ndc {
 namespace fused {
 
-static const int kTabWK = 0, kTabWA = 54, kTabWQ = 126;
-static const int kTabWords = 174;   // packed tap words per channel (54 WK + 72 WA + 48 WQ)
+static const int kTabWK = 0, kTabWA = 54, kTabWQ = 126, kTabWM = 174;
+static const int kTabWords = 246;   // packed tap words per channel (54 WK + 72 WA + 48 WQ + 72 WM)
 
 // idx over C * kTabWords
 NDC_HD void prep_tables(long long idx, const float *h, float *tab)
@@ -54,11 +57,15 @@ NDC_HD void prep_tables(long long idx, const float *h, float *tab)
         const int r = e - 54, s = r / 36, i = (r % 36) / 9, t9 = r % 9;
         w = s == 0 ? pack_bf16x2(hc[i * 27 + 2 * 9 + t9], hc[i * 27 + 1 * 9 + t9])
                    : pack_bf16x2(0.f, hc[i * 27 + t9]);
-    } else {
+    } else if (e < kTabWM) {
         const int r = e - kTabWQ, th = r / 16, i = (r % 16) / 4, n = r % 4;
         const float *ht = hc + i * 27 + th * 3;   // the tap row h[i][0][th][0..2]
         w = n == 0 ? pack_bf16x2(ht[1], ht[0]) : n == 1 ? pack_bf16x2(0.f, ht[2])
           : n == 2 ? pack_bf16x2(ht[2], ht[1]) : pack_bf16x2(ht[0], 0.f);
+    } else {
+        const int r = e - kTabWM, m = r / 18, t9 = (r % 18) / 2, half = r % 2;
+        const int tau = (2 - m) * 9 + t9;
+        w = m == 3 ? 0u : pack_bf16x2(hc[(2 * half) * 27 + tau], hc[(2 * half + 1) * 27 + tau]);
     }
     tab[idx] = bits_to_float(w);
 }

@@ -1,0 +1,361 @@
+// bfloat16 kernels of the 3x3x3, SC = 4 depthwise geometry built on the 4x4x4 matrix
+// instruction (mfma_bf16_4x4x4 in ndc_common.h): 1024 multiply-accumulates per wavefront
+// instruction in about 10 clocks, where v_dot2c_f32_bf16 does 128 in 4.5.  Same work
+// decomposition and march as ndc_fused_bf16.h (a thread owns RH rows x 2 columns); what
+// changes is how the tap sums map to instructions.
+//
+//   K-type applications (4 -> 1 channels, scattered into the three pending output planes):
+//     per (th, tw) one instruction per output voxel column,
+//       D[m][n] += sum_i  H[m][i] * S[i][n],   H[m][i] = h[i][2 - m][th][tw]  (m = 3: zeros)
+//     n = the lane's voxel, S[.][n] = its four source channels at the tap's neighbour,
+//     D[m][n] = pending output plane m at the lane's voxel.  The source is staged as four
+//     bf16 channels (8 bytes) per voxel; a thread reads the 4-voxel window of a row once
+//     (two 16-byte reads) and picks the neighbour per tap from registers.  The tap rows H
+//     sit in 18 registers per lane (lane & 3 selects the row m).
+//
+//   Filter-gradient terms  gh[i][tap] = sum_voxels g_i[v] * u[v + shift(tap)]  (g = gn or gd
+//     with u = x or t1):  per (td, th) and 4-voxel group of a row
+//       D[i][j] += sum_{k<4} g_i[c + k] * u[c + k + j - 1]        (j <-> tw = 2 - j)
+//     lane (b, i) reads channel i of the staged g row (channel-major copy), lane (b, j) the
+//     window of u starting at column c + j - 1.  LDS reads of 8 or 16 bytes must be aligned
+//     to their size, so each u row is staged three times, shifted by -1, 0 and +1 column;
+//     lane j reads copy j at the block's own (aligned) position.  The shifted words are made
+//     from the lane's own column pair and its left neighbour's (one wavefront shift).
+//     Each lane ends with the 9 x 4 sums of its block for ONE tw; the block reduction at the
+//     end of the kernel adds lanes with equal (lane & 3).
+//
+// Both forms need whole 4-lane blocks inside one image row and a row inside one wavefront:
+// W a multiple of 8 and W / 2 a divisor of 64.
+#pragma once
+
+#include "ndc_fused_bf16.h"
+
+namespace ndc {
+namespace fused {
+
+// (hi half of `left`, lo half of `own`): the bf16 pair one column to the left of `own`
+NDC_HD uint32_t shift_in_left(uint32_t own, uint32_t left) { return (left >> 16) | (own << 16); }
+
+// =================================================================== backward pass 1 (bf16, matrix instruction)
+
+// Reads the forward's s/d and n/d (the form every training step uses): gn = g s/d,
+// gd = -gn n/d, gx = K(gn), gt1 = K(gd), and the A-side filter-gradient terms.
+template <int RH_> struct Bwd1KernelM {
+    static constexpr bool SAVED = true;
+    static constexpr int KD = 3, KH = 3, KW = 3, SC = 4, RH = RH_, RW = 2;
+    static constexpr int PD = 1, PH = 1, PW = 1, KT = 27;
+    static constexpr int NXS = RH + 1;   // x / t1 rows a thread stages (the last: first two strips)
+    static constexpr int NX = 3;         // ring slots of x / t1 planes
+    static constexpr int NRED = SC * KT;
+    typedef bf16_t T;
+    typedef BwdParams<T> Params;
+
+    struct State {
+        Lane ln;
+        int lane4, blk4;      // lane & 3; first word of the lane's block in a row of pairs
+        unsigned xoff[NXS], ooff[RH], hoff;
+        unsigned xok;
+        MfmaRows wm[9];
+        f4_t accx[RH][RW], acct[RH][RW];
+        f4_t gacc[KD][KH];
+        uint32_t px[NXS], pt[NXS];
+        uint32_t qg[SC][RH + 1], qd[SC][RH + 1], qr[SC][RH + 1];
+    };
+
+    static NDC_HD bool covers(int W) { return W % 8 == 0 && W <= 128 && 64 % (W / 2) == 0; }
+    static NDC_HD int rows_g(int TH) { return TH + 2; }
+    // strides of the channel rows of the channel-major copy and of the shifted copies: a
+    // multiple of 64 words plus 16, so that the four lanes of a block, which read four
+    // different channels (copies) at one position, hit different banks
+    static NDC_HD int stride_gc(int TH, int W) { return round_up_hd(TH * (W / 2), 64) + 16; }
+    static NDC_HD int stride_xs(int TH, int W) { return round_up_hd((TH + 2) * (W / 2), 64) + 16; }
+    static NDC_HD int round_up_hd(int v, int a) { return (v + a - 1) / a * a; }
+    static NDC_HD int lds_floats(const Tile &t)
+    {
+        const int W = t.CPW * RW;
+        const int main_ = 2 * rows_g(t.TH) * 2 * t.P + 2 * SC * stride_gc(t.TH, W) +
+                          NX * 2 * 3 * stride_xs(t.TH, W);
+        const int red = (t.NT / 64) * NRED;
+        return main_ > red ? main_ : red;
+    }
+
+    template <class Exec> static NDC_D void run(Exec &ex, const Params &p, int block_id)
+    {
+        const Tile t = p.t;
+        const BlockId id = decode_block(block_id, p.C, t, p.D);
+        const int S = t.S, PL = t.PL, TH = t.TH, W = p.W, H = p.H, D = p.D;
+        const int P2 = 2 * t.P, WH = W / 2;
+        const int RG = rows_g(TH), RXS = TH + 2;
+        const int GCS = stride_gc(TH, W), XCS = stride_xs(TH, W);
+        const int off_gp = 0, off_gc = 2 * RG * P2, off_xs = off_gc + 2 * SC * GCS;
+        const int total = off_xs + NX * 2 * 3 * XCS;
+        const int plane = H * W;
+        const long long cplane = (long long)D * plane;
+        const long long cbase = ((long long)id.b * p.C + id.c) * cplane;
+        const size_t xbytes = (size_t)cplane * sizeof(T), sbytes = xbytes * SC;
+        const unsigned plane2 = (unsigned)plane * 2u, cplane2 = (unsigned)cplane * 2u;
+        const BufRef xb_ = make_buf(p.x + cbase, xbytes), tb_ = make_buf(p.t1 + cbase, xbytes);
+        const BufRef gb_ = make_buf(p.gout + cbase * SC, sbytes);
+        const BufRef db_ = make_buf(p.s_over_den + cbase * SC, sbytes);
+        const BufRef rb_ = make_buf(p.ratio + cbase * SC, sbytes);
+        const BufRef gxb_ = make_buf(p.gx ? p.gx + cbase : nullptr, xbytes);
+        const BufRef gtb_ = make_buf(p.gt1 + cbase, xbytes);
+        const float *tabm = p.wtab + (long long)id.c * kTabWords + kTabWM;
+        const int r0 = id.r0;
+        const int nthreads = ex.nthreads;
+        const int need_gh = p.need_gh;
+
+        auto load_plane = [&](State &st, int k) NDC_LAMBDA {
+            if (!st.ln.active) return;
+            const bool live = k < D;
+            const unsigned ko = (unsigned)clampi(k, 0, D - 1) * plane2;
+            NDC_UNROLL
+            for (int n = 0; n < NXS; ++n) {
+                const uint32_t vx = buf_ld(xb_, st.xoff[n], ko);
+                const uint32_t vt = buf_ld(tb_, st.xoff[n], ko);
+                st.px[n] = live ? vx : 0u;
+                st.pt[n] = live ? vt : 0u;
+            }
+        };
+        // plane k of x and t1 (in the registers since load_plane) goes to ring slot k % 3 as
+        // three copies per row: pairs starting one column left of the even columns (copy 0),
+        // at them (copy 1), one column right of them (copy 2)
+        auto store_plane = [&](State &st, int k) NDC_LAMBDA {
+            if (!st.ln.active) return;
+            const int slot = wrap(k % NX, NX);
+            const bool live = k < D;
+            const unsigned ko = (unsigned)clampi(k, 0, D - 1) * plane2;
+            NDC_UNROLL
+            for (int n = 0; n < NXS; ++n) {
+                NDC_UNROLL
+                for (int op = 0; op < 2; ++op) {
+                    const uint32_t own = op ? st.pt[n] : st.px[n];
+                    uint32_t left = from_left_lane(own, [&]() NDC_LAMBDA {
+                        if (st.ln.c0 == 0 || st.xoff[n] >= kNoAccess || !live) return 0u;
+                        return buf_ld(op ? tb_ : xb_, st.xoff[n] - 4u, ko);
+                    });
+                    if (st.ln.c0 == 0) left = 0u;
+                    const uint32_t sh = shift_in_left(own, left);
+                    if ((st.xok >> n) & 1u) {
+                        const int row = off_xs + (slot * 2 + op) * 3 * XCS +
+                                        (st.ln.strip + n * S) * WH + st.ln.c0 / 2;
+                        ex.stw(row, sh);
+                        ex.stw(row + XCS, own);
+                        if (st.ln.c0 > 0) ex.stw(row + 2 * XCS - 1, sh);
+                        if (st.ln.c0 == W - 2) ex.stw(row + 2 * XCS, own >> 16);
+                    }
+                }
+            }
+        };
+        // gout, s/d, n/d words of plane jn into the state, a phase before they are used (own
+        // rows, then the halo row of the first two strips)
+        auto prefetch_g = [&](State &st, int jn) NDC_LAMBDA {
+            if (jn >= D) return;
+            const unsigned jo = (unsigned)jn * plane2;
+            NDC_UNROLL
+            for (int r = 0; r < RH + 1; ++r) {
+                if (r == RH && st.ln.strip >= 2) continue;
+                const unsigned o = r < RH ? st.ooff[r < RH ? r : 0] : st.hoff;
+                NDC_UNROLL
+                for (int i = 0; i < SC; ++i) {
+                    st.qg[i][r] = buf_ld<true>(gb_, o, jo + i * cplane2);
+                    st.qd[i][r] = buf_ld<true>(db_, o, jo + i * cplane2);
+                    st.qr[i][r] = buf_ld<true>(rb_, o, jo + i * cplane2);
+                }
+            }
+        };
+        // gn, gd of the prefetched row `pr` -> tile row j of the per-voxel copy (four channels
+        // per voxel) and, for own rows, row `own` of the channel-major copy
+        auto publish_row = [&](State &st, int pr, int j, int own) NDC_LAMBDA {
+            float gn[SC][RW], gd[SC][RW];
+            NDC_UNROLL
+            for (int i = 0; i < SC; ++i)
+                NDC_UNROLL
+                for (int c = 0; c < RW; ++c) {
+                    // (the words of a row outside the image were read as zeros)
+                    const float gv = c ? bf_hi(st.qg[i][pr]) : bf_lo(st.qg[i][pr]);
+                    gn[i][c] = gv * (c ? bf_hi(st.qd[i][pr]) : bf_lo(st.qd[i][pr]));
+                    gd[i][c] = -(gn[i][c] * (c ? bf_hi(st.qr[i][pr]) : bf_lo(st.qr[i][pr])));
+                }
+            const int o = off_gp + j * P2 + (PL + st.ln.c0) * 2;
+            NDC_UNROLL
+            for (int c = 0; c < RW; ++c) {
+                ex.st2(o + 2 * c, pack_bf16x2(gn[0][c], gn[1][c]), pack_bf16x2(gn[2][c], gn[3][c]));
+                ex.st2(o + RG * P2 + 2 * c, pack_bf16x2(gd[0][c], gd[1][c]),
+                       pack_bf16x2(gd[2][c], gd[3][c]));
+            }
+            if (own >= 0) {
+                const int oc = off_gc + own * WH + st.ln.c0 / 2;
+                NDC_UNROLL
+                for (int i = 0; i < SC; ++i) {
+                    ex.stw(oc + i * GCS, pack_bf16x2(gn[i][0], gn[i][1]));
+                    ex.stw(oc + (SC + i) * GCS, pack_bf16x2(gd[i][0], gd[i][1]));
+                }
+            }
+        };
+
+        ex.each([&](State &st, int tid) NDC_LAMBDA {
+            st.ln = make_lane(tid, t, RW);
+            st.lane4 = tid & 3;
+            st.blk4 = (st.ln.c0 / 8) * 4;
+            st.xok = 0u;
+            NDC_UNROLL
+            for (int n = 0; n < NXS; ++n) {
+                const int j = st.ln.strip + n * S, row = r0 - PH + j;
+                if (j < RXS) st.xok |= 1u << n;
+                st.xoff[n] = j < RXS && row >= 0 && row < H ? (unsigned)(row * W + st.ln.c0) * 2u : kNoAccess;
+                st.px[n] = st.pt[n] = 0u;
+            }
+            NDC_UNROLL
+            for (int r = 0; r < RH; ++r) {
+                const int row = r0 + st.ln.strip * RH + r;
+                st.ooff[r] = row < H ? (unsigned)(row * W + st.ln.c0) * 2u : kNoAccess;
+            }
+            {
+                const int hrow = r0 - PH + halo_row(st.ln.strip, PH, TH);
+                st.hoff = hrow >= 0 && hrow < H ? (unsigned)(hrow * W + st.ln.c0) * 2u : kNoAccess;
+                NDC_UNROLL
+                for (int i = 0; i < SC; ++i)
+                    NDC_UNROLL
+                    for (int r = 0; r < RH + 1; ++r) st.qg[i][r] = st.qd[i][r] = st.qr[i][r] = 0u;
+            }
+            NDC_UNROLL
+            for (int t9 = 0; t9 < 9; ++t9)
+                mfma_rows(st.wm[t9], tid, [&](int m, uint32_t (&w)[2]) NDC_LAMBDA {
+                    w[0] = float_to_bits(tabm[(m * 9 + t9) * 2]);
+                    w[1] = float_to_bits(tabm[(m * 9 + t9) * 2 + 1]);
+                });
+            const f4_t zero = {0.f, 0.f, 0.f, 0.f};
+            NDC_UNROLL
+            for (int r = 0; r < RH; ++r)
+                NDC_UNROLL
+                for (int c = 0; c < RW; ++c) st.accx[r][c] = st.acct[r][c] = zero;
+            NDC_UNROLL
+            for (int a = 0; a < KD; ++a)
+                NDC_UNROLL
+                for (int b = 0; b < KH; ++b) st.gacc[a][b] = zero;
+            for (int i = tid; i < total; i += nthreads) ex.st_(i, 0.f);
+            load_plane(st, 0);
+        });
+        ex.sync();
+
+        // Two barriers per plane step.  Phase 1 of step k stages plane k of x / t1 (fetched
+        // during the step before) and publishes gn / gd of plane k - 1; phase 2 fetches the
+        // next planes and does all tap sums of plane k - 1.
+        for (int kk = 0; kk < D + 2; ++kk) {
+            const int k = uniform_int(kk);
+            const int j1 = k - 1;
+            const bool live1 = j1 >= 0 && j1 < D;
+            ex.each([&](State &st, int) NDC_LAMBDA {
+                if (!st.ln.active) return;
+                store_plane(st, k);
+                if (!live1) return;
+                NDC_UNROLL
+                for (int r = 0; r < RH; ++r)
+                    publish_row(st, r, PH + st.ln.strip * RH + r, st.ln.strip * RH + r);
+                if (st.ln.strip < 2) publish_row(st, RH, halo_row(st.ln.strip, PH, TH), -1);
+            });
+            ex.sync();
+
+            ex.each([&](State &st, int) NDC_LAMBDA {
+                if (!st.ln.active) return;
+                load_plane(st, k + 1);
+                prefetch_g(st, k);
+                if (live1) {
+                    // K-type: gn rows feed gx, gd rows feed gt1
+                    NDC_UNROLL
+                    for (int kind = 0; kind < 2; ++kind) {
+                        const int base = off_gp + (kind * RG + st.ln.strip * RH) * P2 +
+                                         (PL + st.ln.c0 - PW) * 2;
+                        NDC_UNROLL
+                        for (int q = 0; q < RH + 2; ++q) {
+                            uint32_t v[8];
+                            uint32_t lo[4], hi[4];
+                            ex.ld4a(base + q * P2, lo);
+                            ex.ld4a(base + q * P2 + 4, hi);
+                            NDC_UNROLL
+                            for (int u = 0; u < 4; ++u) {
+                                v[u] = lo[u];
+                                v[4 + u] = hi[u];
+                            }
+                            NDC_UNROLL
+                            for (int th = 0; th < KH; ++th) {
+                                const int rr = q - th;
+                                if (rr < 0 || rr >= RH) continue;
+                                NDC_UNROLL
+                                for (int tw = 0; tw < KW; ++tw)
+                                    NDC_UNROLL
+                                    for (int c = 0; c < RW; ++c)
+                                        mfma_bf16_4x4x4(kind ? st.acct[rr][c] : st.accx[rr][c],
+                                                        st.wm[th * 3 + tw], v[(c + tw) * 2],
+                                                        v[(c + tw) * 2 + 1]);
+                            }
+                        }
+                    }
+                    if (need_gh) {
+                        const int copy = st.lane4 < 3 ? st.lane4 : 1;
+                        NDC_UNROLL
+                        for (int op = 0; op < 2; ++op) {
+                            // the block's 8 columns of gn (gd), channel = lane & 3, own rows
+                            MfmaRows ga[RH][2];
+                            NDC_UNROLL
+                            for (int r = 0; r < RH; ++r) {
+                                const int at = off_gc + op * SC * GCS + (st.ln.strip * RH + r) * WH + st.blk4;
+                                mfma_rows2(ga[r][0], ga[r][1], st.lane4,
+                                           [&](int m, uint32_t (&w4)[4]) NDC_LAMBDA { ex.ld4a(at + m * GCS, w4); });
+                            }
+                            NDC_UNROLL
+                            for (int td = 0; td < KD; ++td) {
+                                const int slot = wrap((j1 + 1 - td) % NX, NX);
+                                const int xb = off_xs + ((slot * 2 + op) * 3 + copy) * XCS +
+                                               (st.ln.strip * RH) * WH + st.blk4;
+                                NDC_UNROLL
+                                for (int q = 0; q < RH + 2; ++q) {
+                                    uint32_t bw[4];
+                                    ex.ld4a(xb + q * WH, bw);
+                                    NDC_UNROLL
+                                    for (int r = 0; r < RH; ++r) {
+                                        const int th = r + 2 - q;
+                                        if (th < 0 || th >= KH) continue;
+                                        mfma_bf16_4x4x4(st.gacc[td][th], ga[r][0], bw[0], bw[1]);
+                                        mfma_bf16_4x4x4(st.gacc[td][th], ga[r][1], bw[2], bw[3]);
+                                    }
+                                }
+                            }
+                        }
+                    }
+                }
+                const int pf = k - 2;
+                NDC_UNROLL
+                for (int r = 0; r < RH; ++r) {
+                    if (pf >= 0) {   // rows outside the image: the stores go nowhere
+                        buf_st<true>(gxb_, st.ooff[r], (unsigned)pf * plane2,
+                                     pack_bf16x2(st.accx[r][0][0], st.accx[r][1][0]));
+                        buf_st(gtb_, st.ooff[r], (unsigned)pf * plane2,
+                               pack_bf16x2(st.acct[r][0][0], st.acct[r][1][0]));
+                    }
+                    NDC_UNROLL
+                    for (int c = 0; c < RW; ++c) {
+                        st.accx[r][c] = f4_t{st.accx[r][c][1], st.accx[r][c][2], 0.f, 0.f};
+                        st.acct[r][c] = f4_t{st.acct[r][c][1], st.acct[r][c][2], 0.f, 0.f};
+                    }
+                }
+            });
+            ex.sync();
+        }
+
+        if (need_gh) {
+            float *dst = p.part + (long long)block_id * p.part_stride;
+            // element (i, td, th, tw) is summed over the lanes whose window shift is 1 - tw
+            ex.template block_reduce<NRED>(
+                [](State &st, int e) NDC_LAMBDA {
+                    const int i = e / KT, tap = e % KT, tw = tap % 3;
+                    return st.lane4 == 2 - tw ? st.gacc[tap / 9][(tap % 9) / 3][i] : 0.f;
+                },
+                [&](int e, float v) NDC_LAMBDA { dst[e] = v; });
+        }
+    }
+};
+
+}  // namespace fused
+}  // namespace ndc
