@@ -75,6 +75,8 @@ template <class State> struct DeviceExec {
     // The instruction scheduler may not move anything across this point: used to keep the LDS
     // reads of the next row ahead of the arithmetic on the current one.
     NDC_D void fence() const { __builtin_amdgcn_sched_barrier(0); }
+    // every global load this thread has issued has returned (s_waitcnt vmcnt(0))
+    NDC_D void wait_loads() const { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
     // Sum N per-thread values over the workgroup: butterfly inside each wavefront, one LDS
     // row per wavefront, then thread i < N adds the rows in a fixed order and hands the sum
@@ -136,6 +138,7 @@ template <class State> struct HostExec {
     }
     void sync() { ++epoch; }
     void fence() const {}
+    void wait_loads() const {}
 
     float ld(int i)
     {

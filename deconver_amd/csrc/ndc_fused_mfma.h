@@ -234,6 +234,9 @@ template <int RH_> struct Bwd1KernelM {
             for (int a = 0; a < KD; ++a)
                 NDC_UNROLL
                 for (int b = 0; b < KH; ++b) st.gacc[a][b] = zero;
+            // the tap rows have arrived before the march starts (otherwise every step's first
+            // matrix instruction is made to wait for the loads issued just before it)
+            ex.wait_loads();
             for (int i = tid; i < total; i += nthreads) ex.st_(i, 0.f);
             load_plane(st, 0);
         });
@@ -262,66 +265,95 @@ template <int RH_> struct Bwd1KernelM {
                 load_plane(st, k + 1);
                 prefetch_g(st, k);
                 if (live1) {
-                    // K-type: gn rows feed gx, gd rows feed gt1
-                    NDC_UNROLL
-                    for (int kind = 0; kind < 2; ++kind) {
-                        const int base = off_gp + (kind * RG + st.ln.strip * RH) * P2 +
-                                         (PL + st.ln.c0 - PW) * 2;
+                    // LDS reads run ahead of the matrix instructions that use them (two
+                    // wavefronts per SIMD do not hide their latency): the K-type rows two
+                    // rows ahead, the filter-gradient rows a whole tap plane ahead.  The
+                    // scheduling fences keep that order.
+                    const int kbase = off_gp + (st.ln.strip * RH) * P2 + (PL + st.ln.c0 - PW) * 2;
+                    // K-type group g = (kind, input row q): the 4-voxel window of gn (gd)
+                    auto read_k = [&](int g, uint32_t (&v)[8]) NDC_LAMBDA {
+                        const int at = kbase + ((g / (RH + 2)) * RG + g % (RH + 2)) * P2;
+                        uint32_t lo[4], hi[4];
+                        ex.ld4a(at, lo);
+                        ex.ld4a(at + 4, hi);
                         NDC_UNROLL
-                        for (int q = 0; q < RH + 2; ++q) {
-                            uint32_t v[8];
-                            uint32_t lo[4], hi[4];
-                            ex.ld4a(base + q * P2, lo);
-                            ex.ld4a(base + q * P2 + 4, hi);
-                            NDC_UNROLL
-                            for (int u = 0; u < 4; ++u) {
-                                v[u] = lo[u];
-                                v[4 + u] = hi[u];
-                            }
-                            NDC_UNROLL
-                            for (int th = 0; th < KH; ++th) {
-                                const int rr = q - th;
-                                if (rr < 0 || rr >= RH) continue;
-                                NDC_UNROLL
-                                for (int tw = 0; tw < KW; ++tw)
-                                    NDC_UNROLL
-                                    for (int c = 0; c < RW; ++c)
-                                        mfma_bf16_4x4x4(kind ? st.acct[rr][c] : st.accx[rr][c],
-                                                        st.wm[th * 3 + tw], v[(c + tw) * 2],
-                                                        v[(c + tw) * 2 + 1]);
-                            }
+                        for (int u = 0; u < 4; ++u) {
+                            v[u] = lo[u];
+                            v[4 + u] = hi[u];
                         }
-                    }
-                    if (need_gh) {
-                        const int copy = st.lane4 < 3 ? st.lane4 : 1;
+                    };
+                    // gn rows feed gx, gd rows feed gt1
+                    auto mfma_k = [&](int g, const uint32_t (&v)[8]) NDC_LAMBDA {
+                        const int kind = g / (RH + 2), q = g % (RH + 2);
                         NDC_UNROLL
-                        for (int op = 0; op < 2; ++op) {
-                            // the block's 8 columns of gn (gd), channel = lane & 3, own rows
-                            MfmaRows ga[RH][2];
+                        for (int th = 0; th < KH; ++th) {
+                            const int rr = q - th;
+                            if (rr < 0 || rr >= RH) continue;
+                            NDC_UNROLL
+                            for (int tw = 0; tw < KW; ++tw)
+                                NDC_UNROLL
+                                for (int c = 0; c < RW; ++c)
+                                    mfma_bf16_4x4x4(kind ? st.acct[rr][c] : st.accx[rr][c],
+                                                    st.wm[th * 3 + tw], v[(c + tw) * 2],
+                                                    v[(c + tw) * 2 + 1]);
+                        }
+                    };
+                    // filter-gradient group g = (operand, td): the RH + 2 rows of x (t1) of
+                    // plane j1 + 1 - td around the own rows, in the lane's shifted copy
+                    const int copy = st.lane4 < 3 ? st.lane4 : 1;
+                    auto read_g = [&](int g, uint32_t (&bw)[RH + 2][4]) NDC_LAMBDA {
+                        const int op = g / KD, td = g % KD;
+                        const int slot = wrap((j1 + 1 - td) % NX, NX);
+                        const int xb = off_xs + ((slot * 2 + op) * 3 + copy) * XCS +
+                                       (st.ln.strip * RH) * WH + st.blk4;
+                        NDC_UNROLL
+                        for (int q = 0; q < RH + 2; ++q) ex.ld4a(xb + q * WH, bw[q]);
+                    };
+                    // the block's 8 columns of gn (gd), channel = lane & 3, own rows
+                    MfmaRows ga[2][RH][2];
+                    auto read_ga = [&]() NDC_LAMBDA {
+                        NDC_UNROLL
+                        for (int op = 0; op < 2; ++op)
                             NDC_UNROLL
                             for (int r = 0; r < RH; ++r) {
                                 const int at = off_gc + op * SC * GCS + (st.ln.strip * RH + r) * WH + st.blk4;
-                                mfma_rows2(ga[r][0], ga[r][1], st.lane4,
+                                mfma_rows2(ga[op][r][0], ga[op][r][1], st.lane4,
                                            [&](int m, uint32_t (&w4)[4]) NDC_LAMBDA { ex.ld4a(at + m * GCS, w4); });
                             }
+                    };
+                    auto mfma_g = [&](int g, const uint32_t (&bw)[RH + 2][4]) NDC_LAMBDA {
+                        const int op = g / KD, td = g % KD;
+                        NDC_UNROLL
+                        for (int q = 0; q < RH + 2; ++q)
                             NDC_UNROLL
-                            for (int td = 0; td < KD; ++td) {
-                                const int slot = wrap((j1 + 1 - td) % NX, NX);
-                                const int xb = off_xs + ((slot * 2 + op) * 3 + copy) * XCS +
-                                               (st.ln.strip * RH) * WH + st.blk4;
-                                NDC_UNROLL
-                                for (int q = 0; q < RH + 2; ++q) {
-                                    uint32_t bw[4];
-                                    ex.ld4a(xb + q * WH, bw);
-                                    NDC_UNROLL
-                                    for (int r = 0; r < RH; ++r) {
-                                        const int th = r + 2 - q;
-                                        if (th < 0 || th >= KH) continue;
-                                        mfma_bf16_4x4x4(st.gacc[td][th], ga[r][0], bw[0], bw[1]);
-                                        mfma_bf16_4x4x4(st.gacc[td][th], ga[r][1], bw[2], bw[3]);
-                                    }
-                                }
+                            for (int r = 0; r < RH; ++r) {
+                                const int th = r + 2 - q;
+                                if (th < 0 || th >= KH) continue;
+                                mfma_bf16_4x4x4(st.gacc[td][th], ga[op][r][0], bw[q][0], bw[q][1]);
+                                mfma_bf16_4x4x4(st.gacc[td][th], ga[op][r][1], bw[q][2], bw[q][3]);
                             }
+                    };
+                    constexpr int NKG = 2 * (RH + 2), NGG = 2 * KD;
+                    uint32_t kv[3][8];
+                    uint32_t bw[2][RH + 2][4];
+                    read_k(0, kv[0]);
+                    read_k(1, kv[1]);
+                    NDC_UNROLL
+                    for (int g = 0; g < NKG; ++g) {
+                        if (g + 2 < NKG) read_k(g + 2, kv[(g + 2) % 3]);
+                        if (need_gh && g + 2 == NKG) read_ga();
+                        if (need_gh && g + 1 == NKG) read_g(0, bw[0]);
+                        ex.fence();
+                        mfma_k(g, kv[g % 3]);
+                        ex.fence();
+                    }
+                    if (need_gh) {
+                        NDC_UNROLL
+                        for (int g = 0; g < NGG; ++g) {
+                            if (g + 1 < NGG) read_g(g + 1, bw[(g + 1) & 1]);
+                            ex.fence();
+                            mfma_g(g, bw[g & 1]);
+                            ex.fence();
                         }
                     }
                 }
