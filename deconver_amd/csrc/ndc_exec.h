@@ -72,6 +72,12 @@ template <class State> struct DeviceExec {
         *reinterpret_cast<u2_t *>(lds + i) = v;
     }
     NDC_D void stw(int i, uint32_t a) { lds[i] = __uint_as_float(a); }
+    // two consecutive words from any word index (one ds_read2_b32)
+    NDC_D void ld2w(int i, uint32_t (&v)[2]) const
+    {
+        v[0] = __float_as_uint(lds[i]);
+        v[1] = __float_as_uint(lds[i + 1]);
+    }
     // The instruction scheduler may not move anything across this point: used to keep the LDS
     // reads of the next row ahead of the arithmetic on the current one.
     NDC_D void fence() const { __builtin_amdgcn_sched_barrier(0); }
@@ -193,6 +199,13 @@ template <class State> struct HostExec {
             hf.note("misaligned 16-byte read", i, cur, -1);
         }
         for (int u = 0; u < 4; ++u) {
+            const float f = ld(i + u);
+            memcpy(&v[u], &f, 4);
+        }
+    }
+    void ld2w(int i, uint32_t (&v)[2])
+    {
+        for (int u = 0; u < 2; ++u) {
             const float f = ld(i + u);
             memcpy(&v[u], &f, 4);
         }

@@ -101,7 +101,7 @@ struct Plan {
     Variant v;
     March m;
     bool dot2;            // bf16 dot2 kernels (3x3x3, SC = 4, even W, aligned pairs)
-    bool mfma1;           // ... with pass 1 on the matrix instruction when it reads the forward's ratios
+    bool mfma1, mfma2;    // ... with pass 1 / pass 2 on the matrix instruction when they read the forward's ratios
     Tile tf, tb;          // forward / backward launch shapes
     int lds_f, lds_b1, lds_b2;
     int nblk_f, nblk_b;
@@ -126,7 +126,7 @@ static inline bool make_plan_for(const KGeom &q, Plan &pl, bool pairs_ok, int dt
 {
     pl.m = march_of(q);
     pl.dot2 = false;
-    pl.mfma1 = false;
+    pl.mfma1 = pl.mfma2 = false;
     // 32-bit offsets inside one (sample, channel) volume
     if ((long long)q.sc * q.SP >= (1LL << 31)) return false;
     if (!find_variant(q, pl.m, pairs_ok, pl.v)) return false;
@@ -162,6 +162,8 @@ static inline bool make_plan_for(const KGeom &q, Plan &pl, bool pairs_ok, int dt
                 pl.lds_b2 = l2;
                 pl.mfma1 = tn.mfma && Bwd1KernelM<kDot2RH>::covers(pl.m.W) &&
                            Bwd1KernelM<kDot2RH>::lds_floats(tb) <= cap2;
+                pl.mfma2 = tn.mfma && Bwd2KernelM<kDot2RH>::covers(pl.m.W) &&
+                           Bwd2KernelM<kDot2RH>::lds_floats(tb) <= cap2;
             }
         }
     }
@@ -251,6 +253,9 @@ template <class BE> struct Dot2Launch<BE, bf16_t> {
     }
     static int bwd2(const BwdParams<bf16_t> &p, const Plan &pl, void *stream, bool saved)
     {
+        if (saved && pl.mfma2)
+            return BE::template block_kernel<Bwd2KernelM<kDot2RH>>(
+                p, pl.nblk_b, pl.tb.NT, Bwd2KernelM<kDot2RH>::lds_floats(pl.tb), stream);
         if (saved)
             return BE::template block_kernel<Bwd2KernelB<kDot2RH, true>>(
                 p, pl.nblk_b, pl.tb.NT, Bwd2KernelB<kDot2RH, true>::lds_floats(pl.tb), stream);

@@ -34,6 +34,9 @@
 //   WM[m][th][tw]     = rows of the 4x4 tap matrices of the matrix-instruction kernels
 //                       (ndc_fused_mfma.h): the four source channels' taps of tap plane
 //                       2 - m, (h[0], h[1]) then (h[2], h[3]); m = 3: zeros        72 words
+//   WG[i][td][th]     = rows of the tap matrices of the A-type applications there: the
+//                       tap row against a 4-column window, (h2, h1) then (h0, 0),
+//                       h_tw = h[i][td][th][tw]                                     72 words
 #pragma once
 
 #include "ndc_fused.h"
@@ -41,8 +44,8 @@
 namespace ndc {
 namespace fused {
 
-static const int kTabWK = 0, kTabWA = 54, kTabWQ = 126, kTabWM = 174;
-static const int kTabWords = 246;   // packed tap words per channel (54 WK + 72 WA + 48 WQ + 72 WM)
+static const int kTabWK = 0, kTabWA = 54, kTabWQ = 126, kTabWM = 174, kTabWG = 246;
+static const int kTabWords = 318;   // packed tap words per channel (54 WK + 72 WA + 48 WQ + 72 WM + 72 WG)
 
 // idx over C * kTabWords
 NDC_HD void prep_tables(long long idx, const float *h, float *tab)
@@ -62,10 +65,14 @@ NDC_HD void prep_tables(long long idx, const float *h, float *tab)
         const float *ht = hc + i * 27 + th * 3;   // the tap row h[i][0][th][0..2]
         w = n == 0 ? pack_bf16x2(ht[1], ht[0]) : n == 1 ? pack_bf16x2(0.f, ht[2])
           : n == 2 ? pack_bf16x2(ht[2], ht[1]) : pack_bf16x2(ht[0], 0.f);
-    } else {
+    } else if (e < kTabWG) {
         const int r = e - kTabWM, m = r / 18, t9 = (r % 18) / 2, half = r % 2;
         const int tau = (2 - m) * 9 + t9;
         w = m == 3 ? 0u : pack_bf16x2(hc[(2 * half) * 27 + tau], hc[(2 * half + 1) * 27 + tau]);
+    } else {
+        const int r = e - kTabWG, i = r / 18, t9 = (r % 18) / 2, half = r % 2;
+        const float *ht = hc + i * 27 + t9 * 3;   // the tap row h[i][td][th][0..2]
+        w = half == 0 ? pack_bf16x2(ht[2], ht[1]) : pack_bf16x2(ht[0], 0.f);
     }
     tab[idx] = bits_to_float(w);
 }

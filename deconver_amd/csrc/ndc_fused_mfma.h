@@ -33,6 +33,10 @@
 namespace ndc {
 namespace fused {
 
+// the smallest stride >= n words that is 16 modulo 64: rows of four channels (copies) that
+// far apart put the four lanes of a block, which read them at one position, on different banks
+NDC_HD int stride16(int n) { return (n + 47) / 64 * 64 + 16; }
+
 // (hi half of `left`, lo half of `own`): the bf16 pair one column to the left of `own`
 NDC_HD uint32_t shift_in_left(uint32_t own, uint32_t left) { return (left >> 16) | (own << 16); }
 
@@ -67,9 +71,8 @@ template <int RH_> struct Bwd1KernelM {
     // strides of the channel rows of the channel-major copy and of the shifted copies: a
     // multiple of 64 words plus 16, so that the four lanes of a block, which read four
     // different channels (copies) at one position, hit different banks
-    static NDC_HD int stride_gc(int TH, int W) { return round_up_hd(TH * (W / 2), 64) + 16; }
-    static NDC_HD int stride_xs(int TH, int W) { return round_up_hd((TH + 2) * (W / 2), 64) + 16; }
-    static NDC_HD int round_up_hd(int v, int a) { return (v + a - 1) / a * a; }
+    static NDC_HD int stride_gc(int TH, int W) { return stride16(TH * (W / 2)); }
+    static NDC_HD int stride_xs(int TH, int W) { return stride16((TH + 2) * (W / 2)); }
     static NDC_HD int lds_floats(const Tile &t)
     {
         const int W = t.CPW * RW;
@@ -383,6 +386,294 @@ template <int RH_> struct Bwd1KernelM {
                 [](State &st, int e) NDC_LAMBDA {
                     const int i = e / KT, tap = e % KT, tw = tap % 3;
                     return st.lane4 == 2 - tw ? st.gacc[tap / 9][(tap % 9) / 3][i] : 0.f;
+                },
+                [&](int e, float v) NDC_LAMBDA { dst[e] = v; });
+        }
+    }
+};
+
+// =================================================================== backward pass 2 (bf16, matrix instruction)
+
+//   A-type applications (1 -> 4 channels): per (td, th) one instruction per output voxel column,
+//       D[i][n] += sum_{k<4} T[i][k] * V[k][n],   T[i][k] = h[i][td][th][2 - k]  (k = 3: zero)
+//     V[.][n] = the four columns n - 1 .. n + 2 of the operand's row: two words of the copy
+//     shifted by -1 column for the lane's even column, of the unshifted copy for its odd one.
+//
+// Reads the forward's n/d: gz = [s > 0] (g n/d + A(gt1)), gb, and the K-side filter-gradient
+// term sum_v s_i[v] gt1[v + shift(tap)], in the block form described at the top of this file
+// (lane (b, i) reads channel i of the staged s row).  One barrier per plane step: the step of
+// plane j0 stages s of plane j0 channel-major in one of two buffers, and the filter-gradient
+// instructions of that plane run a step later, after the barrier; the gt1 ring therefore
+// holds five planes.
+template <int RH_> struct Bwd2KernelM {
+    static constexpr bool SAVED = true;
+    static constexpr int KD = 3, KH = 3, KW = 3, SC = 4, RH = RH_, RW = 2;
+    static constexpr int PD = 1, PH = 1, PW = 1, KT = 27;
+    static constexpr int NXS = RH + 1;
+    static constexpr int NG = 5;   // ring slots of gt1 planes
+    static constexpr int NRED = SC * KT + SC;
+    typedef bf16_t T;
+    typedef BwdParams<T> Params;
+
+    struct State {
+        Lane ln;
+        int lane4, blk4;
+        unsigned xoff[NXS], ooff[RH];
+        unsigned xok;
+        float bvr[SC][RH];
+        float okf[RH];
+        MfmaRows wg[9];
+        f4_t gacc[KD][KH];
+        float gbacc[SC];
+        uint32_t pg[NXS];
+        uint32_t qz[SC][RH], qg[SC][RH], qr[SC][RH];
+    };
+
+    static NDC_HD bool covers(int W) { return W % 8 == 0 && W <= 128 && 64 % (W / 2) == 0; }
+    static NDC_HD int pitch_xs(int W) { return W / 2 + 4; }   // one zero word past the row, rows 16-byte aligned
+    static NDC_HD int stride_xs(int TH, int W) { return stride16((TH + 2) * pitch_xs(W)); }
+    static NDC_HD int stride_sc(int TH, int W) { return stride16(TH * (W / 2)); }
+    static NDC_HD int lds_floats(const Tile &t)
+    {
+        const int W = t.CPW * RW;
+        const int main_ = NG * 3 * stride_xs(t.TH, W) + 2 * SC * stride_sc(t.TH, W);
+        const int red = (t.NT / 64) * NRED;
+        return main_ > red ? main_ : red;
+    }
+
+    template <class Exec> static NDC_D void run(Exec &ex, const Params &p, int block_id)
+    {
+        const Tile t = p.t;
+        const BlockId id = decode_block(block_id, p.C, t, p.D);
+        const int S = t.S, TH = t.TH, W = p.W, H = p.H, D = p.D;
+        const int WH = W / 2, PX = pitch_xs(W), RXS = TH + 2;
+        const int XCS = stride_xs(TH, W), SCS = stride_sc(TH, W);
+        const int off_xs = 0, off_sc = NG * 3 * XCS;
+        const int total = off_sc + 2 * SC * SCS;
+        const int plane = H * W;
+        const long long cplane = (long long)D * plane;
+        const long long cbase = ((long long)id.b * p.C + id.c) * cplane;
+        const size_t xbytes = (size_t)cplane * sizeof(T), sbytes = xbytes * SC;
+        const unsigned plane2 = (unsigned)plane * 2u, cplane2 = (unsigned)cplane * 2u;
+        const BufRef gtb_ = make_buf(p.gt1 + cbase, xbytes);
+        const BufRef zb_ = make_buf(p.z + cbase * SC, sbytes), gb_ = make_buf(p.gout + cbase * SC, sbytes);
+        const BufRef rb_ = make_buf(p.ratio + cbase * SC, sbytes);
+        const BufRef gzb_ = make_buf(p.gz ? p.gz + cbase * SC : nullptr, sbytes);
+        const float *tabg = p.wtab + (long long)id.c * kTabWords + kTabWG;
+        const int r0 = id.r0;
+        const int nthreads = ex.nthreads;
+        const float floor_ = p.relu ? 0.f : pass_through_floor();
+        const int need_gh = p.need_gh;
+        const int relu = p.relu;
+
+        auto load_plane = [&](State &st, int k) NDC_LAMBDA {
+            if (!st.ln.active) return;
+            const bool live = k < D;
+            const unsigned ko = (unsigned)clampi(k, 0, D - 1) * plane2;
+            NDC_UNROLL
+            for (int n = 0; n < NXS; ++n) {
+                const uint32_t vg = buf_ld(gtb_, st.xoff[n], ko);
+                st.pg[n] = live ? vg : 0u;
+            }
+        };
+        // plane k of gt1 -> ring slot k % NG as three copies per row (see Bwd1KernelM)
+        auto store_plane = [&](State &st, int k) NDC_LAMBDA {
+            if (!st.ln.active) return;
+            const int slot = wrap(k % NG, NG);
+            const bool live = k < D;
+            const unsigned ko = (unsigned)clampi(k, 0, D - 1) * plane2;
+            NDC_UNROLL
+            for (int n = 0; n < NXS; ++n) {
+                const uint32_t own = st.pg[n];
+                uint32_t left = from_left_lane(own, [&]() NDC_LAMBDA {
+                    if (st.ln.c0 == 0 || st.xoff[n] >= kNoAccess || !live) return 0u;
+                    return buf_ld(gtb_, st.xoff[n] - 4u, ko);
+                });
+                if (st.ln.c0 == 0) left = 0u;
+                const uint32_t sh = shift_in_left(own, left);
+                if ((st.xok >> n) & 1u) {
+                    const int row = off_xs + slot * 3 * XCS + (st.ln.strip + n * S) * PX + st.ln.c0 / 2;
+                    ex.stw(row, sh);
+                    ex.stw(row + XCS, own);
+                    if (st.ln.c0 > 0) ex.stw(row + 2 * XCS - 1, sh);
+                    if (st.ln.c0 == W - 2) {
+                        ex.stw(row + 2 * XCS, own >> 16);
+                        ex.stw(row + 1, own >> 16);
+                    }
+                }
+            }
+        };
+
+        ex.each([&](State &st, int tid) NDC_LAMBDA {
+            st.ln = make_lane(tid, t, RW);
+            st.lane4 = tid & 3;
+            st.blk4 = (st.ln.c0 / 8) * 4;
+            st.xok = 0u;
+            NDC_UNROLL
+            for (int n = 0; n < NXS; ++n) {
+                const int j = st.ln.strip + n * S, row = r0 - PH + j;
+                if (j < RXS) st.xok |= 1u << n;
+                st.xoff[n] = j < RXS && row >= 0 && row < H ? (unsigned)(row * W + st.ln.c0) * 2u : kNoAccess;
+                st.pg[n] = 0u;
+            }
+            NDC_UNROLL
+            for (int r = 0; r < RH; ++r) {
+                const int row = r0 + st.ln.strip * RH + r;
+                st.ooff[r] = row < H ? (unsigned)(row * W + st.ln.c0) * 2u : kNoAccess;
+                st.okf[r] = row < H ? 1.f : 0.f;
+                NDC_UNROLL
+                for (int i = 0; i < SC; ++i) {
+                    // a row outside the image reads zeros; -1 (rectified) or 0 makes its source 0
+                    st.bvr[i][r] = row < H ? (p.bias ? p.bias[id.c * SC + i] : 0.f) : (p.relu ? -1.f : 0.f);
+                    st.qz[i][r] = st.qg[i][r] = st.qr[i][r] = 0u;
+                }
+            }
+            NDC_UNROLL
+            for (int t9 = 0; t9 < 9; ++t9)
+                mfma_rows(st.wg[t9], tid, [&](int m, uint32_t (&w)[2]) NDC_LAMBDA {
+                    w[0] = float_to_bits(tabg[(m * 9 + t9) * 2]);
+                    w[1] = float_to_bits(tabg[(m * 9 + t9) * 2 + 1]);
+                });
+            const f4_t zero = {0.f, 0.f, 0.f, 0.f};
+            NDC_UNROLL
+            for (int a = 0; a < KD; ++a)
+                NDC_UNROLL
+                for (int b = 0; b < KH; ++b) st.gacc[a][b] = zero;
+            NDC_UNROLL
+            for (int i = 0; i < SC; ++i) st.gbacc[i] = 0.f;
+            ex.wait_loads();
+            for (int i = tid; i < total; i += nthreads) ex.st_(i, 0.f);
+            load_plane(st, 0);
+        });
+        ex.sync();
+
+        for (int kk = 0; kk < D + 2; ++kk) {
+            const int k = uniform_int(kk);
+            ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k); });
+            ex.sync();
+            ex.each([&](State &st, int) NDC_LAMBDA {
+                if (!st.ln.active) return;
+                const int j0 = k - 1;
+                load_plane(st, k + 1);
+                const int lc = st.ln.c0 / 2;
+                if (j0 >= 0 && j0 < D) {
+                    // A(gt1) of plane j0: windows of plane j0 + 1 - td, read a tap plane ahead
+                    f4_t acc[RH][RW];
+                    const f4_t zero = {0.f, 0.f, 0.f, 0.f};
+                    NDC_UNROLL
+                    for (int r = 0; r < RH; ++r)
+                        NDC_UNROLL
+                        for (int c = 0; c < RW; ++c) acc[r][c] = zero;
+                    auto read_a = [&](int td, uint32_t (&v)[RH + 2][RW][2]) NDC_LAMBDA {
+                        const int slot = wrap((j0 + 1 - td) % NG, NG);
+                        const int at = off_xs + slot * 3 * XCS + (st.ln.strip * RH) * PX + lc;
+                        NDC_UNROLL
+                        for (int q = 0; q < RH + 2; ++q)
+                            NDC_UNROLL
+                            for (int c = 0; c < RW; ++c) ex.ld2w(at + c * XCS + q * PX, v[q][c]);
+                    };
+                    auto mfma_a = [&](int td, const uint32_t (&v)[RH + 2][RW][2]) NDC_LAMBDA {
+                        NDC_UNROLL
+                        for (int q = 0; q < RH + 2; ++q)
+                            NDC_UNROLL
+                            for (int r = 0; r < RH; ++r) {
+                                const int th = r + 2 - q;
+                                if (th < 0 || th >= KH) continue;
+                                NDC_UNROLL
+                                for (int c = 0; c < RW; ++c)
+                                    mfma_bf16_4x4x4(acc[r][c], st.wg[td * 3 + th], v[q][c][0], v[q][c][1]);
+                            }
+                    };
+                    uint32_t av[2][RH + 2][RW][2];
+                    read_a(0, av[0]);
+                    NDC_UNROLL
+                    for (int td = 0; td < KD; ++td) {
+                        if (td + 1 < KD) read_a(td + 1, av[(td + 1) & 1]);
+                        ex.fence();
+                        mfma_a(td, av[td & 1]);
+                        ex.fence();
+                    }
+                    // gz, gb; s of this plane to the channel-major buffer k & 1
+                    const unsigned jo = (unsigned)j0 * plane2;
+                    const int osc = off_sc + (k & 1) * SC * SCS + (st.ln.strip * RH) * WH + lc;
+                    NDC_UNROLL
+                    for (int r = 0; r < RH; ++r)
+                        NDC_UNROLL
+                        for (int i = 0; i < SC; ++i) {
+                            float v[RW], sv[RW];
+                            NDC_UNROLL
+                            for (int c = 0; c < RW; ++c) {
+                                const float s = floor_f((c ? bf_hi(st.qz[i][r]) : bf_lo(st.qz[i][r])) + st.bvr[i][r], floor_);
+                                const float g = c ? bf_hi(st.qg[i][r]) : bf_lo(st.qg[i][r]);
+                                float gzv = g * (c ? bf_hi(st.qr[i][r]) : bf_lo(st.qr[i][r])) + acc[r][c][i];
+                                if (relu && s <= 0.f) gzv = 0.f;   // a NaN passes
+                                sv[c] = s;
+                                st.gbacc[i] += gzv * st.okf[r];
+                                v[c] = gzv;
+                            }
+                            buf_st<true>(gzb_, st.ooff[r], jo + i * cplane2, pack_bf16x2(v[0], v[1]));
+                            ex.stw(osc + i * SCS + r * WH, pack_bf16x2(sv[0], sv[1]));
+                        }
+                }
+                // the next plane's z, gout, n/d words (this plane's have just been consumed)
+                {
+                    const unsigned jn = (unsigned)clampi(k, 0, D - 1) * plane2;
+                    NDC_UNROLL
+                    for (int r = 0; r < RH; ++r)
+                        NDC_UNROLL
+                        for (int i = 0; i < SC; ++i) {
+                            st.qz[i][r] = buf_ld(zb_, st.ooff[r], jn + i * cplane2);
+                            st.qg[i][r] = buf_ld<true>(gb_, st.ooff[r], jn + i * cplane2);
+                            st.qr[i][r] = buf_ld<true>(rb_, st.ooff[r], jn + i * cplane2);
+                        }
+                }
+                const int js = j0 - 1;   // the plane whose s was staged a step ago
+                if (need_gh && js >= 0 && js < D) {
+                    const int copy = st.lane4 < 3 ? st.lane4 : 1;
+                    MfmaRows ga[RH][2];
+                    NDC_UNROLL
+                    for (int r = 0; r < RH; ++r) {
+                        const int at = off_sc + ((k - 1) & 1) * SC * SCS + (st.ln.strip * RH + r) * WH + st.blk4;
+                        mfma_rows2(ga[r][0], ga[r][1], st.lane4,
+                                   [&](int m, uint32_t (&w4)[4]) NDC_LAMBDA { ex.ld4a(at + m * SCS, w4); });
+                    }
+                    auto read_g = [&](int td, uint32_t (&bw)[RH + 2][4]) NDC_LAMBDA {
+                        const int slot = wrap((js + 1 - td) % NG, NG);
+                        const int xb = off_xs + (slot * 3 + copy) * XCS + (st.ln.strip * RH) * PX + st.blk4;
+                        NDC_UNROLL
+                        for (int q = 0; q < RH + 2; ++q) ex.ld4a(xb + q * PX, bw[q]);
+                    };
+                    auto mfma_g = [&](int td, const uint32_t (&bw)[RH + 2][4]) NDC_LAMBDA {
+                        NDC_UNROLL
+                        for (int q = 0; q < RH + 2; ++q)
+                            NDC_UNROLL
+                            for (int r = 0; r < RH; ++r) {
+                                const int th = r + 2 - q;
+                                if (th < 0 || th >= KH) continue;
+                                mfma_bf16_4x4x4(st.gacc[td][th], ga[r][0], bw[q][0], bw[q][1]);
+                                mfma_bf16_4x4x4(st.gacc[td][th], ga[r][1], bw[q][2], bw[q][3]);
+                            }
+                    };
+                    uint32_t bw[2][RH + 2][4];
+                    read_g(0, bw[0]);
+                    NDC_UNROLL
+                    for (int td = 0; td < KD; ++td) {
+                        if (td + 1 < KD) read_g(td + 1, bw[(td + 1) & 1]);
+                        ex.fence();
+                        mfma_g(td, bw[td & 1]);
+                        ex.fence();
+                    }
+                }
+            });
+        }
+
+        if (p.need_gh || p.need_gb) {
+            float *dst = p.part + (long long)block_id * p.part_stride;
+            ex.template block_reduce<NRED>(
+                [](State &st, int e) NDC_LAMBDA {
+                    if (e >= SC * KT) return st.gbacc[e >= SC * KT ? e - SC * KT : 0];
+                    const int i = e / KT, tap = e % KT, tw = tap % 3;
+                    return st.lane4 == 2 - tw ? st.gacc[tap / 9][(tap % 9) / 3][i < SC ? i : 0] : 0.f;
                 },
                 [&](int e, float v) NDC_LAMBDA { dst[e] = v; });
         }
