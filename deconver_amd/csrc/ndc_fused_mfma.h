@@ -426,7 +426,11 @@ template <int RH_> struct Bwd2KernelM {
         f4_t gacc[KD][KH];
         float gbacc[SC];
         uint32_t pg[NXS];
-        uint32_t qz[SC][RH], qg[SC][RH], qr[SC][RH];
+        // the z, gout, n/d words of two planes: the step of plane parity P consumes set 1 - P
+        // (fetched at the start of the step before) and starts the fetch of its own plane's
+        // into set P, so a fetch has more than a whole step to arrive.  The plane loop is
+        // unrolled twice: the sets are fixed registers.
+        uint32_t qz[2][SC][RH], qg[2][SC][RH], qr[2][SC][RH];
     };
 
     static NDC_HD bool covers(int W) { return W % 8 == 0 && W <= 128 && 64 % (W / 2) == 0; }
@@ -525,7 +529,8 @@ template <int RH_> struct Bwd2KernelM {
                 for (int i = 0; i < SC; ++i) {
                     // a row outside the image reads zeros; -1 (rectified) or 0 makes its source 0
                     st.bvr[i][r] = row < H ? (p.bias ? p.bias[id.c * SC + i] : 0.f) : (p.relu ? -1.f : 0.f);
-                    st.qz[i][r] = st.qg[i][r] = st.qr[i][r] = 0u;
+                    st.qz[0][i][r] = st.qg[0][i][r] = st.qr[0][i][r] = 0u;
+                    st.qz[1][i][r] = st.qg[1][i][r] = st.qr[1][i][r] = 0u;
                 }
             }
             NDC_UNROLL
@@ -547,14 +552,24 @@ template <int RH_> struct Bwd2KernelM {
         });
         ex.sync();
 
-        for (int kk = 0; kk < D + 2; ++kk) {
-            const int k = uniform_int(kk);
-            ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k); });
-            ex.sync();
-            ex.each([&](State &st, int) NDC_LAMBDA {
+        // one plane step; PAR = k % 2, known at compile time (the loop below is unrolled twice)
+        auto compute = [&](State &st, int k, auto par_tag) NDC_LAMBDA {
+                constexpr int PAR = decltype(par_tag)::value;
                 if (!st.ln.active) return;
                 const int j0 = k - 1;
                 load_plane(st, k + 1);
+                // plane k's z, gout, n/d words, consumed by the next step
+                {
+                    const unsigned jn = (unsigned)clampi(k, 0, D - 1) * plane2;
+                    NDC_UNROLL
+                    for (int r = 0; r < RH; ++r)
+                        NDC_UNROLL
+                        for (int i = 0; i < SC; ++i) {
+                            st.qz[PAR][i][r] = buf_ld(zb_, st.ooff[r], jn + i * cplane2);
+                            st.qg[PAR][i][r] = buf_ld<true>(gb_, st.ooff[r], jn + i * cplane2);
+                            st.qr[PAR][i][r] = buf_ld<true>(rb_, st.ooff[r], jn + i * cplane2);
+                        }
+                }
                 const int lc = st.ln.c0 / 2;
                 if (j0 >= 0 && j0 < D) {
                     // A(gt1) of plane j0: windows of plane j0 + 1 - td, read a tap plane ahead
@@ -603,9 +618,9 @@ template <int RH_> struct Bwd2KernelM {
                             float v[RW], sv[RW];
                             NDC_UNROLL
                             for (int c = 0; c < RW; ++c) {
-                                const float s = floor_f((c ? bf_hi(st.qz[i][r]) : bf_lo(st.qz[i][r])) + st.bvr[i][r], floor_);
-                                const float g = c ? bf_hi(st.qg[i][r]) : bf_lo(st.qg[i][r]);
-                                float gzv = g * (c ? bf_hi(st.qr[i][r]) : bf_lo(st.qr[i][r])) + acc[r][c][i];
+                                const float s = floor_f((c ? bf_hi(st.qz[1 - PAR][i][r]) : bf_lo(st.qz[1 - PAR][i][r])) + st.bvr[i][r], floor_);
+                                const float g = c ? bf_hi(st.qg[1 - PAR][i][r]) : bf_lo(st.qg[1 - PAR][i][r]);
+                                float gzv = g * (c ? bf_hi(st.qr[1 - PAR][i][r]) : bf_lo(st.qr[1 - PAR][i][r])) + acc[r][c][i];
                                 if (relu && s <= 0.f) gzv = 0.f;   // a NaN passes
                                 sv[c] = s;
                                 st.gbacc[i] += gzv * st.okf[r];
@@ -613,18 +628,6 @@ template <int RH_> struct Bwd2KernelM {
                             }
                             buf_st<true>(gzb_, st.ooff[r], jo + i * cplane2, pack_bf16x2(v[0], v[1]));
                             ex.stw(osc + i * SCS + r * WH, pack_bf16x2(sv[0], sv[1]));
-                        }
-                }
-                // the next plane's z, gout, n/d words (this plane's have just been consumed)
-                {
-                    const unsigned jn = (unsigned)clampi(k, 0, D - 1) * plane2;
-                    NDC_UNROLL
-                    for (int r = 0; r < RH; ++r)
-                        NDC_UNROLL
-                        for (int i = 0; i < SC; ++i) {
-                            st.qz[i][r] = buf_ld(zb_, st.ooff[r], jn + i * cplane2);
-                            st.qg[i][r] = buf_ld<true>(gb_, st.ooff[r], jn + i * cplane2);
-                            st.qr[i][r] = buf_ld<true>(rb_, st.ooff[r], jn + i * cplane2);
                         }
                 }
                 const int js = j0 - 1;   // the plane whose s was staged a step ago
@@ -664,7 +667,20 @@ template <int RH_> struct Bwd2KernelM {
                         ex.fence();
                     }
                 }
-            });
+        };
+        for (int kk = 0; kk < D + 2; kk += 2) {
+            {
+                const int k = uniform_int(kk);
+                ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k); });
+                ex.sync();
+                ex.each([&](State &st, int) NDC_LAMBDA { compute(st, k, IntTag<0>()); });
+            }
+            if (kk + 1 < D + 2) {
+                const int k = uniform_int(kk + 1);
+                ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k); });
+                ex.sync();
+                ex.each([&](State &st, int) NDC_LAMBDA { compute(st, k, IntTag<1>()); });
+            }
         }
 
         if (p.need_gh || p.need_gb) {
