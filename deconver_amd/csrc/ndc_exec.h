@@ -81,6 +81,12 @@ template <class State> struct DeviceExec {
     // The instruction scheduler may not move anything across this point: used to keep the LDS
     // reads of the next row ahead of the arithmetic on the current one.
     NDC_D void fence() const { __builtin_amdgcn_sched_barrier(0); }
+    // The word `get(state)` of the lane to the left (lane - 1 of the wavefront); lane 0 gets 0.
+    // For values a kernel computes (nothing in memory to fetch them from again).
+    template <class G> NDC_D uint32_t left_lane(G get)
+    {
+        return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)get(st), 0x138 /* wave_shr:1 */, 0xf, 0xf, true);
+    }
     // every global load this thread has issued has returned (s_waitcnt vmcnt(0))
     NDC_D void wait_loads() const { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
@@ -145,6 +151,9 @@ template <class State> struct HostExec {
     void sync() { ++epoch; }
     void fence() const {}
     void wait_loads() const {}
+    // threads of a phase run in order, so the left neighbour has already computed its word
+    // (both must have taken the same path through the phase up to here)
+    template <class G> uint32_t left_lane(G get) { return cur & 63 ? get(states[cur - 1]) : 0u; }
 
     float ld(int i)
     {

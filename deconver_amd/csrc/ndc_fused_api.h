@@ -102,6 +102,7 @@ struct Plan {
     March m;
     bool dot2;            // bf16 dot2 kernels (3x3x3, SC = 4, even W, aligned pairs)
     bool mfma1, mfma2;    // ... with pass 1 / pass 2 on the matrix instruction when they read the forward's ratios
+    bool mfmaf;           // ... with the forward on the matrix instruction
     Tile tf, tb;          // forward / backward launch shapes
     int lds_f, lds_b1, lds_b2;
     int nblk_f, nblk_b;
@@ -126,7 +127,7 @@ static inline bool make_plan_for(const KGeom &q, Plan &pl, bool pairs_ok, int dt
 {
     pl.m = march_of(q);
     pl.dot2 = false;
-    pl.mfma1 = pl.mfma2 = false;
+    pl.mfma1 = pl.mfma2 = pl.mfmaf = false;
     // 32-bit offsets inside one (sample, channel) volume
     if ((long long)q.sc * q.SP >= (1LL << 31)) return false;
     if (!find_variant(q, pl.m, pairs_ok, pl.v)) return false;
@@ -162,6 +163,8 @@ static inline bool make_plan_for(const KGeom &q, Plan &pl, bool pairs_ok, int dt
                 pl.lds_b2 = l2;
                 pl.mfma1 = tn.mfma && Bwd1KernelM<kDot2RH>::covers(pl.m.W) &&
                            Bwd1KernelM<kDot2RH>::lds_floats(tb) <= cap2;
+                pl.mfmaf = tn.mfma && FwdKernelM<kDot2RH>::covers(pl.m.W) &&
+                           FwdKernelM<kDot2RH>::lds_floats(tf) <= cap2;
                 pl.mfma2 = tn.mfma && Bwd2KernelM<kDot2RH>::covers(pl.m.W) &&
                            Bwd2KernelM<kDot2RH>::lds_floats(tb) <= cap2;
             }
@@ -238,6 +241,9 @@ template <class BE, typename T> struct Dot2Launch {
 template <class BE> struct Dot2Launch<BE, bf16_t> {
     static int fwd(const FwdParams<bf16_t> &p, const Plan &pl, void *stream)
     {
+        if (pl.mfmaf)
+            return BE::template block_kernel<FwdKernelM<kDot2RH>>(p, pl.nblk_f, pl.tf.NT,
+                                                                   FwdKernelM<kDot2RH>::lds_floats(pl.tf), stream);
         return BE::template block_kernel<FwdKernelB<kDot2RH>>(p, pl.nblk_f, pl.tf.NT, pl.lds_f, stream);
     }
     // saved: the call brought the forward's s/d and n/d

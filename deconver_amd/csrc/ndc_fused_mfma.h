@@ -40,6 +40,360 @@ NDC_HD int stride16(int n) { return (n + 47) / 64 * 64 + 16; }
 // (hi half of `left`, lo half of `own`): the bf16 pair one column to the left of `own`
 NDC_HD uint32_t shift_in_left(uint32_t own, uint32_t left) { return (left >> 16) | (own << 16); }
 
+// =================================================================== forward (bf16, matrix instruction)
+
+//   A-type applications (1 -> 4 channels): per (td, th) one instruction per output voxel column,
+//       D[i][n] += sum_{k<4} T[i][k] * V[k][n],   T[i][k] = h[i][td][th][2 - k]  (k = 3: zero)
+//     V[.][n] = the four columns n - 1 .. n + 2 of the operand's row.  A row is staged twice,
+//     as bf16 pairs starting at the odd columns (copy 0, first pair (0, v[0])) and at the even
+//     ones (copy 1): the window of the lane's even column is two consecutive words of copy 0,
+//     that of its odd column two consecutive words of copy 1.
+//
+// out = s (A(x) + eps) / (A(K(s)) + eps); the pipeline is that of FwdKernelB: step k scatters
+// source plane k into the three pending t1 planes and completes t1 plane k - 1 (phase 1), then
+// gathers numerator and denominator of plane k - 2 and stages source plane k + 1 (phase 2).
+template <int RH_> struct FwdKernelM {
+    static constexpr int KD = 3, KH = 3, KW = 3, SC = 4, RH = RH_, RW = 2;
+    static constexpr int PD = 1, PH = 1, PW = 1, KT = 27;
+    static constexpr int kMinStrips = 4;
+    static constexpr int RHK = RH + 1, NZR = RH + 1, NXR = RH + 1;
+    static constexpr int NX = 3;   // ring slots of x and of t1 planes
+    typedef bf16_t T;
+    typedef FwdParams<T> Params;
+
+    struct State {
+        Lane ln;
+        unsigned zoff[NZR], xoff[NXR], ooff[RH];
+        unsigned zok, xok;
+        float bv[SC];
+        MfmaRows wm[9], wg[9];
+        f4_t t1acc[RHK][RW];
+        uint32_t tq[RHK];       // the t1 plane just completed, own rows, as column pairs
+        uint32_t pz[SC][NZR];
+        uint32_t px[NXR];
+    };
+
+    static NDC_HD bool covers(int W) { return W % 8 == 0 && W <= 128 && 64 % (W / 2) == 0; }
+    static NDC_HD int rows_s(int TH) { return TH + 4; }
+    static NDC_HD int rows_x(int TH) { return TH + 2; }
+    static NDC_HD int pitch_x(int W) { return W / 2 + 1; }   // one word past the row: (v[W-1], 0) / zeros
+    static NDC_HD int lds_floats(const Tile &t)
+    {
+        const int W = t.CPW * RW;
+        return rows_s(t.TH) * 2 * t.P + 2 * NX * 2 * rows_x(t.TH) * pitch_x(W);
+    }
+
+    template <class Exec> static NDC_D void run(Exec &ex, const Params &p, int block_id)
+    {
+        const Tile t = p.t;
+        const BlockId id = decode_block(block_id, p.C, t, p.D);
+        const int S = t.S, PL = t.PL, TH = t.TH, W = p.W, H = p.H, D = p.D;
+        const int P2 = 2 * t.P, PX = pitch_x(W);
+        const int RS = rows_s(TH), RX = rows_x(TH);
+        const int CPS = RX * PX;                       // one staged copy of a plane
+        const int off_s = 0, off_x = RS * P2, off_t = off_x + NX * 2 * CPS;
+        const int total = off_t + NX * 2 * CPS;
+        const int plane = H * W;
+        const long long cplane = (long long)D * plane;
+        const long long cbase = ((long long)id.b * p.C + id.c) * cplane;
+        const size_t xbytes = (size_t)cplane * sizeof(T), sbytes = xbytes * SC;
+        const unsigned plane2 = (unsigned)plane * 2u, cplane2 = (unsigned)cplane * 2u;
+        const BufRef xb_ = make_buf(p.x + cbase, xbytes), zb_ = make_buf(p.z + cbase * SC, sbytes);
+        const BufRef ob_ = make_buf(p.out + cbase * SC, sbytes);
+        const BufRef tb_ = make_buf(p.t1 ? p.t1 + cbase : nullptr, xbytes);
+        const BufRef db_ = make_buf(p.s_over_den ? p.s_over_den + cbase * SC : nullptr, sbytes);
+        const BufRef rb_ = make_buf(p.ratio ? p.ratio + cbase * SC : nullptr, sbytes);
+        const bool have_saved = p.s_over_den != nullptr;
+        const float *tabm = p.wtab + (long long)id.c * kTabWords + kTabWM;
+        const float *tabg = p.wtab + (long long)id.c * kTabWords + kTabWG;
+        const int r0 = id.r0;
+        const int nthreads = ex.nthreads;
+        const float floor_ = p.relu ? 0.f : pass_through_floor();
+        const float eps = p.eps;
+
+        // source plane k and x plane k - 1 into the staging registers
+        auto load_plane = [&](State &st, int k) NDC_LAMBDA {
+            if (!st.ln.active) return;
+            if (k < D) {
+                NDC_UNROLL
+                for (int n = 0; n < NZR; ++n)
+                    NDC_UNROLL
+                    for (int i = 0; i < SC; ++i)
+                        st.pz[i][n] = buf_ld(zb_, st.zoff[n], (unsigned)k * plane2 + i * cplane2);
+            }
+            const int kx = k - PD;
+            const bool xlive = kx >= 0 && kx < D;
+            const unsigned xk = (unsigned)clampi(kx, 0, D - 1) * plane2;
+            NDC_UNROLL
+            for (int n = 0; n < NXR; ++n) {
+                const uint32_t v = buf_ld(xb_, st.xoff[n], xk);
+                st.px[n] = xlive ? v : 0u;
+            }
+        };
+        // registers -> LDS: source plane k, four bf16 channels per voxel
+        auto store_plane = [&](State &st, int k) NDC_LAMBDA {
+            if (!st.ln.active) return;
+            // planes past the end are never K-scattered, so the slot may keep stale words
+            NDC_UNROLL
+            for (int n = 0; n < NZR; ++n) {
+                if (k >= D || !((st.zok >> n) & 1u)) continue;
+                const int j = st.ln.strip + n * S;
+                float s[SC][RW];
+                NDC_UNROLL
+                for (int i = 0; i < SC; ++i) {
+                    s[i][0] = floor_f(bf_lo(st.pz[i][n]) + st.bv[i], floor_);
+                    s[i][1] = floor_f(bf_hi(st.pz[i][n]) + st.bv[i], floor_);
+                }
+                const int o = off_s + j * P2 + (PL + st.ln.c0) * 2;
+                NDC_UNROLL
+                for (int c = 0; c < RW; ++c)
+                    ex.st2(o + 2 * c, pack_bf16x2(s[0][c], s[1][c]), pack_bf16x2(s[2][c], s[3][c]));
+            }
+        };
+        // a row of column pairs -> its two staged copies (`left`: the pair of the lane to the left)
+        auto stage_row = [&](State &st, int at, uint32_t own, uint32_t left) NDC_LAMBDA {
+            if (st.ln.c0 == 0) left = 0u;
+            ex.stw(at, shift_in_left(own, left));
+            ex.stw(at + CPS, own);
+            if (st.ln.c0 == W - 2) ex.stw(at + 1, own >> 16);
+        };
+        // x plane k - 1 (fetched during the step before) -> ring slot (k - 1) % NX
+        auto store_x = [&](State &st, int k) NDC_LAMBDA {
+            const int kx = k - PD;
+            const bool xlive = kx >= 0 && kx < D;
+            const unsigned xk = (unsigned)clampi(kx, 0, D - 1) * plane2;
+            const int xb = off_x + wrap(kx % NX, NX) * 2 * CPS + st.ln.c0 / 2;
+            NDC_UNROLL
+            for (int n = 0; n < NXR; ++n) {
+                const uint32_t own = st.px[n];
+                const uint32_t left = from_left_lane(own, [&]() NDC_LAMBDA {
+                    if (st.ln.c0 == 0 || st.xoff[n] >= kNoAccess || !xlive) return 0u;
+                    return buf_ld(xb_, st.xoff[n] - 4u, xk);
+                });
+                if ((st.xok >> n) & 1u) stage_row(st, xb + (st.ln.strip + n * S) * PX, own, left);
+            }
+        };
+
+        ex.each([&](State &st, int tid) NDC_LAMBDA {
+            st.ln = make_lane(tid, t, RW);
+            st.zok = st.xok = 0u;
+            NDC_UNROLL
+            for (int n = 0; n < NZR; ++n) {
+                const int j = st.ln.strip + n * S, row = r0 - 2 * PH + j;
+                if (j < RS && row >= 0 && row < H) st.zok |= 1u << n;
+                st.zoff[n] = (unsigned)(clampi(row, 0, H - 1) * W + st.ln.c0) * 2u;
+                NDC_UNROLL
+                for (int i = 0; i < SC; ++i) st.pz[i][n] = 0u;
+            }
+            NDC_UNROLL
+            for (int n = 0; n < NXR; ++n) {
+                const int j = st.ln.strip + n * S, row = r0 - PH + j;
+                if (j < RX) st.xok |= 1u << n;
+                st.xoff[n] = j < RX && row >= 0 && row < H ? (unsigned)(row * W + st.ln.c0) * 2u : kNoAccess;
+                st.px[n] = 0u;
+            }
+            NDC_UNROLL
+            for (int r = 0; r < RH; ++r) {
+                const int row = r0 + st.ln.strip * RH + r;
+                st.ooff[r] = row < H ? (unsigned)(row * W + st.ln.c0) * 2u : kNoAccess;
+            }
+            NDC_UNROLL
+            for (int i = 0; i < SC; ++i) st.bv[i] = p.bias ? p.bias[id.c * SC + i] : 0.f;
+            NDC_UNROLL
+            for (int t9 = 0; t9 < 9; ++t9) {
+                mfma_rows(st.wm[t9], tid, [&](int m, uint32_t (&w)[2]) NDC_LAMBDA {
+                    w[0] = float_to_bits(tabm[(m * 9 + t9) * 2]);
+                    w[1] = float_to_bits(tabm[(m * 9 + t9) * 2 + 1]);
+                });
+                mfma_rows(st.wg[t9], tid, [&](int m, uint32_t (&w)[2]) NDC_LAMBDA {
+                    w[0] = float_to_bits(tabg[(m * 9 + t9) * 2]);
+                    w[1] = float_to_bits(tabg[(m * 9 + t9) * 2 + 1]);
+                });
+            }
+            const f4_t zero = {0.f, 0.f, 0.f, 0.f};
+            NDC_UNROLL
+            for (int r = 0; r < RHK; ++r) {
+                st.tq[r] = 0u;
+                NDC_UNROLL
+                for (int c = 0; c < RW; ++c) st.t1acc[r][c] = zero;
+            }
+            ex.wait_loads();
+            for (int i = tid; i < total; i += nthreads) ex.st_(i, 0.f);
+            load_plane(st, 0);
+        });
+        ex.sync();
+        ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, 0); });
+        ex.sync();
+
+        for (int kk = 0; kk < D + 2; ++kk) {
+            const int k = uniform_int(kk);
+
+            // ---- x plane k - 1 staged; K-scatter of source plane k; t1 plane k - 1 completed
+            ex.each([&](State &st, int) NDC_LAMBDA {
+                if (!st.ln.active) return;
+                store_x(st, k);
+                const bool extra = st.ln.strip < 2;
+                const int jx = halo_row(st.ln.strip, PH, TH);
+                if (k < D) {
+                    const int cb = off_s + (PL + st.ln.c0 - PW) * 2;
+                    // the 4-voxel window of source row `at`, every tap of it that feeds the NR
+                    // rows acc[r_off ...]; q = the window's row among the NR + 2 input rows
+                    auto read_w = [&](int at, uint32_t (&v)[8]) NDC_LAMBDA {
+                        uint32_t lo[4], hi[4];
+                        ex.ld4a(at, lo);
+                        ex.ld4a(at + 4, hi);
+                        NDC_UNROLL
+                        for (int u = 0; u < 4; ++u) {
+                            v[u] = lo[u];
+                            v[4 + u] = hi[u];
+                        }
+                    };
+                    auto scatter = [&](int q, auto nr_tag, int r_off, const uint32_t (&v)[8]) NDC_LAMBDA {
+                        constexpr int NR = decltype(nr_tag)::value;
+                        NDC_UNROLL
+                        for (int th = 0; th < KH; ++th) {
+                            const int rr = q - th;
+                            if (rr < 0 || rr >= NR) continue;
+                            NDC_UNROLL
+                            for (int tw = 0; tw < KW; ++tw)
+                                NDC_UNROLL
+                                for (int c = 0; c < RW; ++c)
+                                    mfma_bf16_4x4x4(st.t1acc[r_off + rr][c], st.wm[th * 3 + tw],
+                                                    v[(c + tw) * 2], v[(c + tw) * 2 + 1]);
+                        }
+                    };
+                    const int b0 = cb + (PH + st.ln.strip * RH) * P2;
+                    uint32_t kv[2][8];
+                    read_w(b0, kv[0]);
+                    NDC_UNROLL
+                    for (int q = 0; q < RH + 2; ++q) {
+                        if (q + 1 < RH + 2) read_w(b0 + (q + 1) * P2, kv[(q + 1) & 1]);
+                        ex.fence();
+                        scatter(q, IntTag<RH>(), 0, kv[q & 1]);
+                        ex.fence();
+                    }
+                    if (extra) {
+                        const int b1 = cb + jx * P2;
+                        NDC_UNROLL
+                        for (int q = 0; q < 3; ++q) {
+                            uint32_t v[8];
+                            read_w(b1 + q * P2, v);
+                            scatter(q, IntTag<1>(), RH, v);
+                        }
+                    }
+                }
+                // t1 plane k - 1 is complete: to ring slot (k - 1) % NX and to global memory
+                const int pf = k - PD;
+                const bool inplane = pf >= 0 && pf < D;
+                const int tb = off_t + wrap(pf % NX, NX) * 2 * CPS + st.ln.c0 / 2;
+                NDC_UNROLL
+                for (int r = 0; r < RHK; ++r) {
+                    const bool mine = r < RH || extra;
+                    const int j = r < RH ? PH + st.ln.strip * RH + r : jx;
+                    const int row = r0 - PH + j;
+                    const bool live = inplane && row >= 0 && row < H;
+                    const uint32_t vq = live ? pack_bf16x2(st.t1acc[r][0][0], st.t1acc[r][1][0]) : 0u;
+                    st.tq[r] = vq;
+                    const uint32_t left = ex.left_lane([&](State &o) NDC_LAMBDA { return o.tq[r]; });
+                    if (mine) stage_row(st, tb + j * PX, vq, left);
+                    if (r < RH && live) buf_st(tb_, st.ooff[r < RH ? r : 0], (unsigned)pf * plane2, vq);
+                    NDC_UNROLL
+                    for (int c = 0; c < RW; ++c)
+                        st.t1acc[r][c] = f4_t{st.t1acc[r][c][1], st.t1acc[r][c][2], 0.f, 0.f};
+                }
+            });
+            ex.sync();
+
+            // ---- prefetch, then A-gather + epilogue of plane k - 2, then staging of plane k + 1
+            ex.each([&](State &st, int) NDC_LAMBDA {
+                if (!st.ln.active) return;
+                load_plane(st, k + 1);
+                const int j0 = k - 2;
+                if (j0 < 0) {
+                    store_plane(st, k + 1);
+                    return;
+                }
+                // the own source values of plane j0: z is read again (staged two steps ago: L2)
+                uint32_t own[SC][RH];
+                NDC_UNROLL
+                for (int r = 0; r < RH; ++r)
+                    NDC_UNROLL
+                    for (int i = 0; i < SC; ++i)
+                        own[i][r] = buf_ld(zb_, st.ooff[r], (unsigned)j0 * plane2 + i * cplane2);
+                f4_t acc[2][RH][RW];   // numerator, denominator; four channels each
+                NDC_UNROLL
+                for (int a = 0; a < 2; ++a)
+                    NDC_UNROLL
+                    for (int r = 0; r < RH; ++r)
+                        NDC_UNROLL
+                        for (int c = 0; c < RW; ++c) acc[a][r][c] = f4_t{eps, eps, eps, eps};
+                {
+                    const int lc = st.ln.c0 / 2;
+                    // group g = (operand, td): the windows of the RH + 2 rows of plane
+                    // j0 + 1 - td; read a group ahead of the instructions that use them
+                    auto read_a = [&](int g, uint32_t (&v)[RH + 2][RW][2]) NDC_LAMBDA {
+                        const int op = g / KD, td = g % KD;
+                        const int at = (op ? off_t : off_x) + wrap((j0 + 1 - td) % NX, NX) * 2 * CPS +
+                                       (st.ln.strip * RH) * PX + lc;
+                        NDC_UNROLL
+                        for (int q = 0; q < RH + 2; ++q)
+                            NDC_UNROLL
+                            for (int c = 0; c < RW; ++c) ex.ld2w(at + c * CPS + q * PX, v[q][c]);
+                    };
+                    auto mfma_a = [&](int g, const uint32_t (&v)[RH + 2][RW][2]) NDC_LAMBDA {
+                        const int op = g / KD, td = g % KD;
+                        NDC_UNROLL
+                        for (int q = 0; q < RH + 2; ++q)
+                            NDC_UNROLL
+                            for (int r = 0; r < RH; ++r) {
+                                const int th = r + 2 - q;
+                                if (th < 0 || th >= KH) continue;
+                                NDC_UNROLL
+                                for (int c = 0; c < RW; ++c)
+                                    mfma_bf16_4x4x4(acc[op][r][c], st.wg[td * 3 + th], v[q][c][0], v[q][c][1]);
+                            }
+                    };
+                    uint32_t av[2][RH + 2][RW][2];
+                    read_a(0, av[0]);
+                    NDC_UNROLL
+                    for (int g = 0; g < 2 * KD; ++g) {
+                        if (g + 1 < 2 * KD) read_a(g + 1, av[(g + 1) & 1]);
+                        ex.fence();
+                        mfma_a(g, av[g & 1]);
+                        ex.fence();
+                    }
+                }
+                const unsigned oj = (unsigned)j0 * plane2;
+                NDC_UNROLL
+                for (int r = 0; r < RH; ++r) {
+                    // (a row outside the image: its stores go nowhere)
+                    NDC_UNROLL
+                    for (int i = 0; i < SC; ++i) {
+                        float v[RW], rd[RW], rt[RW];
+                        NDC_UNROLL
+                        for (int c = 0; c < RW; ++c) {
+                            const uint32_t w = own[i][r];
+                            // same arithmetic as the staging: the staged value before its rounding
+                            const float s = floor_f((c ? bf_hi(w) : bf_lo(w)) + st.bv[i], floor_);
+                            const float inv = fast_rcp(acc[1][r][c][i]);
+                            rd[c] = s * inv;
+                            rt[c] = acc[0][r][c][i] * inv;
+                            v[c] = s * rt[c];
+                        }
+                        buf_st<true>(ob_, st.ooff[r], oj + i * cplane2, pack_bf16x2(v[0], v[1]));
+                        if (have_saved) {
+                            buf_st<true>(db_, st.ooff[r], oj + i * cplane2, pack_bf16x2(rd[0], rd[1]));
+                            buf_st<true>(rb_, st.ooff[r], oj + i * cplane2, pack_bf16x2(rt[0], rt[1]));
+                        }
+                    }
+                }
+                store_plane(st, k + 1);
+            });
+            ex.sync();
+        }
+    }
+};
+
 // =================================================================== backward pass 1 (bf16, matrix instruction)
 
 // Reads the forward's s/d and n/d (the form every training step uses): gn = g s/d,
