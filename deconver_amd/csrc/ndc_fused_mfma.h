@@ -65,12 +65,14 @@ template <int RH_> struct FwdKernelM {
         Lane ln;
         unsigned zoff[NZR], xoff[NXR], ooff[RH];
         unsigned zok, xok;
-        float bv[SC];
         MfmaRows wm[9], wg[9];
         f4_t t1acc[RHK][RW];
         uint32_t tq[RHK];       // the t1 plane just completed, own rows, as column pairs
-        uint32_t pz[SC][NZR];
-        uint32_t px[NXR];
+        // staging registers, two sets: set (plane & 1) holds a source (x) plane from its fetch,
+        // two steps before it is staged, until then.  The plane loop is unrolled twice, so the
+        // sets are fixed registers.
+        uint32_t pz[2][SC][NZR];
+        uint32_t px[2][NXR];
     };
 
     static NDC_HD bool covers(int W) { return W % 8 == 0 && W <= 128 && 64 % (W / 2) == 0; }
@@ -110,28 +112,39 @@ template <int RH_> struct FwdKernelM {
         const int nthreads = ex.nthreads;
         const float floor_ = p.relu ? 0.f : pass_through_floor();
         const float eps = p.eps;
+        // the channel's four bias values: wave-uniform, fetched through the scalar unit
+        float bv[SC];
+        {
+            UniformF bu = as_uniform(p.bias ? p.bias + id.c * SC : p.wtab);
+            NDC_UNROLL
+            for (int i = 0; i < SC; ++i) bv[i] = p.bias ? bu[i] : 0.f;
+        }
 
-        // source plane k and x plane k - 1 into the staging registers
-        auto load_plane = [&](State &st, int k) NDC_LAMBDA {
-            if (!st.ln.active) return;
-            if (k < D) {
+        // source plane k / x plane kx into staging set `set` (= the plane's parity)
+        auto load_z = [&](State &st, int k, auto set_tag) NDC_LAMBDA {
+            constexpr int SET = decltype(set_tag)::value;
+            if (!st.ln.active || k >= D) return;
+            NDC_UNROLL
+            for (int n = 0; n < NZR; ++n)
                 NDC_UNROLL
-                for (int n = 0; n < NZR; ++n)
-                    NDC_UNROLL
-                    for (int i = 0; i < SC; ++i)
-                        st.pz[i][n] = buf_ld(zb_, st.zoff[n], (unsigned)k * plane2 + i * cplane2);
-            }
-            const int kx = k - PD;
+                for (int i = 0; i < SC; ++i)
+                    st.pz[SET][i][n] = buf_ld(zb_, st.zoff[n], (unsigned)k * plane2 + i * cplane2);
+        };
+        auto load_x = [&](State &st, int kx, auto set_tag) NDC_LAMBDA {
+            constexpr int SET = decltype(set_tag)::value;
+            if (!st.ln.active) return;
+            // planes outside the volume: a clamped plane is loaded and zero selected
             const bool xlive = kx >= 0 && kx < D;
             const unsigned xk = (unsigned)clampi(kx, 0, D - 1) * plane2;
             NDC_UNROLL
             for (int n = 0; n < NXR; ++n) {
                 const uint32_t v = buf_ld(xb_, st.xoff[n], xk);
-                st.px[n] = xlive ? v : 0u;
+                st.px[SET][n] = xlive ? v : 0u;
             }
         };
         // registers -> LDS: source plane k, four bf16 channels per voxel
-        auto store_plane = [&](State &st, int k) NDC_LAMBDA {
+        auto store_plane = [&](State &st, int k, auto set_tag) NDC_LAMBDA {
+            constexpr int SET = decltype(set_tag)::value;
             if (!st.ln.active) return;
             // planes past the end are never K-scattered, so the slot may keep stale words
             NDC_UNROLL
@@ -141,8 +154,8 @@ template <int RH_> struct FwdKernelM {
                 float s[SC][RW];
                 NDC_UNROLL
                 for (int i = 0; i < SC; ++i) {
-                    s[i][0] = floor_f(bf_lo(st.pz[i][n]) + st.bv[i], floor_);
-                    s[i][1] = floor_f(bf_hi(st.pz[i][n]) + st.bv[i], floor_);
+                    s[i][0] = floor_f(bf_lo(st.pz[SET][i][n]) + bv[i], floor_);
+                    s[i][1] = floor_f(bf_hi(st.pz[SET][i][n]) + bv[i], floor_);
                 }
                 const int o = off_s + j * P2 + (PL + st.ln.c0) * 2;
                 NDC_UNROLL
@@ -158,14 +171,15 @@ template <int RH_> struct FwdKernelM {
             if (st.ln.c0 == W - 2) ex.stw(at + 1, own >> 16);
         };
         // x plane k - 1 (fetched during the step before) -> ring slot (k - 1) % NX
-        auto store_x = [&](State &st, int k) NDC_LAMBDA {
+        auto store_x = [&](State &st, int k, auto set_tag) NDC_LAMBDA {
+            constexpr int SET = decltype(set_tag)::value;
             const int kx = k - PD;
             const bool xlive = kx >= 0 && kx < D;
             const unsigned xk = (unsigned)clampi(kx, 0, D - 1) * plane2;
             const int xb = off_x + wrap(kx % NX, NX) * 2 * CPS + st.ln.c0 / 2;
             NDC_UNROLL
             for (int n = 0; n < NXR; ++n) {
-                const uint32_t own = st.px[n];
+                const uint32_t own = st.px[SET][n];
                 const uint32_t left = from_left_lane(own, [&]() NDC_LAMBDA {
                     if (st.ln.c0 == 0 || st.xoff[n] >= kNoAccess || !xlive) return 0u;
                     return buf_ld(xb_, st.xoff[n] - 4u, xk);
@@ -183,22 +197,20 @@ template <int RH_> struct FwdKernelM {
                 if (j < RS && row >= 0 && row < H) st.zok |= 1u << n;
                 st.zoff[n] = (unsigned)(clampi(row, 0, H - 1) * W + st.ln.c0) * 2u;
                 NDC_UNROLL
-                for (int i = 0; i < SC; ++i) st.pz[i][n] = 0u;
+                for (int i = 0; i < SC; ++i) st.pz[0][i][n] = st.pz[1][i][n] = 0u;
             }
             NDC_UNROLL
             for (int n = 0; n < NXR; ++n) {
                 const int j = st.ln.strip + n * S, row = r0 - PH + j;
                 if (j < RX) st.xok |= 1u << n;
                 st.xoff[n] = j < RX && row >= 0 && row < H ? (unsigned)(row * W + st.ln.c0) * 2u : kNoAccess;
-                st.px[n] = 0u;
+                st.px[0][n] = st.px[1][n] = 0u;
             }
             NDC_UNROLL
             for (int r = 0; r < RH; ++r) {
                 const int row = r0 + st.ln.strip * RH + r;
                 st.ooff[r] = row < H ? (unsigned)(row * W + st.ln.c0) * 2u : kNoAccess;
             }
-            NDC_UNROLL
-            for (int i = 0; i < SC; ++i) st.bv[i] = p.bias ? p.bias[id.c * SC + i] : 0.f;
             NDC_UNROLL
             for (int t9 = 0; t9 < 9; ++t9) {
                 mfma_rows(st.wm[t9], tid, [&](int m, uint32_t (&w)[2]) NDC_LAMBDA {
@@ -219,19 +231,24 @@ template <int RH_> struct FwdKernelM {
             }
             ex.wait_loads();
             for (int i = tid; i < total; i += nthreads) ex.st_(i, 0.f);
-            load_plane(st, 0);
+            load_z(st, 0, IntTag<0>());
+            load_x(st, 0, IntTag<0>());
         });
         ex.sync();
-        ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, 0); });
+        ex.each([&](State &st, int) NDC_LAMBDA {
+            store_plane(st, 0, IntTag<0>());
+            load_z(st, 1, IntTag<1>());
+        });
         ex.sync();
 
-        for (int kk = 0; kk < D + 2; ++kk) {
-            const int k = uniform_int(kk);
+        // one plane step; PAR = k % 2, known at compile time (the loop below is unrolled twice)
+        auto step = [&](int k, auto par_tag) NDC_LAMBDA {
+            constexpr int PAR = decltype(par_tag)::value;
 
             // ---- x plane k - 1 staged; K-scatter of source plane k; t1 plane k - 1 completed
             ex.each([&](State &st, int) NDC_LAMBDA {
                 if (!st.ln.active) return;
-                store_x(st, k);
+                store_x(st, k, IntTag<1 - PAR>());
                 const bool extra = st.ln.strip < 2;
                 const int jx = halo_row(st.ln.strip, PH, TH);
                 if (k < D) {
@@ -307,19 +324,16 @@ template <int RH_> struct FwdKernelM {
             // ---- prefetch, then A-gather + epilogue of plane k - 2, then staging of plane k + 1
             ex.each([&](State &st, int) NDC_LAMBDA {
                 if (!st.ln.active) return;
-                load_plane(st, k + 1);
+                // fetched now, staged two steps on: source plane k + 2, x plane k + 1
+                load_z(st, k + 2, IntTag<PAR>());
+                load_x(st, k + 1, IntTag<1 - PAR>());
                 const int j0 = k - 2;
                 if (j0 < 0) {
-                    store_plane(st, k + 1);
+                    store_plane(st, k + 1, IntTag<1 - PAR>());
                     return;
                 }
                 // the own source values of plane j0: z is read again (staged two steps ago: L2)
                 uint32_t own[SC][RH];
-                NDC_UNROLL
-                for (int r = 0; r < RH; ++r)
-                    NDC_UNROLL
-                    for (int i = 0; i < SC; ++i)
-                        own[i][r] = buf_ld(zb_, st.ooff[r], (unsigned)j0 * plane2 + i * cplane2);
                 f4_t acc[2][RH][RW];   // numerator, denominator; four channels each
                 NDC_UNROLL
                 for (int a = 0; a < 2; ++a)
@@ -329,37 +343,49 @@ template <int RH_> struct FwdKernelM {
                         for (int c = 0; c < RW; ++c) acc[a][r][c] = f4_t{eps, eps, eps, eps};
                 {
                     const int lc = st.ln.c0 / 2;
-                    // group g = (operand, td): the windows of the RH + 2 rows of plane
-                    // j0 + 1 - td; read a group ahead of the instructions that use them
-                    auto read_a = [&](int g, uint32_t (&v)[RH + 2][RW][2]) NDC_LAMBDA {
-                        const int op = g / KD, td = g % KD;
+                    // unit u = (operand, td, row pair): the windows of two of the RH + 2 rows of
+                    // plane j0 + 1 - td; read two units ahead of the instructions that use them
+                    static_assert(RH == 2, "the units below pair the RH + 2 = 4 input rows");
+                    auto read_a = [&](int u, uint32_t (&v)[2][RW][2]) NDC_LAMBDA {
+                        const int op = u / (2 * KD), td = (u / 2) % KD, q0 = (u % 2) * 2;
                         const int at = (op ? off_t : off_x) + wrap((j0 + 1 - td) % NX, NX) * 2 * CPS +
-                                       (st.ln.strip * RH) * PX + lc;
+                                       (st.ln.strip * RH + q0) * PX + lc;
                         NDC_UNROLL
-                        for (int q = 0; q < RH + 2; ++q)
+                        for (int q = 0; q < 2; ++q)
                             NDC_UNROLL
                             for (int c = 0; c < RW; ++c) ex.ld2w(at + c * CPS + q * PX, v[q][c]);
                     };
-                    auto mfma_a = [&](int g, const uint32_t (&v)[RH + 2][RW][2]) NDC_LAMBDA {
-                        const int op = g / KD, td = g % KD;
+                    auto mfma_a = [&](int u, const uint32_t (&v)[2][RW][2]) NDC_LAMBDA {
+                        const int op = u / (2 * KD), td = (u / 2) % KD, q0 = (u % 2) * 2;
                         NDC_UNROLL
-                        for (int q = 0; q < RH + 2; ++q)
+                        for (int q = 0; q < 2; ++q)
                             NDC_UNROLL
                             for (int r = 0; r < RH; ++r) {
-                                const int th = r + 2 - q;
+                                const int th = r + 2 - (q0 + q);
                                 if (th < 0 || th >= KH) continue;
                                 NDC_UNROLL
                                 for (int c = 0; c < RW; ++c)
                                     mfma_bf16_4x4x4(acc[op][r][c], st.wg[td * 3 + th], v[q][c][0], v[q][c][1]);
                             }
                     };
-                    uint32_t av[2][RH + 2][RW][2];
+                    constexpr int NU = 2 * KD * 2;
+                    uint32_t av[3][2][RW][2];
                     read_a(0, av[0]);
+                    read_a(1, av[1]);
                     NDC_UNROLL
-                    for (int g = 0; g < 2 * KD; ++g) {
-                        if (g + 1 < 2 * KD) read_a(g + 1, av[(g + 1) & 1]);
+                    for (int u = 0; u < NU; ++u) {
+                        if (u + 2 < NU) read_a(u + 2, av[(u + 2) % 3]);
+                        if (u == NU - 3) {
+                            // (issued here, when the last windows have been requested: before
+                            // the loop they would hold eight more registers through it)
+                            NDC_UNROLL
+                            for (int r = 0; r < RH; ++r)
+                                NDC_UNROLL
+                                for (int i = 0; i < SC; ++i)
+                                    own[i][r] = buf_ld(zb_, st.ooff[r], (unsigned)j0 * plane2 + i * cplane2);
+                        }
                         ex.fence();
-                        mfma_a(g, av[g & 1]);
+                        mfma_a(u, av[u % 3]);
                         ex.fence();
                     }
                 }
@@ -374,7 +400,7 @@ template <int RH_> struct FwdKernelM {
                         for (int c = 0; c < RW; ++c) {
                             const uint32_t w = own[i][r];
                             // same arithmetic as the staging: the staged value before its rounding
-                            const float s = floor_f((c ? bf_hi(w) : bf_lo(w)) + st.bv[i], floor_);
+                            const float s = floor_f((c ? bf_hi(w) : bf_lo(w)) + bv[i], floor_);
                             const float inv = fast_rcp(acc[1][r][c][i]);
                             rd[c] = s * inv;
                             rt[c] = acc[0][r][c][i] * inv;
@@ -387,9 +413,13 @@ template <int RH_> struct FwdKernelM {
                         }
                     }
                 }
-                store_plane(st, k + 1);
+                store_plane(st, k + 1, IntTag<1 - PAR>());
             });
             ex.sync();
+        };
+        for (int kk = 0; kk < D + 2; kk += 2) {
+            step(uniform_int(kk), IntTag<0>());
+            if (kk + 1 < D + 2) step(uniform_int(kk + 1), IntTag<1>());
         }
     }
 };
