@@ -123,12 +123,15 @@ template <int RH_> struct FwdKernelM {
         // source plane k / x plane kx into staging set `set` (= the plane's parity)
         auto load_z = [&](State &st, int k, auto set_tag) NDC_LAMBDA {
             constexpr int SET = decltype(set_tag)::value;
-            if (!st.ln.active || k >= D) return;
+            if (!st.ln.active) return;
+            // (planes past the end: a clamped plane is fetched and never staged; a branch
+            // around the loads would keep the compiler from counting the outstanding ones)
+            const unsigned ko = (unsigned)clampi(k, 0, D - 1) * plane2;
             NDC_UNROLL
             for (int n = 0; n < NZR; ++n)
                 NDC_UNROLL
                 for (int i = 0; i < SC; ++i)
-                    st.pz[SET][i][n] = buf_ld(zb_, st.zoff[n], (unsigned)k * plane2 + i * cplane2);
+                    st.pz[SET][i][n] = buf_ld(zb_, st.zoff[n], ko + i * cplane2);
         };
         auto load_x = [&](State &st, int kx, auto set_tag) NDC_LAMBDA {
             constexpr int SET = decltype(set_tag)::value;
@@ -447,7 +450,9 @@ template <int RH_> struct Bwd1KernelM {
         f4_t accx[RH][RW], acct[RH][RW];
         f4_t gacc[KD][KH];
         uint32_t px[NXS], pt[NXS];
-        uint32_t qg[SC][RH + 1], qd[SC][RH + 1], qr[SC][RH + 1];
+        // gout, s/d, n/d words of two planes: set (plane & 1) holds a plane from its fetch, two
+        // steps before it is used, until then (the plane loop is unrolled twice: fixed registers)
+        uint32_t qg[2][SC][RH + 1], qd[2][SC][RH + 1], qr[2][SC][RH + 1];
     };
 
     static NDC_HD bool covers(int W) { return W % 8 == 0 && W <= 128 && 64 % (W / 2) == 0; }
@@ -536,33 +541,37 @@ template <int RH_> struct Bwd1KernelM {
         };
         // gout, s/d, n/d words of plane jn into the state, a phase before they are used (own
         // rows, then the halo row of the first two strips)
-        auto prefetch_g = [&](State &st, int jn) NDC_LAMBDA {
-            if (jn >= D) return;
-            const unsigned jo = (unsigned)jn * plane2;
+        auto prefetch_g = [&](State &st, int jn, auto set_tag) NDC_LAMBDA {
+            constexpr int SET = decltype(set_tag)::value;
+            // (no branch around the loads, also past the last plane, where a clamped plane is
+            // fetched and never used: with loads on one path only the compiler cannot count
+            // the outstanding ones, and makes the next user of ANY load wait for all)
+            const unsigned jo = (unsigned)clampi(jn, 0, D - 1) * plane2;
             NDC_UNROLL
             for (int r = 0; r < RH + 1; ++r) {
                 if (r == RH && st.ln.strip >= 2) continue;
                 const unsigned o = r < RH ? st.ooff[r < RH ? r : 0] : st.hoff;
                 NDC_UNROLL
                 for (int i = 0; i < SC; ++i) {
-                    st.qg[i][r] = buf_ld<true>(gb_, o, jo + i * cplane2);
-                    st.qd[i][r] = buf_ld<true>(db_, o, jo + i * cplane2);
-                    st.qr[i][r] = buf_ld<true>(rb_, o, jo + i * cplane2);
+                    st.qg[SET][i][r] = buf_ld<true>(gb_, o, jo + i * cplane2);
+                    st.qd[SET][i][r] = buf_ld<true>(db_, o, jo + i * cplane2);
+                    st.qr[SET][i][r] = buf_ld<true>(rb_, o, jo + i * cplane2);
                 }
             }
         };
         // gn, gd of the prefetched row `pr` -> tile row j of the per-voxel copy (four channels
         // per voxel) and, for own rows, row `own` of the channel-major copy
-        auto publish_row = [&](State &st, int pr, int j, int own) NDC_LAMBDA {
+        auto publish_row = [&](State &st, auto set_tag, int pr, int j, int own) NDC_LAMBDA {
+            constexpr int SET = decltype(set_tag)::value;
             float gn[SC][RW], gd[SC][RW];
             NDC_UNROLL
             for (int i = 0; i < SC; ++i)
                 NDC_UNROLL
                 for (int c = 0; c < RW; ++c) {
                     // (the words of a row outside the image were read as zeros)
-                    const float gv = c ? bf_hi(st.qg[i][pr]) : bf_lo(st.qg[i][pr]);
-                    gn[i][c] = gv * (c ? bf_hi(st.qd[i][pr]) : bf_lo(st.qd[i][pr]));
-                    gd[i][c] = -(gn[i][c] * (c ? bf_hi(st.qr[i][pr]) : bf_lo(st.qr[i][pr])));
+                    const float gv = c ? bf_hi(st.qg[SET][i][pr]) : bf_lo(st.qg[SET][i][pr]);
+                    gn[i][c] = gv * (c ? bf_hi(st.qd[SET][i][pr]) : bf_lo(st.qd[SET][i][pr]));
+                    gd[i][c] = -(gn[i][c] * (c ? bf_hi(st.qr[SET][i][pr]) : bf_lo(st.qr[SET][i][pr])));
                 }
             const int o = off_gp + j * P2 + (PL + st.ln.c0) * 2;
             NDC_UNROLL
@@ -604,7 +613,9 @@ template <int RH_> struct Bwd1KernelM {
                 NDC_UNROLL
                 for (int i = 0; i < SC; ++i)
                     NDC_UNROLL
-                    for (int r = 0; r < RH + 1; ++r) st.qg[i][r] = st.qd[i][r] = st.qr[i][r] = 0u;
+                    for (int r = 0; r < RH + 1; ++r)
+                        NDC_UNROLL
+                        for (int a = 0; a < 2; ++a) st.qg[a][i][r] = st.qd[a][i][r] = st.qr[a][i][r] = 0u;
             }
             NDC_UNROLL
             for (int t9 = 0; t9 < 9; ++t9)
@@ -626,14 +637,16 @@ template <int RH_> struct Bwd1KernelM {
             ex.wait_loads();
             for (int i = tid; i < total; i += nthreads) ex.st_(i, 0.f);
             load_plane(st, 0);
+            if (st.ln.active) prefetch_g(st, 0, IntTag<0>());
         });
         ex.sync();
 
         // Two barriers per plane step.  Phase 1 of step k stages plane k of x / t1 (fetched
         // during the step before) and publishes gn / gd of plane k - 1; phase 2 fetches the
         // next planes and does all tap sums of plane k - 1.
-        for (int kk = 0; kk < D + 2; ++kk) {
-            const int k = uniform_int(kk);
+        // one plane step; PAR = k % 2, known at compile time (the loop below is unrolled twice)
+        auto step = [&](int k, auto par_tag) NDC_LAMBDA {
+            constexpr int PAR = decltype(par_tag)::value;
             const int j1 = k - 1;
             const bool live1 = j1 >= 0 && j1 < D;
             ex.each([&](State &st, int) NDC_LAMBDA {
@@ -642,15 +655,15 @@ template <int RH_> struct Bwd1KernelM {
                 if (!live1) return;
                 NDC_UNROLL
                 for (int r = 0; r < RH; ++r)
-                    publish_row(st, r, PH + st.ln.strip * RH + r, st.ln.strip * RH + r);
-                if (st.ln.strip < 2) publish_row(st, RH, halo_row(st.ln.strip, PH, TH), -1);
+                    publish_row(st, IntTag<1 - PAR>(), r, PH + st.ln.strip * RH + r, st.ln.strip * RH + r);
+                if (st.ln.strip < 2) publish_row(st, IntTag<1 - PAR>(), RH, halo_row(st.ln.strip, PH, TH), -1);
             });
             ex.sync();
 
             ex.each([&](State &st, int) NDC_LAMBDA {
                 if (!st.ln.active) return;
                 load_plane(st, k + 1);
-                prefetch_g(st, k);
+                prefetch_g(st, k + 1, IntTag<1 - PAR>());
                 if (live1) {
                     // LDS reads run ahead of the matrix instructions that use them (two
                     // wavefronts per SIMD do not hide their latency): the K-type rows two
@@ -685,16 +698,16 @@ template <int RH_> struct Bwd1KernelM {
                                                     v[(c + tw) * 2 + 1]);
                         }
                     };
-                    // filter-gradient group g = (operand, td): the RH + 2 rows of x (t1) of
-                    // plane j1 + 1 - td around the own rows, in the lane's shifted copy
+                    // filter-gradient unit u = (operand, td, row pair): two of the RH + 2 rows of x
+                    // (t1) of plane j1 + 1 - td around the own rows, in the lane's shifted copy
                     const int copy = st.lane4 < 3 ? st.lane4 : 1;
-                    auto read_g = [&](int g, uint32_t (&bw)[RH + 2][4]) NDC_LAMBDA {
-                        const int op = g / KD, td = g % KD;
+                    auto read_g = [&](int u, uint32_t (&bw)[2][4]) NDC_LAMBDA {
+                        const int op = u / (2 * KD), td = (u / 2) % KD, q0 = (u % 2) * 2;
                         const int slot = wrap((j1 + 1 - td) % NX, NX);
                         const int xb = off_xs + ((slot * 2 + op) * 3 + copy) * XCS +
-                                       (st.ln.strip * RH) * WH + st.blk4;
+                                       (st.ln.strip * RH + q0) * WH + st.blk4;
                         NDC_UNROLL
-                        for (int q = 0; q < RH + 2; ++q) ex.ld4a(xb + q * WH, bw[q]);
+                        for (int q = 0; q < 2; ++q) ex.ld4a(xb + q * WH, bw[q]);
                     };
                     // the block's 8 columns of gn (gd), channel = lane & 3, own rows
                     MfmaRows ga[2][RH][2];
@@ -708,38 +721,41 @@ template <int RH_> struct Bwd1KernelM {
                                            [&](int m, uint32_t (&w4)[4]) NDC_LAMBDA { ex.ld4a(at + m * GCS, w4); });
                             }
                     };
-                    auto mfma_g = [&](int g, const uint32_t (&bw)[RH + 2][4]) NDC_LAMBDA {
-                        const int op = g / KD, td = g % KD;
+                    auto mfma_g = [&](int u, const uint32_t (&bw)[2][4]) NDC_LAMBDA {
+                        const int op = u / (2 * KD), td = (u / 2) % KD, q0 = (u % 2) * 2;
                         NDC_UNROLL
-                        for (int q = 0; q < RH + 2; ++q)
+                        for (int q = 0; q < 2; ++q)
                             NDC_UNROLL
                             for (int r = 0; r < RH; ++r) {
-                                const int th = r + 2 - q;
+                                const int th = r + 2 - (q0 + q);
                                 if (th < 0 || th >= KH) continue;
                                 mfma_bf16_4x4x4(st.gacc[td][th], ga[op][r][0], bw[q][0], bw[q][1]);
                                 mfma_bf16_4x4x4(st.gacc[td][th], ga[op][r][1], bw[q][2], bw[q][3]);
                             }
                     };
-                    constexpr int NKG = 2 * (RH + 2), NGG = 2 * KD;
-                    uint32_t kv[3][8];
-                    uint32_t bw[2][RH + 2][4];
+                    static_assert(RH == 2, "the units pair the RH + 2 = 4 input rows");
+                    constexpr int NKG = 2 * (RH + 2), NGG = 2 * KD * 2;
+                    uint32_t kv[2][8];
+                    uint32_t bw[3][2][4];
                     read_k(0, kv[0]);
-                    read_k(1, kv[1]);
                     NDC_UNROLL
                     for (int g = 0; g < NKG; ++g) {
-                        if (g + 2 < NKG) read_k(g + 2, kv[(g + 2) % 3]);
+                        if (g + 1 < NKG) read_k(g + 1, kv[(g + 1) & 1]);
                         if (need_gh && g + 2 == NKG) read_ga();
-                        if (need_gh && g + 1 == NKG) read_g(0, bw[0]);
+                        if (need_gh && g + 1 == NKG) {
+                            read_g(0, bw[0]);
+                            read_g(1, bw[1]);
+                        }
                         ex.fence();
-                        mfma_k(g, kv[g % 3]);
+                        mfma_k(g, kv[g & 1]);
                         ex.fence();
                     }
                     if (need_gh) {
                         NDC_UNROLL
                         for (int g = 0; g < NGG; ++g) {
-                            if (g + 1 < NGG) read_g(g + 1, bw[(g + 1) & 1]);
+                            if (g + 2 < NGG) read_g(g + 2, bw[(g + 2) % 3]);
                             ex.fence();
-                            mfma_g(g, bw[g & 1]);
+                            mfma_g(g, bw[g % 3]);
                             ex.fence();
                         }
                     }
@@ -761,6 +777,10 @@ template <int RH_> struct Bwd1KernelM {
                 }
             });
             ex.sync();
+        };
+        for (int kk = 0; kk < D + 2; kk += 2) {
+            step(uniform_int(kk), IntTag<0>());
+            if (kk + 1 < D + 2) step(uniform_int(kk + 1), IntTag<1>());
         }
 
         if (need_gh) {
