@@ -123,7 +123,6 @@ template <int RH_> struct FwdKernelM {
         // source plane k / x plane kx into staging set `set` (= the plane's parity)
         auto load_z = [&](State &st, int k, auto set_tag) NDC_LAMBDA {
             constexpr int SET = decltype(set_tag)::value;
-            if (!st.ln.active) return;
             // (planes past the end: a clamped plane is fetched and never staged; a branch
             // around the loads would keep the compiler from counting the outstanding ones)
             const unsigned ko = (unsigned)clampi(k, 0, D - 1) * plane2;
@@ -135,7 +134,6 @@ template <int RH_> struct FwdKernelM {
         };
         auto load_x = [&](State &st, int kx, auto set_tag) NDC_LAMBDA {
             constexpr int SET = decltype(set_tag)::value;
-            if (!st.ln.active) return;
             // planes outside the volume: a clamped plane is loaded and zero selected
             const bool xlive = kx >= 0 && kx < D;
             const unsigned xk = (unsigned)clampi(kx, 0, D - 1) * plane2;
@@ -198,7 +196,7 @@ template <int RH_> struct FwdKernelM {
             for (int n = 0; n < NZR; ++n) {
                 const int j = st.ln.strip + n * S, row = r0 - 2 * PH + j;
                 if (j < RS && row >= 0 && row < H) st.zok |= 1u << n;
-                st.zoff[n] = (unsigned)(clampi(row, 0, H - 1) * W + st.ln.c0) * 2u;
+                st.zoff[n] = st.ln.active ? (unsigned)(clampi(row, 0, H - 1) * W + st.ln.c0) * 2u : kNoAccess;
                 NDC_UNROLL
                 for (int i = 0; i < SC; ++i) st.pz[0][i][n] = st.pz[1][i][n] = 0u;
             }
@@ -206,7 +204,7 @@ template <int RH_> struct FwdKernelM {
             for (int n = 0; n < NXR; ++n) {
                 const int j = st.ln.strip + n * S, row = r0 - PH + j;
                 if (j < RX) st.xok |= 1u << n;
-                st.xoff[n] = j < RX && row >= 0 && row < H ? (unsigned)(row * W + st.ln.c0) * 2u : kNoAccess;
+                st.xoff[n] = st.ln.active && j < RX && row >= 0 && row < H ? (unsigned)(row * W + st.ln.c0) * 2u : kNoAccess;
                 st.px[0][n] = st.px[1][n] = 0u;
             }
             NDC_UNROLL
@@ -326,12 +324,16 @@ template <int RH_> struct FwdKernelM {
 
             // ---- prefetch, then A-gather + epilogue of plane k - 2, then staging of plane k + 1
             ex.each([&](State &st, int) NDC_LAMBDA {
-                if (!st.ln.active) return;
                 // fetched now, staged two steps on: source plane k + 2, x plane k + 1
+            // (every lane issues every fetch, lanes outside the tile with offsets outside the
+            // slices: a fetch under a condition gives the compiler a path without it, on which
+            // it cannot count the outstanding loads, and then every use of a prefetched
+            // register waits for ALL loads)
                 load_z(st, k + 2, IntTag<PAR>());
                 load_x(st, k + 1, IntTag<1 - PAR>());
+                if (!st.ln.active) return;
                 const int j0 = k - 2;
-                if (j0 < 0) {
+                if (j0 < 0 || j0 >= D) {
                     store_plane(st, k + 1, IntTag<1 - PAR>());
                     return;
                 }
@@ -420,9 +422,13 @@ template <int RH_> struct FwdKernelM {
             });
             ex.sync();
         };
+        // An even number of steps, the last possibly one past the end of the march (it finds
+        // nothing to do): with the second step of an iteration under a condition the compiler
+        // sees a path from one even step straight to the next and, unable to count the loads
+        // outstanding on it, makes every use of a prefetched register wait for all loads.
         for (int kk = 0; kk < D + 2; kk += 2) {
             step(uniform_int(kk), IntTag<0>());
-            if (kk + 1 < D + 2) step(uniform_int(kk + 1), IntTag<1>());
+            step(uniform_int(kk + 1), IntTag<1>());
         }
     }
 };
@@ -498,7 +504,6 @@ template <int RH_> struct Bwd1KernelM {
         const int need_gh = p.need_gh;
 
         auto load_plane = [&](State &st, int k) NDC_LAMBDA {
-            if (!st.ln.active) return;
             const bool live = k < D;
             const unsigned ko = (unsigned)clampi(k, 0, D - 1) * plane2;
             NDC_UNROLL
@@ -599,17 +604,17 @@ template <int RH_> struct Bwd1KernelM {
             for (int n = 0; n < NXS; ++n) {
                 const int j = st.ln.strip + n * S, row = r0 - PH + j;
                 if (j < RXS) st.xok |= 1u << n;
-                st.xoff[n] = j < RXS && row >= 0 && row < H ? (unsigned)(row * W + st.ln.c0) * 2u : kNoAccess;
+                st.xoff[n] = st.ln.active && j < RXS && row >= 0 && row < H ? (unsigned)(row * W + st.ln.c0) * 2u : kNoAccess;
                 st.px[n] = st.pt[n] = 0u;
             }
             NDC_UNROLL
             for (int r = 0; r < RH; ++r) {
                 const int row = r0 + st.ln.strip * RH + r;
-                st.ooff[r] = row < H ? (unsigned)(row * W + st.ln.c0) * 2u : kNoAccess;
+                st.ooff[r] = st.ln.active && row < H ? (unsigned)(row * W + st.ln.c0) * 2u : kNoAccess;
             }
             {
                 const int hrow = r0 - PH + halo_row(st.ln.strip, PH, TH);
-                st.hoff = hrow >= 0 && hrow < H ? (unsigned)(hrow * W + st.ln.c0) * 2u : kNoAccess;
+                st.hoff = st.ln.active && hrow >= 0 && hrow < H ? (unsigned)(hrow * W + st.ln.c0) * 2u : kNoAccess;
                 NDC_UNROLL
                 for (int i = 0; i < SC; ++i)
                     NDC_UNROLL
@@ -637,7 +642,7 @@ template <int RH_> struct Bwd1KernelM {
             ex.wait_loads();
             for (int i = tid; i < total; i += nthreads) ex.st_(i, 0.f);
             load_plane(st, 0);
-            if (st.ln.active) prefetch_g(st, 0, IntTag<0>());
+            prefetch_g(st, 0, IntTag<0>());
         });
         ex.sync();
 
@@ -661,9 +666,13 @@ template <int RH_> struct Bwd1KernelM {
             ex.sync();
 
             ex.each([&](State &st, int) NDC_LAMBDA {
-                if (!st.ln.active) return;
+            // (every lane issues every fetch, lanes outside the tile with offsets outside the
+            // slices: a fetch under a condition gives the compiler a path without it, on which
+            // it cannot count the outstanding loads, and then every use of a prefetched
+            // register waits for ALL loads)
                 load_plane(st, k + 1);
                 prefetch_g(st, k + 1, IntTag<1 - PAR>());
+                if (!st.ln.active) return;
                 if (live1) {
                     // LDS reads run ahead of the matrix instructions that use them (two
                     // wavefronts per SIMD do not hide their latency): the K-type rows two
@@ -763,7 +772,7 @@ template <int RH_> struct Bwd1KernelM {
                 const int pf = k - 2;
                 NDC_UNROLL
                 for (int r = 0; r < RH; ++r) {
-                    if (pf >= 0) {   // rows outside the image: the stores go nowhere
+                    if (pf >= 0 && pf < D) {   // rows outside the image: the stores go nowhere
                         buf_st<true>(gxb_, st.ooff[r], (unsigned)pf * plane2,
                                      pack_bf16x2(st.accx[r][0][0], st.accx[r][1][0]));
                         buf_st(gtb_, st.ooff[r], (unsigned)pf * plane2,
@@ -778,9 +787,10 @@ template <int RH_> struct Bwd1KernelM {
             });
             ex.sync();
         };
+        // (an even number of steps, see FwdKernelM)
         for (int kk = 0; kk < D + 2; kk += 2) {
             step(uniform_int(kk), IntTag<0>());
-            if (kk + 1 < D + 2) step(uniform_int(kk + 1), IntTag<1>());
+            step(uniform_int(kk + 1), IntTag<1>());
         }
 
         if (need_gh) {
@@ -875,7 +885,6 @@ template <int RH_> struct Bwd2KernelM {
         const int relu = p.relu;
 
         auto load_plane = [&](State &st, int k) NDC_LAMBDA {
-            if (!st.ln.active) return;
             const bool live = k < D;
             const unsigned ko = (unsigned)clampi(k, 0, D - 1) * plane2;
             NDC_UNROLL
@@ -921,13 +930,13 @@ template <int RH_> struct Bwd2KernelM {
             for (int n = 0; n < NXS; ++n) {
                 const int j = st.ln.strip + n * S, row = r0 - PH + j;
                 if (j < RXS) st.xok |= 1u << n;
-                st.xoff[n] = j < RXS && row >= 0 && row < H ? (unsigned)(row * W + st.ln.c0) * 2u : kNoAccess;
+                st.xoff[n] = st.ln.active && j < RXS && row >= 0 && row < H ? (unsigned)(row * W + st.ln.c0) * 2u : kNoAccess;
                 st.pg[n] = 0u;
             }
             NDC_UNROLL
             for (int r = 0; r < RH; ++r) {
                 const int row = r0 + st.ln.strip * RH + r;
-                st.ooff[r] = row < H ? (unsigned)(row * W + st.ln.c0) * 2u : kNoAccess;
+                st.ooff[r] = st.ln.active && row < H ? (unsigned)(row * W + st.ln.c0) * 2u : kNoAccess;
                 st.okf[r] = row < H ? 1.f : 0.f;
                 NDC_UNROLL
                 for (int i = 0; i < SC; ++i) {
@@ -959,8 +968,11 @@ template <int RH_> struct Bwd2KernelM {
         // one plane step; PAR = k % 2, known at compile time (the loop below is unrolled twice)
         auto compute = [&](State &st, int k, auto par_tag) NDC_LAMBDA {
                 constexpr int PAR = decltype(par_tag)::value;
-                if (!st.ln.active) return;
                 const int j0 = k - 1;
+                // (every lane issues every fetch, lanes outside the tile with offsets outside the
+                // slices: a fetch under a condition gives the compiler a path without it, on which
+                // it cannot count the outstanding loads, and then every use of a prefetched
+                // register waits for ALL loads)
                 load_plane(st, k + 1);
                 // plane k's z, gout, n/d words, consumed by the next step
                 {
@@ -974,6 +986,7 @@ template <int RH_> struct Bwd2KernelM {
                             st.qr[PAR][i][r] = buf_ld<true>(rb_, st.ooff[r], jn + i * cplane2);
                         }
                 }
+                if (!st.ln.active) return;
                 const int lc = st.ln.c0 / 2;
                 if (j0 >= 0 && j0 < D) {
                     // A(gt1) of plane j0: windows of plane j0 + 1 - td, read a tap plane ahead
@@ -1079,7 +1092,7 @@ template <int RH_> struct Bwd2KernelM {
                 ex.sync();
                 ex.each([&](State &st, int) NDC_LAMBDA { compute(st, k, IntTag<0>()); });
             }
-            if (kk + 1 < D + 2) {
+            {   // (an even number of steps, see FwdKernelM)
                 const int k = uniform_int(kk + 1);
                 ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k); });
                 ex.sync();
