@@ -647,17 +647,19 @@ template <int RH_> struct Bwd1KernelM {
         ex.sync();
 
         // Two barriers per plane step.  Phase 1 of step k stages plane k of x / t1 (fetched
-        // during the step before) and publishes gn / gd of plane k - 1; phase 2 fetches the
-        // next planes and does all tap sums of plane k - 1.
+        // during the step before), fetches the next, and publishes gn / gd of plane k - 1;
+        // phase 2 fetches gout, s/d, n/d of plane k + 1 and does all tap sums of plane k - 1.
         // one plane step; PAR = k % 2, known at compile time (the loop below is unrolled twice)
         auto step = [&](int k, auto par_tag) NDC_LAMBDA {
             constexpr int PAR = decltype(par_tag)::value;
             const int j1 = k - 1;
             const bool live1 = j1 >= 0 && j1 < D;
             ex.each([&](State &st, int) NDC_LAMBDA {
-                if (!st.ln.active) return;
-                store_plane(st, k);
-                if (!live1) return;
+                if (st.ln.active) store_plane(st, k);
+                // (x and t1 are fetched again as soon as consumed: they are needed at the start
+                // of the next step; every lane issues every fetch, see below)
+                load_plane(st, k + 1);
+                if (!st.ln.active || !live1) return;
                 NDC_UNROLL
                 for (int r = 0; r < RH; ++r)
                     publish_row(st, IntTag<1 - PAR>(), r, PH + st.ln.strip * RH + r, st.ln.strip * RH + r);
@@ -666,11 +668,10 @@ template <int RH_> struct Bwd1KernelM {
             ex.sync();
 
             ex.each([&](State &st, int) NDC_LAMBDA {
-            // (every lane issues every fetch, lanes outside the tile with offsets outside the
-            // slices: a fetch under a condition gives the compiler a path without it, on which
-            // it cannot count the outstanding loads, and then every use of a prefetched
-            // register waits for ALL loads)
-                load_plane(st, k + 1);
+                // (every lane issues every fetch, lanes outside the tile with offsets outside
+                // the slices: a fetch under a condition gives the compiler a path without it, on
+                // which it cannot count the outstanding loads, and then every use of a
+                // prefetched register waits for ALL loads)
                 prefetch_g(st, k + 1, IntTag<1 - PAR>());
                 if (!st.ln.active) return;
                 if (live1) {
