@@ -108,7 +108,7 @@ int ndc_forward(const ndc_geom *g, const void *x, const void *z, const float *h,
                 void *workspace, size_t workspace_bytes, void *stream);
 
 /* Size of the device array behind ndc_forward_noalloc: room for the packed filter tables of
- * 1506 depthwise channels (696 bytes per channel). */
+ * 824 depthwise channels (1272 bytes per channel). */
 #define NDC_NOALLOC_SCRATCH_BYTES (1u << 20)
 
 /*
@@ -128,7 +128,7 @@ int ndc_forward_noalloc(const ndc_geom *g, const void *x, const void *z, const f
 
 /*
  * Prepared filter tables.  Some kernel families read the filter from a packed table instead
- * of `h` (today: the bfloat16 3x3x3 kernels, 696 bytes per channel).  ndc_forward and
+ * of `h` (today: the bfloat16 3x3x3 kernels, 1272 bytes per channel).  ndc_forward and
  * ndc_backward pack it into their workspace on every call; a caller that runs several calls
  * with one filter (forward and backward of one step, several iterations of one layer) can
  * pack it once with ndc_prepare_taps and hand it to ndc_forward_taps / ndc_backward_taps,

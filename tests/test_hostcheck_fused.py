@@ -286,7 +286,7 @@ def test_prepared_taps_give_the_same_results(dtype):
     out0, t0, saved0 = ops.update_forward(lib, x, z, h, bias, save_ratio=True, **kw)
     if taps is None:
         return
-    assert taps.numel() == lib.taps_bytes(ops.make_geom_for(x, h, C, 1, sc, 0.0, True)) >= C * 696
+    assert taps.numel() == lib.taps_bytes(ops.make_geom_for(x, h, C, 1, sc, 0.0, True)) >= C * 1272
     out1, t1, saved1 = ops.update_forward(lib, x, z, h, bias, save_ratio=True, taps=taps, **kw)
     assert torch.equal(out0, out1) and torch.equal(t0, t1)
     assert torch.equal(saved0[0], saved1[0]) and torch.equal(saved0[1], saved1[1])

@@ -48,7 +48,7 @@ def test_noalloc_forward_matches_forward_twice_in_a_row(dtype):
 
 def test_noalloc_forward_refuses_what_does_not_fit():
     lib = _lib.get_library()
-    C = 2304   # 2304 channels x 696 bytes of packed taps > 1 MiB
+    C = 2304   # 2304 channels x 1272 bytes of packed taps > 1 MiB
     g = _lib.make_geom(1, C, 1, 4, (2, 2, 2), (3, 3, 3), _lib.NDC_BF16, True, 1e-16)
     assert lib.forward_workspace_bytes(g) > SCRATCH_BYTES
     x = torch.zeros(1, C, 2, 2, 2, dtype=torch.bfloat16, device="cuda")
