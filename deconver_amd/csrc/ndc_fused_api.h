@@ -161,8 +161,11 @@ static inline bool make_plan_for(const KGeom &q, Plan &pl, bool pairs_ok, int dt
                 pl.lds_f = lf;
                 pl.lds_b1 = l1;
                 pl.lds_b2 = l2;
+                // (pass 1 only where two of its workgroups fit a CU: with 128 columns its LDS
+                // need leaves room for one, and the dot2 kernel is faster, 2.73 against 2.96 ms
+                // at 64 channels of 128^3)
                 pl.mfma1 = tn.mfma && Bwd1KernelM<kDot2RH>::covers(pl.m.W) &&
-                           Bwd1KernelM<kDot2RH>::lds_floats(tb) <= cap2;
+                           Bwd1KernelM<kDot2RH>::lds_floats(tb) <= cap2 / 2;
                 pl.mfmaf = tn.mfma && FwdKernelM<kDot2RH>::covers(pl.m.W) &&
                            FwdKernelM<kDot2RH>::lds_floats(tf) <= cap2;
                 pl.mfma2 = tn.mfma && Bwd2KernelM<kDot2RH>::covers(pl.m.W) &&

@@ -848,7 +848,9 @@ template <int RH_> struct Bwd2KernelM {
         uint32_t qz[2][SC][RH], qg[2][SC][RH], qr[2][SC][RH];
     };
 
-    static NDC_HD bool covers(int W) { return W % 8 == 0 && W <= 128 && 64 % (W / 2) == 0; }
+    // (below 32 columns the dot2 kernel is the faster one: measured 0.095 against 0.134 ms at
+    // 512 channels of 16^3)
+    static NDC_HD bool covers(int W) { return W % 8 == 0 && W >= 32 && W <= 128 && 64 % (W / 2) == 0; }
     static NDC_HD int pitch_xs(int W) { return W / 2 + 4; }   // one zero word past the row, rows 16-byte aligned
     static NDC_HD int stride_xs(int TH, int W) { return stride16((TH + 2) * pitch_xs(W)); }
     static NDC_HD int stride_sc(int TH, int W) { return stride16(TH * (W / 2)); }

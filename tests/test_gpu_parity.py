@@ -40,6 +40,11 @@ FUSED_GEOMS = [
     # widest row of the bf16 dot2 kernels (512 threads, > 64 KiB of LDS); in float32 the
     # column-pair kernels' LDS does not fit and the plan falls back to the one-column ones
     (4, 4, 4, (3, 3, 3), (6, 10, 256), 1),
+    # widths the bf16 matrix-instruction kernels cover (multiples of 8 that divide 128): the
+    # widest, one with several rows per wavefront, one below the width from which pass 2 uses them
+    (4, 4, 4, (3, 3, 3), (6, 12, 128), 1),
+    (8, 8, 4, (3, 3, 3), (7, 9, 32), 2),
+    (8, 8, 4, (3, 3, 3), (5, 6, 16), 2),
 ]
 
 

@@ -140,6 +140,8 @@ FULL_WG_GEOMS = [
     (2, 4, (3, 3, 3), (2, 32, 32), 1),    # 16 lanes per row, 16 strips
     (1, 4, (3, 3, 3), (4, 9, 128), 2),    # 64 lanes per row, 4 strips, ragged band
     (1, 4, (3, 3, 3), (5, 40, 64), 1),    # several row bands
+    (2, 4, (3, 3, 3), (4, 7, 16), 1),     # 8 lanes per row: bf16 matrix-instruction forward and pass 1, dot2 pass 2
+    (1, 4, (3, 3, 3), (3, 5, 8), 2),      # 4 lanes per row: one block of the matrix instruction per row
 ]
 
 
