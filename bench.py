@@ -12,9 +12,9 @@
 One step = one forward + one backward (input-, source-, filter- and bias-gradient) of the
 update node on config 3 of the baseline: batch 2, 128 depthwise channels, 64^3 voxels,
 3x3x3 filter, ratio 4, bfloat16 storage with float32 accumulation; inputs resident in HBM.
-Prints ONE JSON line: whole-step throughput in Gvoxel/s, a ``vector_ceiling`` object (bf16:
-time the kernels' v_dot2c_f32_bf16 alone would take at the measured issue rate, over the
-measured time), plus a ``roofline`` object for the
+Prints ONE JSON line: whole-step throughput in Gvoxel/s, a ``matrix_ceiling`` object (bf16:
+time the kernels' 4x4x4 matrix instructions alone would take at the measured issue rate, over
+the measured time), plus a ``roofline`` object for the
 slowest kernel (device time from events on the launch stream, algorithmic bytes as stated
 below) and a ``cpu_baseline`` object (the oracle timed on the host cores on a bounded
 sample of the same workload).
@@ -354,7 +354,13 @@ def grid_workload(args) -> int:
     return 0
 
 
+# Config 3's bf16 kernels issue v_mfma_f32_4x4x4_16b_bf16 (16 blocks of 4 lanes; one
+# instruction covers 64 channel-voxel columns of a K- or A-type tap pair, or 64 positions of a
+# filter-gradient tap row): instructions per 64 channel-voxels, and what the same sums took
+# as v_dot2c_f32_bf16 per channel-voxel in the kernels they replace.
+MFMA_PER_64_CHANNEL_VOXELS = {"forward": 27, "backward_pass1": 36, "backward_pass2": 18}
 DOT2_PER_CHANNEL_VOXEL = {"forward": 181, "backward_pass1": 216, "backward_pass2": 126}
+CLOCKS_PER_MFMA = 9.85    # per SIMD, measured by `--workload valu` (2 passes of 4 clocks + issue)
 CLOCKS_PER_DOT2C = 4.52   # per SIMD, four wavefronts resident: measured by `--workload valu`
 
 
@@ -400,6 +406,10 @@ def valu_workload(args) -> int:
     ceiling = lanes * 2 / dot2 * hz   # two multiply-accumulates per lane per instruction
     U = 2 * 128 * 64 ** 3
     least_ms = {k: U * n / lanes * dot2 / hz * 1e3 for k, n in DOT2_PER_CHANNEL_VOXEL.items()}
+    mfma = clk.get(("v_mfma_f32_4x4x4_16b_bf16", 2))
+    least_mfma = None if mfma is None else {
+        k: U / 64 * n / (probe["compute_units"] * 4) * mfma / hz * 1e3
+        for k, n in MFMA_PER_64_CHANNEL_VOXELS.items()}
     print(json.dumps({
         "metric": "vector multiply-accumulate ceiling (v_dot2c_f32_bf16 issue rate)",
         "value": ceiling / 1e12, "unit": "TMAC/s", "n_gpus": 1, "steps": 1, "warmup": 0,
@@ -411,6 +421,10 @@ def valu_workload(args) -> int:
         "fmac_vector_operands_TMACs": lanes / clk[("v_fmac_f32 (vector operands)", 4)] * hz / 1e12,
         "config3_dot2c_per_channel_voxel": DOT2_PER_CHANNEL_VOXEL,
         "config3_least_ms_for_dot2c_alone": least_ms,
+        "clocks_per_mfma_4x4x4_bf16": mfma,
+        "mfma_TMACs": None if mfma is None else probe["compute_units"] * 4 * 1024 / mfma * hz / 1e12,
+        "config3_mfma_per_64_channel_voxels": MFMA_PER_64_CHANNEL_VOXELS,
+        "config3_least_ms_for_mfma_alone": least_mfma,
         "probe": probe, "roofline": None, "cpu_baseline": None}))
     return 0
 
@@ -730,6 +744,11 @@ def main() -> int:
         "traffic_measured_at_commit": traffic_at,
         "algorithmic_bytes": alg[dominant],
         "avg_launch_ms": k_ms[dominant],
+        # the three kernels side by side (two of them are within a few percent of each other,
+        # so which one is "dominant" can differ from run to run)
+        "per_kernel": {k: {"algorithmic_bytes": alg[k], "avg_launch_ms": k_ms[k],
+                           "achieved": alg[k] / (k_ms[k] * 1e-3) / 1e9,
+                           "frac": alg[k] / (k_ms[k] * 1e-3) / 1e9 / HBM_PEAK_GBS} for k in alg},
     }
     step_bytes = 23 * U * esz
     result = {
@@ -762,14 +781,15 @@ def main() -> int:
         "roofline": roofline,
     }
     if dtype == torch.bfloat16 and keep:
-        # the path is bound by vector issue, not by HBM: the least time the kernels'
-        # v_dot2c_f32_bf16 alone take, at the issue rate `--workload valu` measured
+        # how far the kernels are from their matrix-instruction floor: the least time their
+        # v_mfma_f32_4x4x4_16b_bf16 alone take at the issue rate `--workload valu` measured
+        # (the kernels are bound by HBM and by staging work, not by these)
         props = torch.cuda.get_device_properties(dev)
-        lanes = props.multi_processor_count * 4 * 64
+        simds = props.multi_processor_count * 4
         hz = getattr(props, "clock_rate", 2400000) * 1e3   # kHz; MI355X peak engine clock 2.4 GHz
-        least = {k: U * n / lanes * CLOCKS_PER_DOT2C / hz * 1e3 for k, n in DOT2_PER_CHANNEL_VOXEL.items()}
-        result["vector_ceiling"] = {
-            "dot2c_per_channel_voxel": DOT2_PER_CHANNEL_VOXEL, "clocks_per_dot2c": CLOCKS_PER_DOT2C,
+        least = {k: U / 64 * n / simds * CLOCKS_PER_MFMA / hz * 1e3 for k, n in MFMA_PER_64_CHANNEL_VOXELS.items()}
+        result["matrix_ceiling"] = {
+            "mfma_per_64_channel_voxels": MFMA_PER_64_CHANNEL_VOXELS, "clocks_per_mfma": CLOCKS_PER_MFMA,
             "least_ms": least,
             "frac": {k: least[k] / k_ms[k] for k in least},
             "step_frac": sum(least.values()) / sum(k_ms[k] for k in least),

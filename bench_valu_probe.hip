@@ -77,6 +77,61 @@ template <int OP> __global__ void __launch_bounds__(256) probe(float *out, const
     out[blockIdx.x * blockDim.x + threadIdx.x] = t;
 }
 
+// The 4x4x4 bf16 matrix instruction (1024 multiply-accumulates per wavefront instruction) alone
+// and beside float32 FMAs, and LDS reads / writes of 4, 8 and 16 bytes per lane (dense,
+// conflict-free addresses) with all four SIMDs of a CU issuing them: 4 x 8 instructions of the
+// probed form per loop iteration.
+enum Op2 { MFMA, MFMA_FMA1, MFMA_FMA2, LDS_R32, LDS_R64, LDS_R128, LDS_W32, LDS_W64, LDS_W128 };
+typedef short probe_s4 __attribute__((ext_vector_type(4)));
+typedef float probe_f4 __attribute__((ext_vector_type(4)));
+typedef unsigned probe_u4 __attribute__((ext_vector_type(4)));
+typedef unsigned probe_u2 __attribute__((ext_vector_type(2)));
+
+template <int OP> __global__ void __launch_bounds__(256) probe2(float *out, const unsigned *w, int iters)
+{
+    __shared__ unsigned lds[256 * 4];
+    for (int i = 0; i < 4; ++i) lds[threadIdx.x * 4 + i] = threadIdx.x;
+    __syncthreads();
+    probe_f4 acc[8];
+    for (int i = 0; i < 8; ++i) acc[i] = probe_f4{0.f, 1.f, 2.f, (float)i};
+    probe_s4 a[4], b[4];
+    for (int i = 0; i < 4; ++i) {
+        a[i] = probe_s4{(short)w[i], (short)(w[i] + 1), (short)threadIdx.x, 3};
+        b[i] = probe_s4{(short)w[i + 4], (short)(w[i] + 1), (short)threadIdx.x, 3};
+    }
+    float va[8];
+    for (int i = 0; i < 8; ++i) va[i] = threadIdx.x + i;
+    const float x = threadIdx.x * 1.5f + 1.f;
+    const unsigned t = threadIdx.x;
+    probe_u4 v4 = {t, t, t, t};
+    probe_u2 v2 = {t, t};
+    unsigned v1 = t;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                if (OP <= MFMA_FMA2)
+                    asm volatile("v_mfma_f32_4x4x4_16b_bf16 %0, %1, %2, %0" : "+v"(acc[i]) : "v"(a[(r + i) & 3]), "v"(b[(r + i) & 3]));
+                if (OP == MFMA_FMA1 || OP == MFMA_FMA2)
+                    asm volatile("v_fmac_f32 %0, %1, %2" : "+v"(va[i]) : "v"(x), "v"(x));
+                if (OP == MFMA_FMA2)
+                    asm volatile("v_fmac_f32 %0, %1, %2" : "+v"(va[(i + 3) & 7]) : "v"(x), "v"(x));
+                if (OP == LDS_R32) asm volatile("ds_read_b32 %0, %1" : "=v"(v1) : "v"(t * 4));
+                if (OP == LDS_R64) asm volatile("ds_read_b64 %0, %1" : "=v"(v2) : "v"(t * 8));
+                if (OP == LDS_R128) asm volatile("ds_read_b128 %0, %1" : "=v"(v4) : "v"(t * 16));
+                if (OP == LDS_W32) asm volatile("ds_write_b32 %0, %1" : : "v"(t * 4), "v"(v1));
+                if (OP == LDS_W64) asm volatile("ds_write_b64 %0, %1" : : "v"(t * 8), "v"(v2));
+                if (OP == LDS_W128) asm volatile("ds_write_b128 %0, %1" : : "v"(t * 16), "v"(v4));
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)");
+        }
+    }
+    float s = (float)(v4[0] + v4[3] + v2[0] + v2[1] + v1);
+    for (int i = 0; i < 8; ++i) s += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3] + va[i];
+    out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
 struct Bench {
     float *out;
     unsigned *w;
@@ -105,6 +160,27 @@ struct Bench {
         std::printf("%s\n    {\"op\": \"%s\", \"wavefronts_per_simd\": %d, \"ms\": %.4f, \"clocks_per_instruction\": %.3f}",
                     first ? "" : ",", name, wg_per_cu, ms, ms * 1e-3 * ghz * 1e9 / per_simd);
         first = false;
+    }
+
+    template <int OP> void run2(const char *name, int wg_per_cu)
+    {
+        const int iters = 1000, nblk = cus * wg_per_cu;
+        hipEvent_t a, b;
+        (void)hipEventCreate(&a);
+        (void)hipEventCreate(&b);
+        probe2<OP><<<nblk, 256>>>(out, w, 10);
+        (void)hipDeviceSynchronize();
+        (void)hipEventRecord(a);
+        probe2<OP><<<nblk, 256>>>(out, w, iters);
+        (void)hipEventRecord(b);
+        (void)hipEventSynchronize(b);
+        float ms = 0.f;
+        (void)hipEventElapsedTime(&ms, a, b);
+        (void)hipEventDestroy(a);
+        (void)hipEventDestroy(b);
+        const double per_simd = (double)wg_per_cu * iters * 4 * 8;
+        std::printf(",\n    {\"op\": \"%s\", \"wavefronts_per_simd\": %d, \"ms\": %.4f, \"clocks_per_instruction\": %.3f}",
+                    name, wg_per_cu, ms, ms * 1e-3 * ghz * 1e9 / per_simd);
     }
 };
 
@@ -146,6 +222,17 @@ int main()
         b.run<MIX_LDS>("dot2c stream + ds_read_b32 per 4 (clocks per dot2c)", wg);
         b.run<MIX_READLANE>("dot2c stream + v_readlane_b32 per 4 (clocks per dot2c)", wg);
     }
+    for (int wg = 2; wg <= 4; wg *= 2) {
+        b.run2<MFMA>("v_mfma_f32_4x4x4_16b_bf16", wg);
+        b.run2<MFMA_FMA1>("v_mfma_f32_4x4x4_16b_bf16 + 1 v_fmac_f32 (clocks per pair)", wg);
+        b.run2<MFMA_FMA2>("v_mfma_f32_4x4x4_16b_bf16 + 2 v_fmac_f32 (clocks per triple)", wg);
+    }
+    b.run2<LDS_R32>("ds_read_b32", 4);
+    b.run2<LDS_R64>("ds_read_b64", 4);
+    b.run2<LDS_R128>("ds_read_b128", 4);
+    b.run2<LDS_W32>("ds_write_b32", 4);
+    b.run2<LDS_W64>("ds_write_b64", 4);
+    b.run2<LDS_W128>("ds_write_b128", 4);
     std::printf("\n]}\n");
     (void)hipDeviceSynchronize();
     (void)hipFree(b.out);
