@@ -12,9 +12,11 @@
 One step = one forward + one backward (input-, source-, filter- and bias-gradient) of the
 update node on config 3 of the baseline: batch 2, 128 depthwise channels, 64^3 voxels,
 3x3x3 filter, ratio 4, bfloat16 storage with float32 accumulation; inputs resident in HBM.
-Prints ONE JSON line: whole-step throughput in Gvoxel/s, a ``matrix_ceiling`` object (bf16:
-time the kernels' 4x4x4 matrix instructions alone would take at the measured issue rate, over
-the measured time), plus a ``roofline`` object for the
+Prints ONE JSON line: whole-step throughput in Gvoxel/s, a ``vector_ceiling`` object (bf16:
+time the kernels' v_dot2c_f32_bf16 alone would take at the measured issue rate, over the
+measured time), a ``matrix_instruction_variant`` object (the same step with the library's other
+kernel family switched on, `ndc_matrix_kernels(1)`: outside the specified path, not `value`),
+plus a ``roofline`` object for the
 slowest kernel (device time from events on the launch stream, algorithmic bytes as stated
 below) and a ``cpu_baseline`` object (the oracle timed on the host cores on a bounded
 sample of the same workload).
@@ -360,7 +362,7 @@ def grid_workload(args) -> int:
 # as v_dot2c_f32_bf16 per channel-voxel in the kernels they replace.
 MFMA_PER_64_CHANNEL_VOXELS = {"forward": 27, "backward_pass1": 36, "backward_pass2": 18}
 DOT2_PER_CHANNEL_VOXEL = {"forward": 181, "backward_pass1": 216, "backward_pass2": 126}
-CLOCKS_PER_MFMA = 9.85    # per SIMD, measured by `--workload valu` (2 passes of 4 clocks + issue)
+CLOCKS_PER_MFMA = 9.11    # per SIMD, two wavefronts resident (as the kernels run): measured by `--workload valu`
 CLOCKS_PER_DOT2C = 4.52   # per SIMD, four wavefronts resident: measured by `--workload valu`
 
 
@@ -600,6 +602,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--dtype", choices=("bf16", "fp32"), default="bf16")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--matrix", action="store_true",
+                    help="run with the matrix-instruction kernel family on (ndc_matrix_kernels(1)): "
+                         "not the specified path, reported for comparison")
     ap.add_argument("--no-train", action="store_true",
                     help="skip the Deconver-3D train-step leg that follows the timed region")
     ap.add_argument("--recompute", action="store_true",
@@ -620,6 +625,8 @@ def main() -> int:
         print("bench.py measures the one-GPU hot path only: this build has no multi-GPU code "
               "path (every box has one GPU); run with --gpus 1", file=sys.stderr)
         return 2
+    if args.matrix:
+        os.environ["DECONVER_NDC_MATRIX"] = "1"   # read when the library is loaded
 
     if args.workload == "sweep":
         return sweep_workload(args)
@@ -642,6 +649,7 @@ def main() -> int:
         print("bench.py needs a GPU (the NDC update has no CPU path)", file=sys.stderr)
         return 2
     lib = _lib.get_library()
+    lib.matrix_kernels(bool(args.matrix))
     dev = torch.device("cuda:0")
     dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float32
     esz = 2 if dtype == torch.bfloat16 else 4
@@ -693,27 +701,31 @@ def main() -> int:
 
     # per-kernel device time: events on the stream the library launches on
     n_probe = max(3, min(10, args.steps))
-    fwd_ms, pass_ms = [], []
-    for _ in range(n_probe):
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        # an untimed call first: the previous iteration ended in a host synchronisation, and
-        # the first kernel after an idle gap runs at ramping clocks
-        ops.update_forward(lib, x, z, h, bias, save_ratio=keep, **kw)
-        e0.record()
-        res = ops.update_forward(lib, x, z, h, bias, save_ratio=keep, **kw)
-        e1.record()
-        pt = []
-        ops.update_backward(lib, x, z, res[1], h, bias, g, pass_times=pt,
-                            saved=res[2] if keep else None, **kw)
-        torch.cuda.synchronize()
-        fwd_ms.append(e0.elapsed_time(e1))
-        pass_ms.append(pt)
-    k_ms = {
-        "forward": statistics.mean(fwd_ms),
-        "backward_pass1": statistics.mean(p[0] for p in pass_ms),
-        "backward_pass2": statistics.mean(p[1] for p in pass_ms),
-        "backward_reduce": statistics.mean(p[2] for p in pass_ms),
-    }
+
+    def kernel_times():
+        fwd_ms, pass_ms = [], []
+        for _ in range(n_probe):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            # an untimed call first: the previous iteration ended in a host synchronisation, and
+            # the first kernel after an idle gap runs at ramping clocks
+            ops.update_forward(lib, x, z, h, bias, save_ratio=keep, **kw)
+            e0.record()
+            res = ops.update_forward(lib, x, z, h, bias, save_ratio=keep, **kw)
+            e1.record()
+            pt = []
+            ops.update_backward(lib, x, z, res[1], h, bias, g, pass_times=pt,
+                                saved=res[2] if keep else None, **kw)
+            torch.cuda.synchronize()
+            fwd_ms.append(e0.elapsed_time(e1))
+            pass_ms.append(pt)
+        return {
+            "forward": statistics.mean(fwd_ms),
+            "backward_pass1": statistics.mean(p[0] for p in pass_ms),
+            "backward_pass2": statistics.mean(p[1] for p in pass_ms),
+            "backward_reduce": statistics.mean(p[2] for p in pass_ms),
+        }
+
+    k_ms = kernel_times()
 
     sp = w["spatial"]
     vox = w["batch"] * sp[0] * sp[1] * sp[2]
@@ -780,16 +792,45 @@ def main() -> int:
         "backward_reads_forward_ratio": bool(keep),
         "roofline": roofline,
     }
-    if dtype == torch.bfloat16 and keep:
-        # how far the kernels are from their matrix-instruction floor: the least time their
-        # v_mfma_f32_4x4x4_16b_bf16 alone take at the issue rate `--workload valu` measured
-        # (the kernels are bound by HBM and by staging work, not by these)
+    if dtype == torch.bfloat16 and keep and not args.matrix:
+        # The same step on the OTHER kernel family (ndc_matrix_kernels(1): tap sums on the
+        # 4x4x4 matrix instruction).  The path is specified without matrix instructions, so this
+        # is not `value`; it is reported because it is the faster form on this GPU.
+        lib.matrix_kernels(True)
+        try:
+            for _ in range(args.warmup):
+                step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                step()
+            torch.cuda.synchronize()
+            m_ms = (time.perf_counter() - t0) / args.steps * 1e3
+            mk = kernel_times()
+        finally:
+            lib.matrix_kernels(False)
         props = torch.cuda.get_device_properties(dev)
         simds = props.multi_processor_count * 4
         hz = getattr(props, "clock_rate", 2400000) * 1e3   # kHz; MI355X peak engine clock 2.4 GHz
         least = {k: U / 64 * n / simds * CLOCKS_PER_MFMA / hz * 1e3 for k, n in MFMA_PER_64_CHANNEL_VOXELS.items()}
-        result["matrix_ceiling"] = {
+        result["matrix_instruction_variant"] = {
+            "ms_per_step": m_ms, "value": vox / (m_ms * 1e-3) / 1e9, "unit": "Gvoxel/s",
+            "step_hbm_frac": step_bytes / (m_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "kernel_ms": mk,
+            "hbm_frac": {k: alg[k] / (mk[k] * 1e-3) / 1e9 / HBM_PEAK_GBS for k in alg},
+            # the least time its matrix instructions alone take at the measured issue rate
             "mfma_per_64_channel_voxels": MFMA_PER_64_CHANNEL_VOXELS, "clocks_per_mfma": CLOCKS_PER_MFMA,
+            "mfma_least_ms": least,
+        }
+    if dtype == torch.bfloat16 and keep and not args.matrix:
+        # the default kernels are bound by vector issue, not by HBM: the least time their
+        # v_dot2c_f32_bf16 alone take, at the issue rate `--workload valu` measured
+        props = torch.cuda.get_device_properties(dev)
+        lanes = props.multi_processor_count * 4 * 64
+        hz = getattr(props, "clock_rate", 2400000) * 1e3
+        least = {k: U * n / lanes * CLOCKS_PER_DOT2C / hz * 1e3 for k, n in DOT2_PER_CHANNEL_VOXEL.items()}
+        result["vector_ceiling"] = {
+            "dot2c_per_channel_voxel": DOT2_PER_CHANNEL_VOXEL, "clocks_per_dot2c": CLOCKS_PER_DOT2C,
             "least_ms": least,
             "frac": {k: least[k] / k_ms[k] for k in least},
             "step_frac": sum(least.values()) / sum(k_ms[k] for k in least),
@@ -811,6 +852,14 @@ def main() -> int:
             result["train3d_steps_per_s_pytorch_route"] = t3["pytorch"]["steps_per_s"]
             result["train3d"] = {"workload": MODEL_WORKLOADS["train3d"]["text"], "routes": t3,
                                  "hip_over_pytorch": t3["hip"]["steps_per_s"] / t3["pytorch"]["steps_per_s"]}
+            if not args.matrix:
+                # the same train step with the other kernel family on (see above: not the metric)
+                lib.matrix_kernels(True)
+                try:
+                    tm = run_model_routes("train3d", ["hip"], warmup=2, steps=5)["hip"]
+                finally:
+                    lib.matrix_kernels(False)
+                result["matrix_instruction_variant"]["train3d_steps_per_s"] = tm["steps_per_s"]
         except Exception as exc:   # the headline line above is complete without this leg
             result["train3d_error"] = f"{type(exc).__name__}: {exc}"
     print(json.dumps(result))

@@ -4,7 +4,7 @@
 (one multiplicative update as an autograd node over ``libdeconver_ndc.so``)."""
 
 from . import _lib, ops  # noqa: F401
-from .functional import DeconvUpdate, deconv_update, hip_kernels_apply  # noqa: F401
+from .functional import DeconvUpdate, deconv_update, hip_kernels_apply, matrix_kernels, save_ratio  # noqa: F401
 from .layers import MLP, LayerNorm, Linear  # noqa: F401
 from .model import Deconver, DeconverBlock, DeconverStage, DeconvMixer, Stem  # noqa: F401
 from .ndc import NDC, Deconv, Initializer  # noqa: F401

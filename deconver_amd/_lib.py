@@ -24,6 +24,7 @@ EXPORTS = (
     "ndc_fused_supported",
     "ndc_check_geometry",
     "ndc_backward_uses_saved",
+    "ndc_matrix_kernels",
     "ndc_forward",
     "ndc_forward_workspace_bytes",
     "ndc_forward_noalloc",
@@ -88,6 +89,7 @@ class NdcLibrary:
         d.ndc_fused_supported.argtypes = [gp]
         d.ndc_check_geometry.argtypes = [gp]
         d.ndc_backward_uses_saved.argtypes = [gp]
+        d.ndc_matrix_kernels.argtypes = [ctypes.c_int]
         d.ndc_forward.argtypes = [gp, vp, vp, fp, fp, vp, vp, vp, vp, vp, ctypes.c_size_t, vp]
         if hasattr(d, "ndc_forward_noalloc"):   # HIP build only
             d.ndc_forward_noalloc.argtypes = [gp, vp, vp, fp, fp, vp, vp, vp, vp, vp]
@@ -138,6 +140,11 @@ class NdcLibrary:
 
     def check_geometry(self, g: Geom) -> int:
         return self._cached("check", g, None, lambda: self._dll.ndc_check_geometry(ctypes.byref(g)))
+
+    def matrix_kernels(self, enabled: Optional[bool] = None) -> bool:
+        """Get or set whether the bf16 3x3x3 kernels built on the 4x4x4 matrix instruction may
+        be chosen (off by default)."""
+        return bool(self._dll.ndc_matrix_kernels(-1 if enabled is None else int(bool(enabled))))
 
     def backward_uses_saved(self, g: Geom) -> bool:
         return self._cached("saved", g, None,
@@ -226,4 +233,6 @@ def get_library() -> NdcLibrary:
                         f"{LIB_PATH} is missing: build it with `python -m deconver_amd.build` "
                         "(hipcc, gfx950). The NDC update has no CPU or PyTorch fallback.")
                 _library = NdcLibrary(LIB_PATH)
+                if os.environ.get("DECONVER_NDC_MATRIX", "0") == "1":
+                    _library.matrix_kernels(True)
     return _library

@@ -272,6 +272,12 @@ int ndc_forward_taps(const ndc_geom *g, const void *x, const void *z, const floa
     return forward_impl(g, x, z, h, bias, out, t1, s_over_den, ratio, taps, nullptr, 0, stream);
 }
 
+int ndc_matrix_kernels(int on)
+{
+    if (on >= 0) ndc::fused::matrix_switch() = on ? 1 : 0;
+    return ndc::fused::matrix_switch();
+}
+
 int ndc_backward_uses_saved(const ndc_geom *g)
 {
     using namespace ndc;

@@ -97,6 +97,15 @@ static inline bool find_variant(const KGeom &q, const March &m, bool pairs_ok, V
     return found;
 }
 
+// Whether plans may choose the kernels built on the 4x4x4 matrix instruction
+// (ndc_fused_mfma.h).  Off unless a caller turns it on (ndc_matrix_kernels): the path is
+// specified as a depthwise stencil that keeps matrix instructions out of it.
+static inline int &matrix_switch()
+{
+    static int on = 0;
+    return on;
+}
+
 struct Plan {
     Variant v;
     March m;
@@ -164,11 +173,11 @@ static inline bool make_plan_for(const KGeom &q, Plan &pl, bool pairs_ok, int dt
                 // (pass 1 only where two of its workgroups fit a CU: with 128 columns its LDS
                 // need leaves room for one, and the dot2 kernel is faster, 2.73 against 2.96 ms
                 // at 64 channels of 128^3)
-                pl.mfma1 = tn.mfma && Bwd1KernelM<kDot2RH>::covers(pl.m.W) &&
+                pl.mfma1 = tn.mfma && matrix_switch() && Bwd1KernelM<kDot2RH>::covers(pl.m.W) &&
                            Bwd1KernelM<kDot2RH>::lds_floats(tb) <= cap2 / 2;
-                pl.mfmaf = tn.mfma && FwdKernelM<kDot2RH>::covers(pl.m.W) &&
+                pl.mfmaf = tn.mfma && matrix_switch() && FwdKernelM<kDot2RH>::covers(pl.m.W) &&
                            FwdKernelM<kDot2RH>::lds_floats(tf) <= cap2;
-                pl.mfma2 = tn.mfma && Bwd2KernelM<kDot2RH>::covers(pl.m.W) &&
+                pl.mfma2 = tn.mfma && matrix_switch() && Bwd2KernelM<kDot2RH>::covers(pl.m.W) &&
                            Bwd2KernelM<kDot2RH>::lds_floats(tb) <= cap2;
             }
         }

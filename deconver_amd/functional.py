@@ -20,7 +20,7 @@ from torch import Tensor
 
 from . import _lib, ops
 
-__all__ = ["deconv_update", "hip_kernels_apply", "DeconvUpdate", "save_ratio"]
+__all__ = ["deconv_update", "hip_kernels_apply", "DeconvUpdate", "save_ratio", "matrix_kernels"]
 
 _SAVE_RATIO = os.environ.get("DECONVER_NDC_SAVE_RATIO", "1") != "0"
 
@@ -36,6 +36,14 @@ def save_ratio(enabled: Optional[bool] = None) -> bool:
     if enabled is not None:
         _SAVE_RATIO = bool(enabled)
     return _SAVE_RATIO
+
+
+def matrix_kernels(enabled: Optional[bool] = None) -> bool:
+    """Get or set whether bf16 3x3x3 updates may run on the kernels that use the 4x4x4 matrix
+    instruction (``ndc_matrix_kernels``).  Off by default (environment
+    ``DECONVER_NDC_MATRIX=1`` turns it on when the library is loaded): the path is specified
+    without matrix instructions.  Same results to the bf16 tolerance, less time per step."""
+    return _lib.get_library().matrix_kernels(enabled)
 
 
 def hip_kernels_apply(x: Tensor, m: int, sc: int, kernel_size, dtype=None) -> bool:

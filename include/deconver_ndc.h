@@ -80,6 +80,16 @@ int ndc_check_geometry(const ndc_geom *g);
  * reference. */
 int ndc_backward_uses_saved(const ndc_geom *g);
 
+/* Kernel-family switch, process-wide: on = 1 lets the calls below run the bfloat16 3x3x3
+ * kernels that do their tap sums on the 4x4x4 matrix instruction (row widths 8, 16, 32, 64,
+ * 128), on = 0 keeps them on the vector unit (v_dot2c_f32_bf16), on < 0 only queries; returns
+ * the setting in force.  Default 0: the path is specified as a stencil without matrix
+ * instructions, and the default build measures that; the other family is the faster one on
+ * MI355X (config 3: 1.56 against 1.84 ms per step) and gives the same results to the bf16
+ * tolerance.  Not to be changed while calls are in flight on other threads.  No counterpart
+ * in the reference. */
+int ndc_matrix_kernels(int on);
+
 /* Bytes of scratch `ndc_forward` needs for `g` (0 for most geometries; the bfloat16 3x3x3
  * kernels keep their packed filter tables there).  No counterpart in the reference, whose
  * wrappers allocate their own temporaries (kernels.py:728-788). */

@@ -316,11 +316,14 @@ def test_config1_single_layer_2d_sum_of_squares():
     assert O.rel_err(layer.init.linear.linear.bias.grad.cpu(), b.grad) < 1e-4
 
 
-@pytest.mark.parametrize("dtype,tol", [(torch.bfloat16, 2e-2), (torch.float32, 1e-4)])
-def test_headline_size_channel_slices_match_oracle(dtype, tol):
+@pytest.mark.parametrize("dtype,tol,matrix", [(torch.bfloat16, 2e-2, False), (torch.float32, 1e-4, False),
+                                              (torch.bfloat16, 2e-2, True)])
+def test_headline_size_channel_slices_match_oracle(dtype, tol, matrix):
     """Config 3 at full size (B=2, C=128, 64^3, 3x3x3, ratio 4).  Depthwise channels are
     independent, so any channel slice of the full-size result must equal the oracle run on
-    that slice alone -- which the CPU does in seconds."""
+    that slice alone -- which the CPU does in seconds.  `matrix`: the training form (backward
+    fed with the forward's ratios) on the matrix-instruction kernel family, switched on through
+    the package's own setter."""
     from deconver_amd import _lib, ops
     B, C, sc, sp = 2, 128, 4, (64, 64, 64)
     gen = torch.Generator().manual_seed(0)
@@ -332,9 +335,15 @@ def test_headline_size_channel_slices_match_oracle(dtype, tol):
     lib = _lib.get_library()
     dev = [t.cuda() for t in (x, z, h, bias, gout)]
     kw = dict(groups=C, m=1, sc=sc, eps=1e-16, relu_input=True)
-    out, t1 = ops.update_forward(lib, dev[0], dev[1], dev[2], dev[3], **kw)
-    gx, gz, gh, gb = ops.update_backward(lib, dev[0], dev[1], t1, dev[2], dev[3], dev[4], **kw)
-    torch.cuda.synchronize()
+    assert dc.matrix_kernels(matrix) == matrix
+    try:
+        res = ops.update_forward(lib, dev[0], dev[1], dev[2], dev[3], save_ratio=matrix, **kw)
+        out, t1 = res[0], res[1]
+        gx, gz, gh, gb = ops.update_backward(lib, dev[0], dev[1], t1, dev[2], dev[3], dev[4],
+                                             saved=res[2] if matrix else None, **kw)
+        torch.cuda.synchronize()
+    finally:
+        dc.matrix_kernels(False)
     for c in (0, 77, 127):
         cs = slice(c * sc, (c + 1) * sc)
         xs, zs, hs, bs, gs = (x[:, c:c + 1].double(), z[:, cs].double(), h[c:c + 1].double(),

@@ -59,6 +59,20 @@ def _oracle(x, z, h, bias, gout, G, m, sc, eps, relu):
     return out, t1, grads
 
 
+# (storage type, matrix-instruction kernels on): the bf16 3x3x3 geometries have two kernel
+# families, the default one on the vector unit and the one ndc_matrix_kernels(1) selects
+FAMILIES = [pytest.param(torch.float32, False, id="f32"), pytest.param(torch.bfloat16, False, id="bf16"),
+            pytest.param(torch.bfloat16, True, id="bf16-matrix")]
+
+
+@pytest.fixture
+def matrix_switch():
+    """Sets the library's kernel-family switch for one test and puts it back to off."""
+    lib = _lib.get_library()
+    yield lib.matrix_kernels
+    lib.matrix_kernels(False)
+
+
 def _run_case(geom, dtype, path, relu=True, with_bias=True, saved=False):
     C, G, sc, ks, sp, B = geom
     m = C // G
@@ -99,17 +113,19 @@ def test_direct_kernels(geom, dtype):
 
 
 @pytest.mark.parametrize("geom", FUSED_GEOMS)
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_fused_kernels(geom, dtype):
-    print("case", geom, dtype, flush=True)
+@pytest.mark.parametrize("dtype,matrix", FAMILIES)
+def test_fused_kernels(geom, dtype, matrix, matrix_switch):
+    print("case", geom, dtype, matrix, flush=True)
+    assert matrix_switch(matrix) == matrix
     _run_case(geom, dtype, _lib.PATH_FUSED)
 
 
 @pytest.mark.parametrize("geom", FUSED_GEOMS)
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_fused_kernels_with_saved_ratio(geom, dtype):
+@pytest.mark.parametrize("dtype,matrix", FAMILIES)
+def test_fused_kernels_with_saved_ratio(geom, dtype, matrix, matrix_switch):
     """Backward fed with the forward's denominator and ratio instead of re-gathering them."""
-    print("case saved", geom, dtype, flush=True)
+    print("case saved", geom, dtype, matrix, flush=True)
+    assert matrix_switch(matrix) == matrix
     _run_case(geom, dtype, _lib.PATH_FUSED, saved=True)
 
 
@@ -235,13 +251,15 @@ def test_graph_capture_replays_match_eager(dtype):
             assert torch.equal(a, b), f"replay {replay}: {name}"
 
 
+@pytest.mark.parametrize("matrix", [False, True])
 @pytest.mark.parametrize("geom", [FUSED_GEOMS[2], FUSED_GEOMS[7], (24, 24, 4, (3, 3, 3), (9, 16, 192), 1)])
-def test_prepared_taps_bit_equal_on_gpu(geom):
+def test_prepared_taps_bit_equal_on_gpu(geom, matrix, matrix_switch):
     """ndc_prepare_taps once, then ndc_forward_taps / ndc_backward_taps: the same bits as the
     entry points that pack the filter table on every call (bf16 3x3x3 kernels; the last case
     is a 192-column row, i.e. six wavefronts per workgroup in the forward)."""
     C, G, sc, ks, sp, B = geom
     lib = _lib_gpu()
+    matrix_switch(matrix)
     x, z, h, bias, gout = make_case(C, G, sc, ks, sp, B=B, dtype=torch.bfloat16, bias_shift=0.3,
                                     device="cuda")
     kw = dict(groups=G, m=1, sc=sc, eps=1e-16, relu_input=True)
@@ -259,3 +277,28 @@ def test_prepared_taps_bit_equal_on_gpu(geom):
     assert O.rel_err(out1.float().cpu(), ro) < 2e-2
     for got, ref in zip(g1, (rgx, rgz, rgh, rgb)):
         assert O.rel_err(got.float().cpu(), ref) < 2e-2
+
+
+def test_matrix_kernel_switch_defaults_to_off_and_changes_the_kernels(matrix_switch):
+    """ndc_matrix_kernels: off in a fresh library; turned on, the bf16 3x3x3 update runs other
+    kernels (the filter gradient's float32 sums come out in another order) that agree with the
+    default ones to the bf16 tolerance."""
+    lib = _lib_gpu()
+    assert lib.matrix_kernels() is False
+    C, G, sc, ks, sp, B = FUSED_GEOMS[7]
+    x, z, h, bias, gout = make_case(C, G, sc, ks, sp, B=B, dtype=torch.bfloat16, bias_shift=0.3, device="cuda")
+    kw = dict(groups=G, m=1, sc=sc, eps=1e-16, relu_input=True)
+
+    def run():
+        out, t1, saved = ops.update_forward(lib, x, z, h, bias, save_ratio=True, **kw)
+        return (out, t1) + tuple(ops.update_backward(lib, x, z, t1, h, bias, gout, saved=saved, **kw))
+    base = run()
+    assert matrix_switch(True) is True
+    other = run()
+    assert matrix_switch(False) is False
+    again = run()
+    for a, b in zip(base, again):
+        assert torch.equal(a, b)
+    assert not torch.equal(base[4], other[4])          # gh: float32, other summation order
+    for a, b in zip(base, other):
+        assert O.rel_err(a.float().cpu(), b.float().cpu().double()) < 2e-2

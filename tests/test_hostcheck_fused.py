@@ -118,10 +118,24 @@ BF16_GEOMS = [
 ]
 
 
+@pytest.fixture
+def matrix_switch():
+    """Sets the host build's kernel-family switch for one test and puts it back to off."""
+    lib = hostcheck_library()
+    yield lib.matrix_kernels
+    lib.matrix_kernels(False)
+
+
+def test_matrix_kernels_are_off_by_default():
+    assert hostcheck_library().matrix_kernels() is False
+
+
+@pytest.mark.parametrize("matrix", [False, True])
 @pytest.mark.parametrize("geom", BF16_GEOMS)
-def test_fused_bf16_storage(geom):
+def test_fused_bf16_storage(geom, matrix, matrix_switch):
     C, sc, ks, sp, B = geom
     lib = hostcheck_library()
+    assert matrix_switch(matrix) == matrix
     x, z, h, bias, gout = make_case(C, C, sc, ks, sp, B=B, dtype=torch.bfloat16, bias_shift=0.3)
     out, t1 = ops.update_forward(lib, x, z, h, bias, groups=C, m=1, sc=sc, eps=1e-16,
                                  relu_input=True, path=_lib.PATH_FUSED)
@@ -147,10 +161,12 @@ FULL_WG_GEOMS = [
 
 @pytest.mark.parametrize("geom", FUSED_GEOMS[:3] + FUSED_GEOMS[5:6] + FUSED_GEOMS[7:9] + FUSED_GEOMS[10:11]
                          + FULL_WG_GEOMS)
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype,matrix", [(torch.float32, False), (torch.bfloat16, False), (torch.bfloat16, True)])
 @pytest.mark.parametrize("relu", [True, False])
-def test_fused_saved_denominator_and_ratio(geom, dtype, relu):
-    """The forward's optional s/d and n/d outputs, and a backward that consumes them."""
+def test_fused_saved_denominator_and_ratio(geom, dtype, matrix, relu, matrix_switch):
+    """The forward's optional s/d and n/d outputs, and a backward that consumes them (bf16: on
+    both kernel families)."""
+    assert matrix_switch(matrix) == matrix
     C, sc, ks, sp, B = geom
     tol_f, tol_b = (1e-5, 1e-4) if dtype == torch.float32 else (2e-2, 2e-2)
     lib = hostcheck_library()
@@ -229,20 +245,23 @@ def test_fused_wide_rows(geom, dtype):
     assert n == 0, f"LDS faults: {n} ({first})"
 
 
-@pytest.mark.parametrize("dtype,path,relu", [
-    (torch.float32, _lib.PATH_FUSED, True), (torch.float32, _lib.PATH_FUSED, False),
-    (torch.bfloat16, _lib.PATH_FUSED, True), (torch.bfloat16, _lib.PATH_FUSED, False),
-    (torch.float32, _lib.PATH_DIRECT, True), (torch.float32, _lib.PATH_DIRECT, False),
+@pytest.mark.parametrize("dtype,path,relu,matrix", [
+    (torch.float32, _lib.PATH_FUSED, True, False), (torch.float32, _lib.PATH_FUSED, False, False),
+    (torch.bfloat16, _lib.PATH_FUSED, True, False), (torch.bfloat16, _lib.PATH_FUSED, False, False),
+    (torch.bfloat16, _lib.PATH_FUSED, True, True), (torch.bfloat16, _lib.PATH_FUSED, False, True),
+    (torch.float32, _lib.PATH_DIRECT, True, False), (torch.float32, _lib.PATH_DIRECT, False, False),
 ])
-def test_nan_in_source_propagates_like_torch(dtype, path, relu):
+def test_nan_in_source_propagates_like_torch(dtype, path, relu, matrix, matrix_switch):
     """A NaN in z is handed on where the reference's PyTorch arithmetic hands it on
     (torch.relu and a plain load both propagate it; reference.py:113-118,169-173): the set of
     non-finite entries of out, t1 and of every gradient equals the oracle's.  The bf16 dot2
     kernels multiply the column neighbour of a stencil's edge by a zero tap (half-empty
     column pairs), so there a non-finite value may also reach the entries one column further:
-    every entry the oracle marks is marked, and nothing beyond that one column."""
+    every entry the oracle marks is marked, and nothing beyond that one column.  The
+    matrix-instruction forward multiplies a fourth window column by a zero tap: two columns."""
     C, sc, ks, sp = 2, 4, (3, 3, 3), (4, 16, 16)
     lib = hostcheck_library()
+    assert matrix_switch(matrix) == matrix
     x, z, h, bias, gout = make_case(C, C, sc, ks, sp, B=1, dtype=dtype, bias_shift=0.3,
                                     positive_z=not relu)
     if not relu:
@@ -256,8 +275,11 @@ def test_nan_in_source_propagates_like_torch(dtype, path, relu):
         if not wide or got.dim() != 5 or got.shape[-1] != sp[-1]:
             return torch.equal(bad_got, bad_ref)
         grown = bad_ref.clone()
-        grown[..., 1:] |= bad_ref[..., :-1]
-        grown[..., :-1] |= bad_ref[..., 1:]
+        for _ in range(2 if matrix else 1):
+            wider = grown.clone()
+            wider[..., 1:] |= grown[..., :-1]
+            wider[..., :-1] |= grown[..., 1:]
+            grown = wider
         return bool((bad_got >= bad_ref).all() and (bad_got <= grown).all())
 
     out, t1 = ops.update_forward(lib, x, z, h, bias, groups=C, m=1, sc=sc, eps=1e-16,
@@ -275,12 +297,13 @@ def test_nan_in_source_propagates_like_torch(dtype, path, relu):
     assert ((out.double() - ro)[fin].abs().max() / ro[fin].abs().max()) < tol
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-def test_prepared_taps_give_the_same_results(dtype):
+@pytest.mark.parametrize("dtype,matrix", [(torch.bfloat16, False), (torch.bfloat16, True), (torch.float32, False)])
+def test_prepared_taps_give_the_same_results(dtype, matrix, matrix_switch):
     """ndc_prepare_taps + ndc_forward_taps / ndc_backward_taps against the entry points that
     pack the table themselves: bit-equal.  float32 geometries have no table (0 bytes)."""
     C, sc, ks, sp = 3, 4, (3, 3, 3), (5, 9, 8)
     lib = hostcheck_library()
+    matrix_switch(matrix)
     x, z, h, bias, gout = make_case(C, C, sc, ks, sp, B=2, dtype=dtype, bias_shift=0.3)
     kw = dict(groups=C, m=1, sc=sc, eps=1e-16, relu_input=True)
     taps = ops.prepare_taps(lib, x, h, groups=C, m=1, sc=sc)
