@@ -741,7 +741,7 @@ def main() -> int:
     if os.path.exists(tpath):
         try:
             rec = json.load(open(tpath))
-            traffic = rec.get(args.dtype, {}).get(dominant)
+            traffic = rec.get(args.dtype + ("_matrix" if args.matrix else ""), {}).get(dominant)
             traffic_at = rec.get("measured_at_commit")
         except (ValueError, OSError):
             traffic = None
