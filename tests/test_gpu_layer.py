@@ -316,14 +316,16 @@ def test_config1_single_layer_2d_sum_of_squares():
     assert O.rel_err(layer.init.linear.linear.bias.grad.cpu(), b.grad) < 1e-4
 
 
-@pytest.mark.parametrize("dtype,tol,matrix", [(torch.bfloat16, 2e-2, False), (torch.float32, 1e-4, False),
-                                              (torch.bfloat16, 2e-2, True)])
-def test_headline_size_channel_slices_match_oracle(dtype, tol, matrix):
+@pytest.mark.parametrize("dtype,tol,saved,matrix", [
+    (torch.bfloat16, 2e-2, False, False), (torch.float32, 1e-4, False, False),
+    (torch.bfloat16, 2e-2, True, False), (torch.float32, 1e-4, True, False),   # the form bench.py times
+    (torch.bfloat16, 2e-2, True, True)])
+def test_headline_size_channel_slices_match_oracle(dtype, tol, saved, matrix):
     """Config 3 at full size (B=2, C=128, 64^3, 3x3x3, ratio 4).  Depthwise channels are
     independent, so any channel slice of the full-size result must equal the oracle run on
-    that slice alone -- which the CPU does in seconds.  `matrix`: the training form (backward
-    fed with the forward's ratios) on the matrix-instruction kernel family, switched on through
-    the package's own setter."""
+    that slice alone -- which the CPU does in seconds.  `saved`: the training form (backward
+    fed with the forward's ratios), which is what bench.py times; `matrix`: on the
+    matrix-instruction kernel family, switched on through the package's own setter."""
     from deconver_amd import _lib, ops
     B, C, sc, sp = 2, 128, 4, (64, 64, 64)
     gen = torch.Generator().manual_seed(0)
@@ -337,10 +339,10 @@ def test_headline_size_channel_slices_match_oracle(dtype, tol, matrix):
     kw = dict(groups=C, m=1, sc=sc, eps=1e-16, relu_input=True)
     assert dc.matrix_kernels(matrix) == matrix
     try:
-        res = ops.update_forward(lib, dev[0], dev[1], dev[2], dev[3], save_ratio=matrix, **kw)
+        res = ops.update_forward(lib, dev[0], dev[1], dev[2], dev[3], save_ratio=saved, **kw)
         out, t1 = res[0], res[1]
         gx, gz, gh, gb = ops.update_backward(lib, dev[0], dev[1], t1, dev[2], dev[3], dev[4],
-                                             saved=res[2] if matrix else None, **kw)
+                                             saved=res[2] if saved else None, **kw)
         torch.cuda.synchronize()
     finally:
         dc.matrix_kernels(False)
