@@ -648,7 +648,9 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
         const int need_gh = p.need_gh;
 
         auto load_plane = [&](State &st, int k) NDC_LAMBDA {
-            if (!st.ln.active) return;
+            // (every lane issues every fetch, lanes outside the tile with offsets outside the
+            // slices: a fetch under a condition gives the compiler a path without it, on which
+            // it cannot count the outstanding loads and makes every user wait for all of them)
             // planes past the end: load the last plane and select zero (a store in each arm of
             // a branch would push the staging registers into private memory)
             const bool live = k < D;
@@ -688,8 +690,10 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
         // channel-pair words; returned as operand pairs GG[i][r][c] = (gn_i, gd_i)
         // SAVED: fetch plane jn of gout, s/d, n/d into the state, a phase before it is used
         auto prefetch_g = [&](State &st, int jn) NDC_LAMBDA {
-            if (!SAVED || jn >= D) return;
-            const unsigned jo = (unsigned)jn * plane2;
+            if (!SAVED) return;
+            // (past the last plane a clamped plane is fetched and never used: no branch
+            // around loads, see load_plane)
+            const unsigned jo = (unsigned)clampi(jn, 0, D - 1) * plane2;
             NDC_UNROLL
             for (int r = 0; r < RH + 1; ++r) {
                 if (r == RH && st.ln.strip >= 2) continue;
@@ -793,17 +797,17 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
             for (int n = 0; n < NXR; ++n) {
                 const int j = st.ln.strip + n * S, row = r0 - 2 * PH + j;
                 if (j < RX && row >= 0 && row < H) st.xok |= 1u << n;
-                st.xoff[n] = (unsigned)(clampi(row, 0, H - 1) * W + st.ln.c0) * 2u;
+                st.xoff[n] = st.ln.active ? (unsigned)(clampi(row, 0, H - 1) * W + st.ln.c0) * 2u : kNoAccess;
                 st.px[n] = st.pt[n] = st.pxprev[n] = st.ptprev[n] = 0u;
             }
             NDC_UNROLL
             for (int r = 0; r < RH; ++r) {
                 const int row = r0 + st.ln.strip * RH + r;
-                st.ooff[r] = row < H ? (unsigned)(row * W + st.ln.c0) * 2u : kNoAccess;
+                st.ooff[r] = st.ln.active && row < H ? (unsigned)(row * W + st.ln.c0) * 2u : kNoAccess;
             }
             {
                 const int hrow = r0 - PH + halo_row(st.ln.strip, PH, TH);
-                st.hoff = hrow >= 0 && hrow < H ? (unsigned)(hrow * W + st.ln.c0) * 2u : kNoAccess;
+                st.hoff = st.ln.active && hrow >= 0 && hrow < H ? (unsigned)(hrow * W + st.ln.c0) * 2u : kNoAccess;
                 NDC_UNROLL
                 for (int i = 0; i < SC; ++i)
                     NDC_UNROLL
@@ -883,9 +887,9 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
             ex.sync();
 
             ex.each([&](State &st, int) NDC_LAMBDA {
-                if (!st.ln.active) return;
                 load_plane(st, k + 1);
                 prefetch_g(st, k);
+                if (!st.ln.active) return;
                 if (live1) {
                     const int gb_ = off_g + (st.ln.strip * RH) * P + PL + st.ln.c0 - PW;
                     // the two channel pairs one after the other in straight-line code (as a
@@ -1013,7 +1017,9 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
         const int need_gh = p.need_gh;
 
         auto load_plane = [&](State &st, int k) NDC_LAMBDA {
-            if (!st.ln.active) return;
+            // (every lane issues every fetch, lanes outside the tile with offsets outside the
+            // slices: a fetch under a condition gives the compiler a path without it, on which
+            // it cannot count the outstanding loads and makes every user wait for all of them)
             // planes past the end: load the last plane and select zero (a store in each arm of
             // a branch would push the staging registers into private memory)
             const bool live = k < D;
@@ -1058,14 +1064,14 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
             for (int n = 0; n < NXR; ++n) {
                 const int j = st.ln.strip + n * S, row = r0 - PH + j;
                 if (j < RX && row >= 0 && row < H) st.xok |= 1u << n;
-                st.xoff[n] = (unsigned)(clampi(row, 0, H - 1) * W + st.ln.c0) * 2u;
+                st.xoff[n] = st.ln.active ? (unsigned)(clampi(row, 0, H - 1) * W + st.ln.c0) * 2u : kNoAccess;
                 st.px[n] = st.pt[n] = st.pg[n] = st.pxprev[n] = st.ptprev[n] = st.pgprev[n] = 0u;
             }
             NDC_UNROLL
             for (int r = 0; r < RH; ++r) {
                 const int row = r0 + st.ln.strip * RH + r;
                 // a row outside the image: its loads give 0 and its stores go nowhere
-                st.ooff[r] = row < H ? (unsigned)(row * W + st.ln.c0) * 2u : kNoAccess;
+                st.ooff[r] = st.ln.active && row < H ? (unsigned)(row * W + st.ln.c0) * 2u : kNoAccess;
                 st.okf[r] = row < H ? 1.f : 0.f;
                 NDC_UNROLL
                 for (int i = 0; i < SC; ++i)
@@ -1096,7 +1102,6 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
         auto compute = [&](State &st, int k, auto par_tag) NDC_LAMBDA {
                 constexpr int PAR = decltype(par_tag)::value;
                 const int j0 = k - 1;
-                if (!st.ln.active) return;
                 load_plane(st, k + 1);
                 // SAVED: this plane's z, gout, n/d words were fetched a step ago; take them and
                 // start the fetch of the next plane's
@@ -1115,7 +1120,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
                             st.qr[1 - PAR][i][r] = buf_ld<true>(rb_, st.ooff[r], jn + i * cplane2);
                         }
                 }
-                if (j0 < 0) return;
+                if (!st.ln.active || j0 < 0) return;
                 float sv[SC][RH][RW];
                 NDC_UNROLL
                 for (int i = 0; i < SC; ++i)
@@ -1235,7 +1240,10 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
                 ex.sync();
                 ex.each([&](State &st, int) NDC_LAMBDA { compute(st, k, IntTag<0>()); });
             }
-            if (kk + 1 < D + 2) {
+            {   // (always: an even number of steps, the last possibly past the end of the march,
+                // where it finds nothing to do; under a condition the compiler sees a path
+                // from one even step to the next without this step's loads and can no longer
+                // count the loads outstanding)
                 const int k = uniform_int(kk + 1);
                 ex.each([&](State &st, int) NDC_LAMBDA { store_plane(st, k); });
                 ex.sync();
