@@ -50,21 +50,27 @@ def _slice(c, x, z, h, bias, gout=None):
 SWEEP = [(512, 16, 4), (256, 32, 2), (64, 128, 1), (32, 192, 1)]
 
 
+@pytest.mark.parametrize("matrix", [False, True])
 @pytest.mark.parametrize("C,n,B", SWEEP)
-def test_config5_inference_form_channel_slices(C, n, B):
+def test_config5_inference_form_channel_slices(C, n, B, matrix):
     """Forward only, bfloat16, t1 = null, nothing kept: the call `bench.py --workload sweep`
-    times, at each of its four shapes."""
-    print("case config5", C, n, B, flush=True)
+    times, at each of its four shapes, on both bf16 kernel families (the 192-column shape is
+    outside the matrix-instruction family's widths and runs the default kernels either way)."""
+    print("case config5", C, n, B, matrix, flush=True)
     sp = (n, n, n)
     x, z, h, bias, _ = _inputs(B, C, sp, torch.bfloat16, with_gout=False)
     lib = _lib.get_library()
     dev = [x, z, h, bias]
     g = ops.make_geom_for(dev[0], dev[2], C, 1, SC, EPS, True)
     assert lib.fused_supported(g), "the fused kernels must cover every config-5 shape"
-    out, t1 = ops.update_forward(lib, *dev, groups=C, m=1, sc=SC, eps=EPS, relu_input=True,
-                                 need_t1=False)
+    assert lib.matrix_kernels(matrix) == matrix
+    try:
+        out, t1 = ops.update_forward(lib, *dev, groups=C, m=1, sc=SC, eps=EPS, relu_input=True,
+                                     need_t1=False)
+        torch.cuda.synchronize()
+    finally:
+        lib.matrix_kernels(False)
     assert t1 is None
-    torch.cuda.synchronize()
     for c in (0, C // 3, C - 1):
         cs, d = _slice(c, x, z, h, bias)
         ro, _ = O.update_grouped(d[0], d[1], d[2], d[3], 1, 1, SC, EPS, True)
@@ -72,8 +78,9 @@ def test_config5_inference_form_channel_slices(C, n, B):
         assert e < 2e-2, f"out channel {c}: {e:.3e}"
 
 
-@pytest.mark.parametrize("dtype,tol", [(torch.bfloat16, 2e-2), (torch.float32, 1e-4)])
-def test_config3_kept_ratio_backward_channel_slices(dtype, tol):
+@pytest.mark.parametrize("dtype,tol,matrix", [(torch.bfloat16, 2e-2, False), (torch.float32, 1e-4, False),
+                                              (torch.bfloat16, 2e-2, True)])
+def test_config3_kept_ratio_backward_channel_slices(dtype, tol, matrix):
     """Config 3 at full size with the forward's s/d and n/d kept: the kernels the headline
     benchmark times (forward with four outputs, both kept-ratio backward passes), including
     the two kept tensors themselves."""
@@ -82,10 +89,14 @@ def test_config3_kept_ratio_backward_channel_slices(dtype, tol):
     lib = _lib.get_library()
     dev = [x, z, h, bias, gout]
     kw = dict(groups=C, m=1, sc=SC, eps=EPS, relu_input=True)
-    out, t1, saved = ops.update_forward(lib, *dev[:4], save_ratio=True, **kw)
-    gx, gz, gh, gb = ops.update_backward(lib, dev[0], dev[1], t1, dev[2], dev[3], dev[4],
-                                         saved=saved, **kw)
-    torch.cuda.synchronize()
+    assert lib.matrix_kernels(matrix) == matrix
+    try:
+        out, t1, saved = ops.update_forward(lib, *dev[:4], save_ratio=True, **kw)
+        gx, gz, gh, gb = ops.update_backward(lib, dev[0], dev[1], t1, dev[2], dev[3], dev[4],
+                                             saved=saved, **kw)
+        torch.cuda.synchronize()
+    finally:
+        lib.matrix_kernels(False)
     kept = saved
     for c in (1, 64, 126):
         cs, d = _slice(c, x, z, h, bias, gout)
@@ -103,10 +114,12 @@ def test_config3_kept_ratio_backward_channel_slices(dtype, tol):
         assert not bad, f"channel {c}: {bad} (all: {errs})"
 
 
-def test_config4_stage0_layer_channel_slices():
+@pytest.mark.parametrize("matrix", [False, True])
+def test_config4_stage0_layer_channel_slices(matrix):
     """Config 4's full-resolution layer: batch 2, 64 channels, 128^3, bfloat16.  The source
     tensors hold 2^30 elements (2 GiB) each, so tensor bases need 64-bit arithmetic; rows of
-    128 columns take the widest column strip.  Forward and the kept-ratio backward."""
+    128 columns take the widest column strip.  Forward and the kept-ratio backward, on both
+    bf16 kernel families (at this width the second family's forward and pass 2)."""
     B, C, sp = 2, 64, (128, 128, 128)
     dtype = torch.bfloat16
     x, z, h, bias, gout = _inputs(B, C, sp, dtype, seed=4)
@@ -114,10 +127,14 @@ def test_config4_stage0_layer_channel_slices():
     lib = _lib.get_library()
     dev = [x, z, h, bias, gout]
     kw = dict(groups=C, m=1, sc=SC, eps=EPS, relu_input=True)
-    out, t1, saved = ops.update_forward(lib, *dev[:4], save_ratio=True, **kw)
-    gx, gz, gh, gb = ops.update_backward(lib, dev[0], dev[1], t1, dev[2], dev[3], dev[4],
-                                         saved=saved, **kw)
-    torch.cuda.synchronize()
+    assert lib.matrix_kernels(matrix) == matrix
+    try:
+        out, t1, saved = ops.update_forward(lib, *dev[:4], save_ratio=True, **kw)
+        gx, gz, gh, gb = ops.update_backward(lib, dev[0], dev[1], t1, dev[2], dev[3], dev[4],
+                                             saved=saved, **kw)
+        torch.cuda.synchronize()
+    finally:
+        lib.matrix_kernels(False)
     del saved
     # the last channel of the last sample sits past the 2^31-byte and 2^31-element marks
     for c in (0, C - 1):
