@@ -16,7 +16,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdeconver_ndc.so")
 
 NDC_F32, NDC_BF16 = 0, 1
-PATH_AUTO, PATH_DIRECT, PATH_FUSED = 0, 1, 2
+PATH_AUTO, PATH_DIRECT, PATH_FUSED, PATH_FUSED_MATRIX, PATH_FUSED_VECTOR = 0, 1, 2, 3, 4
 
 EXPORTS = (
     "ndc_version",

@@ -27,7 +27,7 @@ static inline int make_kgeom(const ndc_geom *g, KGeom &q)
     // element counts must stay well inside int64 and block counts inside int32
     const long long cmax = (long long)g->groups * (g->m > g->sc ? g->m : g->sc);
     if (sp > (1LL << 40) || (long double)sp * cmax * g->batch > 9.0e15L) return NDC_ERR_GEOMETRY;
-    if (g->path < NDC_PATH_AUTO || g->path > NDC_PATH_FUSED) return NDC_ERR_GEOMETRY;
+    if (g->path < NDC_PATH_AUTO || g->path > NDC_PATH_FUSED_VECTOR) return NDC_ERR_GEOMETRY;
     q.B = g->batch;
     q.G = g->groups;
     q.m = g->m;
@@ -43,6 +43,10 @@ static inline int make_kgeom(const ndc_geom *g, KGeom &q)
     q.pW = q.kW / 2;
     q.KT = (int)taps;
     q.relu = g->relu_input ? 1 : 0;
+    // the kernel family is fixed here, once per call: named by the call, or the process default
+    q.matrix = g->path == NDC_PATH_FUSED_MATRIX   ? 1
+               : g->path == NDC_PATH_FUSED_VECTOR ? 0
+                                                  : fused::matrix_default().load(std::memory_order_relaxed);
     q.eps = g->eps;
     q.SP = sp;
     return NDC_OK;
@@ -56,7 +60,8 @@ static inline int choose_path(const ndc_geom *g, const KGeom &q)
 {
     const bool fused_ok = fused::supported(q);
     if (g->path == NDC_PATH_DIRECT) return NDC_PATH_DIRECT;
-    if (g->path == NDC_PATH_FUSED) return fused_ok ? (int)NDC_PATH_FUSED : (int)NDC_ERR_GEOMETRY;
+    if (g->path == NDC_PATH_FUSED || g->path == NDC_PATH_FUSED_MATRIX || g->path == NDC_PATH_FUSED_VECTOR)
+        return fused_ok ? (int)NDC_PATH_FUSED : (int)NDC_ERR_GEOMETRY;
     return fused_ok ? (int)NDC_PATH_FUSED : (int)NDC_PATH_DIRECT;
 }
 
@@ -274,8 +279,8 @@ int ndc_forward_taps(const ndc_geom *g, const void *x, const void *z, const floa
 
 int ndc_matrix_kernels(int on)
 {
-    if (on >= 0) ndc::fused::matrix_switch() = on ? 1 : 0;
-    return ndc::fused::matrix_switch();
+    if (on >= 0) ndc::fused::matrix_default().store(on ? 1 : 0, std::memory_order_relaxed);
+    return ndc::fused::matrix_default().load(std::memory_order_relaxed);
 }
 
 int ndc_backward_uses_saved(const ndc_geom *g)

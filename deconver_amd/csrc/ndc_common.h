@@ -327,6 +327,7 @@ struct KGeom {
     int pD, pH, pW;
     int KT;        // kD*kH*kW
     int relu;      // rectify z (+bias) on load
+    int matrix;    // bf16 3x3x3 calls run the matrix-instruction kernel family where it covers them
     float eps;
     long long SP;  // D*H*W
 

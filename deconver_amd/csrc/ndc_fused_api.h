@@ -6,6 +6,8 @@
 #include "../../include/deconver_ndc.h"
 #include <stdlib.h>
 
+#include <atomic>
+
 #include "ndc_fused.h"
 #include "ndc_fused_mfma.h"
 
@@ -97,12 +99,15 @@ static inline bool find_variant(const KGeom &q, const March &m, bool pairs_ok, V
     return found;
 }
 
-// Whether plans may choose the kernels built on the 4x4x4 matrix instruction
-// (ndc_fused_mfma.h).  Off unless a caller turns it on (ndc_matrix_kernels): the path is
-// specified as a depthwise stencil that keeps matrix instructions out of it.
-static inline int &matrix_switch()
+// The process-wide default of the kernel family for calls that do not name one
+// (ndc_matrix_kernels): 0 = vector unit, 1 = the kernels built on the 4x4x4 matrix instruction
+// (ndc_fused_mfma.h) where they cover the geometry.  Off unless a caller turns it on: the path
+// is specified as a depthwise stencil that keeps matrix instructions out of it.  Atomic, so
+// that a thread that sets it and threads that launch do not race; a call that must not depend
+// on it names its family in ndc_geom.path.
+static inline std::atomic<int> &matrix_default()
 {
-    static int on = 0;
+    static std::atomic<int> on{0};
     return on;
 }
 
@@ -132,7 +137,7 @@ static inline void plan_lds(Plan &pl)
 // pairs_ok: every activation pointer of the call is aligned to two elements
 static const int kDot2RH = 2;   // rows per thread of the bf16 dot2 kernels (columns: 2)
 
-static inline bool make_plan_for(const KGeom &q, Plan &pl, bool pairs_ok, int dtype)
+static inline bool make_plan_for(const KGeom &q, Plan &pl, bool pairs_ok, int dtype, bool matrix)
 {
     pl.m = march_of(q);
     pl.dot2 = false;
@@ -173,11 +178,11 @@ static inline bool make_plan_for(const KGeom &q, Plan &pl, bool pairs_ok, int dt
                 // (pass 1 only where two of its workgroups fit a CU: with 128 columns its LDS
                 // need leaves room for one, and the dot2 kernel is faster, 2.73 against 2.96 ms
                 // at 64 channels of 128^3)
-                pl.mfma1 = tn.mfma && matrix_switch() && Bwd1KernelM<kDot2RH>::covers(pl.m.W) &&
+                pl.mfma1 = tn.mfma && matrix && Bwd1KernelM<kDot2RH>::covers(pl.m.W) &&
                            Bwd1KernelM<kDot2RH>::lds_floats(tb) <= cap2 / 2;
-                pl.mfmaf = tn.mfma && matrix_switch() && FwdKernelM<kDot2RH>::covers(pl.m.W) &&
+                pl.mfmaf = tn.mfma && matrix && FwdKernelM<kDot2RH>::covers(pl.m.W) &&
                            FwdKernelM<kDot2RH>::lds_floats(tf) <= cap2;
-                pl.mfma2 = tn.mfma && matrix_switch() && Bwd2KernelM<kDot2RH>::covers(pl.m.W) &&
+                pl.mfma2 = tn.mfma && matrix && Bwd2KernelM<kDot2RH>::covers(pl.m.W) &&
                            Bwd2KernelM<kDot2RH>::lds_floats(tb) <= cap2;
             }
         }
@@ -195,10 +200,13 @@ static inline bool make_plan_for(const KGeom &q, Plan &pl, bool pairs_ok, int dt
 // The column-pair variants hold more of a row per workgroup: where their LDS need exceeds a
 // workgroup's share (wide rows of a tall image) the one-column variants may still fit, and
 // those are what supported() answers for.
-static inline bool make_plan(const KGeom &q, Plan &pl, bool pairs_ok = true, int dtype = NDC_F32)
+// matrix: the call runs the matrix-instruction family where it covers the geometry (the
+// launch shapes, workspace sizes and table sizes are the same for both families)
+static inline bool make_plan(const KGeom &q, Plan &pl, bool pairs_ok = true, int dtype = NDC_F32,
+                             bool matrix = false)
 {
-    if (make_plan_for(q, pl, pairs_ok, dtype)) return true;
-    return pairs_ok && make_plan_for(q, pl, false, dtype);
+    if (make_plan_for(q, pl, pairs_ok, dtype, matrix)) return true;
+    return pairs_ok && make_plan_for(q, pl, false, dtype, matrix);
 }
 
 static inline bool supported(const KGeom &q)
@@ -299,7 +307,7 @@ static int forward(const KGeom &q, const T *x, const T *z, const float *h, const
     const bool pairs = pair_aligned<T>(x) && pair_aligned<T>(z) && pair_aligned<T>(out) &&
                        pair_aligned<T>(t1) && pair_aligned<T>(s_over_den) && pair_aligned<T>(ratio);
     const int dtype = sizeof(T) == 2 ? NDC_BF16 : NDC_F32;
-    if (!make_plan(q, pl, pairs, (ws || taps) ? dtype : NDC_F32)) return NDC_ERR_GEOMETRY;
+    if (!make_plan(q, pl, pairs, (ws || taps) ? dtype : NDC_F32, q.matrix != 0)) return NDC_ERR_GEOMETRY;
     FwdParams<T> p;
     p.wtab = nullptr;
     p.x = x;
@@ -353,7 +361,7 @@ static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const T
                        pair_aligned<T>(s_over_den) && pair_aligned<T>(ratio);
     const bool saved = s_over_den != nullptr && ratio != nullptr;
     const int dtype = sizeof(T) == 2 ? NDC_BF16 : NDC_F32;
-    if (!make_plan(q, pl, pairs, dtype)) return NDC_ERR_GEOMETRY;
+    if (!make_plan(q, pl, pairs, dtype, q.matrix != 0)) return NDC_ERR_GEOMETRY;
     const size_t n_x = (size_t)q.B * q.G * q.SP;
     const int kt = q.sc * q.KT;
     char *w = (char *)ws;

@@ -606,6 +606,11 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
         // then the halo row of the first two strips)
         uint32_t qg[SC][RH + 1], qd[SC][RH + 1], qr[SC][RH + 1];
         unsigned hoff;
+        // LDS word offsets inside a ring slot, formed once: the word (first own row - 1, first
+        // own column - 1) of an (x, t1) slot's rows, the word (row `strip`, first own column),
+        // and the word (halo row, first own column) of a gn/gd plane.  What is added per access
+        // (slot, row) is the same in every lane and stays on the scalar unit.
+        int ob, so, ho;
     };
 
     static NDC_HD int rows_x(int TH) { return TH + 4; }
@@ -623,6 +628,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
         const BlockId id = decode_block(block_id, p.C, t, p.D);
         const int S = t.S, P = t.P, PL = t.PL, TH = t.TH, W = p.W, H = p.H, D = p.D;
         const int RX = rows_x(TH), RG = rows_g(TH);
+        const int SP = S * P;
         const int off_xp = 0, off_tp = NP * RX * P, off_xt = SAVED ? 0 : 2 * NP * RX * P;
         const int off_g = off_xt + NXT * RX * P;
         const int total = off_g + 4 * RG * P;
@@ -671,7 +677,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
             NDC_UNROLL
             for (int n = 0; n < NXR; ++n) {
                 if ((st.xok >> n) & 1u) {
-                    const int o = (st.ln.strip + n * S) * P + PL + st.ln.c0;
+                    const int o = st.so + n * SP;
                     if (!SAVED) {
                         ex.st_(off_xp + ps + o, bits_to_float(zip_lo(st.pxprev[n], st.px[n])));
                         ex.st_(off_xp + ps + o + 1, bits_to_float(zip_hi(st.pxprev[n], st.px[n])));
@@ -708,7 +714,8 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
         };
 
         // roff: where the rows sit in the prefetched words (0: own rows, RH: halo row)
-        auto gn_gd_rows = [&](State &st, int j1, int j, auto nr_tag, int roff,
+        // lo: LDS word offset of (tile row j, first own column) inside a plane
+        auto gn_gd_rows = [&](State &st, int j1, int j, int lo, auto nr_tag, int roff,
                               uint32_t (&gg_out)[SC][decltype(nr_tag)::value][RW]) NDC_LAMBDA {
             constexpr int NR = decltype(nr_tag)::value;
             uint32_t zw[SC][NR], gw[SC][NR], dw[SC][NR], rw[SC][NR];
@@ -748,7 +755,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
                     float wt[SC][9];
                     load_plane_taps<SC, 9, 9>(tab + 54 + s * 36, wt);
                     const int m = j1 - 1 + s;
-                    const int ob = (wrap(m % NP, NP) * RX + j) * P + PL + st.ln.c0 - PW;
+                    const int ob = lo - PW + wrap(m % NP, NP) * RX * P;
                     const int base[2] = {off_xp + ob, off_tp + ob};
                     a_plane_d2<NR, RW, 2, true>(ex, base, P, wt, acc);
                 }
@@ -776,7 +783,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
                     }
                 // (the two columns of each word plane one after the other: adjacent words, one
                 // ds_write2_b32)
-                const int o = off_g + (j + r) * P + PL + st.ln.c0;
+                const int o = lo + (off_g + r * P);
                 NDC_UNROLL
                 for (int pr = 0; pr < 2; ++pr)
                     NDC_UNROLL
@@ -793,6 +800,9 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
         ex.each([&](State &st, int tid) NDC_LAMBDA {
             st.ln = make_lane(tid, t, RW);
             st.xok = 0u;
+            st.ob = st.ln.strip * RH * P + PL + st.ln.c0 - PW;
+            st.so = st.ln.strip * P + PL + st.ln.c0;
+            st.ho = halo_row(st.ln.strip, PH, TH) * P + PL + st.ln.c0;
             NDC_UNROLL
             for (int n = 0; n < NXR; ++n) {
                 const int j = st.ln.strip + n * S, row = r0 - 2 * PH + j;
@@ -844,17 +854,16 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
                 {
                     uint32_t gg2[SC][RH][RW];
                     const int j = PH + st.ln.strip * RH;
-                    const int cb = PL + st.ln.c0 - PW;
                     auto xt_row = [&](int n) NDC_LAMBDA {
                         const int td = n / (RH + 2), q = n % (RH + 2);
-                        return off_xt + (wrap((j1 + 1 - td) % NXT, NXT) * RX + j + q) * P + cb;
+                        return st.ob + (off_xt + (wrap((j1 + 1 - td) % NXT, NXT) * RX + PH + q) * P);
                     };
                     // the first (x, t1) row of the filter-gradient stream is requested before
                     // the elementwise work, so that it has arrived when that is done
                     uint32_t row0[RW + 2];
                     read_row<RW + 2>(ex, xt_row(0), row0);
                     ex.fence();
-                    gn_gd_rows(st, j1, j, IntTag<RH>(), 0, gg2);
+                    gn_gd_rows(st, j1, j, st.ob + (PW + PH * P), IntTag<RH>(), 0, gg2);
                     if (need_gh) {
                         // A-side filter-gradient terms: (gn_i, gd_i) . (x, t1)[neighbour]
                         stream_rows<KD * (RH + 2), RW + 2, true>(
@@ -881,7 +890,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
                 }
                 if (st.ln.strip < 2) {
                     uint32_t gg1[SC][1][RW];
-                    gn_gd_rows(st, j1, halo_row(st.ln.strip, PH, TH), IntTag<1>(), RH, gg1);
+                    gn_gd_rows(st, j1, halo_row(st.ln.strip, PH, TH), st.ho, IntTag<1>(), RH, gg1);
                 }
             });
             ex.sync();
@@ -891,7 +900,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd1KernelB {
                 prefetch_g(st, k);
                 if (!st.ln.active) return;
                 if (live1) {
-                    const int gb_ = off_g + (st.ln.strip * RH) * P + PL + st.ln.c0 - PW;
+                    const int gb_ = st.ob + off_g;
                     // the two channel pairs one after the other in straight-line code (as a
                     // rolled loop the accumulators it carries were permuted by register copies
                     // on every trip); the fence keeps the second pair's tap loads behind the
@@ -970,7 +979,9 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
         // n/d words read as zeros) -1 when the source is rectified and 0 when it is not, so
         // that its source values and rectified gradients come out as zeros without a select
         float bvr[SC][RH];
-        float okf[RH];   // 1 for a row inside the image, 0 outside: weight of its gz in gb
+        // (1, 1) as a bf16 pair for a row inside the image, (0, 0) outside: the weights of the
+        // row's gz words in gb (gb sums the gz values as they are stored, one dot2 per word)
+        uint32_t okw[RH];
         float gacc[SC][KT];
         float gbacc[SC];
         float sprev[SC][RH][RW];   // own source values of the previous plane
@@ -979,6 +990,10 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
         // and fetches the next plane's into set 1 - P (the plane loop is unrolled twice, so
         // the sets are fixed registers and nothing is copied from step to step)
         uint32_t qz[2][SC][RH], qg[2][SC][RH], qr[2][SC][RH];
+        // LDS word offsets inside a ring slot, formed once: the word (first own row - 1, first
+        // own column - 1) and the word (row `strip`, first own column).  What is added per
+        // access (slot, row) is the same in every lane and stays on the scalar unit.
+        int ob, so;
     };
 
     static NDC_HD int rows_x(int TH) { return TH + 2; }
@@ -995,6 +1010,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
         const BlockId id = decode_block(block_id, p.C, t, p.D);
         const int S = t.S, P = t.P, PL = t.PL, TH = t.TH, W = p.W, H = p.H, D = p.D;
         const int RX = rows_x(TH);
+        const int SP = S * P;
         const int off_xp = 0, off_tp = NP * RX * P, off_gp = SAVED ? 0 : 2 * NP * RX * P;
         const int total = off_gp + NG * RX * P;
         const int plane = H * W;
@@ -1041,7 +1057,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
             NDC_UNROLL
             for (int n = 0; n < NXR; ++n) {
                 if ((st.xok >> n) & 1u) {
-                    const int o = (st.ln.strip + n * S) * P + PL + st.ln.c0;
+                    const int o = st.so + n * SP;
                     if (!SAVED) {
                         ex.st_(off_xp + ps + o, bits_to_float(zip_lo(st.pxprev[n], st.px[n])));
                         ex.st_(off_xp + ps + o + 1, bits_to_float(zip_hi(st.pxprev[n], st.px[n])));
@@ -1060,6 +1076,8 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
         ex.each([&](State &st, int tid) NDC_LAMBDA {
             st.ln = make_lane(tid, t, RW);
             st.xok = 0u;
+            st.ob = st.ln.strip * RH * P + PL + st.ln.c0 - PW;
+            st.so = st.ln.strip * P + PL + st.ln.c0;
             NDC_UNROLL
             for (int n = 0; n < NXR; ++n) {
                 const int j = st.ln.strip + n * S, row = r0 - PH + j;
@@ -1072,7 +1090,7 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
                 const int row = r0 + st.ln.strip * RH + r;
                 // a row outside the image: its loads give 0 and its stores go nowhere
                 st.ooff[r] = st.ln.active && row < H ? (unsigned)(row * W + st.ln.c0) * 2u : kNoAccess;
-                st.okf[r] = row < H ? 1.f : 0.f;
+                st.okw[r] = row < H ? 0x3f803f80u : 0u;
                 NDC_UNROLL
                 for (int i = 0; i < SC; ++i)
                     st.bvr[i][r] = row < H ? (p.bias ? p.bias[id.c * SC + i] : 0.f) : (p.relu ? -1.f : 0.f);
@@ -1148,18 +1166,24 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
                             NDC_UNROLL
                             for (int r = 0; r < RH; ++r)
                                 NDC_UNROLL
-                                for (int c = 0; c < RW; ++c) acc[a][i][r][c] = a < NA - 1 ? eps : 0.f;
+                                for (int c = 0; c < RW; ++c) {
+                                    // SAVED: the sum starts from g (n/d), the other term of gz
+                                    if (SAVED)
+                                        acc[a][i][r][c] = (c ? bf_hi(gw[i][r]) : bf_lo(gw[i][r])) *
+                                                          (c ? bf_hi(rw[i][r]) : bf_lo(rw[i][r]));
+                                    else
+                                        acc[a][i][r][c] = a < NA - 1 ? eps : 0.f;
+                                }
                     NDC_ROLLED
                     for (int s = 0; s < 2; ++s) {
                         float wt[SC][9];
                         load_plane_taps<SC, 9, 9>(tab + 54 + s * 36, wt);
                         const int m = j0 - 1 + s;
-                        const int ob = (st.ln.strip * RH) * P + PL + st.ln.c0 - PW;
                         int base[NA];
-                        base[NA - 1] = off_gp + wrap(m % NG, NG) * RX * P + ob;
+                        base[NA - 1] = st.ob + (off_gp + wrap(m % NG, NG) * RX * P);
                         if (!SAVED) {
-                            base[0] = off_xp + wrap(m % NP, NP) * RX * P + ob;
-                            base[NA > 1 ? 1 : 0] = off_tp + wrap(m % NP, NP) * RX * P + ob;
+                            base[0] = st.ob + (off_xp + wrap(m % NP, NP) * RX * P);
+                            base[NA > 1 ? 1 : 0] = st.ob + (off_tp + wrap(m % NP, NP) * RX * P);
                         }
                         a_plane_d2<RH, RW, NA, SAVED>(ex, base, P, wt, acc);
                     }
@@ -1171,20 +1195,21 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
                             NDC_UNROLL
                             for (int c = 0; c < RW; ++c) {
                                 const float s = floor_f((c ? bf_hi(zw[i][r]) : bf_lo(zw[i][r])) + st.bvr[i][r], floor_);
-                                const float g = c ? bf_hi(gw[i][r]) : bf_lo(gw[i][r]);
                                 float gzv;
                                 if (SAVED)
-                                    gzv = g * (c ? bf_hi(rw[i][r]) : bf_lo(rw[i][r])) + acc[NA - 1][i][r][c];
+                                    gzv = acc[NA - 1][i][r][c];
                                 else
-                                    gzv = g * acc[0][i][r][c] * fast_rcp(acc[NA > 1 ? 1 : 0][i][r][c]) +
+                                    gzv = (c ? bf_hi(gw[i][r]) : bf_lo(gw[i][r])) * acc[0][i][r][c] *
+                                              fast_rcp(acc[NA > 1 ? 1 : 0][i][r][c]) +
                                           acc[NA - 1][i][r][c];
                                 if (p.relu && s <= 0.f) gzv = 0.f;   // a NaN passes
                                 sv[i][r][c] = s;
-                                st.gbacc[i] += gzv * st.okf[r];
                                 v[c] = gzv;
                             }
+                            const uint32_t gzw = pack_bf16x2(v[0], v[1]);
+                            st.gbacc[i] = dot2_bf16(gzw, st.okw[r], st.gbacc[i]);
                             // (no gz asked for: gzb_ is an empty slice and the store goes nowhere)
-                            buf_st<true>(gzb_, st.ooff[r], jo + i * cplane2, pack_bf16x2(v[0], v[1]));
+                            buf_st<true>(gzb_, st.ooff[r], jo + i * cplane2, gzw);
                         }
                     }
                 }
@@ -1198,12 +1223,11 @@ template <int RH_, bool SAVED_ = false> struct Bwd2KernelB {
                         for (int r = 0; r < RH; ++r)
                             NDC_UNROLL
                             for (int c = 0; c < RW; ++c) ss[i][r][c] = pack_bf16x2(st.sprev[i][r][c], sv[i][r][c]);
-                    const int cb = PL + st.ln.c0 - PW;
                     stream_rows<KD * (RH + 2), RW + 2, SAVED>(
                         ex,
                         [&](int n) NDC_LAMBDA {
                             const int td = n / (RH + 2), q = n % (RH + 2);
-                            return off_gp + (wrap((j0 - td) % NG, NG) * RX + st.ln.strip * RH + q) * P + cb;
+                            return st.ob + (off_gp + (wrap((j0 - td) % NG, NG) * RX + q) * P);
                         },
                         [&](int n, const uint32_t (&v)[RW + 2]) NDC_LAMBDA {
                             const int td = n / (RH + 2), q = n % (RH + 2);

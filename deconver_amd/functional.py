@@ -40,9 +40,11 @@ def save_ratio(enabled: Optional[bool] = None) -> bool:
 
 def matrix_kernels(enabled: Optional[bool] = None) -> bool:
     """Get or set whether bf16 3x3x3 updates may run on the kernels that use the 4x4x4 matrix
-    instruction (``ndc_matrix_kernels``).  Off by default (environment
+    instruction (the process default, ``ndc_matrix_kernels``).  Off by default (environment
     ``DECONVER_NDC_MATRIX=1`` turns it on when the library is loaded): the path is specified
-    without matrix instructions.  Same results to the bf16 tolerance, less time per step."""
+    without matrix instructions.  Same results to the bf16 tolerance, less time per step.
+    An update node reads the setting once, in its forward, and names the family in its forward
+    and backward calls (``ndc_geom.path``), so a change takes effect from the next forward."""
     return _lib.get_library().matrix_kernels(enabled)
 
 
@@ -83,20 +85,26 @@ class DeconvUpdate(torch.autograd.Function):
         hc = h.contiguous()
         need_t1 = any(ctx.needs_input_grad[:4])
         keep = need_t1 and _SAVE_RATIO
+        # The kernel family is read once, here, and named in both calls of this node: backward
+        # runs on an autograd thread, possibly after the process default has changed.
+        path = _lib.PATH_AUTO
+        if lib.fused_supported(ops.make_geom_for(x, hc, groups, m, sc, eps, relu_input)):
+            path = _lib.PATH_FUSED_MATRIX if lib.matrix_kernels() else _lib.PATH_FUSED_VECTOR
         if keep:
             # only where the backward kernels for this geometry read them
             keep = lib.backward_uses_saved(
-                ops.make_geom_for(x, hc, groups, m, sc, eps, relu_input))
+                ops.make_geom_for(x, hc, groups, m, sc, eps, relu_input, path))
         with torch.cuda.device(x.device):
             if taps is None:
                 # packed once here, used by the forward kernel and again by the backward's
                 taps = ops.prepare_taps(lib, x, hc, groups=groups, m=m, sc=sc)
             res = ops.update_forward(lib, x, z, hc, bias, groups=groups, m=m, sc=sc, eps=eps,
                                      relu_input=relu_input, need_t1=need_t1, save_ratio=keep,
-                                     taps=taps)
+                                     taps=taps, path=path)
         out, t1 = res[0], res[1]
         s_over_den, ratio = res[2] if keep else (None, None)
         ctx.cfg = (groups, m, sc, eps, relu_input)
+        ctx.path = path
         ctx.taps = taps if need_t1 else None   # a function of h alone; h is saved below
         ctx.save_for_backward(x, z, t1, hc, bias, s_over_den, ratio)
         return out
@@ -123,7 +131,7 @@ class DeconvUpdate(torch.autograd.Function):
             gx, gz, gh, gb = ops.update_backward(
                 lib, x, z, t1, h, bias, gout, groups=groups, m=m, sc=sc, eps=eps,
                 relu_input=relu_input, need_x=need_x, need_z=need_z, need_h=need_h,
-                need_b=need_b and bias is not None,
+                need_b=need_b and bias is not None, path=ctx.path,
                 saved=None if s_over_den is None else (s_over_den, ratio), taps=ctx.taps)
         return gx, gz, gh, gb, None, None, None, None, None, None
 

@@ -45,8 +45,21 @@ enum ndc_status {
 };
 
 /* Which implementation a call may use.  AUTO picks the fused LDS-tiled kernels when the
- * geometry is one they cover and the direct kernels otherwise. */
-enum ndc_path { NDC_PATH_AUTO = 0, NDC_PATH_DIRECT = 1, NDC_PATH_FUSED = 2 };
+ * geometry is one they cover and the direct kernels otherwise; FUSED insists on the fused
+ * kernels.  For both, the kernel FAMILY of bfloat16 3x3x3 calls is the process default
+ * (ndc_matrix_kernels).  FUSED_VECTOR and FUSED_MATRIX are FUSED with the family named by
+ * the call itself: tap sums on the vector unit (v_dot2c_f32_bf16), or on the 4x4x4 matrix
+ * instruction where those kernels cover the geometry (row widths 8, 16, 32, 64, 128; the
+ * vector-unit kernels elsewhere).  A call that names its family reads no process-wide state,
+ * so a forward call on one thread and its backward call on another (an autograd engine
+ * thread) cannot disagree, whatever a third thread does to the default. */
+enum ndc_path {
+    NDC_PATH_AUTO = 0,
+    NDC_PATH_DIRECT = 1,
+    NDC_PATH_FUSED = 2,
+    NDC_PATH_FUSED_MATRIX = 3,
+    NDC_PATH_FUSED_VECTOR = 4
+};
 
 typedef struct ndc_geom {
     int32_t batch;       /* B */
@@ -80,14 +93,15 @@ int ndc_check_geometry(const ndc_geom *g);
  * reference. */
 int ndc_backward_uses_saved(const ndc_geom *g);
 
-/* Kernel-family switch, process-wide: on = 1 lets the calls below run the bfloat16 3x3x3
- * kernels that do their tap sums on the 4x4x4 matrix instruction (row widths 8, 16, 32, 64,
- * 128), on = 0 keeps them on the vector unit (v_dot2c_f32_bf16), on < 0 only queries; returns
- * the setting in force.  Default 0: the path is specified as a stencil without matrix
+/* Process-wide DEFAULT of the kernel family, used by calls whose ndc_geom.path is AUTO or
+ * FUSED (calls with FUSED_VECTOR / FUSED_MATRIX ignore it): on = 1 lets them run the bfloat16
+ * 3x3x3 kernels that do their tap sums on the 4x4x4 matrix instruction (row widths 8, 16, 32,
+ * 64, 128), on = 0 keeps them on the vector unit (v_dot2c_f32_bf16), on < 0 only queries;
+ * returns the setting in force.  Default 0: the path is specified as a stencil without matrix
  * instructions, and the default build measures that; the other family is the faster one on
- * MI355X (config 3: 1.56 against 1.84 ms per step) and gives the same results to the bf16
- * tolerance.  Not to be changed while calls are in flight on other threads.  No counterpart
- * in the reference. */
+ * MI355X and gives the same results to the bf16 tolerance.  The setting is an atomic integer
+ * read once per call; it is the only state the library keeps between calls (besides the
+ * scratch array of ndc_forward_noalloc).  No counterpart in the reference. */
 int ndc_matrix_kernels(int on);
 
 /* Bytes of scratch `ndc_forward` needs for `g` (0 for most geometries; the bfloat16 3x3x3
@@ -202,8 +216,9 @@ int ndc_backward_profiled(const ndc_geom *g, const void *x, const void *z, const
 /*
  * Plain grouped convolution with the same tap conventions (adjoint = 0: K, 1: A), input
  * and output in g->dtype; optional on-load bias + ReLU of the input as in the forward.
- * Replaces kernels.gconv (deconver/deconvolution/kernels.py:728-759); used for
- * `reconstruct` and by tests that probe K and A separately.
+ * Replaces kernels.gconv (deconver/deconvolution/kernels.py:728-759).  The update entry points
+ * above do not call it (they apply K and A inside their own kernels); it is exported for
+ * callers and tests that need K or A alone.  Runs the direct kernels for every geometry.
  */
 int ndc_gconv(const ndc_geom *g, const void *in, const float *h, const float *bias, int adjoint,
               void *out, void *stream);

@@ -8,6 +8,7 @@ bfloat16 storage with float32 accumulation; the oracle is evaluated in float64 o
 import pytest
 import torch
 
+import deconver_amd as dc
 from deconver_amd import _lib, ops
 from oracle import ndc_oracle as O
 from tests.helpers import make_case
@@ -302,3 +303,77 @@ def test_matrix_kernel_switch_defaults_to_off_and_changes_the_kernels(matrix_swi
     assert not torch.equal(base[4], other[4])          # gh: float32, other summation order
     for a, b in zip(base, other):
         assert O.rel_err(a.float().cpu(), b.float().cpu().double()) < 2e-2
+
+
+def test_family_named_per_call_from_two_threads(matrix_switch):
+    """ndc_geom.path = FUSED_VECTOR / FUSED_MATRIX names the kernel family of one call: two
+    threads run the two families at the same time, each on its own stream, while the main thread
+    keeps flipping the process default; every call returns the bits of the family it named
+    (forward on one thread and backward on another cannot disagree)."""
+    import threading
+
+    lib = _lib_gpu()
+    C, G, sc, ks, sp, B = FUSED_GEOMS[7]
+    x, z, h, bias, gout = make_case(C, G, sc, ks, sp, B=B, dtype=torch.bfloat16, bias_shift=0.3, device="cuda")
+    kw = dict(groups=G, m=1, sc=sc, eps=1e-16, relu_input=True)
+
+    def run(path):
+        out, t1, saved = ops.update_forward(lib, x, z, h, bias, save_ratio=True, path=path, **kw)
+        return (out, t1) + tuple(ops.update_backward(lib, x, z, t1, h, bias, gout, saved=saved, path=path, **kw))
+
+    # what each family returns, from the process-wide switch with the default path
+    assert matrix_switch(False) is False
+    want = {_lib.PATH_FUSED_VECTOR: run(_lib.PATH_AUTO)}
+    assert matrix_switch(True) is True
+    want[_lib.PATH_FUSED_MATRIX] = run(_lib.PATH_AUTO)
+    matrix_switch(False)
+    torch.cuda.synchronize()
+    assert not torch.equal(want[_lib.PATH_FUSED_VECTOR][4], want[_lib.PATH_FUSED_MATRIX][4])
+
+    failures, stop = [], threading.Event()
+
+    def worker(path):
+        try:
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                for _ in range(6):
+                    got = run(path)
+                    stream.synchronize()
+                    for a, b in zip(got, want[path]):
+                        if not torch.equal(a, b):
+                            failures.append(path)
+        except Exception as e:   # noqa: BLE001 - reported below
+            failures.append(repr(e))
+
+    threads = [threading.Thread(target=worker, args=(p,)) for p in (_lib.PATH_FUSED_VECTOR, _lib.PATH_FUSED_MATRIX)]
+    for t in threads:
+        t.start()
+    flips = 0
+    while any(t.is_alive() for t in threads):
+        matrix_switch(bool(flips & 1))
+        flips += 1
+        stop.wait(0.001)
+    for t in threads:
+        t.join()
+    assert not failures, failures
+    assert flips > 0
+
+
+def test_autograd_node_names_its_family_once(matrix_switch):
+    """The update node reads the family in its forward and names it in both calls: flipping
+    the process default between forward and backward does not change the backward."""
+    C, G, sc, ks, sp, B = FUSED_GEOMS[7]
+    x, z, h, bias, gout = make_case(C, G, sc, ks, sp, B=B, dtype=torch.bfloat16, bias_shift=0.3, device="cuda")
+
+    def run(flip):
+        leaves = [t.clone().requires_grad_(True) for t in (x, z, h, bias)]
+        matrix_switch(True)
+        out = dc.deconv_update(*leaves, groups=G, m=1, sc=sc, eps=1e-16, relu_input=True)
+        if flip:
+            matrix_switch(False)
+        out.backward(gout)
+        matrix_switch(False)
+        return [t.grad.clone() for t in leaves]
+
+    for a, b in zip(run(False), run(True)):
+        assert torch.equal(a, b)

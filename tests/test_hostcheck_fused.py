@@ -192,22 +192,64 @@ def test_fused_saved_denominator_and_ratio(geom, dtype, matrix, relu, matrix_swi
                      gout.data_ptr(), None, out.data_ptr(), None, None, None, 0, None)
 
 
-def test_fused_partial_outputs():
-    C, sc, ks, sp = 2, 4, (3, 3, 3), (4, 6, 8)
+@pytest.mark.parametrize("dtype,saved,matrix,sp", [
+    (torch.float32, False, False, (4, 6, 8)),
+    (torch.float32, True, False, (4, 6, 8)),
+    (torch.bfloat16, False, False, (4, 6, 8)),
+    (torch.bfloat16, True, False, (4, 6, 8)),
+    (torch.bfloat16, True, True, (4, 7, 16)),    # matrix-instruction forward and pass 1
+    (torch.bfloat16, True, True, (3, 5, 32)),    # ... and pass 2
+])
+def test_fused_partial_outputs(dtype, saved, matrix, sp, matrix_switch):
+    """Null gx / gz / gh / gb outputs (what autograd passes for a leaf that needs no gradient):
+    every subset that is asked for equals the full call's, on the FMA kernels, the bf16 dot2
+    kernels and the bf16 matrix-instruction kernels, with and without the kept ratios."""
+    assert matrix_switch(matrix) == matrix
+    C, sc, ks = 2, 4, (3, 3, 3)
     lib = hostcheck_library()
-    x, z, h, bias, gout = make_case(C, C, sc, ks, sp, bias_shift=0.3)
-    out, t1 = ops.update_forward(lib, x, z, h, bias, groups=C, m=1, sc=sc, eps=1e-16,
-                                 relu_input=True, path=_lib.PATH_FUSED)
+    x, z, h, bias, gout = make_case(C, C, sc, ks, sp, dtype=dtype, bias_shift=0.3)
     kw = dict(groups=C, m=1, sc=sc, eps=1e-16, relu_input=True, path=_lib.PATH_FUSED)
-    full = ops.update_backward(lib, x, z, t1, h, bias, gout, **kw)
-    for mask in ((1, 0, 0, 0), (0, 1, 0, 0), (0, 0, 1, 0), (0, 0, 0, 1)):
+    host_faults(lib)
+    res = ops.update_forward(lib, x, z, h, bias, save_ratio=saved, **kw)
+    t1, sv = res[1], (res[2] if saved else None)
+    full = ops.update_backward(lib, x, z, t1, h, bias, gout, saved=sv, **kw)
+    for mask in ((1, 0, 0, 0), (0, 1, 0, 0), (0, 0, 1, 0), (0, 0, 0, 1), (0, 1, 0, 1), (1, 0, 1, 0)):
         part = ops.update_backward(lib, x, z, t1, h, bias, gout, need_x=bool(mask[0]),
                                    need_z=bool(mask[1]), need_h=bool(mask[2]),
-                                   need_b=bool(mask[3]), **kw)
+                                   need_b=bool(mask[3]), saved=sv, **kw)
         for want, a, b in zip(mask, part, full):
             assert (a is None) == (not want)
             if want:
                 assert torch.equal(a, b)
+    n, first = host_faults(lib)
+    assert n == 0, f"LDS faults: {n} ({first})"
+
+
+def test_family_named_per_call(matrix_switch):
+    """ndc_geom.path = FUSED_VECTOR / FUSED_MATRIX fixes the kernel family of a call whatever
+    the process default says; AUTO and FUSED follow the default."""
+    C, sc, ks, sp = 2, 4, (3, 3, 3), (4, 7, 16)
+    lib = hostcheck_library()
+    x, z, h, bias, gout = make_case(C, C, sc, ks, sp, dtype=torch.bfloat16, bias_shift=0.3)
+    kw = dict(groups=C, m=1, sc=sc, eps=1e-16, relu_input=True)
+
+    def run(path):
+        out, t1, sv = ops.update_forward(lib, x, z, h, bias, save_ratio=True, path=path, **kw)
+        return (out, t1) + tuple(ops.update_backward(lib, x, z, t1, h, bias, gout, saved=sv, path=path, **kw))
+
+    assert matrix_switch(False) is False
+    vec = run(_lib.PATH_FUSED)
+    assert matrix_switch(True) is True
+    mat = run(_lib.PATH_FUSED)
+    assert not torch.equal(vec[4], mat[4])   # gh: float32 sums in another order
+    for default in (False, True):
+        matrix_switch(default)
+        for path, want in ((_lib.PATH_FUSED_VECTOR, vec), (_lib.PATH_FUSED_MATRIX, mat),
+                           (_lib.PATH_AUTO, mat if default else vec)):
+            for a, b in zip(run(path), want):
+                assert torch.equal(a, b)
+    g = ops.make_geom_for(x, h, C, 1, sc, 1e-16, True, 5)
+    assert lib.check_geometry(g) != 0        # no such path value
 
 
 # rows as wide as the large 3-D configurations use (128^3, 192^3 and the widest the 3-D
