@@ -852,7 +852,7 @@ def main() -> int:
             result["train3d_steps_per_s_pytorch_route"] = t3["pytorch"]["steps_per_s"]
             result["train3d"] = {"workload": MODEL_WORKLOADS["train3d"]["text"], "routes": t3,
                                  "hip_over_pytorch": t3["hip"]["steps_per_s"] / t3["pytorch"]["steps_per_s"]}
-            if not args.matrix:
+            if "matrix_instruction_variant" in result:
                 # the same train step with the other kernel family on (see above: not the metric)
                 lib.matrix_kernels(True)
                 try:

@@ -28,6 +28,7 @@ EXPORTS = (
     "ndc_forward",
     "ndc_forward_workspace_bytes",
     "ndc_forward_noalloc",
+    "ndc_noalloc_init",
     "ndc_taps_bytes",
     "ndc_prepare_taps",
     "ndc_forward_taps",
@@ -186,6 +187,10 @@ class NdcLibrary:
         """``forward`` with the scratch in the library's own device array (no workspace)."""
         self._check(self._dll.ndc_forward_noalloc(ctypes.byref(g), x, z, h, bias, out, t1,
                                                   s_over_den, ratio, stream), "ndc_forward_noalloc")
+
+    def noalloc_init(self) -> None:
+        """Set-up of ``forward_noalloc`` on the current device (needed before a stream capture)."""
+        self._check(self._dll.ndc_noalloc_init(), "ndc_noalloc_init")
 
     def backward_workspace_bytes(self, g: Geom, need_gx, need_gz, need_gh, need_gb) -> int:
         flags = (int(need_gx), int(need_gz), int(need_gh), int(need_gb))

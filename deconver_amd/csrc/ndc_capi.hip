@@ -57,19 +57,6 @@ block_kernel_entry_w4(typename Kernel::Params p)
     Kernel::run(ex, p, (int)blockIdx.x);
 }
 
-// ... `kWavesPerSimd = 3`: 168 VGPRs.
-template <class Kernel>
-__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(3, 3)))
-block_kernel_entry_w3(typename Kernel::Params p)
-{
-    extern __shared__ __attribute__((aligned(16))) float ndc_lds[];
-    DeviceExec<typename Kernel::State> ex;
-    ex.lds = ndc_lds;
-    ex.tid = threadIdx.x;
-    ex.nthreads = blockDim.x;
-    Kernel::run(ex, p, (int)blockIdx.x);
-}
-
 template <class K, class = void> struct WavesWanted {
     static constexpr int value = 0;
 };
@@ -121,7 +108,6 @@ struct Backend {
         const size_t bytes = (size_t)lds_floats * sizeof(float);
         void (*entry)(typename Kernel::Params) = block_kernel_entry<Kernel>;
         if constexpr (WavesWanted<Kernel>::value == 4) entry = block_kernel_entry_w4<Kernel>;
-        if constexpr (WavesWanted<Kernel>::value == 3) entry = block_kernel_entry_w3<Kernel>;
         if (bytes > 64 * 1024) {
             // more dynamic LDS than the default cap: raise it for this kernel (idempotent)
             if (hipFuncSetAttribute((const void *)entry, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -198,6 +184,12 @@ int scratch_address(void **out)
 }
 
 }  // namespace
+
+extern "C" int ndc_noalloc_init(void)
+{
+    void *ptr = nullptr;
+    return scratch_address(&ptr);
+}
 
 extern "C" int ndc_forward_noalloc(const ndc_geom *g, const void *x, const void *z, const float *h,
                                    const float *bias, void *out, void *t1, void *s_over_den,

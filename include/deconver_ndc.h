@@ -145,10 +145,21 @@ int ndc_forward(const ndc_geom *g, const void *x, const void *z, const float *h,
  * with NDC_ERR_SCRATCH_LIMIT before anything is launched.  All calls on one GPU share the one
  * array: calls that may overlap on a GPU (different streams, different threads) race on it
  * and must be serialised by the caller, or use ndc_forward with a workspace of their own.
+ * The array's device address is looked up once per device (hipGetSymbolAddress, no
+ * allocation), for the device that is current when the call is made, which must be the
+ * stream's device: by ndc_noalloc_init, or else by the first ndc_forward_noalloc call on that
+ * device.  That lookup is not a stream operation and may be refused while a stream capture is
+ * in progress, so a caller that captures calls ndc_noalloc_init (or makes one call) on each
+ * device beforehand; every later call only launches kernels on `stream`.
  */
 int ndc_forward_noalloc(const ndc_geom *g, const void *x, const void *z, const float *h,
                         const float *bias, void *out, void *t1, void *s_over_den, void *ratio,
                         void *stream);
+
+/* Set-up of ndc_forward_noalloc for the current device (see above): looks up the scratch
+ * array's address there.  Allocates nothing, launches nothing; 0 or a negative ndc_status.
+ * Optional outside stream capture, idempotent, thread-safe.  No counterpart in the reference. */
+int ndc_noalloc_init(void);
 
 /*
  * Prepared filter tables.  Some kernel families read the filter from a packed table instead

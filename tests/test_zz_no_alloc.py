@@ -60,3 +60,45 @@ def test_noalloc_forward_refuses_what_does_not_fit():
                             None, None, None, torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
     assert bool((out == 7.0).all()), "a refused call must not launch anything"
+
+
+def test_noalloc_forward_allocates_nothing_and_replays_in_a_graph():
+    """After ndc_noalloc_init the entry point only launches kernels: device memory in use
+    (the driver's count and torch's) is the same before and after a call, and a call captured
+    in a HIP graph replays to the eager result, several times, with eager work and
+    synchronisations between the replays."""
+    lib = _lib.get_library()
+    lib.noalloc_init()
+    C, sp, B = 24, (8, 10, 16), 2
+    x, z, h, bias, _ = make_case(C, C, 4, (3, 3, 3), sp, B=B, dtype=torch.bfloat16, bias_shift=0.3,
+                                 seed=3, device="cuda")
+    kw = dict(groups=C, m=1, sc=4, eps=1e-16, relu_input=True)
+    ref = ops.update_forward(lib, x, z, h, bias, save_ratio=True, **kw)
+    ref = [ref[0], ref[1], *ref[2]]
+    g = ops.make_geom_for(x, h, C, 1, 4, 1e-16, True)
+    assert lib.forward_workspace_bytes(g) > 0
+    got = [torch.empty_like(z), torch.empty_like(x), torch.empty_like(z), torch.empty_like(z)]
+    args = (g, x.data_ptr(), z.data_ptr(), h.data_ptr(), bias.data_ptr(), *[t.data_ptr() for t in got])
+
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    used0, reserved0 = torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+    lib.forward_noalloc(*args, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert (torch.cuda.memory_allocated(), torch.cuda.memory_reserved()) == (used0, reserved0)
+    assert free1 == free0, "the call changed the device memory in use"
+    for a, b in zip(got, ref):
+        assert torch.equal(a, b)
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):   # (captures on a side stream, which is then the current one)
+        lib.forward_noalloc(*args, torch.cuda.current_stream().cuda_stream)
+    for rep in range(3):
+        for t in got:
+            t.fill_(float("nan"))            # the program's own eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, a, b in zip(("out", "t1", "s_over_den", "ratio"), got, ref):
+            assert torch.equal(a, b), f"{name} differs on replay {rep}"
