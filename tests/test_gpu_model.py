@@ -101,12 +101,25 @@ def test_config2_model_at_full_width_matches_float64(batch):
     backward of the Dice+BCE loss, against the same network evaluated in float64 (which takes
     the layers' PyTorch route).  Sizes the CPU oracle would need minutes for.
 
-    Forward: 1e-4 outright.  Gradients: a float32 network with ~10^7 rectifier and GELU inputs
-    sits 1e-3..1e-2 from its float64 self in single entries whatever computes the
-    deconvolution (units within rounding of zero), so every parameter gradient is held to
-    2e-2 of its largest entry and to a cosine of 0.9999 with the float64 gradient (at most one
-    tensor to 8e-2, see below)."""
+    Forward: 1e-4 outright.  Gradients: every parameter gradient within 2e-2 of the float64
+    gradient's largest entry and at a cosine above 0.9999 with it.  A float32 network with
+    ~10^7 rectifier inputs has some within rounding of zero; which of those are on depends on
+    the summation order of the library routines around the layer (it varies from process to
+    process), and one such unit can move the weight gradient of the layer it feeds by a few
+    percent.  A tensor outside the bound is therefore accepted only with that cause shown
+    (tests/kink_audit.py): the rectifier units that differ between the two networks are found
+    (mixer activations and NDC source rectifiers, the HIP route's from the very z its kernels
+    rectified), they must be few and within rounding of zero in float64, and with the float32
+    network's on/off patterns imposed on the float64 network every gradient must be within
+    1e-3 (measured: 0-10 switched units per rectifier, all below 2e-7 of their layer's scale;
+    worst gradient 1.95e-2 from the plain float64 network and 2.4e-5 from the one with the
+    patterns imposed).  That second comparison is made on every run, so the test holds the
+    whole float32 network on the HIP route to 1e-3 of float64 in every parameter gradient.
+    (tests/test_kink_audit_cpu.py: a planted 3e-2 error in one filter gradient is not
+    explained away by this.)"""
     import copy
+
+    from tests import kink_audit as KA
     net = dict(in_channels=3, out_channels=1, spatial_dims=2, encoder_depth=(1, 1, 1, 1, 1),
                encoder_width=(32, 64, 128, 256, 512), strides=(1, 2, 2, 2, 2),
                decoder_depth=(1, 1, 1, 1), kernel_size=(5, 5), groups=-1, ratio=4,
@@ -117,25 +130,65 @@ def test_config2_model_at_full_width_matches_float64(batch):
     exact = copy.deepcopy(model).double()
     for layer in _ndc_layers(model):
         assert layer.fast_path_applicable(torch.empty(1, layer.channels, 16, 16, device="cuda"))
-    y, ye = model(images), exact(images.double())
-    assert O.rel_err(y.detach(), ye.detach()) < 1e-4
+    kept = {}
+    masks = KA.record_patterns(model, lambda: kept.__setitem__("y", model(images)))
+    assert sum(k.endswith(".source") for k in masks) == len(_ndc_layers(model))
+    y = kept["y"]
     T.dice_bce_loss(y, targets).backward()
-    T.dice_bce_loss(ye, targets.double()).backward()
-    worst = {}
-    for (name, p), pe in zip(model.named_parameters(), exact.parameters()):
-        a, b = p.grad.double().flatten(), pe.grad.flatten()
-        cos = float(torch.dot(a, b) / (a.norm() * b.norm()).clamp_min(1e-300))
-        worst[name] = (O.rel_err(p.grad, pe.grad), cos)
-    bad = {k: v for k, v in worst.items() if not (v[0] < 2e-2 and v[1] > 0.9999)}
-    # Which borderline unit is on depends on the summation order of the library routines
-    # around the layer (the convolution algorithm MIOpen picks varies from process to process),
-    # so on some runs ONE unit that lies within rounding of zero differs from the float64
-    # network and moves the weight gradient of the layer it feeds by a few percent of its
-    # largest entry (seen: 3.6e-2 on one projection weight, cosine 0.99999, the other 100
-    # tensors within 1e-2).  One such tensor is accepted if it still points the same way.
-    assert len(bad) <= 1, bad
-    for k, (err, cos) in bad.items():
-        assert err < 8e-2 and cos > 0.9999, (k, err, cos)
+    grads = {n: p.grad.detach() for n, p in model.named_parameters()}
+
+    def run_exact():
+        exact.zero_grad(set_to_none=True)
+        ye = exact(images.double())
+        kept.setdefault("ye", ye.detach())     # the first, ungated evaluation
+        T.dice_bce_loss(ye, targets.double()).backward()
+        return {n: p.grad.detach().clone() for n, p in exact.named_parameters()}
+
+    report = KA.audit_gradients(grads, masks, exact, run_exact, tol=2e-2, cos_min=0.9999, gated_tol=1e-3)
+    assert O.rel_err(y.detach(), kept["ye"]) < 1e-4
+    print("switched rectifier units:", report["switched"], "outliers:", report["outliers"],
+          "worst on the same patterns:", max(e for e, _ in report["gated_errors"].values()))
+
+
+def test_rectifier_patterns_of_the_hip_route_are_recorded_and_imposed():
+    """The pieces of the criterion above on a small network: the on/off patterns recorded on
+    the HIP route (from the z handed to the kernels) agree with the float64 network's
+    pre-activation signs except for borderline units, and the float64 network evaluated with
+    those patterns imposed is the float64 network (same gradients) when none is switched."""
+    import copy
+
+    from tests import kink_audit as KA
+    cfg = dict(NET_2D)
+    torch.manual_seed(0)
+    model = dc.Deconver(**cfg).cuda()
+    exact = copy.deepcopy(model).double()
+    x = torch.rand(2, 3, 32, 24, device="cuda")
+    g = torch.randn(2, 2, 32, 24, device="cuda")
+    kept = {}
+    masks = KA.record_patterns(model, lambda: kept.__setitem__("y", model(x)))
+    n_src = sum(k.endswith(".source") for k in masks)
+    assert n_src == len(_ndc_layers(model)) and len(masks) == 2 * n_src
+    kept["y"].backward(g)
+    grads = {n: p.grad.detach() for n, p in model.named_parameters()}
+
+    def run_exact():
+        exact.zero_grad(set_to_none=True)
+        exact(x.double()).backward(g.double())
+        return {n: p.grad.detach().clone() for n, p in exact.named_parameters()}
+
+    _, pres = KA.record_patterns(exact, run_exact, keep_pre=True)
+    sw = KA.switched_units(masks, pres)
+    assert set(sw) == set(masks)
+    for name, (n, rel) in sw.items():
+        assert n <= 4 and rel < 1e-5, (name, n, rel)
+    plain = run_exact()
+    with KA.imposed_patterns(exact, masks):
+        gated = run_exact()
+    if not any(n for n, _ in sw.values()):
+        for k in plain:
+            assert torch.allclose(plain[k], gated[k], rtol=1e-9, atol=1e-12), k
+    errs = KA.grad_errors(grads, gated)
+    assert max(e for e, _ in errs.values()) < 5e-3, errs
 
 
 def test_training_step_reduces_loss_and_matches_pytorch_route():
