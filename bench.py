@@ -129,10 +129,88 @@ SWEEP_SHAPES = [   # config 5: (channels, extent, batch), bottleneck to full res
 ]
 
 
-def sweep_workload(args) -> int:
+def sweep_rows(torch, lib, ops, dev, warmup, steps):
     """Config 5: forward-only (inference: no t1, nothing kept for backward) NDC update,
-    3x3x3, ratio 4, bf16, half-normal inputs; Gvoxel/s and HBM-roofline fraction (9 U e
-    algorithmic bytes) per shape.  `value` is the geometric mean over the shapes."""
+    3x3x3, ratio 4, bf16, half-normal inputs; per shape the time of one call, Gvoxel/s and the
+    HBM-roofline fraction on the 9 U e algorithmic bytes."""
+    rows = []
+    for C, n, B in SWEEP_SHAPES:
+        x, z, h, bias, _, sc = make_inputs(torch, torch.bfloat16, dev, B, C, (n, n, n), (3, 3, 3), 4)
+        kw = dict(groups=C, m=1, sc=sc, eps=1e-16, relu_input=True, need_t1=False)
+        for _ in range(warmup):
+            ops.update_forward(lib, x, z, h, bias, **kw)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            ops.update_forward(lib, x, z, h, bias, **kw)
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / steps
+        vox, U = B * n ** 3, B * C * n ** 3
+        rows.append({"channels": C, "extent": n, "batch": B, "ms": ms,
+                     "Gvoxel_per_s": vox / (ms * 1e-3) / 1e9,
+                     "channel_voxels_per_s": U / (ms * 1e-3),
+                     "algorithmic_bytes": 9 * U * 2,
+                     "hbm_frac": 9 * U * 2 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS})
+        del x, z
+    return rows
+
+
+LAYERS_2D = [   # the 2-D 5x5 form: (name, channels, extent, batch)
+    ("config 1: B 1, 32 ch, 64^2", 32, 64, 1),
+    ("config 2 stage 0: B 8, 32 ch, 256^2", 32, 256, 8),
+]
+
+
+def layers_2d_rows(torch, lib, ops, dev, warmup, steps):
+    """The 2-D 5x5 form of the update node (depthwise, ratio 4, float32 storage: the reference's
+    own precision): forward + backward with the forward's ratios kept, per shape the time of
+    one step, of its kernels, Gvoxel/s and the HBM-roofline fraction on 23 U e (forward alone
+    on 9 U e)."""
+    rows = []
+    for name, C, n, B in LAYERS_2D:
+        x, z, h, bias, g, sc = make_inputs(torch, torch.float32, dev, B, C, (n, n), (5, 5), 4)
+        kw = dict(groups=C, m=1, sc=sc, eps=1e-16, relu_input=True)
+        keep = lib.backward_uses_saved(ops.make_geom_for(x, h, C, 1, sc, 1e-16, True))
+
+        def step(pt=None):
+            res = ops.update_forward(lib, x, z, h, bias, save_ratio=keep, **kw)
+            return ops.update_backward(lib, x, z, res[1], h, bias, g, pass_times=pt,
+                                       saved=res[2] if keep else None, **kw)
+
+        for _ in range(warmup):
+            step()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            step()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / steps
+        f0, f1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        f0.record()
+        for _ in range(steps):
+            ops.update_forward(lib, x, z, h, bias, save_ratio=keep, **kw)
+        f1.record()
+        torch.cuda.synchronize()
+        fwd_ms = f0.elapsed_time(f1) / steps
+        pt = []
+        step(pt)
+        vox, U = B * n * n, B * C * n * n
+        rows.append({"layer": name, "channels": C, "extent": n, "batch": B, "dtype": "f32",
+                     "ms": ms, "forward_ms": fwd_ms,
+                     "backward_kernel_ms": {"pass1": pt[0], "pass2": pt[1], "reduce": pt[2]},
+                     "Gvoxel_per_s": vox / (ms * 1e-3) / 1e9,
+                     "channel_voxels_per_s": U / (ms * 1e-3),
+                     "algorithmic_bytes": 23 * U * 4,
+                     "hbm_frac": 23 * U * 4 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "forward_hbm_frac": 9 * U * 4 / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS})
+        del x, z, g
+    return rows
+
+
+def sweep_workload(args) -> int:
+    """Config 5 alone (see sweep_rows); `value` is the geometric mean over the shapes."""
     import torch
 
     from deconver_amd import _lib, ops
@@ -142,25 +220,7 @@ def sweep_workload(args) -> int:
         return 2
     lib = _lib.get_library()
     dev = torch.device("cuda:0")
-    rows = []
-    for C, n, B in SWEEP_SHAPES:
-        x, z, h, bias, _, sc = make_inputs(torch, torch.bfloat16, dev, B, C, (n, n, n), (3, 3, 3), 4)
-        kw = dict(groups=C, m=1, sc=sc, eps=1e-16, relu_input=True, need_t1=False)
-        for _ in range(args.warmup):
-            ops.update_forward(lib, x, z, h, bias, **kw)
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(args.steps):
-            ops.update_forward(lib, x, z, h, bias, **kw)
-        e1.record()
-        torch.cuda.synchronize()
-        ms = e0.elapsed_time(e1) / args.steps
-        vox, U = B * n ** 3, B * C * n ** 3
-        rows.append({"channels": C, "extent": n, "batch": B, "ms": ms,
-                     "Gvoxel_per_s": vox / (ms * 1e-3) / 1e9,
-                     "channel_voxels_per_s": U / (ms * 1e-3),
-                     "hbm_frac": 9 * U * 2 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS})
-        del x, z
+    rows = sweep_rows(torch, lib, ops, dev, args.warmup, args.steps)
     gmean = math.exp(sum(math.log(r["Gvoxel_per_s"]) for r in rows) / len(rows))
     print(json.dumps({
         "metric": "NDC mixer forward-only Gvoxel/s (geometric mean over the sweep)",
@@ -170,7 +230,8 @@ def sweep_workload(args) -> int:
         "data": "synthetic",
         "config": {"workload": "config 5: forward-only NDC update shape sweep, 3x3x3, ratio 4, "
                                "bf16 storage / float32 accumulation, inference form"},
-        "shapes": rows, "roofline": None, "cpu_baseline": None}))
+        "shapes": rows, "layers_2d": layers_2d_rows(torch, lib, ops, dev, args.warmup, args.steps),
+        "roofline": None, "cpu_baseline": None}))
     return 0
 
 
@@ -607,6 +668,8 @@ def main() -> int:
                          "not the specified path, reported for comparison")
     ap.add_argument("--no-train", action="store_true",
                     help="skip the Deconver-3D train-step leg that follows the timed region")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the config-5 forward sweep and the 2-D 5x5 layers that follow the timed region")
     ap.add_argument("--recompute", action="store_true",
                     help="backward re-gathers the denominator and ratio (as the reference does) "
                          "instead of reading the forward's copies")
@@ -836,6 +899,19 @@ def main() -> int:
             "step_frac": sum(least.values()) / sum(k_ms[k] for k in least),
         }
     _progress(f"update node: {ms_per_step:.3f} ms per step")
+    if not args.no_extras and not args.matrix:
+        # outside the timed region, about a second: the other shapes the baseline asks to be
+        # reported -- config 5's forward-only sweep (bf16) and the 2-D 5x5 form (float32)
+        del x, z, g
+        torch.cuda.empty_cache()
+        x = z = g = None
+        result["sweep"] = {"workload": "config 5: forward-only NDC update, 3x3x3, ratio 4, bf16, inference "
+                                       "form; hbm_frac on 9 U e",
+                           "shapes": sweep_rows(torch, lib, ops, dev, 3, 10)}
+        result["layers_2d"] = {"workload": "2-D 5x5 update node, depthwise, ratio 4, float32, forward + "
+                                           "backward; hbm_frac on 23 U e",
+                               "layers": layers_2d_rows(torch, lib, ops, dev, 3, 10)}
+        _progress("config-5 sweep and 2-D layers done")
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(torch)
         _progress("CPU baseline done")
@@ -843,9 +919,15 @@ def main() -> int:
         # the second half of the metric, outside the timed region above: Deconver-3D train
         # steps per second (config 4) with the NDC layers on the HIP kernels and, for
         # reference, on the layers' PyTorch route on the same GPU
-        del x, z, g
+        x = z = g = None
         torch.cuda.empty_cache()
         try:
+            if "layers_2d" in result:
+                # config 2 (model level): the 2-D network's forward + backward on the HIP route
+                m2 = run_model_routes("model2d", ["hip"], warmup=2, steps=5)["hip"]
+                result["layers_2d"]["model2d_steps_per_s"] = m2["steps_per_s"]
+                result["layers_2d"]["model2d_ms_per_step"] = m2["ms_per_step"]
+                result["layers_2d"]["model2d_workload"] = MODEL_WORKLOADS["model2d"]["text"]
             t3 = run_model_routes("train3d", ["hip"], warmup=2, steps=5)
             t3.update(run_model_routes("train3d", ["pytorch"], warmup=1, steps=2))
             result["train3d_steps_per_s"] = t3["hip"]["steps_per_s"]

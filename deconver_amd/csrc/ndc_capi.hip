@@ -30,6 +30,29 @@ __global__ void __launch_bounds__(256) block_reduce_kernel(float *out, F partial
     if (tid == 0) out[blockIdx.x] = buf[0];
 }
 
+// out[o] = sum over p < nparts of term(o, p) for o < nout.  A workgroup sums 32 outputs:
+// thread (o, j), j < 8, adds the terms p = j, j + 8, ... in order, then thread (o, 0) adds the
+// eight partial sums in order -- a fixed association, so results are reproducible.  Threads
+// with consecutive o are neighbours, so a `term` that is contiguous in o reads coalesced.
+template <class F>
+__global__ void __launch_bounds__(256) strided_sum_kernel(int nout, int nparts, float *out, F term)
+{
+    __shared__ float buf[8][33];
+    const int ox = threadIdx.x & 31, j = threadIdx.x >> 5;
+    const int o = (int)blockIdx.x * 32 + ox;
+    float acc = 0.f;
+    if (o < nout)
+        for (int p = j; p < nparts; p += 8) acc += term(o, p);
+    buf[j][ox] = acc;
+    __syncthreads();
+    if (j == 0 && o < nout) {
+        float total = 0.f;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) total += buf[k][ox];
+        out[o] = total;
+    }
+}
+
 // One workgroup of an LDS-tiled kernel.  512 threads at most, so up to 256 VGPRs per lane.
 template <class Kernel>
 __global__ void __launch_bounds__(512) block_kernel_entry(typename Kernel::Params p)
@@ -131,6 +154,15 @@ struct Backend {
         if (blocks > (1LL << 20)) blocks = 1LL << 20;  // grid-stride beyond that
         hipLaunchKernelGGL(elementwise_kernel<F>, dim3((unsigned)blocks), dim3(256), 0,
                            (hipStream_t)stream, n, f);
+        return check();
+    }
+
+    static constexpr int kSumSlices = 8;
+    template <class F> static int strided_sum(int nout, int nparts, void *stream, float *out, F term)
+    {
+        if (nout <= 0) return 0;
+        hipLaunchKernelGGL(strided_sum_kernel<F>, dim3((unsigned)((nout + 31) / 32)), dim3(256), 0,
+                           (hipStream_t)stream, nout, nparts, out, term);
         return check();
     }
 

@@ -917,10 +917,13 @@ struct Bwd1Kernel {
                                             NDC_UNROLL
                                             for (int i = 0; i < SC; ++i)
                                                 NDC_UNROLL
-                                                for (int c = 0; c < RW; ++c)
-                                                    st.gacc[i][(td * KH + th) * KW + tw] +=
-                                                        acc[0][i][rr][c] * v[0][c + KW - 1 - tw] +
-                                                        acc[1][i][rr][c] * v[1][c + KW - 1 - tw];
+                                                for (int c = 0; c < RW; ++c) {
+                                                    // two fused multiply-adds (a sum of two
+                                                    // products added on costs a third instruction)
+                                                    float &ga = st.gacc[i][(td * KH + th) * KW + tw];
+                                                    ga += acc[0][i][rr][c] * v[0][c + KW - 1 - tw];
+                                                    ga += acc[1][i][rr][c] * v[1][c + KW - 1 - tw];
+                                                }
                                     }
                                 }
                             });

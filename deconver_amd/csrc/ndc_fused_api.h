@@ -451,31 +451,21 @@ static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const T
     if (st) return st;
     tm.mark();
 
-    // combine the per-workgroup partial sums: fixed order, so results are reproducible
+    // combine the per-workgroup partial sums: a fixed association, so results are reproducible
     const int C = q.G, SC = q.sc, ntile = pl.tb.ntile * pl.tb.nseg, B = q.B;
     if (gh) {
-        st = BE::elementwise((long long)C * kt, stream, [=] NDC_LAMBDA(long long idx) {
-            const int c = (int)(idx / kt), r = (int)(idx % kt);
-            float acc = 0.f;
-            for (int b = 0; b < B; ++b)
-                for (int tl = 0; tl < ntile; ++tl) {
-                    const long long blk = ((long long)b * C + c) * ntile + tl;
-                    acc += part1[blk * kt + r] + part2[blk * (kt + SC) + r];
-                }
-            gh[idx] = acc;
+        st = BE::strided_sum(C * kt, B * ntile, stream, gh, [=] NDC_LAMBDA(int o, int pi) {
+            const int c = o / kt, r = o % kt;
+            const long long blk = ((long long)(pi / ntile) * C + c) * ntile + pi % ntile;
+            return part1[blk * kt + r] + part2[blk * (kt + SC) + r];
         });
         if (st) return st;
     }
     if (gb) {
-        st = BE::elementwise((long long)C * SC, stream, [=] NDC_LAMBDA(long long idx) {
-            const int c = (int)(idx / SC), i = (int)(idx % SC);
-            float acc = 0.f;
-            for (int b = 0; b < B; ++b)
-                for (int tl = 0; tl < ntile; ++tl) {
-                    const long long blk = ((long long)b * C + c) * ntile + tl;
-                    acc += part2[blk * (kt + SC) + kt + i];
-                }
-            gb[idx] = acc;
+        st = BE::strided_sum(C * SC, B * ntile, stream, gb, [=] NDC_LAMBDA(int o, int pi) {
+            const int c = o / SC, i = o % SC;
+            const long long blk = ((long long)(pi / ntile) * C + c) * ntile + pi % ntile;
+            return part2[blk * (kt + SC) + kt + i];
         });
         if (st) return st;
     }

@@ -22,6 +22,7 @@ struct NoTimer {
 
 struct Backend {
     static constexpr bool is_device = false;
+    static constexpr int kSumSlices = 8;
     typedef NoTimer Timer;
 
     template <class Kernel>
@@ -38,6 +39,22 @@ struct Backend {
     template <class F> static int elementwise(long long n, void *, F f)
     {
         for (long long idx = 0; idx < n; ++idx) f(idx);
+        return 0;
+    }
+
+    // out[o] = sum_p term(o, p) in the association of the HIP build (kSumSlices interleaved
+    // partial sums, then those in order)
+    template <class F> static int strided_sum(int nout, int nparts, void *, float *out, F term)
+    {
+        for (int o = 0; o < nout; ++o) {
+            float total = 0.f;
+            for (int j = 0; j < kSumSlices; ++j) {
+                float acc = 0.f;
+                for (int p = j; p < nparts; p += kSumSlices) acc += term(o, p);
+                total += acc;
+            }
+            out[o] = total;
+        }
         return 0;
     }
 
