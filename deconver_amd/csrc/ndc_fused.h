@@ -124,12 +124,16 @@ static inline bool make_tile(const March &m, int RH, int RW, int target_threads,
 // Split the marching axis so that a launch has enough wavefronts to fill the chip: a
 // workgroup that owns planes [d0, d1) marches over them plus 2*PD warm-up planes on each
 // side (whose outputs its neighbours own), so segments are kept >= 16*PD planes long.
-static inline void split_march(const March &m, long long blocks, Tile &t)
+// target: wavefronts the launch should have (about the number resident at once: more segments
+// than that only add warm-up planes)
+static inline void split_march(const March &m, long long blocks, Tile &t, long long target)
 {
     const int PD = m.KD / 2;
     const long long waves = blocks * (t.NT / 64);
-    const long long target = 4096;   // about four wavefronts per SIMD
-    const int min_seg = PD > 0 ? 16 * PD : m.D;
+#ifndef NDC_MIN_SEG
+#define NDC_MIN_SEG 4
+#endif
+    const int min_seg = PD > 0 ? NDC_MIN_SEG * PD : m.D;
     if (waves >= target || m.D < 2 * min_seg) return;
     long long want = (target + waves - 1) / waves;
     const int max_seg = m.D / min_seg;

@@ -111,6 +111,14 @@ static inline std::atomic<int> &matrix_default()
     return on;
 }
 
+#ifndef NDC_SPLIT_F
+#define NDC_SPLIT_F 4096
+#endif
+#ifndef NDC_SPLIT_B
+#define NDC_SPLIT_B 2048
+#endif
+static const long long kSplitWavesF = NDC_SPLIT_F, kSplitWavesB = NDC_SPLIT_B;
+
 struct Plan {
     Variant v;
     March m;
@@ -149,8 +157,9 @@ static inline bool make_plan_for(const KGeom &q, Plan &pl, bool pairs_ok, int dt
     if (!make_tile(pl.m, pl.v.RHF, pl.v.RWF, tn.threads_f, pl.tf)) return false;
     if (!make_tile(pl.m, pl.v.RHB, pl.v.RWB, tn.threads_b, pl.tb)) return false;
     if (tn.split) {
-        split_march(pl.m, (long long)q.B * q.G * pl.tf.ntile, pl.tf);
-        split_march(pl.m, (long long)q.B * q.G * pl.tb.ntile, pl.tb);
+        // the forward keeps four wavefronts per SIMD resident, the backward kernels two
+        split_march(pl.m, (long long)q.B * q.G * pl.tf.ntile, pl.tf, kSplitWavesF);
+        split_march(pl.m, (long long)q.B * q.G * pl.tb.ntile, pl.tb, kSplitWavesB);
     }
 #define X(kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_)                                        \
     if (NDC_IS_VARIANT(pl, kd_, kh_, kw_, sc_, rhf_, rwf_, rhb_, rwb_))                      \
