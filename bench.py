@@ -8,6 +8,7 @@
     python bench.py --workload valu                                       (instruction-issue ceiling probe)
     python bench.py --workload train3d|model2d [--ndc hip|pytorch|both]   (model level, below)
     python bench.py --workload mixer [--dtype bf16|fp32]                  (one DeconvMixer, fwd+bwd)
+    python bench.py --workload layout                                     (channels-last copies around the update)
 
 One step = one forward + one backward (input-, source-, filter- and bias-gradient) of the
 update node on config 3 of the baseline: batch 2, 128 depthwise channels, 64^3 voxels,
@@ -656,6 +657,74 @@ def mixer_workload(args) -> int:
     return 0
 
 
+LAYOUT_SHAPES = [   # (name, batch, channels, extent): the update's x has C channels, its z 4 C
+    ("config 3: B 2, 128 ch, 64^3", 2, 128, 64),
+    ("config 4 stage 0: B 2, 64 ch, 128^3", 2, 64, 128),
+]
+
+
+def layout_workload(args) -> int:
+    """What a caller that holds channels-last tensors pays before the update: the kernels read
+    channel-first (B, C, D, H, W) tensors, so `torch.channels_last_3d` inputs are copied into
+    that layout by the autograd node (x and z before the forward, gout before the backward,
+    and gx / gz come back channel-first).  Times those copies (bf16) next to the update's own
+    forward + backward on the same shapes."""
+    import torch
+
+    from deconver_amd import _lib, ops
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    lib = _lib.get_library()
+    dev = torch.device("cuda:0")
+    rows = []
+
+    def timed(fn):
+        for _ in range(args.warmup):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / args.steps
+
+    for name, B, C, n in LAYOUT_SHAPES:
+        x, z, h, bias, g, sc = make_inputs(torch, torch.bfloat16, dev, B, C, (n, n, n), (3, 3, 3), 4)
+        kw = dict(groups=C, m=1, sc=sc, eps=1e-16, relu_input=True)
+        x_cl = x.contiguous(memory_format=torch.channels_last_3d)
+        z_cl = z.contiguous(memory_format=torch.channels_last_3d)
+        ms_x = timed(lambda: x_cl.contiguous())
+        ms_z = timed(lambda: z_cl.contiguous())
+        ms_back = timed(lambda: z.contiguous(memory_format=torch.channels_last_3d))
+
+        def step():
+            res = ops.update_forward(lib, x, z, h, bias, save_ratio=True, **kw)
+            ops.update_backward(lib, x, z, res[1], h, bias, g, saved=res[2], **kw)
+
+        ms_step = timed(step)
+        U = B * C * n ** 3
+        # a step that is handed x, z, gout channels-last and must return gx, gz channels-last
+        extra = ms_x + 2 * ms_z + (ms_back + ms_x)
+        rows.append({"shape": name, "update_fwd_bwd_ms": ms_step,
+                     "x_to_channel_first_ms": ms_x, "z_to_channel_first_ms": ms_z,
+                     "z_to_channels_last_ms": ms_back,
+                     "copy_GBs_z": 2 * 4 * U * 2 / (ms_z * 1e-3) / 1e9,
+                     "copies_per_step_ms": extra, "copies_over_update": extra / ms_step})
+        del x, z, g, x_cl, z_cl
+    print(json.dumps({
+        "metric": "layout copies around the NDC update, ms", "value": rows[0]["copies_per_step_ms"],
+        "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": rows[0]["copies_per_step_ms"], "higher_is_better": False, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "torch.channels_last_3d <-> channel-first copies of the update's "
+                               "operands (x, z, gout in; gx, gz out), bf16"},
+        "shapes": rows, "roofline": None, "cpu_baseline": None}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -678,7 +747,7 @@ def main() -> int:
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     ap.add_argument("--build-probe", action="store_true",
                     help="with --workload valu: compile the probe (no GPU needed) and exit")
-    ap.add_argument("--workload", choices=("ndc", "sweep", "accuracy", "grid", "valu", "train3d", "model2d", "mixer"),
+    ap.add_argument("--workload", choices=("ndc", "sweep", "accuracy", "grid", "valu", "train3d", "model2d", "mixer", "layout"),
                     default="ndc",
                     help="ndc: the headline update node (default); the others are model level")
     ap.add_argument("--ndc", choices=("hip", "pytorch", "both"), default="hip",
@@ -701,6 +770,8 @@ def main() -> int:
         return valu_workload(args)
     if args.workload == "mixer":
         return mixer_workload(args)
+    if args.workload == "layout":
+        return layout_workload(args)
     if args.workload != "ndc":
         return model_workload(args)
 

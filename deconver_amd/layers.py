@@ -72,7 +72,10 @@ class _PointwiseLinear(torch.autograd.Function):
                     acc += torch.bmm(a, c).float().sum(0)
                 gw = acc.to(weight.dtype)
         if ctx.has_bias and ctx.needs_input_grad[2]:
-            gb = gy.sum((0, 2), dtype=torch.float32)
+            # rows first (contiguous runs of the voxel axis), then the few per-sample sums: the
+            # library's one-call reduction of a (B, C, N) tensor over B and N runs at a tenth of
+            # the memory bandwidth (0.19 ms at 2 x 128 x 64^3 in bf16)
+            gb = gy.sum(2, dtype=torch.float32).sum(0)
         return gx, gw, gb
 
 
