@@ -273,6 +273,8 @@ template <class BE> struct Dot2Launch<BE, bf16_t> {
         if (pl.mfmaf)
             return BE::template block_kernel<FwdKernelM<kDot2RH>>(p, pl.nblk_f, pl.tf.NT,
                                                                    FwdKernelM<kDot2RH>::lds_floats(pl.tf), stream);
+        if (p.s_over_den && p.ratio)
+            return BE::template block_kernel<FwdKernelB<kDot2RH, true>>(p, pl.nblk_f, pl.tf.NT, pl.lds_f, stream);
         return BE::template block_kernel<FwdKernelB<kDot2RH>>(p, pl.nblk_f, pl.tf.NT, pl.lds_f, stream);
     }
     // saved: the call brought the forward's s/d and n/d

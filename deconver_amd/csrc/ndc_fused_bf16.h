@@ -283,7 +283,11 @@ NDC_D void stream_rows(Exec &ex, Addr addr, Body body, const uint32_t (*first)[N
 
 // =================================================================== forward (bf16, dot2)
 
-template <int RH_> struct FwdKernelB {
+// KEEP: the call keeps s/d and n/d for backward (both tensors are there); without it the code
+// that forms and stores them is not compiled in (as a run-time condition it cost a branch per
+// row and channel, each reloading a spilled buffer resource).
+template <int RH_, bool KEEP_ = false> struct FwdKernelB {
+    static constexpr bool KEEP = KEEP_;
     static constexpr int KD = 3, KH = 3, KW = 3, SC = 4, RH = RH_, RW = 2;
     static constexpr int PD = 1, PH = 1, PW = 1, KT = 27;
     // staging slots per thread: thread (strip, lane) stages rows strip, strip + S, ... of the
@@ -339,9 +343,9 @@ template <int RH_> struct FwdKernelB {
         const BufRef xb_ = make_buf(p.x + cbase, xbytes), zb_ = make_buf(p.z + cbase * SC, sbytes);
         const BufRef ob_ = make_buf(p.out + cbase * SC, sbytes);
         const BufRef tb_ = make_buf(p.t1 ? p.t1 + cbase : nullptr, xbytes);
-        const BufRef db_ = make_buf(p.s_over_den ? p.s_over_den + cbase * SC : nullptr, sbytes);
-        const BufRef rb_ = make_buf(p.ratio ? p.ratio + cbase * SC : nullptr, sbytes);
-        const bool have_t1 = p.t1 != nullptr, have_saved = p.s_over_den != nullptr;
+        const BufRef db_ = make_buf(KEEP ? p.s_over_den + cbase * SC : nullptr, sbytes);
+        const BufRef rb_ = make_buf(KEEP ? p.ratio + cbase * SC : nullptr, sbytes);
+        const bool have_t1 = p.t1 != nullptr;
         UniformF tab = as_uniform(p.wtab + (long long)id.c * kTabWords);
         const int r0 = id.r0;
         const int nthreads = ex.nthreads;
@@ -565,7 +569,7 @@ template <int RH_> struct FwdKernelB {
                             v[c] = s * rt[c];
                         }
                         buf_st<true>(ob_, st.ooff[r], oj + i * cplane2, pack_bf16x2(v[0], v[1]));
-                        if (have_saved) {
+                        if (KEEP) {
                             buf_st<true>(db_, st.ooff[r], oj + i * cplane2, pack_bf16x2(rd[0], rd[1]));
                             buf_st<true>(rb_, st.ooff[r], oj + i * cplane2, pack_bf16x2(rt[0], rt[1]));
                         }
