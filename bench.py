@@ -699,6 +699,11 @@ def layout_workload(args) -> int:
         ms_x = timed(lambda: x_cl.contiguous())
         ms_z = timed(lambda: z_cl.contiguous())
         ms_back = timed(lambda: z.contiguous(memory_format=torch.channels_last_3d))
+        # the same copies by the library's tiled transposition (ndc_relayout)
+        lx = timed(lambda: ops.to_channel_first(lib, x_cl))
+        lz = timed(lambda: ops.to_channel_first(lib, z_cl))
+        lback = timed(lambda: ops.to_channels_last(lib, z))
+        assert torch.equal(ops.to_channel_first(lib, z_cl), z) and torch.equal(ops.to_channels_last(lib, z), z_cl)
 
         def step():
             res = ops.update_forward(lib, x, z, h, bias, save_ratio=True, **kw)
@@ -707,17 +712,23 @@ def layout_workload(args) -> int:
         ms_step = timed(step)
         U = B * C * n ** 3
         # a step that is handed x, z, gout channels-last and must return gx, gz channels-last
-        extra = ms_x + 2 * ms_z + (ms_back + ms_x)
+        # (x, z, gout in; out, gz and gx out: gx takes about what x does)
+        extra = ms_x + 2 * ms_z + 2 * ms_back + ms_x
+        lextra = lx + 2 * lz + 2 * lback + lx
         rows.append({"shape": name, "update_fwd_bwd_ms": ms_step,
-                     "x_to_channel_first_ms": ms_x, "z_to_channel_first_ms": ms_z,
-                     "z_to_channels_last_ms": ms_back,
-                     "copy_GBs_z": 2 * 4 * U * 2 / (ms_z * 1e-3) / 1e9,
-                     "copies_per_step_ms": extra, "copies_over_update": extra / ms_step})
+                     "torch_copy": {"x_to_channel_first_ms": ms_x, "z_to_channel_first_ms": ms_z,
+                                    "z_to_channels_last_ms": ms_back,
+                                    "GBs_z_to_channel_first": 2 * 4 * U * 2 / (ms_z * 1e-3) / 1e9,
+                                    "per_step_ms": extra, "over_update": extra / ms_step},
+                     "ndc_relayout": {"x_to_channel_first_ms": lx, "z_to_channel_first_ms": lz,
+                                      "z_to_channels_last_ms": lback,
+                                      "GBs_z_to_channel_first": 2 * 4 * U * 2 / (lz * 1e-3) / 1e9,
+                                      "per_step_ms": lextra, "over_update": lextra / ms_step}})
         del x, z, g, x_cl, z_cl
     print(json.dumps({
-        "metric": "layout copies around the NDC update, ms", "value": rows[0]["copies_per_step_ms"],
+        "metric": "layout copies around the NDC update, ms", "value": rows[0]["ndc_relayout"]["per_step_ms"],
         "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": rows[0]["copies_per_step_ms"], "higher_is_better": False, "scaling": "weak",
+        "ms_per_step": rows[0]["ndc_relayout"]["per_step_ms"], "higher_is_better": False, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "torch.channels_last_3d <-> channel-first copies of the update's "
                                "operands (x, z, gout in; gx, gz out), bf16"},

@@ -37,6 +37,7 @@ EXPORTS = (
     "ndc_backward",
     "ndc_backward_profiled",
     "ndc_gconv",
+    "ndc_relayout",
 )
 
 
@@ -102,6 +103,8 @@ class NdcLibrary:
                                    ctypes.c_size_t, vp]
         d.ndc_backward_profiled.argtypes = d.ndc_backward.argtypes + [ctypes.POINTER(ctypes.c_float)]
         d.ndc_gconv.argtypes = [gp, vp, fp, fp, ctypes.c_int, vp, vp]
+        d.ndc_relayout.argtypes = [vp, vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                                   ctypes.c_int, ctypes.c_int, vp]
         d.ndc_taps_bytes.restype = ctypes.c_size_t
         d.ndc_taps_bytes.argtypes = [gp]
         d.ndc_prepare_taps.argtypes = [gp, fp, vp, ctypes.c_size_t, vp]
@@ -217,6 +220,13 @@ class NdcLibrary:
     def gconv(self, g: Geom, inp, h, bias, adjoint: bool, out, stream) -> None:
         self._check(self._dll.ndc_gconv(ctypes.byref(g), inp, h, bias, int(adjoint), out, stream),
                     "ndc_gconv")
+
+
+    def relayout(self, src: int, dst: int, batch: int, channels: int, spatial: int, dtype: int,
+                 to_channels_last: bool, stream) -> None:
+        """Channels-last (B, S, C) <-> channel-first (B, C, S) copy of an activation tensor."""
+        self._check(self._dll.ndc_relayout(src, dst, batch, channels, spatial, dtype,
+                                           int(bool(to_channels_last)), stream), "ndc_relayout")
 
 
 _lock = threading.Lock()

@@ -379,6 +379,22 @@ int ndc_backward_profiled(const ndc_geom *g, const void *x, const void *z, const
                          workspace, workspace_bytes, stream, pass_ms);
 }
 
+int ndc_relayout(const void *src, void *dst, int64_t batch, int64_t channels, int64_t spatial,
+                 int dtype, int to_channels_last, void *stream)
+{
+    if (!src || !dst) return NDC_ERR_NULL;
+    if (dtype != NDC_F32 && dtype != NDC_BF16) return NDC_ERR_DTYPE;
+    if (batch < 1 || channels < 1 || spatial < 1 ||
+        (long double)batch * channels * spatial > 9.0e15L)
+        return NDC_ERR_GEOMETRY;
+    if (src == dst) return NDC_ERR_GEOMETRY;
+    // channels-last (B, S, C) -> channel-first (B, C, S) transposes S x C matrices, the other
+    // direction C x S ones
+    const long long R = to_channels_last ? channels : spatial, K = to_channels_last ? spatial : channels;
+    const int st = ndc::Backend::transpose(src, dst, batch, R, K, dtype == NDC_BF16 ? 2 : 4, stream);
+    return st == -2 ? (int)NDC_ERR_GEOMETRY : st;
+}
+
 int ndc_gconv(const ndc_geom *g, const void *in, const float *h, const float *bias, int adjoint,
               void *out, void *stream)
 {

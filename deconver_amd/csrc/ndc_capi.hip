@@ -53,6 +53,67 @@ __global__ void __launch_bounds__(256) strided_sum_kernel(int nout, int nparts, 
     }
 }
 
+// Batched matrix transposition dst[b][k][r] = src[b][r][k] (R rows, K columns per batch entry)
+// of 16-bit elements, two at a time: a workgroup moves a 64 x 64 tile through LDS, reading
+// 32-bit words along K and writing 32-bit words along R (R, K even, both pointers 4-byte
+// aligned).  The copy between the channels-last layout (B, S, C) and the channel-first layout
+// (B, C, S) the update kernels read is this transposition with (R, K) = (S, C) or (C, S).
+__global__ void __launch_bounds__(256)
+transpose_pairs_kernel(const uint32_t *src, uint32_t *dst, long long R, long long K, long long tiles_r,
+                       long long tiles_k)
+{
+    __shared__ uint16_t tile[64][66];
+    long long blk = blockIdx.x;
+    const long long tk = blk % tiles_k;
+    blk /= tiles_k;
+    const long long tr = blk % tiles_r, b = blk / tiles_r;
+    const long long row0 = tr * 64, col0 = tk * 64;
+    const uint32_t *s = src + b * (R * K / 2);
+    uint32_t *d = dst + b * (R * K / 2);
+    const int w = threadIdx.x & 31, q = threadIdx.x >> 5;
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+        const int r = q + 8 * it;
+        uint32_t v = 0u;
+        if (row0 + r < R && col0 + 2 * w < K) v = s[((row0 + r) * K + col0) / 2 + w];
+        *reinterpret_cast<uint32_t *>(&tile[r][2 * w]) = v;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+        const int k = q + 8 * it;
+        if (col0 + k < K && row0 + 2 * w < R)
+            d[((col0 + k) * R + row0) / 2 + w] = (uint32_t)tile[2 * w][k] | ((uint32_t)tile[2 * w + 1][k] << 16);
+    }
+}
+
+// The same for elements of ESZ bytes (2 or 4), one at a time: any R, K and alignment.
+template <typename E>
+__global__ void __launch_bounds__(256)
+transpose_kernel(const E *src, E *dst, long long R, long long K, long long tiles_r, long long tiles_k)
+{
+    __shared__ E tile[32][33];
+    long long blk = blockIdx.x;
+    const long long tk = blk % tiles_k;
+    blk /= tiles_k;
+    const long long tr = blk % tiles_r, b = blk / tiles_r;
+    const long long row0 = tr * 32, col0 = tk * 32;
+    const E *s = src + b * R * K;
+    E *d = dst + b * R * K;
+    const int w = threadIdx.x & 31, q = threadIdx.x >> 5;
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+        const int r = q + 8 * it;
+        tile[r][w] = (row0 + r < R && col0 + w < K) ? s[(row0 + r) * K + col0 + w] : (E)0;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+        const int k = q + 8 * it;
+        if (col0 + k < K && row0 + w < R) d[(col0 + k) * R + row0 + w] = tile[w][k];
+    }
+}
+
 // One workgroup of an LDS-tiled kernel.  512 threads at most, so up to 256 VGPRs per lane.
 template <class Kernel>
 __global__ void __launch_bounds__(512) block_kernel_entry(typename Kernel::Params p)
@@ -154,6 +215,28 @@ struct Backend {
         if (blocks > (1LL << 20)) blocks = 1LL << 20;  // grid-stride beyond that
         hipLaunchKernelGGL(elementwise_kernel<F>, dim3((unsigned)blocks), dim3(256), 0,
                            (hipStream_t)stream, n, f);
+        return check();
+    }
+
+    // dst[b][k][r] = src[b][r][k] for `batch` matrices of R x K elements of esz (2 or 4) bytes
+    static int transpose(const void *src, void *dst, long long batch, long long R, long long K,
+                         int esz, void *stream)
+    {
+        if (batch <= 0 || R <= 0 || K <= 0) return 0;
+        const bool pairs = esz == 2 && R % 2 == 0 && K % 2 == 0 && (((uintptr_t)src | (uintptr_t)dst) & 3u) == 0;
+        const long long t = pairs ? 64 : 32;
+        const long long tiles_r = (R + t - 1) / t, tiles_k = (K + t - 1) / t;
+        const long long nblk = batch * tiles_r * tiles_k;
+        if (nblk > 0x7fffffffLL) return -2;
+        if (pairs)
+            hipLaunchKernelGGL(transpose_pairs_kernel, dim3((unsigned)nblk), dim3(256), 0, (hipStream_t)stream,
+                               (const uint32_t *)src, (uint32_t *)dst, R, K, tiles_r, tiles_k);
+        else if (esz == 2)
+            hipLaunchKernelGGL(transpose_kernel<uint16_t>, dim3((unsigned)nblk), dim3(256), 0,
+                               (hipStream_t)stream, (const uint16_t *)src, (uint16_t *)dst, R, K, tiles_r, tiles_k);
+        else
+            hipLaunchKernelGGL(transpose_kernel<uint32_t>, dim3((unsigned)nblk), dim3(256), 0,
+                               (hipStream_t)stream, (const uint32_t *)src, (uint32_t *)dst, R, K, tiles_r, tiles_k);
         return check();
     }
 

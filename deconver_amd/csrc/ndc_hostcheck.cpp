@@ -42,6 +42,18 @@ struct Backend {
         return 0;
     }
 
+    static int transpose(const void *src, void *dst, long long batch, long long R, long long K,
+                         int esz, void *)
+    {
+        const char *s = (const char *)src;
+        char *d = (char *)dst;
+        for (long long b = 0; b < batch; ++b)
+            for (long long r = 0; r < R; ++r)
+                for (long long k = 0; k < K; ++k)
+                    memcpy(d + ((b * K + k) * R + r) * esz, s + ((b * R + r) * K + k) * esz, (size_t)esz);
+        return 0;
+    }
+
     // out[o] = sum_p term(o, p) in the association of the HIP build (kSumSlices interleaved
     // partial sums, then those in order)
     template <class F> static int strided_sum(int nout, int nparts, void *, float *out, F term)

@@ -80,8 +80,13 @@ class DeconvUpdate(torch.autograd.Function):
             raise RuntimeError("deconv_update runs on the GPU only (HIP kernels); "
                                "CPU tensors take the layer's general PyTorch path")
         lib = _lib.get_library()
-        x = x.contiguous()
-        z = z.contiguous()
+        # channels-last tensors (torch.channels_last / channels_last_3d) come in through the
+        # library's tiled transposition, and the results go back out the same way, in the
+        # layout of the tensor they belong to
+        ctx.cl = (ops.is_channels_last(x), ops.is_channels_last(z))
+        with torch.cuda.device(x.device):
+            x = ops.to_channel_first(lib, x)
+            z = ops.to_channel_first(lib, z)
         hc = h.contiguous()
         need_t1 = any(ctx.needs_input_grad[:4])
         keep = need_t1 and _SAVE_RATIO
@@ -107,6 +112,9 @@ class DeconvUpdate(torch.autograd.Function):
         ctx.path = path
         ctx.taps = taps if need_t1 else None   # a function of h alone; h is saved below
         ctx.save_for_backward(x, z, t1, hc, bias, s_over_den, ratio)
+        if ctx.cl[1]:
+            with torch.cuda.device(x.device):
+                out = ops.to_channels_last(lib, out)
         return out
 
     @staticmethod
@@ -123,16 +131,20 @@ class DeconvUpdate(torch.autograd.Function):
         need_x, need_z, need_h, need_b = ctx.needs_input_grad[:4]
         if t1 is None:
             raise RuntimeError("backward called on an update that was run without gradients")
-        gout = gout.contiguous()
+        lib = _lib.get_library()
         if gout.dtype != z.dtype:
             gout = gout.to(z.dtype)
-        lib = _lib.get_library()
         with torch.cuda.device(x.device):
+            gout = ops.to_channel_first(lib, gout)
             gx, gz, gh, gb = ops.update_backward(
                 lib, x, z, t1, h, bias, gout, groups=groups, m=m, sc=sc, eps=eps,
                 relu_input=relu_input, need_x=need_x, need_z=need_z, need_h=need_h,
                 need_b=need_b and bias is not None, path=ctx.path,
                 saved=None if s_over_den is None else (s_over_den, ratio), taps=ctx.taps)
+            if ctx.cl[0] and gx is not None:
+                gx = ops.to_channels_last(lib, gx)
+            if ctx.cl[1] and gz is not None:
+                gz = ops.to_channels_last(lib, gz)
         return gx, gz, gh, gb, None, None, None, None, None, None
 
 

@@ -58,6 +58,36 @@ def _check_common(x: Tensor, z: Tensor, h: Tensor, bias: Optional[Tensor], group
     return tuple(h.shape[2:])
 
 
+def is_channels_last(t: Optional[Tensor]) -> bool:
+    """Whether ``t`` is a (B, C, *S) tensor with 2 or 3 spatial dims laid out channels-last
+    (``torch.channels_last`` / ``channels_last_3d``) and not also channel-first contiguous."""
+    if t is None or t.dim() not in (4, 5) or t.is_contiguous():
+        return False
+    fmt = torch.channels_last if t.dim() == 4 else torch.channels_last_3d
+    return t.is_contiguous(memory_format=fmt)
+
+
+def to_channel_first(lib: _lib.NdcLibrary, t: Tensor) -> Tensor:
+    """A channel-first contiguous copy of a channels-last tensor, made by the library's tiled
+    transposition (``ndc_relayout``) instead of a generic strided copy."""
+    if not is_channels_last(t):
+        return t.contiguous()
+    out = torch.empty(t.shape, dtype=t.dtype, device=t.device)
+    lib.relayout(t.data_ptr(), out.data_ptr(), t.shape[0], t.shape[1], t[0, 0].numel(),
+                 dtype_tag(t.dtype), False, _stream_of(t))
+    return out
+
+
+def to_channels_last(lib: _lib.NdcLibrary, t: Tensor) -> Tensor:
+    """The channels-last copy of a channel-first contiguous (B, C, *S) tensor (2 or 3 spatial
+    dims), same shape, by the library's tiled transposition."""
+    fmt = torch.channels_last if t.dim() == 4 else torch.channels_last_3d
+    out = torch.empty(t.shape, dtype=t.dtype, device=t.device, memory_format=fmt)
+    lib.relayout(t.data_ptr(), out.data_ptr(), t.shape[0], t.shape[1], t[0, 0].numel(),
+                 dtype_tag(t.dtype), True, _stream_of(t))
+    return out
+
+
 def make_geom_for(x: Tensor, h: Tensor, groups: int, m: int, sc: int, eps: float,
                   relu_input: bool, path: int = _lib.PATH_AUTO) -> _lib.Geom:
     return _lib.make_geom(x.shape[0], groups, m, sc, x.shape[2:], h.shape[2:],

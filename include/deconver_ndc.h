@@ -234,6 +234,26 @@ int ndc_backward_profiled(const ndc_geom *g, const void *x, const void *z, const
 int ndc_gconv(const ndc_geom *g, const void *in, const float *h, const float *bias, int adjoint,
               void *out, void *stream);
 
+/*
+ * Channels-last entry.  The update kernels read channel-first tensors (B, C, D, H, W): all 64
+ * lanes of a wavefront then work on one channel, whose filter taps are wave-uniform and sit in
+ * scalar registers.  A caller that holds its activations channels-last (B, D, H, W, C in
+ * memory: torch.channels_last / channels_last_3d) brings them in, and takes results out,
+ * through this copy: an LDS-tiled transposition that runs near the device-copy bandwidth,
+ * where a generic strided copy takes 4 to 18 times as long (measured on MI355X, bfloat16:
+ * the 512-channel source tensor of config 3, and the 2 GiB source tensor of a 64-channel
+ * 128^3 layer).
+ *   src, dst           distinct device buffers of batch * channels * spatial elements
+ *   spatial            D * H * W
+ *   dtype              ndc_dtype of the elements
+ *   to_channels_last   0: src is channels-last (B, S, C), dst becomes channel-first (B, C, S);
+ *                      1: the reverse
+ * The reference's fused path accepts contiguous channel-first tensors only and copies
+ * anything else first (deconver/deconvolution/kernels.py:118-127, deconv.py:155).
+ */
+int ndc_relayout(const void *src, void *dst, int64_t batch, int64_t channels, int64_t spatial,
+                 int dtype, int to_channels_last, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
