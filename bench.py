@@ -73,7 +73,9 @@ def make_inputs(torch, dtype, device, batch, channels, spatial, kernel, ratio, s
     proj = layer.init.linear.linear
     x = x.to(device=device, dtype=dtype)
     w = proj.weight.detach().to(device=device, dtype=dtype)
-    z = torch.nn.functional.conv1d(x.flatten(2), w, None).view(batch, channels * sc, *spatial)
+    # (a GEMM per sample: conv1d would send MIOpen searching through its convolution algorithms,
+    # seconds of set-up for tensors this size)
+    z = torch.stack([w.squeeze(-1) @ xb for xb in x.flatten(2)]).view(batch, channels * sc, *spatial)
     torch.manual_seed(seed + 2)
     g = torch.randn(batch, channels * sc, *spatial).to(device=device, dtype=dtype)
     bias = proj.bias.detach().float().to(device)
