@@ -811,9 +811,12 @@ def main() -> int:
     keep = (not args.recompute) and lib.backward_uses_saved(geom)
 
     def step():
-        res = ops.update_forward(lib, x, z, h, bias, save_ratio=keep, **kw)
+        # the launch sequence of the autograd node (deconver_amd/functional.py): the filter
+        # table is packed once per update and serves its forward and its backward
+        taps = ops.prepare_taps(lib, x, h, groups=C, m=1, sc=sc)
+        res = ops.update_forward(lib, x, z, h, bias, save_ratio=keep, taps=taps, **kw)
         return ops.update_backward(lib, x, z, res[1], h, bias, g,
-                                   saved=res[2] if keep else None, **kw)
+                                   saved=res[2] if keep else None, taps=taps, **kw)
 
     if args.calibrate_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()

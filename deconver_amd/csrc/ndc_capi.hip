@@ -30,12 +30,12 @@ __global__ void __launch_bounds__(256) block_reduce_kernel(float *out, F partial
     if (tid == 0) out[blockIdx.x] = buf[0];
 }
 
-// out[o] = sum over p < nparts of term(o, p) for o < nout.  A workgroup sums 32 outputs:
+// put(o, sum over p < nparts of term(o, p)) for o < nout.  A workgroup sums 32 outputs:
 // thread (o, j), j < 8, adds the terms p = j, j + 8, ... in order, then thread (o, 0) adds the
 // eight partial sums in order -- a fixed association, so results are reproducible.  Threads
 // with consecutive o are neighbours, so a `term` that is contiguous in o reads coalesced.
-template <class F>
-__global__ void __launch_bounds__(256) strided_sum_kernel(int nout, int nparts, float *out, F term)
+template <class P, class F>
+__global__ void __launch_bounds__(256) strided_sum_kernel(int nout, int nparts, P put, F term)
 {
     __shared__ float buf[8][33];
     const int ox = threadIdx.x & 31, j = threadIdx.x >> 5;
@@ -49,7 +49,7 @@ __global__ void __launch_bounds__(256) strided_sum_kernel(int nout, int nparts, 
         float total = 0.f;
 #pragma unroll
         for (int k = 0; k < 8; ++k) total += buf[k][ox];
-        out[o] = total;
+        put(o, total);
     }
 }
 
@@ -241,11 +241,11 @@ struct Backend {
     }
 
     static constexpr int kSumSlices = 8;
-    template <class F> static int strided_sum(int nout, int nparts, void *stream, float *out, F term)
+    template <class P, class F> static int strided_sum(int nout, int nparts, void *stream, P put, F term)
     {
         if (nout <= 0) return 0;
-        hipLaunchKernelGGL(strided_sum_kernel<F>, dim3((unsigned)((nout + 31) / 32)), dim3(256), 0,
-                           (hipStream_t)stream, nout, nparts, out, term);
+        hipLaunchKernelGGL((strided_sum_kernel<P, F>), dim3((unsigned)((nout + 31) / 32)), dim3(256), 0,
+                           (hipStream_t)stream, nout, nparts, put, term);
         return check();
     }
 

@@ -464,17 +464,18 @@ static int backward(const KGeom &q, const T *x, const T *z, const T *t1, const T
 
     // combine the per-workgroup partial sums: a fixed association, so results are reproducible
     const int C = q.G, SC = q.sc, ntile = pl.tb.ntile * pl.tb.nseg, B = q.B;
-    if (gh) {
-        st = BE::strided_sum(C * kt, B * ntile, stream, gh, [=] NDC_LAMBDA(int o, int pi) {
-            const int c = o / kt, r = o % kt;
-            const long long blk = ((long long)(pi / ntile) * C + c) * ntile + pi % ntile;
-            return part1[blk * kt + r] + part2[blk * (kt + SC) + r];
-        });
-        if (st) return st;
-    }
-    if (gb) {
-        st = BE::strided_sum(C * SC, B * ntile, stream, gb, [=] NDC_LAMBDA(int o, int pi) {
-            const int c = o / SC, i = o % SC;
+    // (gh and gb in one launch: outputs [0, C kt) are gh, the C SC after them gb)
+    const int n_gh = gh ? C * kt : 0, n_gb = gb ? C * SC : 0;
+    if (n_gh + n_gb) {
+        st = BE::strided_sum(n_gh + n_gb, B * ntile, stream, [=] NDC_LAMBDA(int o, float v) {
+            if (o < n_gh) gh[o] = v; else gb[o - n_gh] = v;
+        }, [=] NDC_LAMBDA(int o, int pi) {
+            if (o < n_gh) {
+                const int c = o / kt, r = o % kt;
+                const long long blk = ((long long)(pi / ntile) * C + c) * ntile + pi % ntile;
+                return part1[blk * kt + r] + part2[blk * (kt + SC) + r];
+            }
+            const int c = (o - n_gh) / SC, i = (o - n_gh) % SC;
             const long long blk = ((long long)(pi / ntile) * C + c) * ntile + pi % ntile;
             return part2[blk * (kt + SC) + kt + i];
         });

@@ -54,9 +54,9 @@ struct Backend {
         return 0;
     }
 
-    // out[o] = sum_p term(o, p) in the association of the HIP build (kSumSlices interleaved
+    // put(o, sum_p term(o, p)) in the association of the HIP build (kSumSlices interleaved
     // partial sums, then those in order)
-    template <class F> static int strided_sum(int nout, int nparts, void *, float *out, F term)
+    template <class P, class F> static int strided_sum(int nout, int nparts, void *, P put, F term)
     {
         for (int o = 0; o < nout; ++o) {
             float total = 0.f;
@@ -65,7 +65,7 @@ struct Backend {
                 for (int p = j; p < nparts; p += kSumSlices) acc += term(o, p);
                 total += acc;
             }
-            out[o] = total;
+            put(o, total);
         }
         return 0;
     }
