@@ -396,6 +396,11 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
         float t1acc[KD][RHK][RW];
         float pz[SC][NZR][RW];
         float px[NXR][RW];
+        // LDS word offsets inside a ring slot, formed once: the word (first own row - PH, first
+        // own column - PW), the word (row `strip`, first own column) and the word (halo row,
+        // first own column - PW).  What is added per access (slot, row, channel) is the same in
+        // every lane and stays on the scalar unit.
+        int ob, so, ho;
     };
 
     // tile rows: s has TH + 4*PH (row j = image r0 - 2*PH + j); x and t1 have TH + 2*PH
@@ -475,32 +480,28 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
 
         auto store_plane = [&](State &st, int k) NDC_LAMBDA {
             if (!st.ln.active) return;
-            const int lb = PL + st.ln.c0;
             // rows outside the image are never written: they keep the zeros of the set-up
             NDC_UNROLL
             for (int n = 0; n < NZR; ++n) {
-                const int j = st.ln.strip + n * S;
                 if ((st.zok >> n) & 1u) {
                     NDC_UNROLL
                     for (int i = 0; i < SC; ++i)
                         NDC_UNROLL
                         for (int c = 0; c < RW; ++c)
-                            ex.st_(off_s + (i * RS + j) * P + lb + c, st.pz[i][n][c]);
+                            ex.st_(st.so + (off_s + (i * RS + n * S) * P) + c, st.pz[i][n][c]);
                 }
             }
         };
         // x plane k - PD into its ring slot.  Runs in the scatter phase: a barrier after the
         // gather that last read that slot, which is what lets KD slots do.
         auto store_x_plane = [&](State &st, int k) NDC_LAMBDA {
-            const int lb = PL + st.ln.c0;
             const int slot = wrap((k - PD) % XR, XR);
             NDC_UNROLL
             for (int n = 0; n < NXR; ++n) {
-                const int j = st.ln.strip + n * S;
                 if ((st.xok >> n) & 1u) {
                     NDC_UNROLL
                     for (int c = 0; c < RW; ++c)
-                        ex.st_(off_x + (slot * RX + j) * P + lb + c, st.px[n][c]);
+                        ex.st_(st.so + (off_x + (slot * RX + n * S) * P) + c, st.px[n][c]);
                 }
             }
         };
@@ -509,6 +510,9 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
         //      columns and never-staged rows stay zero for the whole march)
         ex.each([&](State &st, int tid) NDC_LAMBDA {
             st.ln = make_lane(tid, t, RW);
+            st.ob = st.ln.strip * RH * P + PL + st.ln.c0 - PW;
+            st.so = st.ln.strip * P + PL + st.ln.c0;
+            st.ho = halo_row(st.ln.strip, PH, TH) * P + PL + st.ln.c0 - PW;
             st.zok = st.xok = st.ook = 0u;
             NDC_UNROLL
             for (int n = 0; n < NZR; ++n) {
@@ -554,23 +558,21 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                 store_x_plane(st, k);
                 const bool extra = XT && st.ln.strip < 2 * PH;
                 const int jx = halo_row(st.ln.strip, PH, TH);
-                const int cb = PL + st.ln.c0 - PW;
                 if (k < D) {
                     NDC_ROLLED
                     for (int ii = 0; ii < SC; ++ii) {
                         const int i = uniform_int(ii);
                         float wi[KT];
                         load_taps<KT>(hw + i * KT, wi);
-                        const int sb = off_s + i * RS * P + cb;
-                        k_rows<KD, KH, KW, RH, RW, RHK>(ex, sb + (PH + st.ln.strip * RH) * P, P, wi,
+                        k_rows<KD, KH, KW, RH, RW, RHK>(ex, st.ob + (off_s + (i * RS + PH) * P), P, wi,
                                                         st.t1acc, 0);
-                        if (extra) k_rows<KD, KH, KW, 1, RW, RHK>(ex, sb + jx * P, P, wi, st.t1acc, RH);
+                        if (extra) k_rows<KD, KH, KW, 1, RW, RHK>(ex, st.ho + (off_s + i * RS * P), P, wi, st.t1acc, RH);
                     }
                 }
                 // plane k - PD of t1 is complete: publish it (zero outside the volume)
                 const int pf = k - PD;
                 const bool inplane = pf >= 0 && pf < D;
-                const int tb = off_t + wrap(pf % KD, KD) * RX * P + PL + st.ln.c0;
+                const int tb = off_t + wrap(pf % KD, KD) * RX * P;
                 NDC_UNROLL
                 for (int r = 0; r < RHK; ++r) {
                     const bool mine = r < RH || extra;
@@ -581,7 +583,7 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                     NDC_UNROLL
                     for (int c = 0; c < RW; ++c) {
                         v[c] = live ? st.t1acc[0][r][c] : 0.f;
-                        if (mine) ex.st_(tb + j * P + c, v[c]);
+                        if (mine) ex.st_((r < RH ? st.ob + (tb + (PH + r) * P) : st.ho + tb) + PW + c, v[c]);
                     }
                     if (r < RH && t1g && live && pf >= d0 && pf < d1)
                         IO::store(t1g + (long long)pf * plane + st.ooff[r < RH ? r : 0], v);
@@ -635,9 +637,8 @@ template <int KD_, int KH_, int KW_, int SC_, int RH_, int RW_, typename T> stru
                     float wt[SC][KH * KW];
                     load_plane_taps<SC, KT, KH * KW>(hw + td * KH * KW, wt);
                     const int pl = j0 + PD - td;
-                    const int ob = (st.ln.strip * RH) * P + PL + st.ln.c0 - PW;
-                    const int base[2] = {off_x + wrap(pl % XR, XR) * RX * P + ob,
-                                         off_t + wrap(pl % KD, KD) * RX * P + ob};
+                    const int base[2] = {st.ob + (off_x + wrap(pl % XR, XR) * RX * P),
+                                         st.ob + (off_t + wrap(pl % KD, KD) * RX * P)};
                     a_plane<KH, KW, KT, SC, RH, RW, 2>(ex, base, P, wt, acc);
                 }
                 T *ok_ = og + (long long)j0 * plane;
@@ -693,6 +694,11 @@ struct Bwd1Kernel {
         unsigned xok, ook;
         float bv[SC];
         float gacc[SC][KT];          // A-side filter-gradient terms
+        // LDS word offsets inside a ring slot, formed once: the word (first own row - PH of an
+        // x / t1 slot's rows, first own column - PW), the word (row `strip`, first own column)
+        // and the word (halo row of a gn / gd plane, first own column); what is added per access
+        // (slot, row, channel) is the same in every lane and stays on the scalar unit
+        int ob, so, ho;
         float accx[KD][RH][RW];      // pending planes of gx
         float acct[KD][RH][RW];      // pending planes of gt1
         float px[NXR][RW], pt[NXR][RW];
@@ -761,11 +767,10 @@ struct Bwd1Kernel {
             // rows outside the image are never written: they keep the zeros of the set-up
             NDC_UNROLL
             for (int n = 0; n < NXR; ++n) {
-                const int j = st.ln.strip + n * S;
                 if ((st.xok >> n) & 1u) {
                     NDC_UNROLL
                     for (int c = 0; c < RW; ++c) {
-                        const int o = (slot * RX + j) * P + PL + st.ln.c0 + c;
+                        const int o = st.so + (slot * RX + n * S) * P + c;
                         ex.st_(off_x + o, st.px[n][c]);
                         ex.st_(off_t + o, st.pt[n][c]);
                     }
@@ -775,7 +780,8 @@ struct Bwd1Kernel {
 
         // gn, gd of NR rows starting at gn/gd tile row j (image row r0 - PH + j): computed,
         // published to LDS, and returned in acc[0] / acc[1]
-        auto gn_gd_rows = [&](State &st, int j1, int j, auto nr_tag,
+        // lo: LDS word offset of (tile row j, first own column) inside a plane
+        auto gn_gd_rows = [&](State &st, int j1, int j, int lo, auto nr_tag,
                               float (&acc)[2][SC][decltype(nr_tag)::value][RW]) NDC_LAMBDA {
             constexpr int NR = decltype(nr_tag)::value;
             float sv[SC][NR][RW], gv[SC][NR][RW];
@@ -821,7 +827,7 @@ struct Bwd1Kernel {
                     float wt[SC][KH * KW];
                     load_plane_taps<SC, KT, KH * KW>(hw + td * KH * KW, wt);
                     const int slot = wrap((j1 + PD - td) % XR, XR);
-                    const int ob = (slot * RX + j) * P + PL + st.ln.c0 - PW;
+                    const int ob = lo - PW + slot * RX * P;
                     const int base[2] = {off_x + ob, off_t + ob};
                     a_plane<KH, KW, KT, SC, NR, RW, 2>(ex, base, P, wt, acc);
                 }
@@ -841,8 +847,8 @@ struct Bwd1Kernel {
                             gn = gv[i][r][c] * sv[i][r][c] * inv;
                             gd = -(gn * (acc[0][i][r][c] + eps)) * inv;
                         }
-                        ex.st_(off_g + (i * RG + j + r) * P + PL + st.ln.c0 + c, gn);
-                        ex.st_(off_g + ((SC + i) * RG + j + r) * P + PL + st.ln.c0 + c, gd);
+                        ex.st_(lo + (off_g + (i * RG + r) * P) + c, gn);
+                        ex.st_(lo + (off_g + ((SC + i) * RG + r) * P) + c, gd);
                         acc[0][i][r][c] = gn;
                         acc[1][i][r][c] = gd;
                     }
@@ -850,6 +856,9 @@ struct Bwd1Kernel {
 
         ex.each([&](State &st, int tid) NDC_LAMBDA {
             st.ln = make_lane(tid, t, RW);
+            st.ob = st.ln.strip * RH * P + PL + st.ln.c0 - PW;
+            st.so = st.ln.strip * P + PL + st.ln.c0;
+            st.ho = halo_row(st.ln.strip, PH, TH) * P + PL + st.ln.c0;
             st.xok = st.ook = 0u;
             NDC_UNROLL
             for (int n = 0; n < NXR; ++n) {
@@ -896,19 +905,18 @@ struct Bwd1Kernel {
                 {
                     float acc[2][SC][RH][RW];
                     const int j = PH + st.ln.strip * RH;
-                    gn_gd_rows(st, j1, j, IntTag<RH>(), acc);
+                    gn_gd_rows(st, j1, j, st.ob + (PW + PH * P), IntTag<RH>(), acc);
                     if (need_gh && own1) {
                         // own rows: A-side filter-gradient terms, re-reading the x / t1 windows
                         // (read ahead: for the 2x2 float32 tile this costs two spilled registers
                         // and is still 3 % faster)
                         constexpr int NQ = RH + 2 * PH;
-                        const int cb = PL + st.ln.c0 - PW;
                         stream_rows<KD * NQ, RW + KW - 1, 2, (KH > 1 && SAVED), RW>(
                             ex,
                             [&](int n, int t) NDC_LAMBDA {
                                 const int td = n / NQ, q = n % NQ;
                                 const int slot = wrap((j1 + PD - td) % XR, XR);
-                                return (t ? off_t : off_x) + (slot * RX + j + q) * P + cb;
+                                return st.ob + ((t ? off_t : off_x) + (slot * RX + PH + q) * P);
                             },
                             [&](int n, const float (&v)[2][RW + KW - 1]) NDC_LAMBDA {
                                 const int td = n / NQ, q = n % NQ;
@@ -935,7 +943,7 @@ struct Bwd1Kernel {
                 }
                 if (XT && st.ln.strip < 2 * PH) {
                     float acc[2][SC][1][RW];
-                    gn_gd_rows(st, j1, halo_row(st.ln.strip, PH, TH), IntTag<1>(), acc);
+                    gn_gd_rows(st, j1, halo_row(st.ln.strip, PH, TH), st.ho, IntTag<1>(), acc);
                 }
             });
             ex.sync();
@@ -950,7 +958,7 @@ struct Bwd1Kernel {
                         const int i = uniform_int(ii);
                         float wi[KT];
                         load_taps<KT>(hw + i * KT, wi);
-                        const int gb_ = off_g + (st.ln.strip * RH) * P + PL + st.ln.c0 - PW;
+                        const int gb_ = st.ob + off_g;
                         k_rows<KD, KH, KW, RH, RW, RH, (KH > 1 && SAVED)>(ex, gb_ + i * RG * P, P, wi, st.accx, 0);
                         k_rows<KD, KH, KW, RH, RW, RH, (KH > 1 && SAVED)>(ex, gb_ + (SC + i) * RG * P, P, wi, st.acct, 0);
                     }
@@ -1009,6 +1017,10 @@ struct Bwd2Kernel {
         unsigned xok, ook;
         float bv[SC];
         float gacc[SC][KT];   // K-side filter-gradient term
+        // LDS word offsets inside a ring slot, formed once: the word (first own row - PH, first
+        // own column - PW) and the word (row `strip`, first own column); what is added per
+        // access (slot, row) is the same in every lane and stays on the scalar unit
+        int ob, so;
         float gbacc[SC];
         float px[NXR][RW], pt[NXR][RW], pg[NXR][RW];
     };
@@ -1073,11 +1085,10 @@ struct Bwd2Kernel {
             const int slot = wrap(k % XR, XR);
             NDC_UNROLL
             for (int n = 0; n < NXR; ++n) {
-                const int j = st.ln.strip + n * S;
                 if ((st.xok >> n) & 1u) {
                     NDC_UNROLL
                     for (int c = 0; c < RW; ++c) {
-                        const int o = (slot * RX + j) * P + PL + st.ln.c0 + c;
+                        const int o = st.so + (slot * RX + n * S) * P + c;
                         if (!SAVED) {
                             ex.st_(off_x + o, st.px[n][c]);
                             ex.st_(off_t + o, st.pt[n][c]);
@@ -1090,6 +1101,8 @@ struct Bwd2Kernel {
 
         ex.each([&](State &st, int tid) NDC_LAMBDA {
             st.ln = make_lane(tid, t, RW);
+            st.ob = st.ln.strip * RH * P + PL + st.ln.c0 - PW;
+            st.so = st.ln.strip * P + PL + st.ln.c0;
             st.xok = st.ook = 0u;
             NDC_UNROLL
             for (int n = 0; n < NXR; ++n) {
@@ -1165,7 +1178,7 @@ struct Bwd2Kernel {
                     float wt[SC][KH * KW];
                     load_plane_taps<SC, KT, KH * KW>(hw + td * KH * KW, wt);
                     const int slot = wrap((j0 + PD - td) % XR, XR);
-                    const int ob = (slot * RX + st.ln.strip * RH) * P + PL + st.ln.c0 - PW;
+                    const int ob = st.ob + slot * RX * P;
                     int base[NA];
                     base[NA - 1] = off_g + ob;
                     if (!SAVED) {
@@ -1177,13 +1190,12 @@ struct Bwd2Kernel {
                 if (need_gh) {
                     // K-side filter-gradient term: re-read the gt1 window
                     constexpr int NQ = RH + 2 * PH;
-                    const int cb = PL + st.ln.c0 - PW;
                     stream_rows<KD * NQ, RW + KW - 1, 1, (KH > 1 && SAVED), RW>(
                         ex,
                         [&](int n, int) NDC_LAMBDA {
                             const int td = n / NQ, q = n % NQ;
                             const int slot = wrap((j0 + PD - td) % XR, XR);
-                            return off_g + (slot * RX + st.ln.strip * RH + q) * P + cb;
+                            return st.ob + (off_g + (slot * RX + q) * P);
                         },
                         [&](int n, const float (&v)[1][RW + KW - 1]) NDC_LAMBDA {
                             const int td = n / NQ, q = n % NQ;
