@@ -16,6 +16,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdeconver_ndc.so")
 
 NDC_F32, NDC_BF16 = 0, 1
+ACT_NONE, ACT_RELU, ACT_GELU = 0, 1, 2
 PATH_AUTO, PATH_DIRECT, PATH_FUSED, PATH_FUSED_MATRIX, PATH_FUSED_VECTOR = 0, 1, 2, 3, 4
 
 EXPORTS = (
@@ -38,6 +39,12 @@ EXPORTS = (
     "ndc_backward_profiled",
     "ndc_gconv",
     "ndc_relayout",
+    "ndc_rownorm_workspace_bytes",
+    "ndc_rownorm_forward",
+    "ndc_rownorm_backward",
+    "ndc_bias_act_parts",
+    "ndc_bias_act",
+    "ndc_bias_act_backward",
 )
 
 
@@ -105,6 +112,18 @@ class NdcLibrary:
         d.ndc_gconv.argtypes = [gp, vp, fp, fp, ctypes.c_int, vp, vp]
         d.ndc_relayout.argtypes = [vp, vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                                    ctypes.c_int, ctypes.c_int, vp]
+        d.ndc_rownorm_workspace_bytes.restype = ctypes.c_size_t
+        d.ndc_rownorm_workspace_bytes.argtypes = [ctypes.c_int64, ctypes.c_int64]
+        d.ndc_rownorm_forward.argtypes = [vp, vp, vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int,
+                                          ctypes.c_float, vp, ctypes.c_size_t, vp]
+        d.ndc_rownorm_backward.argtypes = [vp, vp, vp, vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int,
+                                           vp, ctypes.c_size_t, vp]
+        d.ndc_bias_act_parts.restype = ctypes.c_int64
+        d.ndc_bias_act_parts.argtypes = [ctypes.c_int64, ctypes.c_int64]
+        d.ndc_bias_act.argtypes = [vp, vp, vp, vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                                   ctypes.c_int, ctypes.c_int, vp]
+        d.ndc_bias_act_backward.argtypes = [vp, vp, vp, vp, vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                                            ctypes.c_int, ctypes.c_int, vp]
         d.ndc_taps_bytes.restype = ctypes.c_size_t
         d.ndc_taps_bytes.argtypes = [gp]
         d.ndc_prepare_taps.argtypes = [gp, fp, vp, ctypes.c_size_t, vp]
@@ -227,6 +246,35 @@ class NdcLibrary:
         """Channels-last (B, S, C) <-> channel-first (B, C, S) copy of an activation tensor."""
         self._check(self._dll.ndc_relayout(src, dst, batch, channels, spatial, dtype,
                                            int(bool(to_channels_last)), stream), "ndc_relayout")
+
+    def rownorm_workspace_bytes(self, rows: int, n: int) -> int:
+        return int(self._dll.ndc_rownorm_workspace_bytes(rows, n))
+
+    def rownorm_forward(self, x: int, y: int, stats: int, rows: int, n: int, dtype: int, eps: float,
+                        workspace: int, workspace_bytes: int, stream) -> None:
+        """``y = (x - mean) / sqrt(var + eps)`` over each of ``rows`` rows of ``n`` elements;
+        ``stats`` receives (mean, rstd) per row."""
+        self._check(self._dll.ndc_rownorm_forward(x, y, stats, rows, n, dtype, eps, workspace,
+                                                  workspace_bytes, stream), "ndc_rownorm_forward")
+
+    def rownorm_backward(self, gy: int, y: int, stats: int, gx: int, rows: int, n: int, dtype: int,
+                         workspace: int, workspace_bytes: int, stream) -> None:
+        self._check(self._dll.ndc_rownorm_backward(gy, y, stats, gx, rows, n, dtype, workspace,
+                                                   workspace_bytes, stream), "ndc_rownorm_backward")
+
+    def bias_act_parts(self, rows: int, n: int) -> int:
+        return int(self._dll.ndc_bias_act_parts(rows, n))
+
+    def bias_act(self, z: int, bias: Optional[int], residual: Optional[int], y: int, batch: int,
+                 channels: int, n: int, act: int, dtype: int, stream) -> None:
+        """``y = act(z + bias[c]) + residual`` on a channel-first ``(batch, channels, n)`` tensor."""
+        self._check(self._dll.ndc_bias_act(z, bias, residual, y, batch, channels, n, act, dtype, stream),
+                    "ndc_bias_act")
+
+    def bias_act_backward(self, gy: int, z: int, bias: Optional[int], gz: int, gpart: Optional[int],
+                          batch: int, channels: int, n: int, act: int, dtype: int, stream) -> None:
+        self._check(self._dll.ndc_bias_act_backward(gy, z, bias, gz, gpart, batch, channels, n, act, dtype,
+                                                    stream), "ndc_bias_act_backward")
 
 
 _lock = threading.Lock()

@@ -395,6 +395,127 @@ int ndc_relayout(const void *src, void *dst, int64_t batch, int64_t channels, in
     return st == -2 ? (int)NDC_ERR_GEOMETRY : st;
 }
 
+// How a row of n elements is cut for the row normalisation: about 4096 workgroups in all, parts
+// of at least 8192 elements and a multiple of 2048 (every thread's 16-byte vectors stay whole),
+// at most 64 parts (one wavefront adds a row's partial sums).
+static void rownorm_split(long long rows, long long n, int &nsplit, long long &chunk)
+{
+    long long want = (4096 + rows - 1) / rows;
+    if (want > 64) want = 64;
+    if (want > n / 8192) want = n / 8192;
+    if (want < 1) want = 1;
+    chunk = (n + want - 1) / want;
+    chunk = (chunk + 2047) / 2048 * 2048;
+    nsplit = (int)((n + chunk - 1) / chunk);
+}
+
+static int rownorm_check(long long rows, long long n, int dtype)
+{
+    if (dtype != NDC_F32 && dtype != NDC_BF16) return NDC_ERR_DTYPE;
+    if (rows < 1 || n < 1 || (long double)rows * n > 9.0e15L) return NDC_ERR_GEOMETRY;
+    int nsplit;
+    long long chunk;
+    rownorm_split(rows, n, nsplit, chunk);
+    if (rows * nsplit > 0x7fffffffLL) return NDC_ERR_GEOMETRY;
+    return NDC_OK;
+}
+
+size_t ndc_rownorm_workspace_bytes(int64_t rows, int64_t n)
+{
+    if (rows < 1 || n < 1) return 0;
+    int nsplit;
+    long long chunk;
+    rownorm_split(rows, n, nsplit, chunk);
+    return (size_t)rows * nsplit * 2 * sizeof(float);
+}
+
+static bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
+
+int ndc_rownorm_forward(const void *x, void *y, float *stats, int64_t rows, int64_t n, int dtype,
+                        float eps, void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (!x || !y || !stats || !workspace) return NDC_ERR_NULL;
+    int st = rownorm_check(rows, n, dtype);
+    if (st) return st;
+    if (x == (const void *)y || !(eps >= 0.f)) return NDC_ERR_GEOMETRY;
+    if (workspace_bytes < ndc_rownorm_workspace_bytes(rows, n) || ((uintptr_t)workspace & 7u))
+        return NDC_ERR_WORKSPACE;
+    int nsplit;
+    long long chunk;
+    rownorm_split(rows, n, nsplit, chunk);
+    const int esz = dtype == NDC_BF16 ? 2 : 4;
+    const bool vec = n % (16 / esz) == 0 && aligned16(x) && aligned16(y);
+    return ndc::Backend::rownorm(false, x, nullptr, (float *)workspace, stats, y, rows, n, nsplit, chunk,
+                                 esz, vec, eps, stream);
+}
+
+int ndc_rownorm_backward(const void *gy, const void *y, const float *stats, void *gx, int64_t rows,
+                         int64_t n, int dtype, void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (!gy || !y || !stats || !gx || !workspace) return NDC_ERR_NULL;
+    int st = rownorm_check(rows, n, dtype);
+    if (st) return st;
+    if (gx == y) return NDC_ERR_GEOMETRY;
+    if (workspace_bytes < ndc_rownorm_workspace_bytes(rows, n) || ((uintptr_t)workspace & 7u))
+        return NDC_ERR_WORKSPACE;
+    int nsplit;
+    long long chunk;
+    rownorm_split(rows, n, nsplit, chunk);
+    const int esz = dtype == NDC_BF16 ? 2 : 4;
+    const bool vec = n % (16 / esz) == 0 && aligned16(gy) && aligned16(y) && aligned16(gx);
+    return ndc::Backend::rownorm(true, gy, y, (float *)workspace, const_cast<float *>(stats), gx, rows, n,
+                                 nsplit, chunk, esz, vec, 0.f, stream);
+}
+
+static int bias_act_check(long long batch, long long channels, long long n, int act, int dtype)
+{
+    if (dtype != NDC_F32 && dtype != NDC_BF16) return NDC_ERR_DTYPE;
+    if (batch < 1 || channels < 1 || channels > 0x7fffffffLL || n < 1 || act < NDC_ACT_NONE || act > NDC_ACT_GELU)
+        return NDC_ERR_GEOMETRY;
+    if ((long double)batch * channels * n > 9.0e15L) return NDC_ERR_GEOMETRY;
+    return rownorm_check(batch * channels, n, dtype);
+}
+
+int64_t ndc_bias_act_parts(int64_t rows, int64_t n)
+{
+    if (rows < 1 || n < 1) return 0;
+    int nsplit;
+    long long chunk;
+    rownorm_split(rows, n, nsplit, chunk);
+    return nsplit;
+}
+
+int ndc_bias_act(const void *z, const float *bias, const void *residual, void *y, int64_t batch,
+                 int64_t channels, int64_t n, int act, int dtype, void *stream)
+{
+    if (!z || !y) return NDC_ERR_NULL;
+    int st = bias_act_check(batch, channels, n, act, dtype);
+    if (st) return st;
+    int nsplit;
+    long long chunk;
+    rownorm_split(batch * channels, n, nsplit, chunk);
+    const int esz = dtype == NDC_BF16 ? 2 : 4;
+    const bool vec = n % (16 / esz) == 0 && aligned16(z) && aligned16(y) && (!residual || aligned16(residual));
+    return ndc::Backend::bias_act(z, bias, residual, y, batch * channels, (int)channels, n, nsplit, chunk, act,
+                                  esz, vec, stream);
+}
+
+int ndc_bias_act_backward(const void *gy, const void *z, const float *bias, void *gz, float *gpart,
+                          int64_t batch, int64_t channels, int64_t n, int act, int dtype, void *stream)
+{
+    if (!gy || !z || !gz) return NDC_ERR_NULL;
+    int st = bias_act_check(batch, channels, n, act, dtype);
+    if (st) return st;
+    if (act == NDC_ACT_NONE) return NDC_ERR_GEOMETRY;   // gz = gy: nothing to compute
+    int nsplit;
+    long long chunk;
+    rownorm_split(batch * channels, n, nsplit, chunk);
+    const int esz = dtype == NDC_BF16 ? 2 : 4;
+    const bool vec = n % (16 / esz) == 0 && aligned16(gy) && aligned16(z) && aligned16(gz);
+    return ndc::Backend::bias_act_backward(gy, z, bias, gz, gpart, batch * channels, (int)channels, n, nsplit,
+                                           chunk, act, esz, vec, stream);
+}
+
 int ndc_gconv(const ndc_geom *g, const void *in, const float *h, const float *bias, int adjoint,
               void *out, void *stream)
 {

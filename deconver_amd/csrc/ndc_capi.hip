@@ -3,6 +3,8 @@
 
 #include "ndc_common.h"
 #include "ndc_exec.h"
+#include "ndc_rownorm.h"
+#include "ndc_epilogue.h"
 
 #define NDC_LAMBDA __host__ __device__
 
@@ -237,6 +239,112 @@ struct Backend {
         else
             hipLaunchKernelGGL(transpose_kernel<uint32_t>, dim3((unsigned)nblk), dim3(256), 0,
                                (hipStream_t)stream, (const uint32_t *)src, (uint32_t *)dst, R, K, tiles_r, tiles_k);
+        return check();
+    }
+
+    // Row normalisation, one direction: reduce launch then apply launch on rows * nsplit
+    // workgroups.  Forward: a = x, out = y, stats written; backward: a = gy, b = y, stats read,
+    // out = gx.  `vec`: n is a multiple of 16 bytes of elements and every pointer is 16-byte
+    // aligned.
+    template <typename T, bool BWD>
+    static int rownorm_t(const void *a, const void *b, float *partial, float *stats, void *out,
+                         long long rows, long long n, int nsplit, long long chunk, bool vec, float eps,
+                         void *stream)
+    {
+        using namespace rownorm;
+        const Split sp = {n, chunk, nsplit};
+        const dim3 grid((unsigned)(rows * nsplit)), block(kThreads);
+        if (vec) {
+            hipLaunchKernelGGL((reduce_kernel<T, BWD, true>), grid, block, 0, (hipStream_t)stream,
+                               (const T *)a, (const T *)b, (float2 *)partial, sp);
+            hipLaunchKernelGGL((apply_kernel<T, BWD, true>), grid, block, 0, (hipStream_t)stream,
+                               (const T *)a, (const T *)b, (const float2 *)partial, (float2 *)stats, (T *)out, sp, eps);
+        } else {
+            hipLaunchKernelGGL((reduce_kernel<T, BWD, false>), grid, block, 0, (hipStream_t)stream,
+                               (const T *)a, (const T *)b, (float2 *)partial, sp);
+            hipLaunchKernelGGL((apply_kernel<T, BWD, false>), grid, block, 0, (hipStream_t)stream,
+                               (const T *)a, (const T *)b, (const float2 *)partial, (float2 *)stats, (T *)out, sp, eps);
+        }
+        return check();
+    }
+
+    static int rownorm(bool bwd, const void *a, const void *b, float *partial, float *stats, void *out,
+                       long long rows, long long n, int nsplit, long long chunk, int esz, bool vec,
+                       float eps, void *stream)
+    {
+        if (rows <= 0 || n <= 0) return 0;
+        if (esz == 2)
+            return bwd ? rownorm_t<bf16_t, true>(a, b, partial, stats, out, rows, n, nsplit, chunk, vec, eps, stream)
+                       : rownorm_t<bf16_t, false>(a, b, partial, stats, out, rows, n, nsplit, chunk, vec, eps, stream);
+        return bwd ? rownorm_t<float, true>(a, b, partial, stats, out, rows, n, nsplit, chunk, vec, eps, stream)
+                   : rownorm_t<float, false>(a, b, partial, stats, out, rows, n, nsplit, chunk, vec, eps, stream);
+    }
+
+    // y = act(z + bias[channel]) + residual on rows * nsplit workgroups (bias, residual optional)
+    template <typename T, int ACT, bool RES>
+    static void bias_act_launch(const void *z, const float *bias, const void *res, void *y, int channels,
+                                const rownorm::Split &sp, long long rows, bool vec, void *stream)
+    {
+        const dim3 grid((unsigned)(rows * sp.nsplit)), block(rownorm::kThreads);
+        if (vec)
+            hipLaunchKernelGGL((epilogue::forward_kernel<T, ACT, RES, true>), grid, block, 0, (hipStream_t)stream,
+                               (const T *)z, bias, (const T *)res, (T *)y, channels, sp);
+        else
+            hipLaunchKernelGGL((epilogue::forward_kernel<T, ACT, RES, false>), grid, block, 0, (hipStream_t)stream,
+                               (const T *)z, bias, (const T *)res, (T *)y, channels, sp);
+    }
+
+    template <typename T>
+    static int bias_act_t(const void *z, const float *bias, const void *res, void *y, long long rows,
+                          int channels, long long n, int nsplit, long long chunk, int act, bool vec, void *stream)
+    {
+        const rownorm::Split sp = {n, chunk, nsplit};
+#define NDC_BIAS_ACT(ACT)                                                                        \
+    (res ? bias_act_launch<T, ACT, true>(z, bias, res, y, channels, sp, rows, vec, stream)        \
+         : bias_act_launch<T, ACT, false>(z, bias, res, y, channels, sp, rows, vec, stream))
+        if (act == epilogue::kNone) NDC_BIAS_ACT(epilogue::kNone);
+        else if (act == epilogue::kRelu) NDC_BIAS_ACT(epilogue::kRelu);
+        else NDC_BIAS_ACT(epilogue::kGelu);
+#undef NDC_BIAS_ACT
+        return check();
+    }
+
+    static int bias_act(const void *z, const float *bias, const void *res, void *y, long long rows,
+                        int channels, long long n, int nsplit, long long chunk, int act, int esz, bool vec,
+                        void *stream)
+    {
+        if (rows <= 0 || n <= 0) return 0;
+        return esz == 2 ? bias_act_t<bf16_t>(z, bias, res, y, rows, channels, n, nsplit, chunk, act, vec, stream)
+                        : bias_act_t<float>(z, bias, res, y, rows, channels, n, nsplit, chunk, act, vec, stream);
+    }
+
+    template <typename T, int ACT>
+    static void bias_act_bwd_launch(const void *gy, const void *z, const float *bias, void *gz, float *gpart,
+                                    int channels, const rownorm::Split &sp, long long rows, bool vec, void *stream)
+    {
+        const dim3 grid((unsigned)(rows * sp.nsplit)), block(rownorm::kThreads);
+        if (vec)
+            hipLaunchKernelGGL((epilogue::backward_kernel<T, ACT, true>), grid, block, 0, (hipStream_t)stream,
+                               (const T *)gy, (const T *)z, bias, (T *)gz, gpart, channels, sp);
+        else
+            hipLaunchKernelGGL((epilogue::backward_kernel<T, ACT, false>), grid, block, 0, (hipStream_t)stream,
+                               (const T *)gy, (const T *)z, bias, (T *)gz, gpart, channels, sp);
+    }
+
+    // gz = gy * act'(z + bias), gpart[row * nsplit + part] = the part's sum of gz (act: relu, gelu)
+    static int bias_act_backward(const void *gy, const void *z, const float *bias, void *gz, float *gpart,
+                                 long long rows, int channels, long long n, int nsplit, long long chunk, int act,
+                                 int esz, bool vec, void *stream)
+    {
+        if (rows <= 0 || n <= 0) return 0;
+        const rownorm::Split sp = {n, chunk, nsplit};
+        if (esz == 2) {
+            if (act == epilogue::kRelu) bias_act_bwd_launch<bf16_t, epilogue::kRelu>(gy, z, bias, gz, gpart, channels, sp, rows, vec, stream);
+            else bias_act_bwd_launch<bf16_t, epilogue::kGelu>(gy, z, bias, gz, gpart, channels, sp, rows, vec, stream);
+        } else {
+            if (act == epilogue::kRelu) bias_act_bwd_launch<float, epilogue::kRelu>(gy, z, bias, gz, gpart, channels, sp, rows, vec, stream);
+            else bias_act_bwd_launch<float, epilogue::kGelu>(gy, z, bias, gz, gpart, channels, sp, rows, vec, stream);
+        }
         return check();
     }
 

@@ -2,6 +2,7 @@
 // build, executed thread by thread on the CPU, so that the CPU test-suite can check
 // indexing, bounds and barrier placement before anything runs on a GPU.  It is a checker
 // for the kernels' source, not a fallback: the Python package never loads it.
+#include <cmath>
 #include <vector>
 
 #include "ndc_common.h"
@@ -51,6 +52,123 @@ struct Backend {
             for (long long r = 0; r < R; ++r)
                 for (long long k = 0; k < K; ++k)
                     memcpy(d + ((b * K + k) * R + r) * esz, s + ((b * R + r) * K + k) * esz, (size_t)esz);
+        return 0;
+    }
+
+    // Row normalisation as the HIP build computes it (part by part, float32 sums, the same
+    // shift and the same formulas), sequentially.
+    template <typename T>
+    static void rownorm_t(bool bwd, const T *a, const T *b, float *partial, float *stats, T *out,
+                          long long rows, long long n, int nsplit, long long chunk, float eps)
+    {
+        for (long long row = 0; row < rows; ++row) {
+            const T *ar = a + row * n, *br = bwd ? b + row * n : nullptr;
+            const float pivot = bwd ? 0.f : Elem<T>::load(ar);
+            float s1 = 0.f, s2 = 0.f;
+            for (int part = 0; part < nsplit; ++part) {
+                const long long lo = part * chunk, hi = lo + chunk < n ? lo + chunk : n;
+                float p1 = 0.f, p2 = 0.f;
+                for (long long i = lo; i < hi; ++i) {
+                    const float f = Elem<T>::load(ar + i) - pivot;
+                    p1 += f;
+                    p2 += f * (bwd ? Elem<T>::load(br + i) : f);
+                }
+                partial[2 * (row * nsplit + part)] = p1;
+                partial[2 * (row * nsplit + part) + 1] = p2;
+                s1 += p1;
+                s2 += p2;
+            }
+            const float inv_n = 1.f / (float)n;
+            float c0, c1, c2 = 0.f;
+            if (bwd) {
+                c1 = stats[2 * row + 1];
+                c0 = -c1 * s1 * inv_n;
+                c2 = -c1 * s2 * inv_n;
+            } else {
+                const float m = s1 * inv_n;
+                float var = s2 * inv_n - m * m;
+                var = var > 0.f ? var : 0.f;
+                c1 = 1.f / std::sqrt(var + eps);
+                c0 = pivot + m;
+                stats[2 * row] = c0;
+                stats[2 * row + 1] = c1;
+            }
+            for (long long i = 0; i < n; ++i) {
+                const float v = Elem<T>::load(ar + i);
+                Elem<T>::store(out + row * n + i, bwd ? v * c1 + c0 + Elem<T>::load(br + i) * c2 : (v - c0) * c1);
+            }
+        }
+    }
+
+    static int rownorm(bool bwd, const void *a, const void *b, float *partial, float *stats, void *out,
+                       long long rows, long long n, int nsplit, long long chunk, int esz, bool, float eps,
+                       void *)
+    {
+        if (esz == 2)
+            rownorm_t<bf16_t>(bwd, (const bf16_t *)a, (const bf16_t *)b, partial, stats, (bf16_t *)out, rows, n,
+                              nsplit, chunk, eps);
+        else
+            rownorm_t<float>(bwd, (const float *)a, (const float *)b, partial, stats, (float *)out, rows, n,
+                             nsplit, chunk, eps);
+        return 0;
+    }
+
+    static float act_value(int act, float u, bool grad)
+    {
+        const float cdf = 0.5f * (1.f + std::erf(u * 0.70710678118654752f));
+        if (act == 1) return grad ? (u > 0.f ? 1.f : 0.f) : (u > 0.f ? u : 0.f);
+        if (act == 2) return grad ? cdf + u * 0.3989422804014327f * std::exp(-0.5f * u * u) : u * cdf;
+        return grad ? 1.f : u;
+    }
+
+    template <typename T>
+    static void bias_act_t(const T *z, const float *bias, const T *res, T *y, long long rows, int channels,
+                           long long n, int act)
+    {
+        for (long long row = 0; row < rows; ++row) {
+            const float b = bias ? bias[row % channels] : 0.f;
+            for (long long i = row * n; i < (row + 1) * n; ++i)
+                Elem<T>::store(y + i, act_value(act, Elem<T>::load(z + i) + b, false) + (res ? Elem<T>::load(res + i) : 0.f));
+        }
+    }
+
+    static int bias_act(const void *z, const float *bias, const void *res, void *y, long long rows,
+                        int channels, long long n, int, long long, int act, int esz, bool, void *)
+    {
+        if (esz == 2) bias_act_t<bf16_t>((const bf16_t *)z, bias, (const bf16_t *)res, (bf16_t *)y, rows, channels, n, act);
+        else bias_act_t<float>((const float *)z, bias, (const float *)res, (float *)y, rows, channels, n, act);
+        return 0;
+    }
+
+    template <typename T>
+    static void bias_act_bwd_t(const T *gy, const T *z, const float *bias, T *gz, float *gpart, long long rows,
+                               int channels, long long n, int nsplit, long long chunk, int act)
+    {
+        for (long long row = 0; row < rows; ++row) {
+            const float b = bias ? bias[row % channels] : 0.f;
+            for (int part = 0; part < nsplit; ++part) {
+                const long long lo = part * chunk, hi = lo + chunk < n ? lo + chunk : n;
+                float s = 0.f;
+                for (long long i = row * n + lo; i < row * n + hi; ++i) {
+                    const float v = Elem<T>::load(gy + i) * act_value(act, Elem<T>::load(z + i) + b, true);
+                    s += v;
+                    Elem<T>::store(gz + i, v);
+                }
+                if (gpart) gpart[row * nsplit + part] = s;
+            }
+        }
+    }
+
+    static int bias_act_backward(const void *gy, const void *z, const float *bias, void *gz, float *gpart,
+                                 long long rows, int channels, long long n, int nsplit, long long chunk, int act,
+                                 int esz, bool, void *)
+    {
+        if (esz == 2)
+            bias_act_bwd_t<bf16_t>((const bf16_t *)gy, (const bf16_t *)z, bias, (bf16_t *)gz, gpart, rows, channels, n,
+                                   nsplit, chunk, act);
+        else
+            bias_act_bwd_t<float>((const float *)gy, (const float *)z, bias, (float *)gz, gpart, rows, channels, n,
+                                  nsplit, chunk, act);
         return 0;
     }
 

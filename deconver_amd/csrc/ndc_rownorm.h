@@ -1,0 +1,242 @@
+// Row normalisation on the GPU: y = (x - mean(x)) / sqrt(var(x) + eps) over each row of a
+// (rows, n) matrix, and its gradient.  On a channel-first tensor (B, C, *S) the rows are the
+// B*C channel maps, i.e. this is InstanceNorm without affine parameters or running
+// statistics -- the norm that sits between the NDC layers of the 3-D network, where a row is
+// up to 128^3 elements long and there are as few as 128 rows.  A row is therefore cut into
+// `nsplit` parts, one workgroup each, in two launches per direction:
+//
+//   reduce:  partial[row][part] = (sum a', sum a' b')  over the part
+//   apply :  every workgroup adds its row's nsplit partials (same order everywhere), then
+//            transforms its part
+//
+//   forward : a' = b' = x - x[row][0] (a shift that keeps the variance free of cancellation);
+//             y = (x - mean) rstd;  stats[row] = (mean, rstd)
+//   backward: a' = gy, b' = y;  gx = rstd (gy - mean(gy) - y mean(gy y))
+//
+// HBM traffic: forward 2 reads + 1 write of the tensor, backward 4 reads + 1 write.  Sums are
+// float32 whatever the storage type.  Device code only (included by the HIP build).
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "ndc_common.h"
+
+namespace ndc {
+namespace rownorm {
+
+static constexpr int kThreads = 256;
+static constexpr int kMaxSplit = 64;
+
+template <typename T> struct Vec;   // 16 bytes of T
+template <> struct Vec<float> {
+    static constexpr int N = 4;
+    float4 v;
+    __device__ float get(int i) const { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
+    __device__ void set(int i, float f) { (i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w) = f; }
+};
+template <> struct Vec<bf16_t> {
+    static constexpr int N = 8;
+    uint4 v;
+    __device__ uint32_t word(int i) const { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
+    __device__ float get(int i) const
+    {
+        const uint32_t w = word(i >> 1);
+        return __uint_as_float((i & 1) ? (w & 0xffff0000u) : (w << 16));
+    }
+    __device__ void set_pair(int p, float lo, float hi)
+    {
+        (p == 0 ? v.x : p == 1 ? v.y : p == 2 ? v.z : v.w) = pack_bf16x2(lo, hi);
+    }
+};
+
+// (sum over the workgroup of a, of b) in every thread; fixed association
+__device__ inline void block_sum2(float &a, float &b, float (*buf)[2])
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        a += __shfl_down(a, off, 64);
+        b += __shfl_down(b, off, 64);
+    }
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) {
+        buf[wave][0] = a;
+        buf[wave][1] = b;
+    }
+    __syncthreads();
+    a = (buf[0][0] + buf[1][0]) + (buf[2][0] + buf[3][0]);
+    b = (buf[0][1] + buf[1][1]) + (buf[2][1] + buf[3][1]);
+    __syncthreads();
+}
+
+// the row's totals from its nsplit partials, in every thread
+__device__ inline void row_totals(const float2 *partial, int nsplit, float &s1, float &s2, float (*buf)[2])
+{
+    if (threadIdx.x < 64) {
+        float a = 0.f, b = 0.f;
+        if ((int)threadIdx.x < nsplit) {
+            const float2 p = partial[threadIdx.x];
+            a = p.x;
+            b = p.y;
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            a += __shfl_down(a, off, 64);
+            b += __shfl_down(b, off, 64);
+        }
+        if (threadIdx.x == 0) {
+            buf[0][0] = a;
+            buf[0][1] = b;
+        }
+    }
+    __syncthreads();
+    s1 = buf[0][0];
+    s2 = buf[0][1];
+}
+
+struct Split {
+    long long n;        // row length, elements
+    long long chunk;    // elements per part (a multiple of the vector width)
+    int nsplit;
+};
+
+template <typename T, bool BWD, bool VEC>
+__global__ void __launch_bounds__(kThreads)
+reduce_kernel(const T *a, const T *b, float2 *partial, Split sp)
+{
+    __shared__ float buf[4][2];
+    const long long row = blockIdx.x / sp.nsplit;
+    const int part = blockIdx.x % sp.nsplit;
+    const T *ar = a + row * sp.n, *br = BWD ? b + row * sp.n : nullptr;
+    const long long lo = part * sp.chunk, hi = lo + sp.chunk < sp.n ? lo + sp.chunk : sp.n;
+    const float pivot = BWD ? 0.f : Elem<T>::load(ar);
+    float s1 = 0.f, s2 = 0.f;
+    if constexpr (VEC) {
+        typedef Vec<T> V;
+        const long long v0 = lo / V::N, v1 = hi / V::N;
+        const V *av = reinterpret_cast<const V *>(ar), *bv = reinterpret_cast<const V *>(br);
+        float t1[4] = {0.f, 0.f, 0.f, 0.f}, t2[4] = {0.f, 0.f, 0.f, 0.f};
+        long long i = v0 + threadIdx.x;
+        for (; i + 3 * kThreads < v1; i += 4 * kThreads) {
+            V x[4], y[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                x[u] = av[i + u * kThreads];
+                if (BWD) y[u] = bv[i + u * kThreads];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int e = 0; e < V::N; ++e) {
+                    const float f = x[u].get(e) - pivot;
+                    t1[u] += f;
+                    t2[u] += f * (BWD ? y[u].get(e) : f);
+                }
+        }
+        for (; i < v1; i += kThreads) {
+            const V x = av[i];
+            V y;
+            if (BWD) y = bv[i];
+#pragma unroll
+            for (int e = 0; e < V::N; ++e) {
+                const float f = x.get(e) - pivot;
+                t1[0] += f;
+                t2[0] += f * (BWD ? y.get(e) : f);
+            }
+        }
+        s1 = (t1[0] + t1[1]) + (t1[2] + t1[3]);
+        s2 = (t2[0] + t2[1]) + (t2[2] + t2[3]);
+    } else {
+        for (long long i = lo + threadIdx.x; i < hi; i += kThreads) {
+            const float f = Elem<T>::load(ar + i) - pivot;
+            s1 += f;
+            s2 += f * (BWD ? Elem<T>::load(br + i) : f);
+        }
+    }
+    block_sum2(s1, s2, buf);
+    if (threadIdx.x == 0) partial[blockIdx.x] = make_float2(s1, s2);
+}
+
+template <typename T, bool BWD, bool VEC>
+__global__ void __launch_bounds__(kThreads)
+apply_kernel(const T *a, const T *b, const float2 *partial, float2 *stats, T *out, Split sp, float eps)
+{
+    __shared__ float buf[4][2];
+    const long long row = blockIdx.x / sp.nsplit;
+    const int part = blockIdx.x % sp.nsplit;
+    const T *ar = a + row * sp.n, *br = BWD ? b + row * sp.n : nullptr;
+    T *orow = out + row * sp.n;
+    const long long lo = part * sp.chunk, hi = lo + sp.chunk < sp.n ? lo + sp.chunk : sp.n;
+    float s1, s2;
+    row_totals(partial + row * sp.nsplit, sp.nsplit, s1, s2, buf);
+    const float inv_n = 1.f / (float)sp.n;
+    // forward: out = (x - c0) * c1;  backward: out = gy * c1 + y * c2 + c0
+    float c0, c1, c2 = 0.f;
+    if (BWD) {
+        const float rstd = stats[row].y;
+        c1 = rstd;
+        c0 = -rstd * s1 * inv_n;
+        c2 = -rstd * s2 * inv_n;
+    } else {
+        const float pivot = Elem<T>::load(ar);
+        const float m = s1 * inv_n;
+        float var = s2 * inv_n - m * m;
+        var = var > 0.f ? var : 0.f;
+        const float rstd = rsqrtf(var + eps), mean = pivot + m;
+        c1 = rstd;
+        c0 = mean;
+        if (part == 0 && threadIdx.x == 0) stats[row] = make_float2(mean, rstd);
+    }
+    if constexpr (VEC) {
+        typedef Vec<T> V;
+        const long long v0 = lo / V::N, v1 = hi / V::N;
+        const V *av = reinterpret_cast<const V *>(ar), *bv = reinterpret_cast<const V *>(br);
+        V *ov = reinterpret_cast<V *>(orow);
+        auto one = [&](const V &x, const V &y) {
+            V r;
+            if constexpr (sizeof(T) == 2) {
+#pragma unroll
+                for (int p = 0; p < V::N / 2; ++p) {
+                    float f0, f1;
+                    if (BWD) {
+                        f0 = x.get(2 * p) * c1 + c0 + y.get(2 * p) * c2;
+                        f1 = x.get(2 * p + 1) * c1 + c0 + y.get(2 * p + 1) * c2;
+                    } else {
+                        f0 = (x.get(2 * p) - c0) * c1;
+                        f1 = (x.get(2 * p + 1) - c0) * c1;
+                    }
+                    r.set_pair(p, f0, f1);
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < V::N; ++e) {
+                    r.set(e, BWD ? x.get(e) * c1 + c0 + y.get(e) * c2 : (x.get(e) - c0) * c1);
+                }
+            }
+            return r;
+        };
+        long long i = v0 + threadIdx.x;
+        for (; i + 3 * kThreads < v1; i += 4 * kThreads) {
+            V x[4], y[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                x[u] = av[i + u * kThreads];
+                if (BWD) y[u] = bv[i + u * kThreads];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) ov[i + u * kThreads] = one(x[u], y[u]);
+        }
+        for (; i < v1; i += kThreads) {
+            const V x = av[i];
+            V y;
+            if (BWD) y = bv[i];
+            ov[i] = one(x, y);
+        }
+    } else {
+        for (long long i = lo + threadIdx.x; i < hi; i += kThreads) {
+            const float v = Elem<T>::load(ar + i);
+            Elem<T>::store(orow + i, BWD ? v * c1 + c0 + Elem<T>::load(br + i) * c2 : (v - c0) * c1);
+        }
+    }
+}
+
+}  // namespace rownorm
+}  // namespace ndc

@@ -5,11 +5,14 @@ reference so that its checkpoints load unchanged."""
 
 from __future__ import annotations
 
+import math
 from typing import Optional
 
 import torch
 from torch import nn
 from torch.nn.modules.utils import _pair
+
+from . import _lib, ops
 
 
 def _wgrad_chunks(batch: int, n: int) -> int:
@@ -23,11 +26,14 @@ def _wgrad_chunks(batch: int, n: int) -> int:
 
 
 class _PointwiseLinear(torch.autograd.Function):
-    """``y[b] = W x[b] (+ bias)`` for ``x`` of shape ``(B, Cin, N)``: the 1x1 projection as
-    plain GEMMs on the channel-first layout (hipBLASLt through ``torch.matmul`` / ``bmm``).
+    """``y[b] = act(W x[b] + bias) + residual[b]`` for ``x`` of shape ``(B, Cin, N)``: the 1x1
+    projection as plain GEMMs on the channel-first layout (hipBLASLt through ``torch.mm`` /
+    ``bmm``), then ONE pass of the HIP library over the result for bias, activation and
+    residual sum (``ndc_bias_act``).
 
-    The same map as ``nn.Conv1d(kernel_size=1)`` (layers/linear.py:53-58).  The library
-    convolution reaches its GEMM through layout transposes of input and output and a
+    The same map as ``nn.Conv1d(kernel_size=1)`` (layers/linear.py:53-58) followed by the
+    activation and the ``x + ...`` of the block (layers/mlp.py:40-63, deconver.py:60-64).  The
+    library convolution reaches its GEMM through layout transposes of input and output and a
     separate weight-gradient kernel; here forward and input gradient are one GEMM each on
     the tensors as they lie, and the weight gradient (a ``Cout x Cin`` result summed over
     millions of voxels) is a batch of GEMMs over equal chunks of the voxel axis whose
@@ -35,67 +41,205 @@ class _PointwiseLinear(torch.autograd.Function):
     of the 128 -> 512 projection at 2 x 64^3 in bf16."""
 
     @staticmethod
-    def forward(ctx, x, weight, bias):
-        ctx.save_for_backward(x, weight)
-        ctx.has_bias = bias is not None
+    def forward(ctx, x, weight, bias, act, residual):
+        lib = _lib.get_library()
         # one GEMM per sample on the tensors as they lie (torch.matmul would fold the batch into
         # the voxel axis through two transposing copies when its input requires a gradient)
-        y = x.new_empty(x.shape[0], weight.shape[0], x.shape[2])
+        z = x.new_empty(x.shape[0], weight.shape[0], x.shape[2])
         for b in range(x.shape[0]):
-            torch.mm(weight, x[b], out=y[b])
-        if bias is not None:
-            y += bias.to(y.dtype).view(1, -1, 1)
+            torch.mm(weight, x[b], out=z[b])
+        bias32 = None if bias is None else bias.detach().float().contiguous()
+        y = z
+        # the activation's gradient needs z + bias: gelu keeps z; relu alone needs only the
+        # sign of its output, which may then overwrite z
+        keep_z = act == "gelu" or (act == "relu" and residual is not None)
+        if bias is not None or act is not None or residual is not None:
+            with torch.cuda.device(x.device):
+                y = ops.bias_act(lib, z, bias32, residual, act, inplace=not keep_z)
+        kept = z if keep_z else y if act == "relu" else None
+        ctx.save_for_backward(x, weight, kept, bias32 if keep_z else None)
+        ctx.has_bias = bias is not None
+        ctx.act = act
         return y
 
     @staticmethod
     def backward(ctx, gy):
-        x, weight = ctx.saved_tensors
+        x, weight, kept, bias32 = ctx.saved_tensors
         gy = gy.contiguous()
         gx = gw = gb = None
-        if ctx.needs_input_grad[0]:
-            gx = torch.empty_like(x)
-            wt = weight.t()
-            for b in range(x.shape[0]):
-                torch.mm(wt, gy[b], out=gx[b])
-        if ctx.needs_input_grad[1]:
-            B, cout, n = gy.shape
-            cin = x.shape[1]
-            s = _wgrad_chunks(B, n) if gy.dtype in (torch.bfloat16, torch.float16) else 1
-            if s == 1:
-                gw = torch.bmm(gy, x.transpose(1, 2)).sum(0)
-            else:
-                acc = torch.zeros(cout, cin, dtype=torch.float32, device=gy.device)
-                for b in range(B):
-                    # chunk c of the voxel axis as batch entry c: strided views, no copies
-                    a = gy[b].view(cout, s, n // s).transpose(0, 1)
-                    c = x[b].view(cin, s, n // s).permute(1, 2, 0)
-                    acc += torch.bmm(a, c).float().sum(0)
-                gw = acc.to(weight.dtype)
-        if ctx.has_bias and ctx.needs_input_grad[2]:
+        gres = gy if ctx.needs_input_grad[4] else None
+        want_gb = ctx.has_bias and ctx.needs_input_grad[2]
+        gz = gy
+        if ctx.act is not None:
+            with torch.cuda.device(gy.device):
+                gz, gb = ops.bias_act_backward(_lib.get_library(), gy, kept, bias32, ctx.act,
+                                               need_bias_grad=want_gb)
+        elif want_gb:
             # rows first (contiguous runs of the voxel axis), then the few per-sample sums: the
             # library's one-call reduction of a (B, C, N) tensor over B and N runs at a tenth of
             # the memory bandwidth (0.19 ms at 2 x 128 x 64^3 in bf16)
             gb = gy.sum(2, dtype=torch.float32).sum(0)
-        return gx, gw, gb
+        if ctx.needs_input_grad[0]:
+            gx = torch.empty_like(x)
+            wt = weight.t()
+            for b in range(x.shape[0]):
+                torch.mm(wt, gz[b], out=gx[b])
+        if ctx.needs_input_grad[1]:
+            B, cout, n = gz.shape
+            cin = x.shape[1]
+            s = _wgrad_chunks(B, n) if gz.dtype in (torch.bfloat16, torch.float16) else 1
+            if s == 1:
+                gw = torch.bmm(gz, x.transpose(1, 2)).sum(0)
+            else:
+                acc = torch.zeros(cout, cin, dtype=torch.float32, device=gz.device)
+                for b in range(B):
+                    # chunk c of the voxel axis as batch entry c: strided views, no copies
+                    a = gz[b].view(cout, s, n // s).transpose(0, 1)
+                    c = x[b].view(cin, s, n // s).permute(1, 2, 0)
+                    acc += torch.bmm(a, c).float().sum(0)
+                gw = acc.to(weight.dtype)
+        return gx, gw, gb, None, gres
 
 
-def pointwise_linear(x: torch.Tensor, weight: torch.Tensor,
-                     bias: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """The 1x1 projection ``(B, Cin, N) -> (B, Cout, N)`` with ``weight`` of shape
-    ``(Cout, Cin)`` or ``(Cout, Cin, 1)``.  16-bit tensors on the GPU (bfloat16 / float16
-    storage or autocast) run as GEMMs on the channel-first layout; everything else as the
-    reference's ``conv1d``."""
+_ACT_FUNCTIONS = {None: lambda t: t, "relu": torch.relu, "gelu": torch.nn.functional.gelu}
+
+
+def pointwise_linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                     act: Optional[str] = None, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``act(W x + bias) + residual``: the 1x1 projection ``(B, Cin, N) -> (B, Cout, N)`` with
+    ``weight`` of shape ``(Cout, Cin)`` or ``(Cout, Cin, 1)``, optionally followed by an
+    activation (``"relu"`` or ``"gelu"``, the exact one) and the sum with a tensor of the
+    output's shape.  bfloat16 tensors on the GPU (stored or under autocast) run as GEMMs on the
+    channel-first layout plus one pass of the HIP library over the result; everything else as
+    the reference's ``conv1d`` followed by PyTorch's activation and sum."""
     w2 = weight.squeeze(-1) if weight.dim() == 3 else weight
     dtype = x.dtype
     if x.is_cuda and torch.is_autocast_enabled(x.device.type):
         dtype = torch.get_autocast_dtype(x.device.type)
     # 16-bit GPU tensors only: in float32 the library convolution is as fast (2-D network,
     # batch 8: 24.5 against 25.5 ms per step)
-    if not x.is_cuda or x.dim() != 3 or dtype not in (torch.bfloat16, torch.float16):
-        return torch.nn.functional.conv1d(x, w2.unsqueeze(-1), bias)
+    if not x.is_cuda or x.dim() != 3 or dtype != torch.bfloat16:
+        y = _ACT_FUNCTIONS[act](torch.nn.functional.conv1d(x, w2.unsqueeze(-1), bias))
+        return y if residual is None else residual + y
     x, w2 = x.to(dtype), w2.to(dtype)
+    if residual is not None:
+        residual = residual.to(dtype).contiguous()
     with torch.autocast(x.device.type, enabled=False):
-        return _PointwiseLinear.apply(x.contiguous(), w2, bias)
+        return _PointwiseLinear.apply(x.contiguous(), w2, bias, act, residual)
+
+
+def _gemm_route(x: torch.Tensor) -> bool:
+    """True for the tensors ``pointwise_linear`` runs as GEMMs: bfloat16 (stored or under
+    autocast) on the GPU."""
+    dtype = x.dtype
+    if x.is_cuda and torch.is_autocast_enabled(x.device.type):
+        dtype = torch.get_autocast_dtype(x.device.type)
+    return x.is_cuda and dtype == torch.bfloat16
+
+
+def _is_patch_conv(conv) -> bool:
+    """A convolution whose windows tile the input: stride == kernel size, no padding, no
+    dilation, one group (and no output padding on a transposed one)."""
+    return (tuple(conv.stride) == tuple(conv.kernel_size) and all(p == 0 for p in conv.padding)
+            and all(d == 1 for d in conv.dilation) and conv.groups == 1
+            and isinstance(conv.padding, tuple)
+            and all(p == 0 for p in getattr(conv, "output_padding", ())))
+
+
+def patches_to_channels(x: torch.Tensor, k) -> torch.Tensor:
+    """``(B, C, *S) -> (B, C * prod(k), prod(S // k))``: every ``k`` window of the grid becomes
+    one column, channel-major then window offset (the order of a convolution weight's
+    ``(Cin, *k)`` axes).  Rows and planes that do not fill a window are dropped, as a strided
+    convolution drops them."""
+    B, C = x.shape[:2]
+    nd = len(k)
+    if all(v == 1 for v in k):
+        return x.flatten(2)
+    coarse = [s // v for s, v in zip(x.shape[2:], k)]
+    if any(c * v != s for c, v, s in zip(coarse, k, x.shape[2:])):
+        x = x[(slice(None), slice(None), *[slice(0, c * v) for c, v in zip(coarse, k)])]
+    split = [B, C]
+    for c, v in zip(coarse, k):
+        split += [c, v]
+    x = x.reshape(split)
+    order = [0, 1] + [3 + 2 * i for i in range(nd)] + [2 + 2 * i for i in range(nd)]
+    return x.permute(order).reshape(B, C * math.prod(k), math.prod(coarse))
+
+
+def channels_to_patches(y: torch.Tensor, k, coarse) -> torch.Tensor:
+    """Inverse of ``patches_to_channels`` on an exactly tiled grid:
+    ``(B, C * prod(k), prod(coarse)) -> (B, C, *(coarse * k))``."""
+    B = y.shape[0]
+    nd = len(k)
+    C = y.shape[1] // math.prod(k)
+    if all(v == 1 for v in k):
+        return y.view(B, C, *coarse)
+    y = y.view(B, C, *k, *coarse)
+    order = [0, 1]
+    for i in range(nd):
+        order += [2 + nd + i, 2 + i]
+    return y.permute(order).reshape(B, C, *[c * v for c, v in zip(coarse, k)])
+
+
+def patch_conv(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
+    """``conv(x, weight, bias, stride=weight.shape[2:])``, no padding: a strided convolution
+    whose windows tile its input is a regrouping of the grid followed by the 1x1 projection."""
+    k = tuple(weight.shape[2:])
+    coarse = [s // v for s, v in zip(x.shape[2:], k)]
+    y = pointwise_linear(patches_to_channels(x, k), weight.flatten(1), bias)
+    return y.view(x.shape[0], -1, *coarse)
+
+
+def patch_conv_transpose(x: torch.Tensor, weight: torch.Tensor,
+                         bias: Optional[torch.Tensor]) -> torch.Tensor:
+    """``conv_transpose(x, weight, bias, stride=weight.shape[2:])``: the 1x1 projection to
+    ``Cout * prod(k)`` channels, then every column spread over its window of the finer grid."""
+    k = tuple(weight.shape[2:])
+    # weight (Cin, Cout, *k): row (cout, offset) of the projection is weight[:, cout, offset]
+    w = weight.flatten(1).t()
+    if bias is not None:
+        bias = bias.repeat_interleave(math.prod(k))
+    return channels_to_patches(pointwise_linear(x.flatten(2), w, bias), k, x.shape[2:])
+
+
+class _PatchConvMixin:
+    """The network's 2-tap resampling convolutions (unet.py:36-60) and its 1-tap head are
+    convolutions whose windows tile the input.  16-bit tensors on the GPU take the form of
+    ``patch_conv`` here -- one strided copy and the GEMMs of ``pointwise_linear`` instead of
+    the library's column-matrix convolution; everything else, and any other stride or
+    padding, runs the parent class's convolution.  Parameters, their shapes and names are the
+    parent's."""
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if _is_patch_conv(self) and _gemm_route(x) and x.dim() == len(self.kernel_size) + 2:
+            return patch_conv(x, self.weight, self.bias)
+        return super().forward(x)
+
+
+class _PatchConvTransposeMixin:
+    """The transposed counterpart (unet.py:108-131), as ``patch_conv_transpose``."""
+
+    def forward(self, x: torch.Tensor, output_size=None) -> torch.Tensor:
+        if (output_size is None and _is_patch_conv(self) and _gemm_route(x)
+                and x.dim() == len(self.kernel_size) + 2):
+            return patch_conv_transpose(x, self.weight, self.bias)
+        return super().forward(x, output_size)
+
+
+class PatchConv2d(_PatchConvMixin, nn.Conv2d):
+    pass
+
+
+class PatchConv3d(_PatchConvMixin, nn.Conv3d):
+    pass
+
+
+class PatchConvTranspose2d(_PatchConvTransposeMixin, nn.ConvTranspose2d):
+    pass
+
+
+class PatchConvTranspose3d(_PatchConvTransposeMixin, nn.ConvTranspose3d):
+    pass
 
 
 class Linear(nn.Module):
@@ -112,9 +256,14 @@ class Linear(nn.Module):
         self.linear = nn.Conv1d(in_channels, out_channels, kernel_size=1, bias=bias,
                                 device=device, dtype=dtype)
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, act: Optional[str] = None,
+                residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``act(linear(x)) + residual``; ``act`` None, ``"relu"`` or ``"gelu"``; ``residual``
+        of the output's shape."""
         shape = x.shape
-        y = pointwise_linear(self.flatten(x), self.linear.weight, self.linear.bias)
+        if residual is not None:
+            residual = residual.flatten(2)
+        y = pointwise_linear(self.flatten(x), self.linear.weight, self.linear.bias, act, residual)
         return y.view(shape[0], -1, *shape[2:])
 
 
@@ -136,8 +285,16 @@ class MLP(nn.Module):
             nn.Dropout(p_out),
         )
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return self.block(x)
+    def forward(self, x: torch.Tensor, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``block(x)``, plus ``residual`` if given.  With the exact GELU and no active dropout
+        the activation and the sum ride on the projections (``Linear.forward``)."""
+        first, act, drop1, second, drop2 = self.block
+        idle = lambda d: d.p == 0 or not d.training   # noqa: E731
+        if (isinstance(first, Linear) and isinstance(second, Linear) and type(act) is nn.GELU
+                and act.approximate == "none" and idle(drop1) and idle(drop2)):
+            return second(first(x, act="gelu"), residual=residual)
+        y = self.block(x)
+        return y if residual is None else residual + y
 
 
 class LayerNorm(nn.Module):

@@ -29,8 +29,10 @@ from typing import Any, Optional, Sequence
 import torch
 from torch import Tensor, nn
 
+from . import layers
 from .layers import MLP, LayerNorm, Linear
 from .ndc import Deconv
+from .norm import native_norm
 from .spec import as_tuple, build
 
 __all__ = ["DeconvMixer", "DeconverBlock", "DeconverStage", "Stem", "Deconver"]
@@ -52,8 +54,14 @@ class DeconvMixer(nn.Module):
         self.out_proj = Linear(self.deconv.groups * self.deconv.source_channels, out_channels)
         self.dropout = nn.Dropout(dropout)
 
-    def forward(self, x: Tensor) -> Tensor:
-        return self.dropout(self.out_proj(self.deconv(self.act(self.in_proj(x)))))
+    def forward(self, x: Tensor, residual: Optional[Tensor] = None) -> Tensor:
+        """The mixer's output, plus ``residual`` if given (the block's ``x + dcm(...)``, which
+        then rides on ``out_proj`` unless dropout is active)."""
+        sources = self.deconv(self.act(self.in_proj(x)))
+        if self.dropout.p == 0 or not self.training:
+            return self.out_proj(sources, residual=residual)
+        y = self.dropout(self.out_proj(sources))
+        return y if residual is None else residual + y
 
 
 class DeconverBlock(nn.Module):
@@ -62,14 +70,15 @@ class DeconverBlock(nn.Module):
     def __init__(self, channels: int, norm: Any = LayerNorm, dropout: float = 0.0,
                  mlp_ratio: float = 4, **mixer_kwargs):
         super().__init__()
+        norm = native_norm(norm)   # torch's InstanceNorm classes -> their HIP-backed subclasses
         self.norm1 = build(norm, channels)
         self.dcm = DeconvMixer(channels, channels, **mixer_kwargs)
         self.norm2 = build(norm, channels)
         self.mlp = MLP(channels, ratio=mlp_ratio, dropout=dropout)
 
     def forward(self, x: Tensor) -> Tensor:
-        x = x + self.dcm(self.norm1(x))
-        return x + self.mlp(self.norm2(x))
+        x = self.dcm(self.norm1(x), residual=x)
+        return self.mlp(self.norm2(x), residual=x)
 
 
 class DeconverStage(nn.Module):
@@ -99,7 +108,7 @@ class Stem(nn.Sequential):
                  norm: Any = LayerNorm):
         conv = getattr(nn, f"Conv{len(patch_size)}d")
         super().__init__(conv(in_channels, out_channels, patch_size, stride=patch_size),
-                         build(norm, out_channels))
+                         build(native_norm(norm), out_channels))
 
 
 class _Down(nn.Module):
@@ -178,12 +187,14 @@ class Deconver(nn.Module):
         self.spatial_dims = spatial_dims
         self.spatial_size = spatial_size
         conv = getattr(nn, f"Conv{spatial_dims}d")
-        tconv = getattr(nn, f"ConvTranspose{spatial_dims}d")
+        # same modules and parameters; their 16-bit GPU forward is a regrouping + GEMMs
+        pconv = getattr(layers, f"PatchConv{spatial_dims}d")
+        ptconv = getattr(layers, f"PatchConvTranspose{spatial_dims}d")
         if stem is None:
             stem = (conv, {"kernel_size": 3, "padding": 1, "bias": False})
-        downsample = downsample or (conv, {"kernel_size": 2})
-        upsample = upsample or (tconv, {"kernel_size": 2})
-        head = head or (conv, {"kernel_size": 1})
+        downsample = downsample or (pconv, {"kernel_size": 2})
+        upsample = upsample or (ptconv, {"kernel_size": 2})
+        head = head or (pconv, {"kernel_size": 1})
 
         if stem is nn.Identity:
             self.stem, width0 = nn.Identity(), in_channels

@@ -205,3 +205,71 @@ def gconv(lib: _lib.NdcLibrary, inp: Tensor, h: Tensor, *, groups: int, m: int, 
     out = torch.empty((inp.shape[0], cout, *inp.shape[2:]), dtype=inp.dtype, device=inp.device)
     lib.gconv(g, _ptr(inp), _ptr(h), _ptr(bias), adjoint, _ptr(out), _stream_of(inp))
     return out
+
+
+def _rownorm_workspace(lib: _lib.NdcLibrary, rows: int, n: int, device) -> Tensor:
+    return torch.empty(max(lib.rownorm_workspace_bytes(rows, n) // 4, 2), dtype=torch.float32, device=device)
+
+
+def rownorm_forward(lib: _lib.NdcLibrary, x: Tensor, eps: float):
+    """Normalises each row of the contiguous matrix ``x`` (rows, n) to zero mean and unit
+    (biased) variance.  Returns ``(y, stats)``; ``stats`` (rows, 2) holds (mean, rstd)."""
+    if x.dim() != 2 or not x.is_contiguous():
+        raise ValueError("rownorm_forward wants a contiguous (rows, n) matrix")
+    rows, n = x.shape
+    y = torch.empty_like(x)
+    stats = torch.empty(rows, 2, dtype=torch.float32, device=x.device)
+    ws = _rownorm_workspace(lib, rows, n, x.device)
+    lib.rownorm_forward(_ptr(x), _ptr(y), _ptr(stats), rows, n, dtype_tag(x.dtype), eps, _ptr(ws),
+                        ws.numel() * 4, _stream_of(x))
+    return y, stats
+
+
+def rownorm_backward(lib: _lib.NdcLibrary, gy: Tensor, y: Tensor, stats: Tensor) -> Tensor:
+    """Gradient of :func:`rownorm_forward` with respect to its input, from the gradient of
+    its output ``gy``, its output ``y`` and its ``stats``."""
+    if gy.shape != y.shape or gy.dtype != y.dtype or not (gy.is_contiguous() and y.is_contiguous()):
+        raise ValueError("rownorm_backward wants gy and y contiguous, of one shape and dtype")
+    rows, n = y.shape
+    gx = torch.empty_like(y)
+    ws = _rownorm_workspace(lib, rows, n, y.device)
+    lib.rownorm_backward(_ptr(gy), _ptr(y), _ptr(stats), _ptr(gx), rows, n, dtype_tag(y.dtype), _ptr(ws),
+                         ws.numel() * 4, _stream_of(y))
+    return gx
+
+
+ACTS = {None: _lib.ACT_NONE, "none": _lib.ACT_NONE, "relu": _lib.ACT_RELU, "gelu": _lib.ACT_GELU}
+
+
+def bias_act(lib: _lib.NdcLibrary, z: Tensor, bias: Optional[Tensor], residual: Optional[Tensor],
+             act: Optional[str], inplace: bool = False) -> Tensor:
+    """``act(z + bias[c]) + residual`` for a contiguous channel-first ``z`` of shape (B, C, n);
+    ``bias`` float32 of C entries or None, ``residual`` like ``z`` or None.  ``inplace`` writes
+    the result over ``z``."""
+    if z.dim() != 3 or not z.is_contiguous():
+        raise ValueError("bias_act wants a contiguous (B, C, n) tensor")
+    if bias is not None and (bias.dtype != torch.float32 or bias.numel() != z.shape[1] or not bias.is_contiguous()):
+        raise ValueError("bias must be float32 with one entry per channel")
+    if residual is not None and (residual.shape != z.shape or residual.dtype != z.dtype
+                                 or not residual.is_contiguous()):
+        raise ValueError("residual must be contiguous, of the shape and dtype of z")
+    y = z if inplace else torch.empty_like(z)
+    B, C, n = z.shape
+    lib.bias_act(_ptr(z), _ptr(bias), _ptr(residual), _ptr(y), B, C, n, ACTS[act], dtype_tag(z.dtype),
+                 _stream_of(z))
+    return y
+
+
+def bias_act_backward(lib: _lib.NdcLibrary, gy: Tensor, z: Tensor, bias: Optional[Tensor], act: str,
+                      need_bias_grad: bool = True, inplace: bool = False):
+    """``(gz, gbias)`` with ``gz = gy * act'(z + bias)`` and ``gbias`` its sum over batch and
+    voxels in float32 (None unless ``need_bias_grad``).  ``inplace`` writes ``gz`` over ``gy``."""
+    if gy.shape != z.shape or gy.dtype != z.dtype or not (gy.is_contiguous() and z.is_contiguous()):
+        raise ValueError("bias_act_backward wants gy and z contiguous, of one shape and dtype")
+    B, C, n = z.shape
+    gz = gy if inplace else torch.empty_like(gy)
+    parts = lib.bias_act_parts(B * C, n)
+    gpart = torch.empty(B, C, parts, dtype=torch.float32, device=z.device) if need_bias_grad else None
+    lib.bias_act_backward(_ptr(gy), _ptr(z), _ptr(bias), _ptr(gz), _ptr(gpart), B, C, n, ACTS[act],
+                          dtype_tag(z.dtype), _stream_of(z))
+    return gz, (gpart.sum((0, 2)) if need_bias_grad else None)

@@ -254,6 +254,53 @@ int ndc_gconv(const ndc_geom *g, const void *in, const float *h, const float *bi
 int ndc_relayout(const void *src, void *dst, int64_t batch, int64_t channels, int64_t spatial,
                  int dtype, int to_channels_last, void *stream);
 
+/*
+ * Row normalisation: y = (x - mean) / sqrt(var + eps) over each of `rows` contiguous rows of n
+ * elements (biased variance, float32 statistics), and its gradient.  On a channel-first tensor
+ * (B, C, *S) with rows = B * C and n = prod(S) this is InstanceNorm without affine parameters
+ * or running statistics: the norm1 / norm2 of a Deconver block (deconver/deconver.py:52-64) in
+ * the 2-D and 3-D segmentation networks, i.e. the producer of every NDC layer's input and the
+ * consumer of its gradient.  A row of the 3-D network's first level is 128^3 elements long and
+ * there are 128 of them, so each row is cut over many workgroups (two launches per direction:
+ * partial sums, then the transform).  HBM traffic: 2 reads + 1 write of the tensor forward,
+ * 4 reads + 1 write backward.
+ *   x, y         distinct device buffers of rows * n elements of `dtype`
+ *   stats        rows * 2 floats: (mean, 1/sqrt(var + eps)) per row; written by the forward,
+ *                read by the backward
+ *   gy, gx       gradient of y (in), of x (out); gx may be gy
+ *   workspace    ndc_rownorm_workspace_bytes(rows, n) bytes of device memory, 8-byte aligned;
+ *                contents need not survive between calls
+ * The backward takes the forward's OUTPUT y (the normalised rows), not x.
+ */
+size_t ndc_rownorm_workspace_bytes(int64_t rows, int64_t n);
+int ndc_rownorm_forward(const void *x, void *y, float *stats, int64_t rows, int64_t n, int dtype,
+                        float eps, void *workspace, size_t workspace_bytes, void *stream);
+int ndc_rownorm_backward(const void *gy, const void *y, const float *stats, void *gx, int64_t rows,
+                         int64_t n, int dtype, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * What follows a 1x1 projection in a Deconver block, in one pass over the projection's output:
+ *   y[b][c][i] = act(z[b][c][i] + bias[c]) + residual[b][c][i]
+ * on channel-first tensors of batch * channels rows of n elements.  It stands for the bias of
+ * the mixer's out_proj and of the MLP's two projections, the MLP's GELU and the block's
+ * residual sums (deconver/deconver.py:41-46, 60-64; deconver/layers/mlp.py:40-63), which
+ * PyTorch runs as separate passes over the tensor.
+ *   bias       `channels` floats, or NULL
+ *   residual   a tensor like z, or NULL
+ *   y          may be z (in place)
+ *   act        ndc_act; the GELU is the exact one, u * Phi(u)
+ * ndc_bias_act_backward: gz = gy * act'(z + bias) for NDC_ACT_RELU / NDC_ACT_GELU (gz may be
+ * gy), and, if gpart is not NULL, gpart[row * parts + p] = the sum of gz over part p of the
+ * row, parts = ndc_bias_act_parts(batch * channels, n): the bias gradient is their sum over the
+ * batch and the parts.  (With NDC_ACT_NONE the gradient of z is gy itself; the call is refused.)
+ */
+enum ndc_act { NDC_ACT_NONE = 0, NDC_ACT_RELU = 1, NDC_ACT_GELU = 2 };
+int64_t ndc_bias_act_parts(int64_t rows, int64_t n);
+int ndc_bias_act(const void *z, const float *bias, const void *residual, void *y, int64_t batch,
+                 int64_t channels, int64_t n, int act, int dtype, void *stream);
+int ndc_bias_act_backward(const void *gy, const void *z, const float *bias, void *gz, float *gpart,
+                          int64_t batch, int64_t channels, int64_t n, int act, int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,166 @@
+"""The pass that follows a 1x1 projection (ndc_bias_act / ndc_bias_act_backward: bias,
+activation, residual sum; bias-gradient partial sums) against PyTorch in float64, and the
+projections, MLP and block that use it against their unfused PyTorch forms.
+
+CPU tests run the host build of the library; GPU tests the HIP kernels.  Bars: float32 1e-5
+of the largest entry, bfloat16 2e-2."""
+
+import pytest
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+import deconver_amd as dc
+from deconver_amd import _lib, layers, ops
+from tests.helpers import hostcheck_library
+
+ACT = {None: lambda t: t, "relu": torch.relu, "gelu": F.gelu}
+
+
+def _rel(a, b):
+    return float((a.double() - b.double()).abs().max() / b.double().abs().max().clamp_min(1e-30))
+
+
+def _case(shape, dtype, seed, device="cpu"):
+    gen = torch.Generator().manual_seed(seed)
+    z = torch.randn(*shape, generator=gen).to(dtype).to(device)
+    res = torch.randn(*shape, generator=gen).to(dtype).to(device)
+    gy = torch.randn(*shape, generator=gen).to(dtype).to(device)
+    bias = torch.randn(shape[1], generator=gen).to(device)
+    return z, res, gy, bias
+
+
+def _check(lib, shape, dtype, act, with_bias, with_res, device="cpu"):
+    z, res, gy, bias = _case(shape, dtype, sum(shape), device)
+    b = bias if with_bias else None
+    r = res if with_res else None
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    z64 = z.double().requires_grad_(True)
+    u = z64 + (bias.double().view(1, -1, 1) if with_bias else 0)
+    ref = ACT[act](u) + (res.double() if with_res else 0)
+    y = ops.bias_act(lib, z, b, r, act)
+    assert _rel(y, ref.detach()) <= tol
+    y2 = ops.bias_act(lib, z.clone(), b, r, act, inplace=True)
+    assert torch.equal(y, y2)
+    if act is not None:
+        (gz_ref,) = torch.autograd.grad(ref, z64, gy.double())
+        gz, gb = ops.bias_act_backward(lib, gy, z, b, act)
+        assert _rel(gz, gz_ref) <= tol
+        assert gb.dtype == torch.float32
+        assert _rel(gb, gz_ref.sum((0, 2))) <= max(tol, 1e-4)
+        gz2, none = ops.bias_act_backward(lib, gy, z, b, act, need_bias_grad=False)
+        assert none is None and torch.equal(gz, gz2)
+
+
+SHAPES = [(2, 3, 7), (1, 5, 64), (2, 2, 8192 * 2 + 24), (1, 3, 2048 * 5 + 3)]
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("act", [None, "relu", "gelu"])
+def test_host_build_matches_pytorch(shape, dtype, act):
+    lib = hostcheck_library()
+    for with_bias, with_res in ((True, True), (True, False), (False, True)):
+        _check(lib, shape, dtype, act, with_bias, with_res)
+
+
+def test_bad_arguments_are_refused():
+    lib = hostcheck_library()
+    z = torch.zeros(2, 3, 8)
+    with pytest.raises(_lib.NdcError):
+        lib.bias_act(z.data_ptr(), None, None, z.data_ptr(), 2, 3, 8, 5, _lib.NDC_F32, None)
+    with pytest.raises(_lib.NdcError):
+        lib.bias_act(None, None, None, z.data_ptr(), 2, 3, 8, 0, _lib.NDC_F32, None)
+    with pytest.raises(_lib.NdcError):
+        lib.bias_act(z.data_ptr(), None, None, z.data_ptr(), 2, 3, 8, 0, 9, None)
+    with pytest.raises(_lib.NdcError):    # no activation: the gradient is gy itself
+        lib.bias_act_backward(z.data_ptr(), z.data_ptr(), None, z.data_ptr(), None, 2, 3, 8, 0, _lib.NDC_F32, None)
+    with pytest.raises(ValueError):
+        ops.bias_act(lib, z, torch.zeros(4), None, None)
+    assert lib.bias_act_parts(128, 128 ** 3) == 32 and lib.bias_act_parts(4096, 4096) == 1
+
+
+def test_general_route_of_the_fused_arguments_is_the_unfused_arithmetic():
+    """On the CPU ``Linear(x, act, residual)``, ``MLP(x, residual)`` and the block compute
+    exactly what the reference's modules do: conv1d, activation, sum."""
+    torch.manual_seed(0)
+    lin = dc.Linear(4, 6)
+    x, res = torch.randn(2, 4, 5, 3), torch.randn(2, 6, 5, 3)
+    plain = lin(x)
+    assert torch.equal(lin(x, act="gelu"), F.gelu(plain))
+    assert torch.equal(lin(x, act="relu", residual=res), res + torch.relu(plain))
+    mlp = dc.MLP(4, ratio=2)
+    r4 = torch.randn(2, 4, 5, 3)
+    assert torch.equal(mlp(x, residual=r4), r4 + mlp.block(x))
+    assert torch.equal(mlp(x), mlp.block(x))
+    mlp_d = dc.MLP(4, ratio=2, dropout=0.5)           # active dropout: the sequential form
+    torch.manual_seed(1)
+    a = mlp_d(x, residual=r4)
+    torch.manual_seed(1)
+    assert torch.equal(a, r4 + mlp_d.block(x))
+    blk = dc.DeconverBlock(4, kernel_size=(3, 3), ratio=2)
+    xb = torch.rand(1, 4, 6, 6)
+    h = xb + blk.dcm(blk.norm1(xb))
+    assert torch.equal(blk(xb), h + blk.mlp(blk.norm2(h)))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(2, 3, 7), (2, 64, 32 * 32 * 32), (1, 5, 2048 * 9 + 3), (2, 130, 4096)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("act", [None, "relu", "gelu"])
+def test_hip_kernels_match_pytorch(shape, dtype, act):
+    lib = _lib.get_library()
+    for with_bias, with_res in ((True, True), (True, False), (False, False)):
+        _check(lib, shape, dtype, act, with_bias, with_res, device="cuda")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("act,with_res", [(None, False), (None, True), ("gelu", False), ("relu", True)])
+def test_projection_with_fused_tail_matches_the_unfused_form(act, with_res):
+    """bf16 autocast on the GPU: values and every gradient of ``pointwise_linear(x, w, b, act,
+    residual)`` against conv1d + activation + sum on float64 copies of the same bf16-rounded
+    operands."""
+    torch.manual_seed(4)
+    B, cin, cout, n = 2, 32, 48, 4096 + 512
+    x = torch.randn(B, cin, n, device="cuda", requires_grad=True)
+    w = (torch.randn(cout, cin, 1, device="cuda") / cin ** 0.5).requires_grad_(True)
+    b = torch.randn(cout, device="cuda", requires_grad=True)
+    res = torch.randn(B, cout, n, device="cuda", requires_grad=True) if with_res else None
+    g = torch.randn(B, cout, n, device="cuda")
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        y = layers.pointwise_linear(x, w, b, act, res)
+    assert y.dtype == torch.bfloat16
+    leaves = [t for t in (x, w, b, res) if t is not None]
+    got = torch.autograd.grad(y, leaves, g.bfloat16())
+    r64 = lambda t: t.detach().bfloat16().double().requires_grad_(True)   # noqa: E731
+    x64, w64, b64 = r64(x), r64(w), b.detach().double().requires_grad_(True)
+    res64 = r64(res) if with_res else None
+    u64 = F.conv1d(x64, w64, b64)
+    if act == "relu":
+        # the rectifier's on/off pattern as the kernels saw it (from the bf16-rounded GEMM
+        # result): a unit within rounding of zero may differ from the float64 pattern, and
+        # one such unit moves a gradient by a finite amount
+        with torch.autocast("cuda", dtype=torch.bfloat16), torch.no_grad():
+            z_hip = layers.pointwise_linear(x, w, None)
+        ref = u64 * ((z_hip.float() + b.detach().view(1, -1, 1)) > 0) + (res64 if with_res else 0)
+    else:
+        ref = ACT[act](u64) + (res64 if with_res else 0)
+    want = torch.autograd.grad(ref, [t for t in (x64, w64, b64, res64) if t is not None], g.bfloat16().double())
+    assert _rel(y, ref) <= 2e-2
+    for a, r in zip(got, want):
+        assert a.shape == r.shape and _rel(a, r) <= 2e-2
+
+
+@pytest.mark.gpu
+def test_block_on_the_gpu_matches_its_float64_general_route():
+    """A Deconver block under bf16 autocast (HIP norm, NDC kernels, fused projection tails)
+    against the same block in float64 on the CPU's general route: output within the bf16
+    bar."""
+    torch.manual_seed(5)
+    blk = dc.DeconverBlock(16, norm=nn.InstanceNorm3d, kernel_size=(3, 3, 3), ratio=4)
+    x = torch.rand(2, 16, 12, 12, 16)
+    ref = blk.double()(x.double())
+    blk = blk.float().cuda()
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        y = blk(x.cuda())
+    assert _rel(y.cpu(), ref.detach()) <= 2e-2

@@ -1,0 +1,115 @@
+"""The resampling convolutions as regrouping + 1x1 projection (layers.patch_conv,
+layers.patch_conv_transpose) against torch's convolutions: same values, same gradients, same
+parameters.  The reference uses ``nn.ConvNd(kernel_size=2, stride=2)`` and
+``nn.ConvTransposeNd(kernel_size=2, stride=2)`` (unet.py:36-60, 108-131) and a 1-tap head."""
+
+import pytest
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+import deconver_amd as dc
+from deconver_amd import layers
+
+
+@pytest.mark.parametrize("k,size", [((2, 2), (6, 8)), ((2, 2, 2), (4, 6, 8)), ((2, 2, 2), (5, 6, 7)),
+                                     ((1, 1, 1), (3, 4, 5)), ((2, 3), (4, 9)), ((4, 4), (8, 12))])
+def test_patch_conv_is_the_strided_convolution(k, size):
+    torch.manual_seed(0)
+    nd = len(k)
+    conv = getattr(F, f"conv{nd}d")
+    x = torch.randn(2, 3, *size, dtype=torch.float64, requires_grad=True)
+    w = torch.randn(5, 3, *k, dtype=torch.float64, requires_grad=True)
+    b = torch.randn(5, dtype=torch.float64, requires_grad=True)
+    ref = conv(x, w, b, stride=k)
+    got = layers.patch_conv(x, w, b)
+    assert got.shape == ref.shape
+    torch.testing.assert_close(got, ref, rtol=1e-12, atol=1e-12)
+    g = torch.randn_like(ref)
+    for a, r in zip(torch.autograd.grad(got, (x, w, b), g), torch.autograd.grad(ref, (x, w, b), g)):
+        torch.testing.assert_close(a, r, rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(layers.patch_conv(x, w, None), conv(x, w, None, stride=k), rtol=1e-12, atol=1e-12)
+
+
+@pytest.mark.parametrize("k,size", [((2, 2), (3, 4)), ((2, 2, 2), (2, 3, 4)), ((1, 1), (3, 4)), ((3, 2), (2, 5))])
+def test_patch_conv_transpose_is_the_transposed_convolution(k, size):
+    torch.manual_seed(1)
+    nd = len(k)
+    tconv = getattr(F, f"conv_transpose{nd}d")
+    x = torch.randn(2, 4, *size, dtype=torch.float64, requires_grad=True)
+    w = torch.randn(4, 3, *k, dtype=torch.float64, requires_grad=True)
+    b = torch.randn(3, dtype=torch.float64, requires_grad=True)
+    ref = tconv(x, w, b, stride=k)
+    got = layers.patch_conv_transpose(x, w, b)
+    assert got.shape == ref.shape
+    torch.testing.assert_close(got, ref, rtol=1e-12, atol=1e-12)
+    g = torch.randn_like(ref)
+    for a, r in zip(torch.autograd.grad(got, (x, w, b), g), torch.autograd.grad(ref, (x, w, b), g)):
+        torch.testing.assert_close(a, r, rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(layers.patch_conv_transpose(x, w, None), tconv(x, w, None, stride=k),
+                               rtol=1e-12, atol=1e-12)
+
+
+def test_regrouping_round_trip():
+    x = torch.arange(2 * 3 * 4 * 6 * 8, dtype=torch.float32).view(2, 3, 4, 6, 8)
+    cols = layers.patches_to_channels(x, (2, 2, 2))
+    assert cols.shape == (2, 24, 2 * 3 * 4)
+    assert torch.equal(layers.channels_to_patches(cols, (2, 2, 2), (2, 3, 4)), x)
+
+
+def test_modules_keep_the_parent_parameters_and_route():
+    """Same parameter names and shapes as the torch modules, so reference checkpoints load;
+    on the CPU (and in float32) the parent's convolution runs; other strides always do."""
+    torch.manual_seed(2)
+    for cls, parent, args in ((layers.PatchConv3d, nn.Conv3d, (3, 5, 2)), (layers.PatchConvTranspose2d, nn.ConvTranspose2d, (3, 5, 2))):
+        mod, ref = cls(*args, stride=2), parent(*args, stride=2)
+        assert isinstance(mod, parent)
+        assert {k: v.shape for k, v in mod.state_dict().items()} == {k: v.shape for k, v in ref.state_dict().items()}
+        ref.load_state_dict(mod.state_dict())
+        x = torch.randn(2, 3, *([4] * (mod.weight.dim() - 2)))
+        assert torch.equal(mod(x), ref(x))
+    odd = layers.PatchConv2d(3, 5, 3, stride=1, padding=1)
+    assert not layers._is_patch_conv(odd)
+    assert layers._is_patch_conv(layers.PatchConv2d(3, 5, 2, stride=2))
+    assert layers._is_patch_conv(layers.PatchConv3d(3, 5, 1))
+    assert not layers._is_patch_conv(layers.PatchConvTranspose2d(3, 5, 2, stride=2, output_padding=1))
+    assert not layers._is_patch_conv(layers.PatchConv2d(4, 4, 2, stride=2, groups=2))
+    x = torch.randn(1, 3, 6, 6)
+    assert odd(x).shape == (1, 5, 6, 6)
+
+
+def test_network_uses_them_with_the_reference_state_dict_names():
+    net = dc.Deconver(in_channels=1, out_channels=2, spatial_dims=2, encoder_depth=(1, 1), encoder_width=(4, 8),
+                      strides=(1, 2), decoder_depth=(1,), kernel_size=(3, 3), ratio=2)
+    assert isinstance(net.encoder.blocks[1].downsample, layers.PatchConv2d)
+    assert isinstance(net.decoder.blocks[0].upsample, layers.PatchConvTranspose2d)
+    assert isinstance(net.head, layers.PatchConv2d)
+    keys = set(net.state_dict())
+    assert {"encoder.blocks.1.downsample.weight", "encoder.blocks.1.downsample.bias",
+            "decoder.blocks.0.upsample.weight", "decoder.blocks.0.upsample.bias", "head.weight", "head.bias"} <= keys
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("nd", [2, 3])
+def test_gemm_route_matches_the_library_convolution_on_the_gpu(nd):
+    """bf16 autocast on the GPU (the route the 3-D training step takes): values and gradients
+    of the regrouped form against torch's convolution of the same 16-bit operands, to the
+    bf16 bar 2e-2 of the largest entry."""
+    torch.manual_seed(3)
+    size = (16, 12, 20)[:nd]
+    down = getattr(layers, f"PatchConv{nd}d")(16, 32, 2, stride=2).cuda()
+    up = getattr(layers, f"PatchConvTranspose{nd}d")(32, 16, 2, stride=2).cuda()
+    x = torch.randn(2, 16, *size, device="cuda", requires_grad=True)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        y = up(down(x))
+        conv, tconv = getattr(F, f"conv{nd}d"), getattr(F, f"conv_transpose{nd}d")
+        ref = tconv(conv(x, down.weight, down.bias, stride=2), up.weight, up.bias, stride=2)
+    assert y.dtype == torch.bfloat16 and y.shape == ref.shape
+    params = (x, down.weight, down.bias, up.weight, up.bias)
+    g = torch.randn_like(ref)
+    got = torch.autograd.grad(y, params, g)
+    want = torch.autograd.grad(ref, params, g)
+    for a, r in zip((y, *got), (ref, *want)):
+        assert a.shape == r.shape
+        err = float((a.float() - r.float()).abs().max() / r.float().abs().max())
+        assert err <= 2e-2, err
