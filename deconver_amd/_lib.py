@@ -116,7 +116,7 @@ class NdcLibrary:
         d.ndc_rownorm_workspace_bytes.argtypes = [ctypes.c_int64, ctypes.c_int64]
         d.ndc_rownorm_forward.argtypes = [vp, vp, vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int,
                                           ctypes.c_float, vp, ctypes.c_size_t, vp]
-        d.ndc_rownorm_backward.argtypes = [vp, vp, vp, vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int,
+        d.ndc_rownorm_backward.argtypes = [vp, vp, vp, vp, vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int,
                                            vp, ctypes.c_size_t, vp]
         d.ndc_bias_act_parts.restype = ctypes.c_int64
         d.ndc_bias_act_parts.argtypes = [ctypes.c_int64, ctypes.c_int64]
@@ -257,9 +257,9 @@ class NdcLibrary:
         self._check(self._dll.ndc_rownorm_forward(x, y, stats, rows, n, dtype, eps, workspace,
                                                   workspace_bytes, stream), "ndc_rownorm_forward")
 
-    def rownorm_backward(self, gy: int, y: int, stats: int, gx: int, rows: int, n: int, dtype: int,
-                         workspace: int, workspace_bytes: int, stream) -> None:
-        self._check(self._dll.ndc_rownorm_backward(gy, y, stats, gx, rows, n, dtype, workspace,
+    def rownorm_backward(self, gy: int, y: int, stats: int, addend: Optional[int], gx: int, rows: int,
+                         n: int, dtype: int, workspace: int, workspace_bytes: int, stream) -> None:
+        self._check(self._dll.ndc_rownorm_backward(gy, y, stats, addend, gx, rows, n, dtype, workspace,
                                                    workspace_bytes, stream), "ndc_rownorm_backward")
 
     def bias_act_parts(self, rows: int, n: int) -> int:

@@ -445,12 +445,13 @@ int ndc_rownorm_forward(const void *x, void *y, float *stats, int64_t rows, int6
     rownorm_split(rows, n, nsplit, chunk);
     const int esz = dtype == NDC_BF16 ? 2 : 4;
     const bool vec = n % (16 / esz) == 0 && aligned16(x) && aligned16(y);
-    return ndc::Backend::rownorm(false, x, nullptr, (float *)workspace, stats, y, rows, n, nsplit, chunk,
-                                 esz, vec, eps, stream);
+    return ndc::Backend::rownorm(false, x, nullptr, nullptr, (float *)workspace, stats, y, rows, n, nsplit,
+                                 chunk, esz, vec, eps, stream);
 }
 
-int ndc_rownorm_backward(const void *gy, const void *y, const float *stats, void *gx, int64_t rows,
-                         int64_t n, int dtype, void *workspace, size_t workspace_bytes, void *stream)
+int ndc_rownorm_backward(const void *gy, const void *y, const float *stats, const void *addend, void *gx,
+                         int64_t rows, int64_t n, int dtype, void *workspace, size_t workspace_bytes,
+                         void *stream)
 {
     if (!gy || !y || !stats || !gx || !workspace) return NDC_ERR_NULL;
     int st = rownorm_check(rows, n, dtype);
@@ -462,9 +463,10 @@ int ndc_rownorm_backward(const void *gy, const void *y, const float *stats, void
     long long chunk;
     rownorm_split(rows, n, nsplit, chunk);
     const int esz = dtype == NDC_BF16 ? 2 : 4;
-    const bool vec = n % (16 / esz) == 0 && aligned16(gy) && aligned16(y) && aligned16(gx);
-    return ndc::Backend::rownorm(true, gy, y, (float *)workspace, const_cast<float *>(stats), gx, rows, n,
-                                 nsplit, chunk, esz, vec, 0.f, stream);
+    const bool vec = n % (16 / esz) == 0 && aligned16(gy) && aligned16(y) && aligned16(gx) &&
+                     (!addend || aligned16(addend));
+    return ndc::Backend::rownorm(true, gy, y, addend, (float *)workspace, const_cast<float *>(stats), gx, rows,
+                                 n, nsplit, chunk, esz, vec, 0.f, stream);
 }
 
 static int bias_act_check(long long batch, long long channels, long long n, int act, int dtype)

@@ -246,38 +246,50 @@ struct Backend {
     // workgroups.  Forward: a = x, out = y, stats written; backward: a = gy, b = y, stats read,
     // out = gx.  `vec`: n is a multiple of 16 bytes of elements and every pointer is 16-byte
     // aligned.
-    template <typename T, bool BWD>
-    static int rownorm_t(const void *a, const void *b, float *partial, float *stats, void *out,
-                         long long rows, long long n, int nsplit, long long chunk, bool vec, float eps,
-                         void *stream)
+    template <typename T, bool BWD, bool VEC>
+    static void rownorm_launch(const void *a, const void *b, const void *addend, float *partial, float *stats,
+                               void *out, long long rows, const rownorm::Split &sp, float eps, void *stream)
     {
         using namespace rownorm;
-        const Split sp = {n, chunk, nsplit};
-        const dim3 grid((unsigned)(rows * nsplit)), block(kThreads);
-        if (vec) {
-            hipLaunchKernelGGL((reduce_kernel<T, BWD, true>), grid, block, 0, (hipStream_t)stream,
-                               (const T *)a, (const T *)b, (float2 *)partial, sp);
-            hipLaunchKernelGGL((apply_kernel<T, BWD, true>), grid, block, 0, (hipStream_t)stream,
-                               (const T *)a, (const T *)b, (const float2 *)partial, (float2 *)stats, (T *)out, sp, eps);
-        } else {
-            hipLaunchKernelGGL((reduce_kernel<T, BWD, false>), grid, block, 0, (hipStream_t)stream,
-                               (const T *)a, (const T *)b, (float2 *)partial, sp);
-            hipLaunchKernelGGL((apply_kernel<T, BWD, false>), grid, block, 0, (hipStream_t)stream,
-                               (const T *)a, (const T *)b, (const float2 *)partial, (float2 *)stats, (T *)out, sp, eps);
-        }
-        return check();
+        const dim3 grid((unsigned)(rows * sp.nsplit)), block(kThreads);
+        hipLaunchKernelGGL((reduce_kernel<T, BWD, VEC>), grid, block, 0, (hipStream_t)stream, (const T *)a,
+                           (const T *)b, (float2 *)partial, sp);
+        if (BWD && addend)
+            hipLaunchKernelGGL((apply_kernel<T, BWD, VEC, BWD>), grid, block, 0, (hipStream_t)stream, (const T *)a,
+                               (const T *)b, (const T *)addend, (const float2 *)partial, (float2 *)stats, (T *)out,
+                               sp, eps);
+        else
+            hipLaunchKernelGGL((apply_kernel<T, BWD, VEC, false>), grid, block, 0, (hipStream_t)stream,
+                               (const T *)a, (const T *)b, (const T *)nullptr, (const float2 *)partial,
+                               (float2 *)stats, (T *)out, sp, eps);
     }
 
-    static int rownorm(bool bwd, const void *a, const void *b, float *partial, float *stats, void *out,
-                       long long rows, long long n, int nsplit, long long chunk, int esz, bool vec,
+    // Row normalisation, one direction: reduce launch then apply launch on rows * nsplit
+    // workgroups.  Forward: a = x, out = y, stats written; backward: a = gy, b = y, stats read,
+    // out = gx (+ addend, if given).  `vec`: n is a multiple of 16 bytes of elements and every
+    // pointer is 16-byte aligned.
+    template <typename T>
+    static void rownorm_t(bool bwd, const void *a, const void *b, const void *addend, float *partial, float *stats,
+                          void *out, long long rows, const rownorm::Split &sp, bool vec, float eps, void *stream)
+    {
+        if (bwd) {
+            if (vec) rownorm_launch<T, true, true>(a, b, addend, partial, stats, out, rows, sp, eps, stream);
+            else rownorm_launch<T, true, false>(a, b, addend, partial, stats, out, rows, sp, eps, stream);
+        } else {
+            if (vec) rownorm_launch<T, false, true>(a, b, addend, partial, stats, out, rows, sp, eps, stream);
+            else rownorm_launch<T, false, false>(a, b, addend, partial, stats, out, rows, sp, eps, stream);
+        }
+    }
+
+    static int rownorm(bool bwd, const void *a, const void *b, const void *addend, float *partial, float *stats,
+                       void *out, long long rows, long long n, int nsplit, long long chunk, int esz, bool vec,
                        float eps, void *stream)
     {
         if (rows <= 0 || n <= 0) return 0;
-        if (esz == 2)
-            return bwd ? rownorm_t<bf16_t, true>(a, b, partial, stats, out, rows, n, nsplit, chunk, vec, eps, stream)
-                       : rownorm_t<bf16_t, false>(a, b, partial, stats, out, rows, n, nsplit, chunk, vec, eps, stream);
-        return bwd ? rownorm_t<float, true>(a, b, partial, stats, out, rows, n, nsplit, chunk, vec, eps, stream)
-                   : rownorm_t<float, false>(a, b, partial, stats, out, rows, n, nsplit, chunk, vec, eps, stream);
+        const rownorm::Split sp = {n, chunk, nsplit};
+        if (esz == 2) rownorm_t<bf16_t>(bwd, a, b, addend, partial, stats, out, rows, sp, vec, eps, stream);
+        else rownorm_t<float>(bwd, a, b, addend, partial, stats, out, rows, sp, vec, eps, stream);
+        return check();
     }
 
     // y = act(z + bias[channel]) + residual on rows * nsplit workgroups (bias, residual optional)

@@ -58,8 +58,8 @@ struct Backend {
     // Row normalisation as the HIP build computes it (part by part, float32 sums, the same
     // shift and the same formulas), sequentially.
     template <typename T>
-    static void rownorm_t(bool bwd, const T *a, const T *b, float *partial, float *stats, T *out,
-                          long long rows, long long n, int nsplit, long long chunk, float eps)
+    static void rownorm_t(bool bwd, const T *a, const T *b, const T *addend, float *partial, float *stats,
+                          T *out, long long rows, long long n, int nsplit, long long chunk, float eps)
     {
         for (long long row = 0; row < rows; ++row) {
             const T *ar = a + row * n, *br = bwd ? b + row * n : nullptr;
@@ -95,21 +95,23 @@ struct Backend {
             }
             for (long long i = 0; i < n; ++i) {
                 const float v = Elem<T>::load(ar + i);
-                Elem<T>::store(out + row * n + i, bwd ? v * c1 + c0 + Elem<T>::load(br + i) * c2 : (v - c0) * c1);
+                float f = bwd ? v * c1 + c0 + Elem<T>::load(br + i) * c2 : (v - c0) * c1;
+                if (bwd && addend) f += Elem<T>::load(addend + row * n + i);
+                Elem<T>::store(out + row * n + i, f);
             }
         }
     }
 
-    static int rownorm(bool bwd, const void *a, const void *b, float *partial, float *stats, void *out,
-                       long long rows, long long n, int nsplit, long long chunk, int esz, bool, float eps,
-                       void *)
+    static int rownorm(bool bwd, const void *a, const void *b, const void *addend, float *partial, float *stats,
+                       void *out, long long rows, long long n, int nsplit, long long chunk, int esz, bool,
+                       float eps, void *)
     {
         if (esz == 2)
-            rownorm_t<bf16_t>(bwd, (const bf16_t *)a, (const bf16_t *)b, partial, stats, (bf16_t *)out, rows, n,
-                              nsplit, chunk, eps);
+            rownorm_t<bf16_t>(bwd, (const bf16_t *)a, (const bf16_t *)b, (const bf16_t *)addend, partial, stats,
+                              (bf16_t *)out, rows, n, nsplit, chunk, eps);
         else
-            rownorm_t<float>(bwd, (const float *)a, (const float *)b, partial, stats, (float *)out, rows, n,
-                             nsplit, chunk, eps);
+            rownorm_t<float>(bwd, (const float *)a, (const float *)b, (const float *)addend, partial, stats,
+                             (float *)out, rows, n, nsplit, chunk, eps);
         return 0;
     }
 

@@ -11,7 +11,10 @@
 //
 //   forward : a' = b' = x - x[row][0] (a shift that keeps the variance free of cancellation);
 //             y = (x - mean) rstd;  stats[row] = (mean, rstd)
-//   backward: a' = gy, b' = y;  gx = rstd (gy - mean(gy) - y mean(gy y))
+//   backward: a' = gy, b' = y;  gx = rstd (gy - mean(gy) - y mean(gy y)) [+ addend]
+//
+// The backward's optional addend is the gradient that reaches x by another way (the residual
+// branch around a pre-norm block): summed here, it saves the separate pass that would add it.
 //
 // HBM traffic: forward 2 reads + 1 write of the tensor, backward 4 reads + 1 write.  Sums are
 // float32 whatever the storage type.  Device code only (included by the HIP build).
@@ -155,14 +158,16 @@ reduce_kernel(const T *a, const T *b, float2 *partial, Split sp)
     if (threadIdx.x == 0) partial[blockIdx.x] = make_float2(s1, s2);
 }
 
-template <typename T, bool BWD, bool VEC>
+template <typename T, bool BWD, bool VEC, bool ADD = false>
 __global__ void __launch_bounds__(kThreads)
-apply_kernel(const T *a, const T *b, const float2 *partial, float2 *stats, T *out, Split sp, float eps)
+apply_kernel(const T *a, const T *b, const T *addend, const float2 *partial, float2 *stats, T *out, Split sp,
+             float eps)
 {
     __shared__ float buf[4][2];
     const long long row = blockIdx.x / sp.nsplit;
     const int part = blockIdx.x % sp.nsplit;
     const T *ar = a + row * sp.n, *br = BWD ? b + row * sp.n : nullptr;
+    const T *dr = ADD ? addend + row * sp.n : nullptr;
     T *orow = out + row * sp.n;
     const long long lo = part * sp.chunk, hi = lo + sp.chunk < sp.n ? lo + sp.chunk : sp.n;
     float s1, s2;
@@ -189,51 +194,50 @@ apply_kernel(const T *a, const T *b, const float2 *partial, float2 *stats, T *ou
         typedef Vec<T> V;
         const long long v0 = lo / V::N, v1 = hi / V::N;
         const V *av = reinterpret_cast<const V *>(ar), *bv = reinterpret_cast<const V *>(br);
+        const V *dv = reinterpret_cast<const V *>(dr);
         V *ov = reinterpret_cast<V *>(orow);
-        auto one = [&](const V &x, const V &y) {
+        auto one = [&](const V &x, const V &y, const V &d) {
             V r;
+            float v[V::N];
+#pragma unroll
+            for (int e = 0; e < V::N; ++e) {
+                v[e] = BWD ? x.get(e) * c1 + c0 + y.get(e) * c2 : (x.get(e) - c0) * c1;
+                if (ADD) v[e] += d.get(e);
+            }
             if constexpr (sizeof(T) == 2) {
 #pragma unroll
-                for (int p = 0; p < V::N / 2; ++p) {
-                    float f0, f1;
-                    if (BWD) {
-                        f0 = x.get(2 * p) * c1 + c0 + y.get(2 * p) * c2;
-                        f1 = x.get(2 * p + 1) * c1 + c0 + y.get(2 * p + 1) * c2;
-                    } else {
-                        f0 = (x.get(2 * p) - c0) * c1;
-                        f1 = (x.get(2 * p + 1) - c0) * c1;
-                    }
-                    r.set_pair(p, f0, f1);
-                }
+                for (int p = 0; p < V::N / 2; ++p) r.set_pair(p, v[2 * p], v[2 * p + 1]);
             } else {
 #pragma unroll
-                for (int e = 0; e < V::N; ++e) {
-                    r.set(e, BWD ? x.get(e) * c1 + c0 + y.get(e) * c2 : (x.get(e) - c0) * c1);
-                }
+                for (int e = 0; e < V::N; ++e) r.set(e, v[e]);
             }
             return r;
         };
         long long i = v0 + threadIdx.x;
         for (; i + 3 * kThreads < v1; i += 4 * kThreads) {
-            V x[4], y[4];
+            V x[4], y[4], d[4];
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
                 x[u] = av[i + u * kThreads];
                 if (BWD) y[u] = bv[i + u * kThreads];
+                if (ADD) d[u] = dv[i + u * kThreads];
             }
 #pragma unroll
-            for (int u = 0; u < 4; ++u) ov[i + u * kThreads] = one(x[u], y[u]);
+            for (int u = 0; u < 4; ++u) ov[i + u * kThreads] = one(x[u], y[u], d[u]);
         }
         for (; i < v1; i += kThreads) {
             const V x = av[i];
-            V y;
+            V y, d;
             if (BWD) y = bv[i];
-            ov[i] = one(x, y);
+            if (ADD) d = dv[i];
+            ov[i] = one(x, y, d);
         }
     } else {
         for (long long i = lo + threadIdx.x; i < hi; i += kThreads) {
             const float v = Elem<T>::load(ar + i);
-            Elem<T>::store(orow + i, BWD ? v * c1 + c0 + Elem<T>::load(br + i) * c2 : (v - c0) * c1);
+            float f = BWD ? v * c1 + c0 + Elem<T>::load(br + i) * c2 : (v - c0) * c1;
+            if (ADD) f += Elem<T>::load(dr + i);
+            Elem<T>::store(orow + i, f);
         }
     }
 }

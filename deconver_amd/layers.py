@@ -226,6 +226,56 @@ class _PatchConvTransposeMixin:
         return super().forward(x, output_size)
 
 
+def unfold_conv(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
+    """``conv(x, weight, bias, stride=1, padding=k // 2)`` for odd kernel sizes ``k`` as a column
+    matrix (every tap's shifted copy of the zero-padded input, channel-major then tap: the order
+    of the weight's ``(Cin, *k)`` axes) followed by the 1x1 projection."""
+    k = tuple(weight.shape[2:])
+    size = x.shape[2:]
+    pad = []
+    for v in reversed(k):
+        pad += [v // 2, v // 2]
+    xp = torch.nn.functional.pad(x, pad)
+    shifts = [()]
+    for v in k:
+        shifts = [t + (o,) for t in shifts for o in range(v)]
+    cols = torch.stack([xp[(slice(None), slice(None), *[slice(o, o + n) for o, n in zip(t, size)])]
+                        for t in shifts], dim=2)
+    y = pointwise_linear(cols.flatten(1, 2).flatten(2), weight.flatten(1), bias)
+    return y.view(x.shape[0], -1, *size)
+
+
+class _UnfoldConvMixin:
+    """The network's stem (unet.py:175-276: a 3-tap convolution from the few image channels to
+    the first width): with few input channels the column matrix is small next to the output,
+    and bfloat16 tensors on the GPU take ``unfold_conv`` -- one gather and the GEMMs of
+    ``pointwise_linear`` -- instead of the library's convolution, whose weight gradient alone
+    takes longer.  Anything else (more than ``max_columns`` rows in the column matrix, other
+    strides or paddings) runs the parent class's convolution."""
+
+    max_columns = 128
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        k = tuple(self.kernel_size)
+        if (_gemm_route(x) and x.dim() == len(k) + 2 and all(v % 2 == 1 for v in k)
+                and isinstance(self.padding, tuple) and tuple(self.padding) == tuple(v // 2 for v in k)
+                and all(v == 1 for v in self.stride) and all(v == 1 for v in self.dilation)
+                and self.groups == 1 and self.padding_mode == "zeros"
+                and self.in_channels * math.prod(k) <= self.max_columns):
+            if torch.is_autocast_enabled(x.device.type):
+                x = x.to(torch.get_autocast_dtype(x.device.type))    # before the gather, not after
+            return unfold_conv(x, self.weight, self.bias)
+        return super().forward(x)
+
+
+class UnfoldConv2d(_UnfoldConvMixin, nn.Conv2d):
+    pass
+
+
+class UnfoldConv3d(_UnfoldConvMixin, nn.Conv3d):
+    pass
+
+
 class PatchConv2d(_PatchConvMixin, nn.Conv2d):
     pass
 

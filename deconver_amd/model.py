@@ -77,8 +77,11 @@ class DeconverBlock(nn.Module):
         self.mlp = MLP(channels, ratio=mlp_ratio, dropout=dropout)
 
     def forward(self, x: Tensor) -> Tensor:
-        x = self.dcm(self.norm1(x), residual=x)
-        return self.mlp(self.norm2(x), residual=x)
+        # (norm(x), x): on the HIP norm the residual's gradient is summed in the norm's backward
+        y, x = self.norm1.with_skip(x) if hasattr(self.norm1, "with_skip") else (self.norm1(x), x)
+        x = self.dcm(y, residual=x)
+        y, x = self.norm2.with_skip(x) if hasattr(self.norm2, "with_skip") else (self.norm2(x), x)
+        return self.mlp(y, residual=x)
 
 
 class DeconverStage(nn.Module):
@@ -191,7 +194,7 @@ class Deconver(nn.Module):
         pconv = getattr(layers, f"PatchConv{spatial_dims}d")
         ptconv = getattr(layers, f"PatchConvTranspose{spatial_dims}d")
         if stem is None:
-            stem = (conv, {"kernel_size": 3, "padding": 1, "bias": False})
+            stem = (getattr(layers, f"UnfoldConv{spatial_dims}d"), {"kernel_size": 3, "padding": 1, "bias": False})
         downsample = downsample or (pconv, {"kernel_size": 2})
         upsample = upsample or (ptconv, {"kernel_size": 2})
         head = head or (pconv, {"kernel_size": 1})

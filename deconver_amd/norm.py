@@ -45,6 +45,38 @@ class _RowNorm(torch.autograd.Function):
         return gx.view(ctx.shape), None
 
 
+class _RowNormSkip(torch.autograd.Function):
+    """``(norm(x), x)``: the norm and the tensor it was taken of, for a pre-norm residual block
+    ``x + f(norm(x))``.  In backward the gradient that arrives for the second output (the
+    residual branch's) is summed into the norm's own input gradient by the kernel that writes
+    it, instead of by a separate addition."""
+
+    @staticmethod
+    def forward(ctx, x: Tensor, eps: float):
+        lib = _lib.get_library()
+        xc = x.contiguous()
+        rows = xc.shape[0] * xc.shape[1]
+        with torch.cuda.device(xc.device):
+            y, stats = ops.rownorm_forward(lib, xc.view(rows, -1), eps)
+        ctx.save_for_backward(y, stats)
+        ctx.shape = xc.shape
+        ctx.set_materialize_grads(False)     # an unused output's gradient arrives as None
+        return y.view(xc.shape), x.view_as(x)
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, gy, gskip):
+        y, stats = ctx.saved_tensors
+        if gy is None:
+            return gskip, None
+        gy = gy.contiguous().view(y.shape)
+        if gskip is not None:
+            gskip = gskip.to(gy.dtype).contiguous().view(y.shape)
+        with torch.cuda.device(y.device):
+            gx = ops.rownorm_backward(_lib.get_library(), gy, y, stats, addend=gskip)
+        return gx.view(ctx.shape), None
+
+
 def hip_norm_applies(x: Tensor) -> bool:
     return (x.is_cuda and x.dim() >= 3 and x.dtype in (torch.float32, torch.bfloat16) and x.numel() > 0
             and x[0, 0].numel() > 1)
@@ -60,14 +92,24 @@ def instance_norm(x: Tensor, eps: float = 1e-5) -> Tensor:
 
 
 class _HipInstanceNorm:
+    def _on_hip(self, x: Tensor) -> bool:
+        return not (self.affine or self.track_running_stats or not hip_norm_applies(x)
+                    or not _lib.library_available() or x.dim() == self._get_no_batch_dim())
+
     def forward(self, x: Tensor) -> Tensor:
-        if (self.affine or self.track_running_stats or not hip_norm_applies(x)
-                or not _lib.library_available()):
+        if not self._on_hip(x):
             return super().forward(x)
         self._check_input_dim(x)
-        if x.dim() == self._get_no_batch_dim():
-            return super().forward(x)
         return instance_norm(x, self.eps)
+
+    def with_skip(self, x: Tensor):
+        """``(self(x), x)`` for a residual block ``x + f(self(x))``: use the second tensor as
+        the residual term and the two gradients of ``x`` are summed inside the norm's backward
+        kernel (on the HIP route; elsewhere it is ``x`` itself)."""
+        if not self._on_hip(x) or not x.requires_grad:
+            return self(x), x
+        self._check_input_dim(x)
+        return _RowNormSkip.apply(x, float(self.eps))
 
 
 class InstanceNorm1d(_HipInstanceNorm, nn.InstanceNorm1d):

@@ -225,15 +225,19 @@ def rownorm_forward(lib: _lib.NdcLibrary, x: Tensor, eps: float):
     return y, stats
 
 
-def rownorm_backward(lib: _lib.NdcLibrary, gy: Tensor, y: Tensor, stats: Tensor) -> Tensor:
+def rownorm_backward(lib: _lib.NdcLibrary, gy: Tensor, y: Tensor, stats: Tensor,
+                     addend: Optional[Tensor] = None) -> Tensor:
     """Gradient of :func:`rownorm_forward` with respect to its input, from the gradient of
-    its output ``gy``, its output ``y`` and its ``stats``."""
+    its output ``gy``, its output ``y`` and its ``stats``; plus ``addend`` (a tensor like
+    ``gy``: the gradient that reaches the input by another way), if given."""
     if gy.shape != y.shape or gy.dtype != y.dtype or not (gy.is_contiguous() and y.is_contiguous()):
         raise ValueError("rownorm_backward wants gy and y contiguous, of one shape and dtype")
+    if addend is not None and (addend.shape != y.shape or addend.dtype != y.dtype or not addend.is_contiguous()):
+        raise ValueError("addend must be contiguous, of the shape and dtype of gy")
     rows, n = y.shape
     gx = torch.empty_like(y)
     ws = _rownorm_workspace(lib, rows, n, y.device)
-    lib.rownorm_backward(_ptr(gy), _ptr(y), _ptr(stats), _ptr(gx), rows, n, dtype_tag(y.dtype), _ptr(ws),
+    lib.rownorm_backward(_ptr(gy), _ptr(y), _ptr(stats), _ptr(addend), _ptr(gx), rows, n, dtype_tag(y.dtype), _ptr(ws),
                          ws.numel() * 4, _stream_of(y))
     return gx
 

@@ -268,6 +268,10 @@ int ndc_relayout(const void *src, void *dst, int64_t batch, int64_t channels, in
  *   stats        rows * 2 floats: (mean, 1/sqrt(var + eps)) per row; written by the forward,
  *                read by the backward
  *   gy, gx       gradient of y (in), of x (out); gx may be gy
+ *   addend       NULL, or a tensor like gy that is added to gx: the gradient that reaches x
+ *                around the norm (the residual branch of a pre-norm block,
+ *                deconver/deconver.py:63-64), which otherwise costs a pass of its own; gx may
+ *                be addend
  *   workspace    ndc_rownorm_workspace_bytes(rows, n) bytes of device memory, 8-byte aligned;
  *                contents need not survive between calls
  * The backward takes the forward's OUTPUT y (the normalised rows), not x.
@@ -275,8 +279,9 @@ int ndc_relayout(const void *src, void *dst, int64_t batch, int64_t channels, in
 size_t ndc_rownorm_workspace_bytes(int64_t rows, int64_t n);
 int ndc_rownorm_forward(const void *x, void *y, float *stats, int64_t rows, int64_t n, int dtype,
                         float eps, void *workspace, size_t workspace_bytes, void *stream);
-int ndc_rownorm_backward(const void *gy, const void *y, const float *stats, void *gx, int64_t rows,
-                         int64_t n, int dtype, void *workspace, size_t workspace_bytes, void *stream);
+int ndc_rownorm_backward(const void *gy, const void *y, const float *stats, const void *addend, void *gx,
+                         int64_t rows, int64_t n, int dtype, void *workspace, size_t workspace_bytes,
+                         void *stream);
 
 /*
  * What follows a 1x1 projection in a Deconver block, in one pass over the projection's output:

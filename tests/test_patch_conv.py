@@ -50,6 +50,24 @@ def test_patch_conv_transpose_is_the_transposed_convolution(k, size):
                                rtol=1e-12, atol=1e-12)
 
 
+@pytest.mark.parametrize("k,size", [((3, 3), (5, 7)), ((3, 3, 3), (4, 5, 6)), ((1, 3, 5), (3, 4, 7))])
+def test_unfold_conv_is_the_same_padded_convolution(k, size):
+    torch.manual_seed(6)
+    nd = len(k)
+    conv = getattr(F, f"conv{nd}d")
+    x = torch.randn(2, 2, *size, dtype=torch.float64, requires_grad=True)
+    w = torch.randn(5, 2, *k, dtype=torch.float64, requires_grad=True)
+    b = torch.randn(5, dtype=torch.float64, requires_grad=True)
+    ref = conv(x, w, b, padding=tuple(v // 2 for v in k))
+    got = layers.unfold_conv(x, w, b)
+    torch.testing.assert_close(got, ref, rtol=1e-12, atol=1e-12)
+    g = torch.randn_like(ref)
+    for a, r in zip(torch.autograd.grad(got, (x, w, b), g), torch.autograd.grad(ref, (x, w, b), g)):
+        torch.testing.assert_close(a, r, rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(layers.unfold_conv(x, w, None), conv(x, w, None, padding=tuple(v // 2 for v in k)),
+                               rtol=1e-12, atol=1e-12)
+
+
 def test_regrouping_round_trip():
     x = torch.arange(2 * 3 * 4 * 6 * 8, dtype=torch.float32).view(2, 3, 4, 6, 8)
     cols = layers.patches_to_channels(x, (2, 2, 2))
@@ -84,6 +102,8 @@ def test_network_uses_them_with_the_reference_state_dict_names():
     assert isinstance(net.encoder.blocks[1].downsample, layers.PatchConv2d)
     assert isinstance(net.decoder.blocks[0].upsample, layers.PatchConvTranspose2d)
     assert isinstance(net.head, layers.PatchConv2d)
+    assert isinstance(net.stem, layers.UnfoldConv2d) and isinstance(net.stem, nn.Conv2d)
+    assert tuple(net.stem.weight.shape) == (4, 1, 3, 3) and net.stem.bias is None
     keys = set(net.state_dict())
     assert {"encoder.blocks.1.downsample.weight", "encoder.blocks.1.downsample.bias",
             "decoder.blocks.0.upsample.weight", "decoder.blocks.0.upsample.bias", "head.weight", "head.bias"} <= keys
@@ -105,6 +125,16 @@ def test_gemm_route_matches_the_library_convolution_on_the_gpu(nd):
         conv, tconv = getattr(F, f"conv{nd}d"), getattr(F, f"conv_transpose{nd}d")
         ref = tconv(conv(x, down.weight, down.bias, stride=2), up.weight, up.bias, stride=2)
     assert y.dtype == torch.bfloat16 and y.shape == ref.shape
+    stem = getattr(layers, f"UnfoldConv{nd}d")(2, 16, 3, padding=1, bias=False).cuda()
+    img = torch.randn(2, 2, *size, device="cuda")
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        ys = stem(img)
+        rs = conv(img, stem.weight, None, padding=1)
+    assert ys.dtype == torch.bfloat16
+    gs = torch.randn_like(rs)
+    (gw,), (gw_ref,) = torch.autograd.grad(ys, stem.weight, gs), torch.autograd.grad(rs, stem.weight, gs)
+    for a, r in ((ys, rs), (gw, gw_ref)):
+        assert float((a.float() - r.float()).abs().max() / r.float().abs().max()) <= 2e-2
     params = (x, down.weight, down.bias, up.weight, up.bias)
     g = torch.randn_like(ref)
     got = torch.autograd.grad(y, params, g)

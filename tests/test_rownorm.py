@@ -29,6 +29,11 @@ def _rel(a, b):
 def _run(lib, x, gy, eps):
     y, stats = ops.rownorm_forward(lib, x, eps)
     gx = ops.rownorm_backward(lib, gy, y, stats)
+    # with an addend: the same plus that tensor (one rounding of the sum)
+    extra = torch.flip(gy, (1,))
+    gx2 = ops.rownorm_backward(lib, gy, y, stats, addend=extra)
+    tol = 1e-6 if x.dtype == torch.float32 else 1e-2
+    torch.testing.assert_close(gx2.float(), gx.float() + extra.float(), rtol=tol, atol=tol * float(gy.abs().max()))
     return y, stats, gx
 
 
@@ -135,6 +140,33 @@ def test_hip_module_matches_instance_norm(shape, eps, dtype):
     y2 = F.instance_norm(x2, eps=eps)
     (gx2,) = torch.autograd.grad(y2, x2, gy.cuda())
     assert _rel(y.cpu(), y2.double().cpu()) <= tol and _rel(gx.cpu(), gx2.double().cpu()) <= tol
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_with_skip_sums_the_two_gradients(dtype):
+    """x + f(norm(x)) through ``with_skip``: the gradient of x is the norm's plus the residual
+    branch's, as autograd would have summed them."""
+    torch.manual_seed(7)
+    shape = (2, 6, 16, 8, 40)
+    x = torch.randn(*shape, device="cuda").to(dtype).requires_grad_(True)
+    w = torch.randn(*shape, device="cuda").to(dtype)
+    g = torch.randn(*shape, device="cuda").to(dtype)
+    m = dc.InstanceNorm3d(6)
+    y, xs = m.with_skip(x)
+    (gx,) = torch.autograd.grad(xs + y * w, x, g)
+    x64 = x.detach().double().requires_grad_(True)
+    ref = x64 + F.instance_norm(x64) * w.double()
+    (gx_ref,) = torch.autograd.grad(ref, x64, g.double())
+    assert _rel(gx.cpu(), gx_ref.cpu()) <= (1e-5 if dtype == torch.float32 else 2e-2)
+    # only one of the two outputs used
+    y, xs = m.with_skip(x)
+    (ga,) = torch.autograd.grad(y * w, x, g)
+    (gb,) = torch.autograd.grad(m(x) * w, x, g)
+    assert torch.equal(ga, gb)
+    y, xs = m.with_skip(x)
+    (gc,) = torch.autograd.grad(xs * w, x, g)
+    assert torch.equal(gc, (g * w))
 
 
 @pytest.mark.gpu
