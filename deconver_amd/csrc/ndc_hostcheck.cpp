@@ -63,8 +63,13 @@ struct Backend {
     {
         for (long long row = 0; row < rows; ++row) {
             const T *ar = a + row * n, *br = bwd ? b + row * n : nullptr;
-            const float pivot = bwd ? 0.f : Elem<T>::load(ar);
-            float s1 = 0.f, s2 = 0.f;
+            float pivot = 0.f;
+            if (!bwd) {
+                const long long first = n < 256 ? n : 256;
+                for (long long i = 0; i < first; ++i) pivot += Elem<T>::load(ar + i);
+                pivot /= (float)first;
+            }
+            float s1 = 0.f, s2 = 0.f, cnt = 0.f, mean = 0.f, m2 = 0.f;
             for (int part = 0; part < nsplit; ++part) {
                 const long long lo = part * chunk, hi = lo + chunk < n ? lo + chunk : n;
                 float p1 = 0.f, p2 = 0.f;
@@ -73,10 +78,22 @@ struct Backend {
                     p1 += f;
                     p2 += f * (bwd ? Elem<T>::load(br + i) : f);
                 }
-                partial[2 * (row * nsplit + part)] = p1;
-                partial[2 * (row * nsplit + part) + 1] = p2;
-                s1 += p1;
-                s2 += p2;
+                const float np = (float)(hi - lo);
+                if (!bwd) {
+                    // the part's (mean, squared deviations), merged into the row's
+                    const float pm = pivot + p1 / np, pq = p2 - p1 * p1 / np;
+                    partial[2 * (row * nsplit + part)] = pm;
+                    partial[2 * (row * nsplit + part) + 1] = pq;
+                    const float tot = cnt + np, delta = pm - mean;
+                    mean += delta * (np / tot);
+                    m2 += pq + delta * delta * (cnt * np / tot);
+                    cnt = tot;
+                } else {
+                    partial[2 * (row * nsplit + part)] = p1;
+                    partial[2 * (row * nsplit + part) + 1] = p2;
+                    s1 += p1;
+                    s2 += p2;
+                }
             }
             const float inv_n = 1.f / (float)n;
             float c0, c1, c2 = 0.f;
@@ -85,11 +102,10 @@ struct Backend {
                 c0 = -c1 * s1 * inv_n;
                 c2 = -c1 * s2 * inv_n;
             } else {
-                const float m = s1 * inv_n;
-                float var = s2 * inv_n - m * m;
+                float var = m2 * inv_n;
                 var = var > 0.f ? var : 0.f;
                 c1 = 1.f / std::sqrt(var + eps);
-                c0 = pivot + m;
+                c0 = mean;
                 stats[2 * row] = c0;
                 stats[2 * row + 1] = c1;
             }

@@ -5,13 +5,15 @@
 // up to 128^3 elements long and there are as few as 128 rows.  A row is therefore cut into
 // `nsplit` parts, one workgroup each, in two launches per direction:
 //
-//   reduce:  partial[row][part] = (sum a', sum a' b')  over the part
-//   apply :  every workgroup adds its row's nsplit partials (same order everywhere), then
+//   reduce:  one partial result per (row, part)
+//   apply :  every workgroup combines its row's nsplit partials (same order everywhere), then
 //            transforms its part
 //
-//   forward : a' = b' = x - x[row][0] (a shift that keeps the variance free of cancellation);
-//             y = (x - mean) rstd;  stats[row] = (mean, rstd)
-//   backward: a' = gy, b' = y;  gx = rstd (gy - mean(gy) - y mean(gy y)) [+ addend]
+//   forward : partial = (mean, sum of squared deviations from it) of the part, from sums of
+//             x - pivot and (x - pivot)^2 with pivot = the mean of the row's first elements
+//             (so the squares carry no cancellation); parts are combined pairwise-exactly
+//             (Chan et al.); y = (x - mean) rstd;  stats[row] = (mean, rstd)
+//   backward: partial = (sum gy, sum gy y);  gx = rstd (gy - mean(gy) - y mean(gy y)) [+ addend]
 //
 // The backward's optional addend is the gradient that reaches x by another way (the residual
 // branch around a pre-norm block): summed here, it saves the separate pass that would add it.
@@ -110,7 +112,27 @@ reduce_kernel(const T *a, const T *b, float2 *partial, Split sp)
     const int part = blockIdx.x % sp.nsplit;
     const T *ar = a + row * sp.n, *br = BWD ? b + row * sp.n : nullptr;
     const long long lo = part * sp.chunk, hi = lo + sp.chunk < sp.n ? lo + sp.chunk : sp.n;
-    const float pivot = BWD ? 0.f : Elem<T>::load(ar);
+    float pivot = 0.f;
+    if (!BWD) {
+        // the mean of the row's first elements (one access per thread), the same in every part
+        float a = 0.f, unused = 0.f;
+        long long cnt;
+        if constexpr (VEC) {
+            typedef Vec<T> V;
+            const long long nv = sp.n / V::N;
+            cnt = (nv < kThreads ? nv : kThreads) * V::N;
+            if ((long long)threadIdx.x < nv) {
+                const V x = reinterpret_cast<const V *>(ar)[threadIdx.x];
+#pragma unroll
+                for (int e = 0; e < V::N; ++e) a += x.get(e);
+            }
+        } else {
+            cnt = sp.n < kThreads ? sp.n : kThreads;
+            if ((long long)threadIdx.x < sp.n) a = Elem<T>::load(ar + threadIdx.x);
+        }
+        block_sum2(a, unused, buf);
+        pivot = a / (float)cnt;
+    }
     float s1 = 0.f, s2 = 0.f;
     if constexpr (VEC) {
         typedef Vec<T> V;
@@ -155,7 +177,14 @@ reduce_kernel(const T *a, const T *b, float2 *partial, Split sp)
         }
     }
     block_sum2(s1, s2, buf);
-    if (threadIdx.x == 0) partial[blockIdx.x] = make_float2(s1, s2);
+    if (threadIdx.x == 0) {
+        if (!BWD) {
+            const float inv = 1.f / (float)(hi - lo);
+            partial[blockIdx.x] = make_float2(pivot + s1 * inv, s2 - s1 * s1 * inv);
+        } else {
+            partial[blockIdx.x] = make_float2(s1, s2);
+        }
+    }
 }
 
 template <typename T, bool BWD, bool VEC, bool ADD = false>
@@ -170,22 +199,30 @@ apply_kernel(const T *a, const T *b, const T *addend, const float2 *partial, flo
     const T *dr = ADD ? addend + row * sp.n : nullptr;
     T *orow = out + row * sp.n;
     const long long lo = part * sp.chunk, hi = lo + sp.chunk < sp.n ? lo + sp.chunk : sp.n;
-    float s1, s2;
-    row_totals(partial + row * sp.nsplit, sp.nsplit, s1, s2, buf);
     const float inv_n = 1.f / (float)sp.n;
     // forward: out = (x - c0) * c1;  backward: out = gy * c1 + y * c2 + c0
     float c0, c1, c2 = 0.f;
     if (BWD) {
+        float s1, s2;
+        row_totals(partial + row * sp.nsplit, sp.nsplit, s1, s2, buf);
         const float rstd = stats[row].y;
         c1 = rstd;
         c0 = -rstd * s1 * inv_n;
         c2 = -rstd * s2 * inv_n;
     } else {
-        const float pivot = Elem<T>::load(ar);
-        const float m = s1 * inv_n;
-        float var = s2 * inv_n - m * m;
+        // (count, mean, squared deviations) of the parts merged in order, by every thread
+        float cnt = 0.f, mean = 0.f, m2 = 0.f;
+        for (int p = 0; p < sp.nsplit; ++p) {
+            const float2 q = partial[row * sp.nsplit + p];
+            const long long plo = p * sp.chunk, phi = plo + sp.chunk < sp.n ? plo + sp.chunk : sp.n;
+            const float np = (float)(phi - plo), tot = cnt + np, delta = q.x - mean;
+            mean += delta * (np / tot);
+            m2 += q.y + delta * delta * (cnt * np / tot);
+            cnt = tot;
+        }
+        float var = m2 * inv_n;
         var = var > 0.f ? var : 0.f;
-        const float rstd = rsqrtf(var + eps), mean = pivot + m;
+        const float rstd = 1.f / sqrtf(var + eps);
         c1 = rstd;
         c0 = mean;
         if (part == 0 && threadIdx.x == 0) stats[row] = make_float2(mean, rstd);
