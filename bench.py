@@ -7,6 +7,7 @@
     python bench.py --workload grid                                       (ratio x groups x kernel grid)
     python bench.py --workload valu                                       (instruction-issue ceiling probe)
     python bench.py --workload train3d|model2d [--ndc hip|pytorch|both]   (model level, below)
+    python bench.py --workload block      (norm and projection-tail kernels of a Deconver block)
     python bench.py --workload mixer [--dtype bf16|fp32]                  (one DeconvMixer, fwd+bwd)
     python bench.py --workload layout                                     (channels-last copies around the update)
 
@@ -736,6 +737,102 @@ def layout_workload(args) -> int:
     return 0
 
 
+BLOCK_SHAPES = [("config 4, level 0: B 2, 64 ch, 128^3", 2, 64, 128 ** 3),
+                ("config 4, level 1 (= config 3): B 2, 128 ch, 64^3", 2, 128, 64 ** 3),
+                ("config 4, level 3: B 2, 512 ch, 16^3", 2, 512, 16 ** 3)]
+
+
+def block_rows(torch, steps: int, warmup: int) -> list:
+    """The HBM-bound kernels between the NDC layers of a Deconver block (InstanceNorm as row
+    normalisation, and the bias / GELU / residual pass after a 1x1 projection), bf16, forward and
+    backward, next to PyTorch's own kernels for the same arithmetic: ms and achieved GB/s on
+    the bytes each must move (U = B*C*N elements of 2 bytes: norm forward 3 U, backward 5 U;
+    bias + GELU on the 4C hidden tensor forward 8 U, backward 12 U; bias + residual 3 U)."""
+    import torch.nn.functional as F
+
+    import deconver_amd as dc
+    from deconver_amd import _lib, ops
+
+    lib = _lib.get_library()
+    dev = torch.device("cuda:0")
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps
+
+    rows = []
+    for name, B, C, n in BLOCK_SHAPES:
+        U = B * C * n * 2    # bytes of one (B, C, N) bf16 tensor
+        x = torch.randn(B * C, n, device=dev).bfloat16()
+        g = torch.randn(B * C, n, device=dev).bfloat16()
+        y, stats = ops.rownorm_forward(lib, x, 1e-5)
+        x3 = x.view(B, C, n).requires_grad_(True)
+        y3 = F.instance_norm(x3)
+        g3 = g.view(B, C, n)
+        r = {"shape": name}
+
+        def put(key, ms, nbytes):
+            r[key] = {"ms": ms, "GBs": nbytes / (ms * 1e-3) / 1e9, "hbm_frac": nbytes / (ms * 1e-3) / 8e12}
+
+        put("norm_forward", timed(lambda: ops.rownorm_forward(lib, x, 1e-5)), 3 * U)
+        put("norm_backward", timed(lambda: ops.rownorm_backward(lib, g, y, stats)), 5 * U)
+        put("norm_forward_pytorch", timed(lambda: F.instance_norm(x3)), 3 * U)
+        put("norm_backward_pytorch", timed(lambda: torch.autograd.grad(y3, x3, g3, retain_graph=True)), 5 * U)
+        del x, g, y, x3, y3, g3
+        z = torch.randn(B, 4 * C, n, device=dev).bfloat16()
+        gz = torch.randn(B, 4 * C, n, device=dev).bfloat16()
+        bias = torch.randn(4 * C, device=dev)
+        put("bias_gelu_forward", timed(lambda: ops.bias_act(lib, z, bias, None, "gelu")), 8 * U)
+        put("bias_gelu_backward", timed(lambda: ops.bias_act_backward(lib, gz, z, bias, "gelu")), 12 * U)
+        b16 = bias.bfloat16().view(1, -1, 1)
+        put("bias_gelu_forward_pytorch", timed(lambda: F.gelu(z + b16)), 8 * U)
+        zz = (z + b16).requires_grad_(True)
+        yy = F.gelu(zz)
+        put("bias_gelu_backward_pytorch",
+            timed(lambda: (torch.autograd.grad(yy, zz, gz, retain_graph=True)[0].sum(2, dtype=torch.float32).sum(0))), 12 * U)
+        del z, gz, zz, yy
+        z1 = torch.randn(B, C, n, device=dev).bfloat16()
+        res = torch.randn(B, C, n, device=dev).bfloat16()
+        b1 = torch.randn(C, device=dev)
+        put("bias_residual", timed(lambda: ops.bias_act(lib, z1, b1, res, None)), 3 * U)
+        b1h = b1.bfloat16().view(1, -1, 1)
+        put("bias_residual_pytorch", timed(lambda: res + (z1 + b1h)), 3 * U)
+        del z1, res
+        rows.append(r)
+        torch.cuda.empty_cache()
+    return rows
+
+
+def block_workload(args) -> int:
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    rows = block_rows(torch, args.steps, args.warmup)
+    first = rows[0]
+    ms = sum(first[k]["ms"] for k in ("norm_forward", "norm_backward", "bias_gelu_forward", "bias_gelu_backward",
+                                      "bias_residual"))
+    print(json.dumps({
+        "metric": "Deconver block: norm and projection-tail kernels, ms", "value": ms, "unit": "ms", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": False,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "row normalisation (InstanceNorm) and bias / GELU / residual passes of a "
+                               "Deconver block at config 4's levels, bf16, HIP kernels next to PyTorch's"},
+        "shapes": rows,
+        "roofline": {"kernel": "norm_backward", "bound": "hbm", "achieved": first["norm_backward"]["GBs"],
+                     "peak": 8000.0, "unit": "GB/s", "frac": first["norm_backward"]["hbm_frac"], "traffic": None},
+        "cpu_baseline": None}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -758,7 +855,7 @@ def main() -> int:
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     ap.add_argument("--build-probe", action="store_true",
                     help="with --workload valu: compile the probe (no GPU needed) and exit")
-    ap.add_argument("--workload", choices=("ndc", "sweep", "accuracy", "grid", "valu", "train3d", "model2d", "mixer", "layout"),
+    ap.add_argument("--workload", choices=("ndc", "sweep", "accuracy", "grid", "valu", "train3d", "model2d", "mixer", "layout", "block"),
                     default="ndc",
                     help="ndc: the headline update node (default); the others are model level")
     ap.add_argument("--ndc", choices=("hip", "pytorch", "both"), default="hip",
@@ -783,6 +880,8 @@ def main() -> int:
         return mixer_workload(args)
     if args.workload == "layout":
         return layout_workload(args)
+    if args.workload == "block":
+        return block_workload(args)
     if args.workload != "ndc":
         return model_workload(args)
 
