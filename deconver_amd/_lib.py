@@ -45,6 +45,7 @@ EXPORTS = (
     "ndc_bias_act_parts",
     "ndc_bias_act",
     "ndc_bias_act_backward",
+    "ndc_regroup",
 )
 
 
@@ -124,6 +125,8 @@ class NdcLibrary:
                                    ctypes.c_int, ctypes.c_int, vp]
         d.ndc_bias_act_backward.argtypes = [vp, vp, vp, vp, vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                                             ctypes.c_int, ctypes.c_int, vp]
+        d.ndc_regroup.argtypes = [vp, vp, vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                                   ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp]
         d.ndc_taps_bytes.restype = ctypes.c_size_t
         d.ndc_taps_bytes.argtypes = [gp]
         d.ndc_prepare_taps.argtypes = [gp, fp, vp, ctypes.c_size_t, vp]
@@ -275,6 +278,12 @@ class NdcLibrary:
                           batch: int, channels: int, n: int, act: int, dtype: int, stream) -> None:
         self._check(self._dll.ndc_bias_act_backward(gy, z, bias, gz, gpart, batch, channels, n, act, dtype,
                                                     stream), "ndc_bias_act_backward")
+
+    def regroup2(self, src: int, dst: int, bias: Optional[int], rows: int, channels: int, D: int, H: int,
+                 W: int, depth2: bool, dtype: int, to_channels: bool, stream) -> None:
+        """2 x 2 (x 2) windows of the fine grid (rows, D, H, W) <-> 4 (8) planes per row."""
+        self._check(self._dll.ndc_regroup(src, dst, bias, rows, channels, D, H, W, int(bool(depth2)), dtype,
+                                           int(bool(to_channels)), stream), "ndc_regroup")
 
 
 _lock = threading.Lock()

@@ -518,6 +518,24 @@ int ndc_bias_act_backward(const void *gy, const void *z, const float *bias, void
                                            chunk, act, esz, vec, stream);
 }
 
+int ndc_regroup(const void *src, void *dst, const float *bias, int64_t rows, int64_t channels, int64_t D,
+                 int64_t H, int64_t W, int depth2, int dtype, int to_channels, void *stream)
+{
+    if (!src || !dst) return NDC_ERR_NULL;
+    if (dtype != NDC_F32 && dtype != NDC_BF16) return NDC_ERR_DTYPE;
+    const int esz = dtype == NDC_BF16 ? 2 : 4;
+    if (rows < 1 || channels < 1 || D < 1 || H < 2 || W < 2 || D > 0x3fffffff || H > 0x3fffffff ||
+        W > 0x3fffffff || channels > 0x7fffffff || (long double)rows * D * H * W > 9.0e15L)
+        return NDC_ERR_GEOMETRY;
+    // even windows, whole 16-byte vectors per row, aligned buffers; a bias only on the way back
+    if (H % 2 || W % (16 / esz) || (depth2 && D % 2) || src == dst || !aligned16(src) || !aligned16(dst) ||
+        (bias && to_channels))
+        return NDC_ERR_GEOMETRY;
+    const int st = ndc::Backend::regroup2(src, dst, bias, rows, (int)channels, (int)D, (int)H, (int)W,
+                                          depth2 ? 1 : 0, esz, to_channels ? 1 : 0, stream);
+    return st == -2 ? (int)NDC_ERR_GEOMETRY : st;
+}
+
 int ndc_gconv(const ndc_geom *g, const void *in, const float *h, const float *bias, int adjoint,
               void *out, void *stream)
 {

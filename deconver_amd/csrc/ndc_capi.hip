@@ -5,6 +5,7 @@
 #include "ndc_exec.h"
 #include "ndc_rownorm.h"
 #include "ndc_epilogue.h"
+#include "ndc_regroup.h"
 
 #define NDC_LAMBDA __host__ __device__
 
@@ -356,6 +357,26 @@ struct Backend {
         } else {
             if (act == epilogue::kRelu) bias_act_bwd_launch<float, epilogue::kRelu>(gy, z, bias, gz, gpart, channels, sp, rows, vec, stream);
             else bias_act_bwd_launch<float, epilogue::kGelu>(gy, z, bias, gz, gpart, channels, sp, rows, vec, stream);
+        }
+        return check();
+    }
+
+    // 2 x 2 (x 2) windows of a fine grid <-> 4 (8) planes of the coarse grid; see ndc_regroup.h
+    static int regroup2(const void *src, void *dst, const float *bias, long long rows, int channels, int D,
+                        int H, int W, int depth2, int esz, int to_channels, void *stream)
+    {
+        const regroup::Shape sh = {rows, D, H, W, depth2, channels};
+        const long long nvec = rows * D * H * (W / (16 / esz));
+        if (nvec <= 0) return 0;
+        const long long blocks = (nvec + 255) / 256;
+        if (blocks > 0x7fffffffLL) return -2;
+        const dim3 grid((unsigned)blocks), block(256);
+        if (esz == 2) {
+            if (to_channels) hipLaunchKernelGGL((regroup::kernel<2, true>), grid, block, 0, (hipStream_t)stream, src, dst, bias, sh, nvec);
+            else hipLaunchKernelGGL((regroup::kernel<2, false>), grid, block, 0, (hipStream_t)stream, src, dst, bias, sh, nvec);
+        } else {
+            if (to_channels) hipLaunchKernelGGL((regroup::kernel<4, true>), grid, block, 0, (hipStream_t)stream, src, dst, bias, sh, nvec);
+            else hipLaunchKernelGGL((regroup::kernel<4, false>), grid, block, 0, (hipStream_t)stream, src, dst, bias, sh, nvec);
         }
         return check();
     }

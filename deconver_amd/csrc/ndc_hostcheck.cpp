@@ -131,6 +131,32 @@ struct Backend {
         return 0;
     }
 
+    static int regroup2(const void *src, void *dst, const float *bias, long long rows, int channels, int D,
+                        int H, int W, int depth2, int esz, int to_channels, void *)
+    {
+        const int Dc = depth2 ? D / 2 : 1, Hc = H / 2, Wc = W / 2, nk = depth2 ? 8 : 4;
+        const long long plane = (long long)Dc * Hc * Wc;
+        for (long long r = 0; r < rows; ++r)
+            for (int d = 0; d < D; ++d)
+                for (int h = 0; h < H; ++h)
+                    for (int w = 0; w < W; ++w) {
+                        const int kd = depth2 ? (d & 1) : 0, k = (kd * 2 + (h & 1)) * 2 + (w & 1);
+                        const long long fine = ((r * D + d) * H + h) * (long long)W + w;
+                        const long long coarse =
+                            (r * nk + k) * plane + ((long long)(depth2 ? d / 2 : 0) * Hc + h / 2) * Wc + w / 2;
+                        if (to_channels) {
+                            memcpy((char *)dst + coarse * esz, (const char *)src + fine * esz, (size_t)esz);
+                        } else if (esz == 2) {
+                            const float v = Elem<bf16_t>::load((const bf16_t *)src + coarse);
+                            Elem<bf16_t>::store((bf16_t *)dst + fine, bias ? v + bias[r % channels] : v);
+                        } else {
+                            const float v = ((const float *)src)[coarse];
+                            ((float *)dst)[fine] = bias ? v + bias[r % channels] : v;
+                        }
+                    }
+        return 0;
+    }
+
     static float act_value(int act, float u, bool grad)
     {
         const float cdf = 0.5f * (1.f + std::erf(u * 0.70710678118654752f));

@@ -181,12 +181,53 @@ def channels_to_patches(y: torch.Tensor, k, coarse) -> torch.Tensor:
     return y.permute(order).reshape(B, C, *[c * v for c, v in zip(coarse, k)])
 
 
+class _Regroup2(torch.autograd.Function):
+    """2 x 2 (x 2) windows of the grid <-> 2^nd channels per window on the HIP kernel
+    (``ndc_regroup``); each direction's gradient is the other direction.  On the way back to
+    the grid a per-channel bias can be added in the same pass."""
+
+    @staticmethod
+    def forward(ctx, x, to_channels, bias):
+        lib = _lib.get_library()
+        ctx.to_channels = to_channels
+        ctx.has_bias = bias is not None
+        with torch.cuda.device(x.device):
+            if to_channels:
+                return ops.windows_to_channels(lib, x)
+            return ops.channels_to_windows(lib, x, None if bias is None else bias.detach().float().contiguous())
+
+    @staticmethod
+    def backward(ctx, g):
+        lib = _lib.get_library()
+        g = g.contiguous()
+        gb = None
+        with torch.cuda.device(g.device):
+            if ctx.to_channels:
+                return ops.channels_to_windows(lib, g), None, None
+            if ctx.has_bias and ctx.needs_input_grad[2]:
+                gb = g.flatten(2).sum(2, dtype=torch.float32).sum(0)
+            return ops.windows_to_channels(lib, g), None, gb
+
+
+def _regroup_on_hip(fine_shape, t: torch.Tensor, k) -> bool:
+    """2-windows in every dimension, a GPU tensor the kernel takes, and the library is there."""
+    return (t.is_cuda and all(v == 2 for v in k) and len(k) in (2, 3) and _lib.library_available()
+            and ops.regroup2_applies(tuple(fine_shape), t.dtype, t.data_ptr()))
+
+
 def patch_conv(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
     """``conv(x, weight, bias, stride=weight.shape[2:])``, no padding: a strided convolution
     whose windows tile its input is a regrouping of the grid followed by the 1x1 projection."""
     k = tuple(weight.shape[2:])
     coarse = [s // v for s, v in zip(x.shape[2:], k)]
-    y = pointwise_linear(patches_to_channels(x, k), weight.flatten(1), bias)
+    if x.is_cuda and torch.is_autocast_enabled(x.device.type):
+        x = x.to(torch.get_autocast_dtype(x.device.type))     # before the regrouping, not after
+    xc = x.contiguous()
+    if _regroup_on_hip(xc.shape, xc, k):
+        cols = _Regroup2.apply(xc, True, None).flatten(2)
+    else:
+        cols = patches_to_channels(x, k)
+    y = pointwise_linear(cols, weight.flatten(1), bias)
     return y.view(x.shape[0], -1, *coarse)
 
 
@@ -197,6 +238,16 @@ def patch_conv_transpose(x: torch.Tensor, weight: torch.Tensor,
     k = tuple(weight.shape[2:])
     # weight (Cin, Cout, *k): row (cout, offset) of the projection is weight[:, cout, offset]
     w = weight.flatten(1).t()
+    fine = (x.shape[0], weight.shape[1], *[s * v for s, v in zip(x.shape[2:], k)])
+    dtype = x.dtype
+    if x.is_cuda and torch.is_autocast_enabled(x.device.type):
+        dtype = torch.get_autocast_dtype(x.device.type)
+    if x.is_cuda and dtype in (torch.bfloat16, torch.float32) and _regroup_on_hip(fine, x.new_empty(0, dtype=dtype), k):
+        # the bias rides on the regrouping pass
+        y = pointwise_linear(x.flatten(2), w, None)
+        if y.dtype == dtype and y.is_contiguous() and y.data_ptr() % 16 == 0:
+            return _Regroup2.apply(y.view(x.shape[0], -1, *x.shape[2:]), False, bias)
+        return channels_to_patches(y, k, x.shape[2:]) + (0 if bias is None else bias.view(1, -1, *([1] * len(k))))
     if bias is not None:
         bias = bias.repeat_interleave(math.prod(k))
     return channels_to_patches(pointwise_linear(x.flatten(2), w, bias), k, x.shape[2:])

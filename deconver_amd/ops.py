@@ -277,3 +277,40 @@ def bias_act_backward(lib: _lib.NdcLibrary, gy: Tensor, z: Tensor, bias: Optiona
     lib.bias_act_backward(_ptr(gy), _ptr(z), _ptr(bias), _ptr(gz), _ptr(gpart), B, C, n, ACTS[act],
                           dtype_tag(z.dtype), _stream_of(z))
     return gz, (gpart.sum((0, 2)) if need_bias_grad else None)
+
+
+def regroup2_applies(fine_shape, dtype, *ptrs) -> bool:
+    """Whether ``ndc_regroup`` takes a fine-grid tensor ``(B, C, [D,] H, W)``: float32 or
+    bfloat16, even extents, rows of whole 16-byte vectors, 16-byte aligned buffers."""
+    if dtype not in _DTYPES or len(fine_shape) not in (4, 5):
+        return False
+    vn = 16 // (2 if dtype == torch.bfloat16 else 4)
+    return (all(v % 2 == 0 and v > 0 for v in fine_shape[2:]) and fine_shape[-1] % vn == 0
+            and fine_shape[0] * fine_shape[1] > 0 and all(p % 16 == 0 for p in ptrs))
+
+
+def windows_to_channels(lib: _lib.NdcLibrary, x: Tensor) -> Tensor:
+    """``(B, C, [D,] H, W) -> (B, C * 2^nd, [D/2,] H/2, W/2)``: every 2 x 2 (x 2) window becomes
+    2^nd channels, channel-major then window offset.  ``x`` contiguous."""
+    B, C = x.shape[:2]
+    sp = list(x.shape[2:])
+    nd = len(sp)
+    out = torch.empty(B, C * 2 ** nd, *[v // 2 for v in sp], dtype=x.dtype, device=x.device)
+    D = sp[0] if nd == 3 else 1
+    lib.regroup2(_ptr(x), _ptr(out), None, B * C, C, D, sp[-2], sp[-1], nd == 3, dtype_tag(x.dtype), True,
+                 _stream_of(x))
+    return out
+
+
+def channels_to_windows(lib: _lib.NdcLibrary, y: Tensor, bias: Optional[Tensor] = None) -> Tensor:
+    """Inverse of :func:`windows_to_channels`: ``(B, C * 2^nd, *coarse) -> (B, C, *(2 coarse))``,
+    plus ``bias[c]`` (float32, C entries) if given.  ``y`` contiguous."""
+    B = y.shape[0]
+    sp = [2 * v for v in y.shape[2:]]
+    nd = len(sp)
+    C = y.shape[1] // 2 ** nd
+    out = torch.empty(B, C, *sp, dtype=y.dtype, device=y.device)
+    D = sp[0] if nd == 3 else 1
+    lib.regroup2(_ptr(y), _ptr(out), _ptr(bias), B * C, C, D, sp[-2], sp[-1], nd == 3, dtype_tag(y.dtype), False,
+                 _stream_of(y))
+    return out

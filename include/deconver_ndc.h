@@ -306,6 +306,23 @@ int ndc_bias_act(const void *z, const float *bias, const void *residual, void *y
 int ndc_bias_act_backward(const void *gy, const void *z, const float *bias, void *gz, float *gpart,
                           int64_t batch, int64_t channels, int64_t n, int act, int dtype, void *stream);
 
+/*
+ * Regrouping of a grid by 2 x 2 (depth2 = 0) or 2 x 2 x 2 (depth2 = 1) windows: the data
+ * movement of the reference's 2-tap, stride-2 resampling convolutions (nn.ConvNd(kernel_size=2,
+ * stride=2), nn.ConvTransposeNd(kernel_size=2, stride=2), deconver/unet.py:36-60, 108-131) once
+ * their arithmetic is the 1x1 projection.
+ *   to_channels = 1:  dst[r][k][d][h][w] = src[r][2d + kd][2h + kh][2w + kw],  k = (kd, kh, kw)
+ *   to_channels = 0:  dst[r][2d + kd][2h + kh][2w + kw] = src[r][k][d][h][w] + bias[r % channels]
+ *   rows       batch * channels of the fine-grid tensor
+ *   D, H, W    the fine grid (D = 1 for images); H, W (and D with depth2) even, W a multiple of
+ *              16 bytes of elements; src, dst distinct and 16-byte aligned -- anything else is
+ *              refused with NDC_ERR_GEOMETRY and the caller copies by other means
+ *   bias       NULL, or `channels` floats added on the way to the grid (the transposed
+ *              convolution's bias); not allowed with to_channels = 1
+ */
+int ndc_regroup(const void *src, void *dst, const float *bias, int64_t rows, int64_t channels, int64_t D,
+                 int64_t H, int64_t W, int depth2, int dtype, int to_channels, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -9,7 +9,8 @@ import torch.nn.functional as F
 from torch import nn
 
 import deconver_amd as dc
-from deconver_amd import layers
+from deconver_amd import _lib, layers, ops
+from tests.helpers import hostcheck_library
 
 
 @pytest.mark.parametrize("k,size", [((2, 2), (6, 8)), ((2, 2, 2), (4, 6, 8)), ((2, 2, 2), (5, 6, 7)),
@@ -66,6 +67,57 @@ def test_unfold_conv_is_the_same_padded_convolution(k, size):
         torch.testing.assert_close(a, r, rtol=1e-12, atol=1e-12)
     torch.testing.assert_close(layers.unfold_conv(x, w, None), conv(x, w, None, padding=tuple(v // 2 for v in k)),
                                rtol=1e-12, atol=1e-12)
+
+
+@pytest.mark.parametrize("shape", [(2, 3, 4, 8), (1, 2, 6, 16), (2, 2, 4, 6, 8), (1, 3, 2, 2, 24)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_host_regroup_is_the_strided_regrouping(shape, dtype):
+    """ndc_regroup (host build) against the view / permute form, both directions, with bias."""
+    lib = hostcheck_library()
+    if shape[-1] % (16 // (2 if dtype == torch.bfloat16 else 4)):
+        pytest.skip("row is not a whole number of 16-byte vectors")
+    nd = len(shape) - 2
+    x = torch.randn(*shape).to(dtype)
+    assert ops.regroup2_applies(shape, dtype, x.data_ptr())
+    cols = ops.windows_to_channels(lib, x)
+    ref = layers.patches_to_channels(x, (2,) * nd)
+    assert cols.shape == (shape[0], shape[1] * 2 ** nd, *[v // 2 for v in shape[2:]])
+    assert torch.equal(cols.flatten(2), ref)
+    assert torch.equal(ops.channels_to_windows(lib, cols), x)
+    bias = torch.randn(shape[1])
+    want = (x.float() + bias.view(1, -1, *([1] * nd))).to(dtype)
+    assert torch.equal(ops.channels_to_windows(lib, cols, bias), want)
+
+
+def test_regroup_refuses_what_the_kernel_does_not_take():
+    lib = hostcheck_library()
+    x = torch.zeros(1, 1, 3, 8)
+    assert not ops.regroup2_applies((1, 1, 3, 8), torch.float32, x.data_ptr())      # odd extent
+    assert not ops.regroup2_applies((1, 1, 4, 6), torch.float32, x.data_ptr())      # 6 floats: not 16-byte rows
+    assert not ops.regroup2_applies((1, 1, 4, 8), torch.float64, x.data_ptr())
+    assert not ops.regroup2_applies((1, 1, 4, 8), torch.float32, x.data_ptr() + 4)  # unaligned
+    out = torch.zeros(1, 4, 1, 4)
+    with pytest.raises(_lib.NdcError):
+        lib.regroup2(x.data_ptr(), out.data_ptr(), None, 1, 1, 1, 3, 8, False, _lib.NDC_F32, True, None)
+    with pytest.raises(_lib.NdcError):   # a bias only on the way back to the grid
+        lib.regroup2(x.data_ptr(), out.data_ptr(), out.data_ptr(), 1, 1, 1, 2, 8, False, _lib.NDC_F32, True, None)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(2, 3, 4, 8), (2, 5, 64, 128), (2, 4, 8, 16, 32), (1, 3, 6, 10, 24), (2, 16, 32, 32, 64)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_hip_regroup_is_the_strided_regrouping(shape, dtype):
+    lib = _lib.get_library()
+    if shape[-1] % (16 // (2 if dtype == torch.bfloat16 else 4)):
+        pytest.skip("row is not a whole number of 16-byte vectors")
+    nd = len(shape) - 2
+    x = torch.randn(*shape, device="cuda").to(dtype)
+    cols = ops.windows_to_channels(lib, x)
+    assert torch.equal(cols.flatten(2), layers.patches_to_channels(x, (2,) * nd))
+    assert torch.equal(ops.channels_to_windows(lib, cols), x)
+    bias = torch.randn(shape[1], device="cuda")
+    want = (x.float() + bias.view(1, -1, *([1] * nd))).to(dtype)
+    assert torch.equal(ops.channels_to_windows(lib, cols, bias), want)
 
 
 def test_regrouping_round_trip():
