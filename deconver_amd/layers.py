@@ -63,6 +63,7 @@ class _PointwiseLinear(torch.autograd.Function):
         return y
 
     @staticmethod
+    @torch.autograd.function.once_differentiable
     def backward(ctx, gy):
         x, weight, kept, bias32 = ctx.saved_tensors
         gy = gy.contiguous()
@@ -197,6 +198,7 @@ class _Regroup2(torch.autograd.Function):
             return ops.channels_to_windows(lib, x, None if bias is None else bias.detach().float().contiguous())
 
     @staticmethod
+    @torch.autograd.function.once_differentiable
     def backward(ctx, g):
         lib = _lib.get_library()
         g = g.contiguous()
