@@ -102,6 +102,43 @@ class _PointwiseLinear(torch.autograd.Function):
         return gx, gw, gb, None, gres
 
 
+class _BiasAct(torch.autograd.Function):
+    """``act(z + bias[c]) + residual`` for a ``(B, C, N)`` GPU tensor in one pass of the HIP
+    library (``ndc_bias_act``); the activation's gradient and the bias gradient's partial sums
+    in one pass as well.  For projections whose GEMM stays with the library convolution
+    (float32)."""
+
+    @staticmethod
+    def forward(ctx, z, bias, act, residual):
+        lib = _lib.get_library()
+        z = z.contiguous()
+        bias32 = None if bias is None else bias.detach().float().contiguous()
+        if residual is not None:
+            residual = residual.to(z.dtype).contiguous()
+        with torch.cuda.device(z.device):
+            y = ops.bias_act(lib, z, bias32, residual, act)
+        # relu alone needs only the sign of its output
+        keep_z = act == "gelu" or (act == "relu" and residual is not None)
+        ctx.save_for_backward(z if keep_z else y if act == "relu" else None, bias32 if keep_z else None)
+        ctx.act = act
+        ctx.has_bias = bias is not None
+        return y
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, gy):
+        kept, bias32 = ctx.saved_tensors
+        gy = gy.contiguous()
+        want_gb = ctx.has_bias and ctx.needs_input_grad[1]
+        gz, gb = gy, None
+        if ctx.act is not None:
+            with torch.cuda.device(gy.device):
+                gz, gb = ops.bias_act_backward(_lib.get_library(), gy, kept, bias32, ctx.act, need_bias_grad=want_gb)
+        elif want_gb:
+            gb = gy.sum(2, dtype=torch.float32).sum(0)
+        return gz, gb, None, (gy if ctx.needs_input_grad[3] else None)
+
+
 _ACT_FUNCTIONS = {None: lambda t: t, "relu": torch.relu, "gelu": torch.nn.functional.gelu}
 
 
@@ -111,8 +148,9 @@ def pointwise_linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch
     ``weight`` of shape ``(Cout, Cin)`` or ``(Cout, Cin, 1)``, optionally followed by an
     activation (``"relu"`` or ``"gelu"``, the exact one) and the sum with a tensor of the
     output's shape.  bfloat16 tensors on the GPU (stored or under autocast) run as GEMMs on the
-    channel-first layout plus one pass of the HIP library over the result; everything else as
-    the reference's ``conv1d`` followed by PyTorch's activation and sum."""
+    channel-first layout plus one pass of the HIP library over the result; float32 tensors on
+    the GPU as the library's ``conv1d`` without bias plus that pass; everything else as the
+    reference's ``conv1d`` followed by PyTorch's activation and sum."""
     w2 = weight.squeeze(-1) if weight.dim() == 3 else weight
     dtype = x.dtype
     if x.is_cuda and torch.is_autocast_enabled(x.device.type):
@@ -120,6 +158,14 @@ def pointwise_linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch
     # 16-bit GPU tensors only: in float32 the library convolution is as fast (2-D network,
     # batch 8: 24.5 against 25.5 ms per step)
     if not x.is_cuda or x.dim() != 3 or dtype != torch.bfloat16:
+        if (x.is_cuda and x.dim() == 3 and dtype == torch.float32 and _lib.library_available()
+                and (bias is not None or act is not None or residual is not None)):
+            # float32 on the GPU: the library's convolution for the GEMM, its tail in one pass
+            z = torch.nn.functional.conv1d(x, w2.unsqueeze(-1))
+            if z.dtype == torch.float32:
+                return _BiasAct.apply(z, bias, act, residual)
+            y = _ACT_FUNCTIONS[act](z + bias.to(z.dtype).view(1, -1, 1) if bias is not None else z)
+            return y if residual is None else residual + y
         y = _ACT_FUNCTIONS[act](torch.nn.functional.conv1d(x, w2.unsqueeze(-1), bias))
         return y if residual is None else residual + y
     x, w2 = x.to(dtype), w2.to(dtype)
@@ -130,12 +176,13 @@ def pointwise_linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch
 
 
 def _gemm_route(x: torch.Tensor) -> bool:
-    """True for the tensors ``pointwise_linear`` runs as GEMMs: bfloat16 (stored or under
-    autocast) on the GPU."""
+    """True for the tensors whose 1x1 projection ``pointwise_linear`` runs off the library's
+    strided convolutions: bfloat16 (stored or under autocast; channel-first GEMMs) and float32
+    (``conv1d`` on the regrouped tensor) on the GPU."""
     dtype = x.dtype
     if x.is_cuda and torch.is_autocast_enabled(x.device.type):
         dtype = torch.get_autocast_dtype(x.device.type)
-    return x.is_cuda and dtype == torch.bfloat16
+    return x.is_cuda and dtype in (torch.bfloat16, torch.float32)
 
 
 def _is_patch_conv(conv) -> bool:
@@ -211,10 +258,12 @@ class _Regroup2(torch.autograd.Function):
             return ops.windows_to_channels(lib, g), None, gb
 
 
-def _regroup_on_hip(fine_shape, t: torch.Tensor, k) -> bool:
-    """2-windows in every dimension, a GPU tensor the kernel takes, and the library is there."""
-    return (t.is_cuda and all(v == 2 for v in k) and len(k) in (2, 3) and _lib.library_available()
-            and ops.regroup2_applies(tuple(fine_shape), t.dtype, t.data_ptr()))
+def _regroup_on_hip(fine_shape, dtype, k, *tensors) -> bool:
+    """2-windows in every dimension, GPU buffers the kernel takes (``tensors``: the ones that
+    exist already), and the library is there."""
+    return (all(v == 2 for v in k) and len(k) in (2, 3) and all(t.is_cuda for t in tensors)
+            and _lib.library_available()
+            and ops.regroup2_applies(tuple(fine_shape), dtype, *[t.data_ptr() for t in tensors]))
 
 
 def patch_conv(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
@@ -225,7 +274,7 @@ def patch_conv(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tenso
     if x.is_cuda and torch.is_autocast_enabled(x.device.type):
         x = x.to(torch.get_autocast_dtype(x.device.type))     # before the regrouping, not after
     xc = x.contiguous()
-    if _regroup_on_hip(xc.shape, xc, k):
+    if _regroup_on_hip(xc.shape, xc.dtype, k, xc):
         cols = _Regroup2.apply(xc, True, None).flatten(2)
     else:
         cols = patches_to_channels(x, k)
@@ -244,12 +293,13 @@ def patch_conv_transpose(x: torch.Tensor, weight: torch.Tensor,
     dtype = x.dtype
     if x.is_cuda and torch.is_autocast_enabled(x.device.type):
         dtype = torch.get_autocast_dtype(x.device.type)
-    if x.is_cuda and dtype in (torch.bfloat16, torch.float32) and _regroup_on_hip(fine, x.new_empty(0, dtype=dtype), k):
+    if x.is_cuda and _regroup_on_hip(fine, dtype, k):
         # the bias rides on the regrouping pass
-        y = pointwise_linear(x.flatten(2), w, None)
-        if y.dtype == dtype and y.is_contiguous() and y.data_ptr() % 16 == 0:
+        y = pointwise_linear(x.flatten(2), w, None).contiguous()
+        if _regroup_on_hip(fine, y.dtype, k, y):
             return _Regroup2.apply(y.view(x.shape[0], -1, *x.shape[2:]), False, bias)
-        return channels_to_patches(y, k, x.shape[2:]) + (0 if bias is None else bias.view(1, -1, *([1] * len(k))))
+        y = channels_to_patches(y, k, x.shape[2:])
+        return y if bias is None else y + bias.to(y.dtype).view(1, -1, *([1] * len(k)))
     if bias is not None:
         bias = bias.repeat_interleave(math.prod(k))
     return channels_to_patches(pointwise_linear(x.flatten(2), w, bias), k, x.shape[2:])
@@ -257,11 +307,11 @@ def patch_conv_transpose(x: torch.Tensor, weight: torch.Tensor,
 
 class _PatchConvMixin:
     """The network's 2-tap resampling convolutions (unet.py:36-60) and its 1-tap head are
-    convolutions whose windows tile the input.  16-bit tensors on the GPU take the form of
-    ``patch_conv`` here -- one strided copy and the GEMMs of ``pointwise_linear`` instead of
-    the library's column-matrix convolution; everything else, and any other stride or
-    padding, runs the parent class's convolution.  Parameters, their shapes and names are the
-    parent's."""
+    convolutions whose windows tile the input.  bfloat16 and float32 tensors on the GPU take
+    the form of ``patch_conv`` here -- one regrouping copy and the projection of
+    ``pointwise_linear`` instead of the library's column-matrix convolution; everything else,
+    and any other stride or padding, runs the parent class's convolution.  Parameters, their
+    shapes and names are the parent's."""
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if _is_patch_conv(self) and _gemm_route(x) and x.dim() == len(self.kernel_size) + 2:
@@ -301,9 +351,9 @@ def unfold_conv(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tens
 class _UnfoldConvMixin:
     """The network's stem (unet.py:175-276: a 3-tap convolution from the few image channels to
     the first width): with few input channels the column matrix is small next to the output,
-    and bfloat16 tensors on the GPU take ``unfold_conv`` -- one gather and the GEMMs of
-    ``pointwise_linear`` -- instead of the library's convolution, whose weight gradient alone
-    takes longer.  Anything else (more than ``max_columns`` rows in the column matrix, other
+    and bfloat16 / float32 tensors on the GPU take ``unfold_conv`` -- one gather and the
+    projection of ``pointwise_linear`` -- instead of the library's convolution, whose weight
+    gradient alone takes longer.  Anything else (more than ``max_columns`` rows in the column matrix, other
     strides or paddings) runs the parent class's convolution."""
 
     max_columns = 128

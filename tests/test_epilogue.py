@@ -152,6 +152,30 @@ def test_projection_with_fused_tail_matches_the_unfused_form(act, with_res):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("act,with_res", [(None, False), (None, True), ("gelu", False), ("gelu", True)])
+def test_float32_projection_tail_matches_float64(act, with_res):
+    """float32 on the GPU (the 2-D network's regime): conv1d without bias + one pass of the HIP
+    library, values and every gradient against float64, 1e-5 of the largest entry."""
+    torch.manual_seed(8)
+    B, cin, cout, n = 2, 16, 24, 4096 + 40
+    x = torch.randn(B, cin, n, device="cuda", requires_grad=True)
+    w = (torch.randn(cout, cin, 1, device="cuda") / cin ** 0.5).requires_grad_(True)
+    b = torch.randn(cout, device="cuda", requires_grad=True)
+    res = torch.randn(B, cout, n, device="cuda", requires_grad=True) if with_res else None
+    g = torch.randn(B, cout, n, device="cuda")
+    y = layers.pointwise_linear(x, w, b, act, res)
+    assert y.dtype == torch.float32 and type(y.grad_fn).__name__.startswith("_BiasAct")
+    leaves = [t for t in (x, w, b, res) if t is not None]
+    got = torch.autograd.grad(y, leaves, g)
+    l64 = [t.detach().double().requires_grad_(True) for t in leaves]
+    ref = ACT[act](F.conv1d(l64[0], l64[1], l64[2])) + (l64[3] if with_res else 0)
+    want = torch.autograd.grad(ref, l64, g.double())
+    assert _rel(y.detach(), ref.detach()) <= 1e-5
+    for a, r in zip(got, want):
+        assert a.shape == r.shape and _rel(a, r) <= 1e-5
+
+
+@pytest.mark.gpu
 def test_block_on_the_gpu_matches_its_float64_general_route():
     """A Deconver block under bf16 autocast (HIP norm, NDC kernels, fused projection tails)
     against the same block in float64 on the CPU's general route: output within the bf16

@@ -163,35 +163,41 @@ def test_network_uses_them_with_the_reference_state_dict_names():
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("nd", [2, 3])
-def test_gemm_route_matches_the_library_convolution_on_the_gpu(nd):
-    """bf16 autocast on the GPU (the route the 3-D training step takes): values and gradients
-    of the regrouped form against torch's convolution of the same 16-bit operands, to the
-    bf16 bar 2e-2 of the largest entry."""
+@pytest.mark.parametrize("regime", ["bf16 autocast", "float32"])
+def test_regrouped_route_matches_the_library_convolution_on_the_gpu(nd, regime):
+    """The resampling convolutions and the stem on the GPU, in the two regimes that take the
+    regrouped form -- bf16 autocast (the 3-D training step) and float32 (the 2-D network):
+    values and gradients against torch's convolution of the same operands, bf16 to 2e-2 of the
+    largest entry, float32 to 1e-5 (against float64)."""
+    import contextlib
     torch.manual_seed(3)
-    size = (16, 12, 20)[:nd]
+    bf16 = regime == "bf16 autocast"
+    tol = 2e-2 if bf16 else 1e-5
+    ctx = (lambda: torch.autocast("cuda", dtype=torch.bfloat16)) if bf16 else contextlib.nullcontext
+    hi = (lambda t: t) if bf16 else (lambda t: t.double())      # the reference's precision
+    size = (16, 12, 24)[:nd]
+    conv, tconv = getattr(F, f"conv{nd}d"), getattr(F, f"conv_transpose{nd}d")
     down = getattr(layers, f"PatchConv{nd}d")(16, 32, 2, stride=2).cuda()
     up = getattr(layers, f"PatchConvTranspose{nd}d")(32, 16, 2, stride=2).cuda()
-    x = torch.randn(2, 16, *size, device="cuda", requires_grad=True)
-    with torch.autocast("cuda", dtype=torch.bfloat16):
-        y = up(down(x))
-        conv, tconv = getattr(F, f"conv{nd}d"), getattr(F, f"conv_transpose{nd}d")
-        ref = tconv(conv(x, down.weight, down.bias, stride=2), up.weight, up.bias, stride=2)
-    assert y.dtype == torch.bfloat16 and y.shape == ref.shape
     stem = getattr(layers, f"UnfoldConv{nd}d")(2, 16, 3, padding=1, bias=False).cuda()
+    x = torch.randn(2, 16, *size, device="cuda", requires_grad=True)
     img = torch.randn(2, 2, *size, device="cuda")
-    with torch.autocast("cuda", dtype=torch.bfloat16):
-        ys = stem(img)
-        rs = conv(img, stem.weight, None, padding=1)
-    assert ys.dtype == torch.bfloat16
-    gs = torch.randn_like(rs)
-    (gw,), (gw_ref,) = torch.autograd.grad(ys, stem.weight, gs), torch.autograd.grad(rs, stem.weight, gs)
-    for a, r in ((ys, rs), (gw, gw_ref)):
-        assert float((a.float() - r.float()).abs().max() / r.float().abs().max()) <= 2e-2
     params = (x, down.weight, down.bias, up.weight, up.bias)
-    g = torch.randn_like(ref)
-    got = torch.autograd.grad(y, params, g)
-    want = torch.autograd.grad(ref, params, g)
-    for a, r in zip((y, *got), (ref, *want)):
+    with ctx():
+        y = up(down(x))
+        ys = stem(img)
+    ref_params = [hi(p.detach()).requires_grad_(True) for p in params]
+    sw = hi(stem.weight.detach()).requires_grad_(True)
+    with ctx():
+        rx, dw, db, uw, ub = ref_params
+        ref = tconv(conv(rx, dw, db, stride=2), uw, ub, stride=2)
+        rs = conv(hi(img), sw, None, padding=1)
+    assert y.dtype == (torch.bfloat16 if bf16 else torch.float32) and y.shape == ref.shape
+    assert ys.dtype == y.dtype and ys.shape == rs.shape
+    g, gs = torch.randn_like(y), torch.randn_like(ys)
+    got = (y, ys, *torch.autograd.grad(y, params, g), *torch.autograd.grad(ys, stem.weight, gs))
+    want = (ref, rs, *torch.autograd.grad(ref, ref_params, hi(g)), *torch.autograd.grad(rs, sw, hi(gs)))
+    for a, r in zip(got, want):
         assert a.shape == r.shape
-        err = float((a.float() - r.float()).abs().max() / r.float().abs().max())
-        assert err <= 2e-2, err
+        err = float((a.detach().double() - r.detach().double()).abs().max() / r.detach().double().abs().max())
+        assert err <= tol, err
