@@ -167,7 +167,7 @@ static int direct_gconv(const KGeom &q, const TI *in, const float *h, const floa
 
 extern "C" {
 
-int ndc_version(void) { return 100; }
+int ndc_version(void) { return 200; }   // 0.2.0: row normalisation, projection tails, regrouping
 
 const char *ndc_status_string(int status)
 {
