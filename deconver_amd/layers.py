@@ -158,7 +158,7 @@ def pointwise_linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch
     # 16-bit GPU tensors only: in float32 the library convolution is as fast (2-D network,
     # batch 8: 24.5 against 25.5 ms per step)
     if not x.is_cuda or x.dim() != 3 or dtype != torch.bfloat16:
-        if (x.is_cuda and x.dim() == 3 and dtype == torch.float32 and _lib.library_available()
+        if (x.is_cuda and x.dim() == 3 and dtype == torch.float32
                 and (bias is not None or act is not None or residual is not None)):
             # float32 on the GPU: the library's convolution for the GEMM, its tail in one pass
             z = torch.nn.functional.conv1d(x, w2.unsqueeze(-1))
@@ -259,10 +259,9 @@ class _Regroup2(torch.autograd.Function):
 
 
 def _regroup_on_hip(fine_shape, dtype, k, *tensors) -> bool:
-    """2-windows in every dimension, GPU buffers the kernel takes (``tensors``: the ones that
-    exist already), and the library is there."""
+    """2-windows in every dimension and GPU buffers the kernel takes (``tensors``: the ones
+    that exist already)."""
     return (all(v == 2 for v in k) and len(k) in (2, 3) and all(t.is_cuda for t in tensors)
-            and _lib.library_available()
             and ops.regroup2_applies(tuple(fine_shape), dtype, *[t.data_ptr() for t in tensors]))
 
 

@@ -9,7 +9,9 @@ at the 3-D network's first level is 128 workgroups walking 2M elements each; the
 
 ``InstanceNorm{1,2,3}d`` here are subclasses of the ``torch.nn`` modules with the same
 constructor, parameters and state dict.  GPU tensors in float32 / bfloat16 without affine
-parameters and running statistics take the kernels; anything else runs the parent's forward.
+parameters and running statistics take the kernels (a missing library raises, as for the NDC
+update: there is no silent PyTorch path for them); anything else -- CPU tensors, float64,
+affine or tracked statistics -- runs the parent's forward.
 """
 
 from __future__ import annotations
@@ -94,7 +96,7 @@ def instance_norm(x: Tensor, eps: float = 1e-5) -> Tensor:
 class _HipInstanceNorm:
     def _on_hip(self, x: Tensor) -> bool:
         return not (self.affine or self.track_running_stats or not hip_norm_applies(x)
-                    or not _lib.library_available() or x.dim() == self._get_no_batch_dim())
+                    or x.dim() == self._get_no_batch_dim())
 
     def forward(self, x: Tensor) -> Tensor:
         if not self._on_hip(x):
