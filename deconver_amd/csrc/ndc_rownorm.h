@@ -115,7 +115,7 @@ reduce_kernel(const T *a, const T *b, float2 *partial, Split sp)
     float pivot = 0.f;
     if (!BWD) {
         // the mean of the row's first elements (one access per thread), the same in every part
-        float a = 0.f, unused = 0.f;
+        float head = 0.f, unused = 0.f;
         long long cnt;
         if constexpr (VEC) {
             typedef Vec<T> V;
@@ -124,14 +124,14 @@ reduce_kernel(const T *a, const T *b, float2 *partial, Split sp)
             if ((long long)threadIdx.x < nv) {
                 const V x = reinterpret_cast<const V *>(ar)[threadIdx.x];
 #pragma unroll
-                for (int e = 0; e < V::N; ++e) a += x.get(e);
+                for (int e = 0; e < V::N; ++e) head += x.get(e);
             }
         } else {
             cnt = sp.n < kThreads ? sp.n : kThreads;
-            if ((long long)threadIdx.x < sp.n) a = Elem<T>::load(ar + threadIdx.x);
+            if ((long long)threadIdx.x < sp.n) head = Elem<T>::load(ar + threadIdx.x);
         }
-        block_sum2(a, unused, buf);
-        pivot = a / (float)cnt;
+        block_sum2(head, unused, buf);
+        pivot = head / (float)cnt;
     }
     float s1 = 0.f, s2 = 0.f;
     if constexpr (VEC) {
