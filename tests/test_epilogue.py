@@ -188,3 +188,28 @@ def test_block_on_the_gpu_matches_its_float64_general_route():
     with torch.autocast("cuda", dtype=torch.bfloat16):
         y = blk(x.cuda())
     assert _rel(y.cpu(), ref.detach()) <= 2e-2
+
+
+@pytest.mark.gpu
+def test_full_size_hidden_tensor_of_the_3d_network():
+    """bias + GELU and its gradient on the MLP's hidden tensor at the 3-D network's first level
+    (B 2, 256 channels, 128^3, bf16: 2 GiB): sampled channels against float64, the bias gradient
+    against the sum of the stored gradient, and linearity of the backward in gy."""
+    torch.manual_seed(12)
+    B, C, n = 2, 256, 128 ** 3
+    lib = _lib.get_library()
+    z = torch.randn(B, C, n, device="cuda").bfloat16()
+    gy = torch.randn(B, C, n, device="cuda").bfloat16()
+    bias = torch.randn(C, device="cuda")
+    y = ops.bias_act(lib, z, bias, None, "gelu")
+    gz, gb = ops.bias_act_backward(lib, gy, z, bias, "gelu")
+    for c in (0, 101, 255):
+        u = (z[:, c].double() + bias[c].double()).requires_grad_(True)
+        ref = F.gelu(u)
+        (g_ref,) = torch.autograd.grad(ref, u, gy[:, c].double())
+        assert _rel(y[:, c], ref.detach()) <= 2e-2
+        assert _rel(gz[:, c], g_ref) <= 2e-2
+        # the bias gradient is summed from the unrounded values: within bf16 rounding of the stored ones
+        assert abs(float(gb[c]) - float(g_ref.sum())) <= 2e-3 * float(g_ref.abs().sum()) ** 0.5 + 1e-2 * abs(float(g_ref.sum()))
+    gz2, _ = ops.bias_act_backward(lib, (gy.float() * 2).bfloat16(), z, bias, "gelu", need_bias_grad=False)
+    assert torch.equal(gz2, (gz.float() * 2).bfloat16())    # exact: a power of two

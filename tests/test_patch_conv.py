@@ -201,3 +201,21 @@ def test_regrouped_route_matches_the_library_convolution_on_the_gpu(nd, regime):
         assert a.shape == r.shape
         err = float((a.detach().double() - r.detach().double()).abs().max() / r.detach().double().abs().max())
         assert err <= tol, err
+
+
+@pytest.mark.gpu
+def test_full_size_regrouping_round_trip():
+    """The first resampling step of the 3-D network (B 2, 64 channels, 128^3, bf16): to channels
+    and back is the identity, bit for bit, and a sampled window lands where the strided view
+    puts it."""
+    lib = _lib.get_library()
+    torch.manual_seed(13)
+    x = torch.randn(2, 64, 128, 128, 128, device="cuda").bfloat16()
+    cols = ops.windows_to_channels(lib, x)
+    assert cols.shape == (2, 512, 64, 64, 64)
+    assert torch.equal(ops.channels_to_windows(lib, cols), x)
+    for (b, c, d, h, w) in ((0, 0, 0, 0, 0), (1, 63, 63, 63, 63), (1, 17, 5, 40, 9)):
+        for kd in (0, 1):
+            for kh in (0, 1):
+                for kw in (0, 1):
+                    assert cols[b, c * 8 + (kd * 2 + kh) * 2 + kw, d, h, w] == x[b, c, 2 * d + kd, 2 * h + kh, 2 * w + kw]

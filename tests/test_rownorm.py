@@ -178,3 +178,30 @@ def test_hip_rownorm_is_reproducible_and_handles_views():
     xt = x.transpose(2, 4)               # not contiguous: copied first
     ref = F.instance_norm(xt.double())
     assert _rel(dc.instance_norm(xt).cpu(), ref.cpu()) <= 1e-5
+
+
+@pytest.mark.gpu
+def test_full_size_rows_of_the_3d_network():
+    """The first level of the 3-D network (B 2, 64 channels, 128^3, bf16: 128 rows of 2 M
+    elements, cut into 32 parts each) through size-independent properties: normalised rows have
+    zero mean and unit variance, the gradient is orthogonal to the constant and to the
+    normalised row (the two directions the norm removes), and sampled rows agree with float64."""
+    torch.manual_seed(11)
+    B, C, n = 2, 64, 128 ** 3
+    lib = _lib.get_library()
+    x = (torch.randn(B * C, n, device="cuda") * 0.8 + 0.3).bfloat16()
+    gy = torch.randn(B * C, n, device="cuda").bfloat16()
+    assert lib.rownorm_workspace_bytes(B * C, n) == B * C * 32 * 8
+    y, stats = ops.rownorm_forward(lib, x, 1e-5)
+    gx = ops.rownorm_backward(lib, gy, y, stats)
+    yf, gf = y.float(), gx.float()
+    assert float(yf.mean(1).abs().max()) <= 2e-3           # bf16 rounding of y leaves ~1e-4
+    assert float((yf.var(1, unbiased=False) - 1).abs().max()) <= 5e-3
+    scale = float(gf.abs().mean())
+    assert float(gf.mean(1).abs().max()) <= 2e-3 * scale
+    assert float((gf * yf).mean(1).abs().max()) <= 5e-3 * scale
+    for row in (0, 77, 127):
+        y_ref, gx_ref = _reference(x[row:row + 1].cpu(), gy[row:row + 1].cpu(), 1e-5)
+        assert _rel(y[row:row + 1].cpu(), y_ref) <= 2e-2
+        assert _rel(gx[row:row + 1].cpu(), gx_ref) <= 2e-2
+        torch.testing.assert_close(stats[row, 0].double().cpu(), x[row].double().mean().cpu(), rtol=1e-4, atol=1e-5)
