@@ -52,7 +52,7 @@ def _check(lib, shape, dtype, act, with_bias, with_res, device="cpu"):
         assert none is None and torch.equal(gz, gz2)
 
 
-SHAPES = [(2, 3, 7), (1, 5, 64), (2, 2, 8192 * 2 + 24), (1, 3, 2048 * 5 + 3)]
+SHAPES = [(2, 3, 7), (1, 5, 64), (2, 2, 8192 * 2 + 24), (1, 3, 2048 * 5 + 3), (1, 1, 16385), (1, 2, 8192), (3, 1, 1)]
 
 
 @pytest.mark.parametrize("shape", SHAPES)

@@ -38,7 +38,9 @@ def _run(lib, x, gy, eps):
 
 
 # (rows, n): one part; several parts with a ragged last one; not a multiple of the vector width
-SHAPES = [(3, 7), (5, 64), (2, 8192 * 3 + 8), (1, 2048 * 9 + 3), (4, 20000)]
+SHAPES = [(3, 7), (5, 64), (2, 8192 * 3 + 8), (1, 2048 * 9 + 3), (4, 20000),
+          # around the split's thresholds (parts of at least 8 192 elements, multiples of 2 048)
+          (1, 8191), (1, 8192), (2, 16383), (1, 16384), (1, 16385), (1, 2 * 8192 + 2048 + 8), (3, 5)]
 
 
 @pytest.mark.parametrize("rows,n", SHAPES)
