@@ -7,7 +7,7 @@ computes anything in PyTorch.
 
 from __future__ import annotations
 
-from typing import Optional, Sequence, Tuple
+from typing import Optional, Tuple
 
 import torch
 from torch import Tensor
