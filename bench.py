@@ -1131,11 +1131,11 @@ def main() -> int:
         try:
             if "layers_2d" in result:
                 # config 2 (model level): the 2-D network's forward + backward on the HIP route
-                m2 = run_model_routes("model2d", ["hip"], warmup=2, steps=5)["hip"]
+                m2 = run_model_routes("model2d", ["hip"], warmup=5, steps=20)["hip"]
                 result["layers_2d"]["model2d_steps_per_s"] = m2["steps_per_s"]
                 result["layers_2d"]["model2d_ms_per_step"] = m2["ms_per_step"]
                 result["layers_2d"]["model2d_workload"] = MODEL_WORKLOADS["model2d"]["text"]
-            t3 = run_model_routes("train3d", ["hip"], warmup=2, steps=5)
+            t3 = run_model_routes("train3d", ["hip"], warmup=3, steps=10)
             t3.update(run_model_routes("train3d", ["pytorch"], warmup=1, steps=2))
             result["train3d_steps_per_s"] = t3["hip"]["steps_per_s"]
             result["train3d_steps_per_s_pytorch_route"] = t3["pytorch"]["steps_per_s"]
@@ -1145,7 +1145,7 @@ def main() -> int:
                 # the same train step with the other kernel family on (see above: not the metric)
                 lib.matrix_kernels(True)
                 try:
-                    tm = run_model_routes("train3d", ["hip"], warmup=2, steps=5)["hip"]
+                    tm = run_model_routes("train3d", ["hip"], warmup=3, steps=10)["hip"]
                 finally:
                     lib.matrix_kernels(False)
                 result["matrix_instruction_variant"]["train3d_steps_per_s"] = tm["steps_per_s"]
