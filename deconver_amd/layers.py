@@ -15,6 +15,9 @@ from torch.nn.modules.utils import _pair
 from . import _lib, ops
 
 
+_CHUNKED_WGRAD_FROM = 1 << 17   # voxels per sample from which the weight gradient is chunked
+
+
 def _wgrad_chunks(batch: int, n: int) -> int:
     """Number of equal chunks the voxel axis is cut into for the weight-gradient GEMM: a power
     of two that divides ``n``, leaves chunks of at least 2048 voxels and at most 128 GEMMs in
@@ -43,11 +46,11 @@ class _PointwiseLinear(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, weight, bias, act, residual):
         lib = _lib.get_library()
-        # one GEMM per sample on the tensors as they lie (torch.matmul would fold the batch into
-        # the voxel axis through two transposing copies when its input requires a gradient)
-        z = x.new_empty(x.shape[0], weight.shape[0], x.shape[2])
-        for b in range(x.shape[0]):
-            torch.mm(weight, x[b], out=z[b])
+        # one batched GEMM on the tensors as they lie, the weight shared by the batch entries
+        # through a zero stride (no copy; the same bits as one GEMM per sample, in one launch)
+        B = x.shape[0]
+        z = x.new_empty(B, weight.shape[0], x.shape[2])
+        torch.bmm(weight.unsqueeze(0).expand(B, -1, -1), x, out=z)
         bias32 = None if bias is None else bias.detach().float().contiguous()
         y = z
         # the activation's gradient needs z + bias: gelu keeps z; relu alone needs only the
@@ -82,15 +85,15 @@ class _PointwiseLinear(torch.autograd.Function):
             gb = gy.sum(2, dtype=torch.float32).sum(0)
         if ctx.needs_input_grad[0]:
             gx = torch.empty_like(x)
-            wt = weight.t()
-            for b in range(x.shape[0]):
-                torch.mm(wt, gz[b], out=gx[b])
+            torch.bmm(weight.t().unsqueeze(0).expand(x.shape[0], -1, -1), gz, out=gx)
         if ctx.needs_input_grad[1]:
             B, cout, n = gz.shape
             cin = x.shape[1]
-            s = _wgrad_chunks(B, n) if gz.dtype in (torch.bfloat16, torch.float16) else 1
+            # short rows (the 2-D network's levels): one batched GEMM and a sum over the batch
+            # (two launches); long rows: chunks of the voxel axis as batch entries
+            s = _wgrad_chunks(B, n) if n >= _CHUNKED_WGRAD_FROM else 1
             if s == 1:
-                gw = torch.bmm(gz, x.transpose(1, 2)).sum(0)
+                gw = torch.bmm(gz, x.transpose(1, 2)).float().sum(0).to(weight.dtype)
             else:
                 acc = torch.zeros(cout, cin, dtype=torch.float32, device=gz.device)
                 for b in range(B):
