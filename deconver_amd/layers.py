@@ -105,43 +105,6 @@ class _PointwiseLinear(torch.autograd.Function):
         return gx, gw, gb, None, gres
 
 
-class _BiasAct(torch.autograd.Function):
-    """``act(z + bias[c]) + residual`` for a ``(B, C, N)`` GPU tensor in one pass of the HIP
-    library (``ndc_bias_act``); the activation's gradient and the bias gradient's partial sums
-    in one pass as well.  For projections whose GEMM stays with the library convolution
-    (float32)."""
-
-    @staticmethod
-    def forward(ctx, z, bias, act, residual):
-        lib = _lib.get_library()
-        z = z.contiguous()
-        bias32 = None if bias is None else bias.detach().float().contiguous()
-        if residual is not None:
-            residual = residual.to(z.dtype).contiguous()
-        with torch.cuda.device(z.device):
-            y = ops.bias_act(lib, z, bias32, residual, act)
-        # relu alone needs only the sign of its output
-        keep_z = act == "gelu" or (act == "relu" and residual is not None)
-        ctx.save_for_backward(z if keep_z else y if act == "relu" else None, bias32 if keep_z else None)
-        ctx.act = act
-        ctx.has_bias = bias is not None
-        return y
-
-    @staticmethod
-    @torch.autograd.function.once_differentiable
-    def backward(ctx, gy):
-        kept, bias32 = ctx.saved_tensors
-        gy = gy.contiguous()
-        want_gb = ctx.has_bias and ctx.needs_input_grad[1]
-        gz, gb = gy, None
-        if ctx.act is not None:
-            with torch.cuda.device(gy.device):
-                gz, gb = ops.bias_act_backward(_lib.get_library(), gy, kept, bias32, ctx.act, need_bias_grad=want_gb)
-        elif want_gb:
-            gb = gy.sum(2, dtype=torch.float32).sum(0)
-        return gz, gb, None, (gy if ctx.needs_input_grad[3] else None)
-
-
 _ACT_FUNCTIONS = {None: lambda t: t, "relu": torch.relu, "gelu": torch.nn.functional.gelu}
 
 
@@ -150,25 +113,16 @@ def pointwise_linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch
     """``act(W x + bias) + residual``: the 1x1 projection ``(B, Cin, N) -> (B, Cout, N)`` with
     ``weight`` of shape ``(Cout, Cin)`` or ``(Cout, Cin, 1)``, optionally followed by an
     activation (``"relu"`` or ``"gelu"``, the exact one) and the sum with a tensor of the
-    output's shape.  bfloat16 tensors on the GPU (stored or under autocast) run as GEMMs on the
-    channel-first layout plus one pass of the HIP library over the result; float32 tensors on
-    the GPU as the library's ``conv1d`` without bias plus that pass; everything else as the
-    reference's ``conv1d`` followed by PyTorch's activation and sum."""
+    output's shape.  bfloat16 (stored or under autocast) and float32 tensors on the GPU run as
+    batched GEMMs on the channel-first layout plus one pass of the HIP library over the result;
+    everything else as the reference's ``conv1d`` followed by PyTorch's activation and sum."""
     w2 = weight.squeeze(-1) if weight.dim() == 3 else weight
     dtype = x.dtype
     if x.is_cuda and torch.is_autocast_enabled(x.device.type):
         dtype = torch.get_autocast_dtype(x.device.type)
-    # 16-bit GPU tensors only: in float32 the library convolution is as fast (2-D network,
-    # batch 8: 24.5 against 25.5 ms per step)
-    if not x.is_cuda or x.dim() != 3 or dtype != torch.bfloat16:
-        if (x.is_cuda and x.dim() == 3 and dtype == torch.float32
-                and (bias is not None or act is not None or residual is not None)):
-            # float32 on the GPU: the library's convolution for the GEMM, its tail in one pass
-            z = torch.nn.functional.conv1d(x, w2.unsqueeze(-1))
-            if z.dtype == torch.float32:
-                return _BiasAct.apply(z, bias, act, residual)
-            y = _ACT_FUNCTIONS[act](z + bias.to(z.dtype).view(1, -1, 1) if bias is not None else z)
-            return y if residual is None else residual + y
+    # (2-D network in float32, batch 8: 16.6 ms per step this way against 20.8 ms with the
+    # GEMM left to the library's conv1d, whose weight gradient goes through layout transposes)
+    if not x.is_cuda or x.dim() != 3 or dtype not in (torch.bfloat16, torch.float32):
         y = _ACT_FUNCTIONS[act](torch.nn.functional.conv1d(x, w2.unsqueeze(-1), bias))
         return y if residual is None else residual + y
     x, w2 = x.to(dtype), w2.to(dtype)
@@ -179,9 +133,8 @@ def pointwise_linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch
 
 
 def _gemm_route(x: torch.Tensor) -> bool:
-    """True for the tensors whose 1x1 projection ``pointwise_linear`` runs off the library's
-    strided convolutions: bfloat16 (stored or under autocast; channel-first GEMMs) and float32
-    (``conv1d`` on the regrouped tensor) on the GPU."""
+    """True for the tensors whose 1x1 projection ``pointwise_linear`` runs as channel-first
+    GEMMs: bfloat16 (stored or under autocast) and float32 on the GPU."""
     dtype = x.dtype
     if x.is_cuda and torch.is_autocast_enabled(x.device.type):
         dtype = torch.get_autocast_dtype(x.device.type)

@@ -154,7 +154,7 @@ def test_projection_with_fused_tail_matches_the_unfused_form(act, with_res):
 @pytest.mark.gpu
 @pytest.mark.parametrize("act,with_res", [(None, False), (None, True), ("gelu", False), ("gelu", True)])
 def test_float32_projection_tail_matches_float64(act, with_res):
-    """float32 on the GPU (the 2-D network's regime): conv1d without bias + one pass of the HIP
+    """float32 on the GPU (the 2-D network's regime): batched GEMMs + one pass of the HIP
     library, values and every gradient against float64, 1e-5 of the largest entry."""
     torch.manual_seed(8)
     B, cin, cout, n = 2, 16, 24, 4096 + 40
@@ -164,7 +164,7 @@ def test_float32_projection_tail_matches_float64(act, with_res):
     res = torch.randn(B, cout, n, device="cuda", requires_grad=True) if with_res else None
     g = torch.randn(B, cout, n, device="cuda")
     y = layers.pointwise_linear(x, w, b, act, res)
-    assert y.dtype == torch.float32 and type(y.grad_fn).__name__.startswith("_BiasAct")
+    assert y.dtype == torch.float32 and type(y.grad_fn).__name__.startswith("_PointwiseLinear")
     leaves = [t for t in (x, w, b, res) if t is not None]
     got = torch.autograd.grad(y, leaves, g)
     l64 = [t.detach().double().requires_grad_(True) for t in leaves]

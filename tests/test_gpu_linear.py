@@ -60,7 +60,9 @@ def test_linear_module_under_autocast_keeps_float32_parameter_gradients():
     y.float().pow(2).sum().backward()
     assert lin.linear.weight.grad.dtype == torch.float32 and lin.linear.weight.grad.shape == (48, 16, 1)
     assert lin.linear.bias.grad.dtype == torch.float32 and x.grad.dtype == torch.float32
-    # float32 tensors outside autocast take the library convolution, bit for bit
+    # float32 tensors outside autocast take the same GEMM route in float32: the library
+    # convolution's result to float32 rounding
     y32 = lin(x.detach())
-    ref = F.conv1d(x.detach().flatten(2), lin.linear.weight, lin.linear.bias).view_as(y32)
-    assert torch.equal(y32, ref)
+    ref = F.conv1d(x.detach().double().flatten(2), lin.linear.weight.double(), lin.linear.bias.double()).view_as(y32)
+    assert y32.dtype == torch.float32
+    assert float((y32.double() - ref).abs().max() / ref.abs().max()) <= 1e-5
