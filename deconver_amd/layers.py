@@ -93,15 +93,16 @@ class _PointwiseLinear(torch.autograd.Function):
             # (two launches); long rows: chunks of the voxel axis as batch entries
             s = _wgrad_chunks(B, n) if n >= _CHUNKED_WGRAD_FROM else 1
             if s == 1:
-                gw = torch.bmm(gz, x.transpose(1, 2)).float().sum(0).to(weight.dtype)
+                parts = torch.bmm(gz, x.transpose(1, 2))
             else:
-                acc = torch.zeros(cout, cin, dtype=torch.float32, device=gz.device)
+                parts = gz.new_empty(B * s, cout, cin)
                 for b in range(B):
                     # chunk c of the voxel axis as batch entry c: strided views, no copies
                     a = gz[b].view(cout, s, n // s).transpose(0, 1)
                     c = x[b].view(cin, s, n // s).permute(1, 2, 0)
-                    acc += torch.bmm(a, c).float().sum(0)
-                gw = acc.to(weight.dtype)
+                    torch.bmm(a, c, out=parts[b * s:(b + 1) * s])
+            # the partial results are added in float32, in one reduction
+            gw = parts.sum(0, dtype=torch.float32).to(weight.dtype)
         return gx, gw, gb, None, gres
 
 
