@@ -48,9 +48,12 @@ class _PointwiseLinear(torch.autograd.Function):
         lib = _lib.get_library()
         # one batched GEMM on the tensors as they lie, the weight shared by the batch entries
         # through a zero stride (no copy; the same bits as one GEMM per sample, in one launch)
+        # (the weight arrives in its own dtype -- float32 under autocast -- and is cast here, so
+        # that its gradient leaves backward as the float32 sum it is, not rounded to bf16 first)
         B = x.shape[0]
-        z = x.new_empty(B, weight.shape[0], x.shape[2])
-        torch.bmm(weight.unsqueeze(0).expand(B, -1, -1), x, out=z)
+        w = weight.detach().to(x.dtype)
+        z = x.new_empty(B, w.shape[0], x.shape[2])
+        torch.bmm(w.unsqueeze(0).expand(B, -1, -1), x, out=z)
         bias32 = None if bias is None else bias.detach().float().contiguous()
         y = z
         # the activation's gradient needs z + bias: gelu keeps z; relu alone needs only the
@@ -60,7 +63,8 @@ class _PointwiseLinear(torch.autograd.Function):
             with torch.cuda.device(x.device):
                 y = ops.bias_act(lib, z, bias32, residual, act, inplace=not keep_z)
         kept = z if keep_z else y if act == "relu" else None
-        ctx.save_for_backward(x, weight, kept, bias32 if keep_z else None)
+        ctx.save_for_backward(x, w, kept, bias32 if keep_z else None)
+        ctx.weight_dtype = weight.dtype
         ctx.has_bias = bias is not None
         ctx.act = act
         return y
@@ -102,7 +106,7 @@ class _PointwiseLinear(torch.autograd.Function):
                     c = x[b].view(cin, s, n // s).permute(1, 2, 0)
                     torch.bmm(a, c, out=parts[b * s:(b + 1) * s])
             # the partial results are added in float32, in one reduction
-            gw = parts.sum(0, dtype=torch.float32).to(weight.dtype)
+            gw = parts.sum(0, dtype=torch.float32).to(ctx.weight_dtype)
         return gx, gw, gb, None, gres
 
 
@@ -126,7 +130,7 @@ def pointwise_linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch
     if not x.is_cuda or x.dim() != 3 or dtype not in (torch.bfloat16, torch.float32):
         y = _ACT_FUNCTIONS[act](torch.nn.functional.conv1d(x, w2.unsqueeze(-1), bias))
         return y if residual is None else residual + y
-    x, w2 = x.to(dtype), w2.to(dtype)
+    x = x.to(dtype)
     if residual is not None:
         residual = residual.to(dtype).contiguous()
     with torch.autocast(x.device.type, enabled=False):
