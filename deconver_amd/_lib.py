@@ -46,6 +46,7 @@ EXPORTS = (
     "ndc_bias_act",
     "ndc_bias_act_backward",
     "ndc_regroup",
+    "ndc_row_sums",
 )
 
 
@@ -125,6 +126,7 @@ class NdcLibrary:
                                    ctypes.c_int, ctypes.c_int, vp]
         d.ndc_bias_act_backward.argtypes = [vp, vp, vp, vp, vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                                             ctypes.c_int, ctypes.c_int, vp]
+        d.ndc_row_sums.argtypes = [vp, vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int, vp]
         d.ndc_regroup.argtypes = [vp, vp, vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                                    ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp]
         d.ndc_taps_bytes.restype = ctypes.c_size_t
@@ -278,6 +280,9 @@ class NdcLibrary:
                           batch: int, channels: int, n: int, act: int, dtype: int, stream) -> None:
         self._check(self._dll.ndc_bias_act_backward(gy, z, bias, gz, gpart, batch, channels, n, act, dtype,
                                                     stream), "ndc_bias_act_backward")
+
+    def row_sums(self, x: int, partial: int, rows: int, n: int, dtype: int, stream) -> None:
+        self._check(self._dll.ndc_row_sums(x, partial, rows, n, dtype, stream), "ndc_row_sums")
 
     def regroup2(self, src: int, dst: int, bias: Optional[int], rows: int, channels: int, D: int, H: int,
                  W: int, depth2: bool, dtype: int, to_channels: bool, stream) -> None:

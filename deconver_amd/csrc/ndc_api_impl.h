@@ -518,6 +518,19 @@ int ndc_bias_act_backward(const void *gy, const void *z, const float *bias, void
                                            chunk, act, esz, vec, stream);
 }
 
+int ndc_row_sums(const void *x, float *partial, int64_t rows, int64_t n, int dtype, void *stream)
+{
+    if (!x || !partial) return NDC_ERR_NULL;
+    int st = rownorm_check(rows, n, dtype);
+    if (st) return st;
+    int nsplit;
+    long long chunk;
+    rownorm_split(rows, n, nsplit, chunk);
+    const int esz = dtype == NDC_BF16 ? 2 : 4;
+    const bool vec = n % (16 / esz) == 0 && aligned16(x);
+    return ndc::Backend::row_sums(x, partial, rows, n, nsplit, chunk, esz, vec, stream);
+}
+
 int ndc_regroup(const void *src, void *dst, const float *bias, int64_t rows, int64_t channels, int64_t D,
                  int64_t H, int64_t W, int depth2, int dtype, int to_channels, void *stream)
 {

@@ -293,6 +293,22 @@ struct Backend {
         return check();
     }
 
+    static int row_sums(const void *a, float *partial, long long rows, long long n, int nsplit, long long chunk,
+                        int esz, bool vec, void *stream)
+    {
+        if (rows <= 0 || n <= 0) return 0;
+        const rownorm::Split sp = {n, chunk, nsplit};
+        const dim3 grid((unsigned)(rows * nsplit)), block(rownorm::kThreads);
+        if (esz == 2) {
+            if (vec) hipLaunchKernelGGL((rownorm::row_sums_kernel<bf16_t, true>), grid, block, 0, (hipStream_t)stream, (const bf16_t *)a, partial, sp);
+            else hipLaunchKernelGGL((rownorm::row_sums_kernel<bf16_t, false>), grid, block, 0, (hipStream_t)stream, (const bf16_t *)a, partial, sp);
+        } else {
+            if (vec) hipLaunchKernelGGL((rownorm::row_sums_kernel<float, true>), grid, block, 0, (hipStream_t)stream, (const float *)a, partial, sp);
+            else hipLaunchKernelGGL((rownorm::row_sums_kernel<float, false>), grid, block, 0, (hipStream_t)stream, (const float *)a, partial, sp);
+        }
+        return check();
+    }
+
     // y = act(z + bias[channel]) + residual on rows * nsplit workgroups (bias, residual optional)
     template <typename T, int ACT, bool RES>
     static void bias_act_launch(const void *z, const float *bias, const void *res, void *y, int channels,

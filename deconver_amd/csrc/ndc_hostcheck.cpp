@@ -157,6 +157,20 @@ struct Backend {
         return 0;
     }
 
+    static int row_sums(const void *a, float *partial, long long rows, long long n, int nsplit, long long chunk,
+                        int esz, bool, void *)
+    {
+        for (long long row = 0; row < rows; ++row)
+            for (int part = 0; part < nsplit; ++part) {
+                const long long lo = part * chunk, hi = lo + chunk < n ? lo + chunk : n;
+                float s = 0.f;
+                for (long long i = row * n + lo; i < row * n + hi; ++i)
+                    s += esz == 2 ? Elem<bf16_t>::load((const bf16_t *)a + i) : ((const float *)a)[i];
+                partial[row * nsplit + part] = s;
+            }
+        return 0;
+    }
+
     static float act_value(int act, float u, bool grad)
     {
         const float cdf = 0.5f * (1.f + std::erf(u * 0.70710678118654752f));

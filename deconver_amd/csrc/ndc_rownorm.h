@@ -187,6 +187,46 @@ reduce_kernel(const T *a, const T *b, float2 *partial, Split sp)
     }
 }
 
+// partial[row][part] = the sum of the part: the bias gradient of a projection without activation
+// is the sum of its output gradient over batch, parts and voxels (1 U e read).
+template <typename T, bool VEC>
+__global__ void __launch_bounds__(kThreads)
+row_sums_kernel(const T *a, float *partial, Split sp)
+{
+    __shared__ float buf[4][2];
+    const long long row = blockIdx.x / sp.nsplit;
+    const int part = blockIdx.x % sp.nsplit;
+    const T *ar = a + row * sp.n;
+    const long long lo = part * sp.chunk, hi = lo + sp.chunk < sp.n ? lo + sp.chunk : sp.n;
+    float s = 0.f, unused = 0.f;
+    if constexpr (VEC) {
+        typedef Vec<T> V;
+        const long long v0 = lo / V::N, v1 = hi / V::N;
+        const V *av = reinterpret_cast<const V *>(ar);
+        float t[4] = {0.f, 0.f, 0.f, 0.f};
+        long long i = v0 + threadIdx.x;
+        for (; i + 3 * kThreads < v1; i += 4 * kThreads) {
+            V x[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) x[u] = av[i + u * kThreads];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int e = 0; e < V::N; ++e) t[u] += x[u].get(e);
+        }
+        for (; i < v1; i += kThreads) {
+            const V x = av[i];
+#pragma unroll
+            for (int e = 0; e < V::N; ++e) t[0] += x.get(e);
+        }
+        s = (t[0] + t[1]) + (t[2] + t[3]);
+    } else {
+        for (long long i = lo + threadIdx.x; i < hi; i += kThreads) s += Elem<T>::load(ar + i);
+    }
+    block_sum2(s, unused, buf);
+    if (threadIdx.x == 0) partial[blockIdx.x] = s;
+}
+
 template <typename T, bool BWD, bool VEC, bool ADD = false>
 __global__ void __launch_bounds__(kThreads)
 apply_kernel(const T *a, const T *b, const T *addend, const float2 *partial, float2 *stats, T *out, Split sp,

@@ -314,3 +314,15 @@ def channels_to_windows(lib: _lib.NdcLibrary, y: Tensor, bias: Optional[Tensor] 
     lib.regroup2(_ptr(y), _ptr(out), _ptr(bias), B * C, C, D, sp[-2], sp[-1], nd == 3, dtype_tag(y.dtype), False,
                  _stream_of(y))
     return out
+
+
+def channel_sums(lib: _lib.NdcLibrary, g: Tensor) -> Tensor:
+    """Sum of a contiguous ``(B, C, n)`` tensor over batch and voxels, float32, ``C`` entries:
+    the bias gradient of a projection from its output gradient."""
+    if g.dim() != 3 or not g.is_contiguous():
+        raise ValueError("channel_sums wants a contiguous (B, C, n) tensor")
+    B, C, n = g.shape
+    parts = lib.bias_act_parts(B * C, n)
+    partial = torch.empty(B, C, parts, dtype=torch.float32, device=g.device)
+    lib.row_sums(_ptr(g), _ptr(partial), B * C, n, dtype_tag(g.dtype), _stream_of(g))
+    return partial.sum((0, 2))

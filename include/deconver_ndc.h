@@ -300,6 +300,13 @@ int ndc_rownorm_backward(const void *gy, const void *y, const float *stats, cons
  * batch and the parts.  (With NDC_ACT_NONE the gradient of z is gy itself; the call is refused.)
  */
 enum ndc_act { NDC_ACT_NONE = 0, NDC_ACT_RELU = 1, NDC_ACT_GELU = 2 };
+/*
+ * ndc_row_sums: partial[row * parts + p] = the sum of part p of row `row` of a (rows, n) matrix,
+ * parts = ndc_bias_act_parts(rows, n), float32.  The bias gradient of a projection without
+ * activation (nn.Conv1d's in deconver/layers/linear.py:53-58) is the sum of these over the
+ * batch and the parts of its output gradient.
+ */
+int ndc_row_sums(const void *x, float *partial, int64_t rows, int64_t n, int dtype, void *stream);
 int64_t ndc_bias_act_parts(int64_t rows, int64_t n);
 int ndc_bias_act(const void *z, const float *bias, const void *residual, void *y, int64_t batch,
                  int64_t channels, int64_t n, int act, int dtype, void *stream);

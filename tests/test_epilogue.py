@@ -64,6 +64,17 @@ def test_host_build_matches_pytorch(shape, dtype, act):
         _check(lib, shape, dtype, act, with_bias, with_res)
 
 
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_host_channel_sums(shape, dtype):
+    lib = hostcheck_library()
+    g = torch.randn(*shape, generator=torch.Generator().manual_seed(sum(shape))).to(dtype)
+    got = ops.channel_sums(lib, g)
+    ref = g.double().sum((0, 2))
+    assert got.dtype == torch.float32 and got.shape == (shape[1],)
+    assert float((got.double() - ref).abs().max()) <= 1e-5 * float(g.double().abs().sum((0, 2)).max())
+
+
 def test_bad_arguments_are_refused():
     lib = hostcheck_library()
     z = torch.zeros(2, 3, 8)
@@ -112,6 +123,18 @@ def test_hip_kernels_match_pytorch(shape, dtype, act):
     lib = _lib.get_library()
     for with_bias, with_res in ((True, True), (True, False), (False, False)):
         _check(lib, shape, dtype, act, with_bias, with_res, device="cuda")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(2, 3, 7), (2, 64, 32 * 32 * 32), (1, 5, 2048 * 9 + 3), (2, 130, 4096)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_hip_channel_sums(shape, dtype):
+    lib = _lib.get_library()
+    g = torch.randn(*shape, device="cuda").to(dtype)
+    got = ops.channel_sums(lib, g)
+    ref = g.double().sum((0, 2))
+    assert float((got.double() - ref).abs().max()) <= 1e-5 * float(g.double().abs().sum((0, 2)).max())
+    assert torch.equal(got, ops.channel_sums(lib, g))     # fixed association
 
 
 @pytest.mark.gpu
