@@ -47,3 +47,16 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "_library", None)
     with pytest.raises(_lib.NdcError, match="no CPU or PyTorch fallback"):
         _lib.get_library()
+
+
+def test_header_is_plain_c():
+    """The boundary is a C ABI: the header must compile as C99 and as C++ on its own."""
+    import shutil
+    import subprocess
+    if not shutil.which("gcc"):
+        pytest.skip("no C compiler here")
+    for args in (["gcc", "-std=c99", "-x", "c"], ["g++", "-std=c++11", "-x", "c++"]):
+        if not shutil.which(args[0]):
+            continue
+        proc = subprocess.run(args + ["-fsyntax-only", "-Wall", "-Werror", HEADER], capture_output=True, text=True)
+        assert proc.returncode == 0, proc.stderr
