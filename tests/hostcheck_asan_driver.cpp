@@ -67,6 +67,37 @@ static int run_case(const Case &c)
     return st;
 }
 
+// The block-level entry points on exactly sized buffers (rows cut into several parts, a ragged
+// last part, a row length that is not a whole number of 16-byte vectors).
+static int run_block_level(int dtype)
+{
+    const int esz = dtype == NDC_BF16 ? 2 : 4;
+    const long long B = 2, C = 3, n = 2 * 8192 + 2048 + 5, rows = B * C;
+    const size_t bytes = (size_t)(rows * n * esz);
+    void *x = calloc(1, bytes), *y = malloc(bytes), *g = calloc(1, bytes), *gx = malloc(bytes);
+    float *stats = (float *)malloc(sizeof(float) * 2 * rows);
+    float bias[3] = {0.1f, -0.2f, 0.3f};
+    const size_t wsb = ndc_rownorm_workspace_bytes(rows, n);
+    void *ws = malloc(wsb);
+    const long long parts = ndc_bias_act_parts(rows, n);
+    float *gpart = (float *)malloc(sizeof(float) * rows * parts);
+    int st = ndc_rownorm_forward(x, y, stats, rows, n, dtype, 1e-5f, ws, wsb, nullptr);
+    if (!st) st = ndc_rownorm_backward(g, y, stats, x, gx, rows, n, dtype, ws, wsb, nullptr);
+    if (!st) st = ndc_bias_act(x, bias, g, y, B, C, n, NDC_ACT_GELU, dtype, nullptr);
+    if (!st) st = ndc_bias_act_backward(g, x, bias, gx, gpart, B, C, n, NDC_ACT_GELU, dtype, nullptr);
+    if (!st) st = ndc_row_sums(g, gpart, rows, n, dtype, nullptr);
+    if (!st) st = ndc_relayout(x, y, B, C, n, dtype, 1, nullptr);
+    free(gpart); free(ws); free(stats); free(x); free(y); free(g); free(gx);
+    // 2 x 2 x 2 windows of a (rows, 4, 6, 16) grid and back
+    const long long D = 4, H = 6, W = 16, m = rows * D * H * W;
+    void *fine = calloc(1, (size_t)(m * esz)), *coarse = malloc((size_t)(m * esz)), *back = malloc((size_t)(m * esz));
+    if (!st) st = ndc_regroup(fine, coarse, nullptr, rows, C, D, H, W, 1, dtype, 1, nullptr);
+    if (!st) st = ndc_regroup(coarse, back, bias, rows, C, D, H, W, 1, dtype, 0, nullptr);
+    free(fine); free(coarse); free(back);
+    printf("block-level entry points dtype%d -> status %d\n", dtype, st);
+    return st;
+}
+
 int main()
 {
     const Case cases[] = {
@@ -94,5 +125,7 @@ int main()
                c.B, c.G, c.m, c.sc, c.D, c.H, c.W, c.kD, c.kH, c.kW, c.dtype, c.path, st, faults, first);
         if (st || faults) ++bad;
     }
+    if (run_block_level(NDC_F32)) ++bad;
+    if (run_block_level(NDC_BF16)) ++bad;
     return bad ? 1 : 0;
 }
