@@ -638,14 +638,33 @@ def mixer_workload(args) -> int:
             y = mixer(x)
         y.backward(g.to(y.dtype))
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    def timed(fn):
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / args.steps * 1e3
+
+    ms = timed(step)
+    extra = {}
+    if dtype is not None:
+        # the same mixer as it sits inside the network: its input (the norm's output) and the
+        # gradient of its output are bf16 already, so the casts of the autocast boundary above
+        # (float32 input -> bf16, input gradient -> float32) do not occur
+        xb = x.detach().bfloat16().requires_grad_(True)
+        gb = g.bfloat16()
+
+        def step_in_network():
+            mixer.zero_grad(set_to_none=True)
+            xb.grad = None
+            with torch.autocast("cuda", dtype=torch.bfloat16):
+                y = mixer(xb)
+            y.backward(gb)
+
+        extra["in_network_ms_per_step"] = timed(step_in_network)
     vox = w["batch"] * math.prod(w["spatial"])
     print(json.dumps({
         "metric": "DeconvMixer fwd+bwd Gvoxel/s", "value": vox / (ms * 1e-3) / 1e9,
@@ -653,8 +672,9 @@ def mixer_workload(args) -> int:
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype if args.dtype == "bf16" else "f32", "data": "synthetic",
         "config": {"workload": "one DeconvMixer at config 3's shape (batch 2, 128 channels, "
-                               "64^3, 3x3x3, ratio 4), forward + backward"},
-        "roofline": None, "cpu_baseline": None}))
+                               "64^3, 3x3x3, ratio 4), forward + backward; float32 input and "
+                               "upstream gradient under bf16 autocast"},
+        **extra, "roofline": None, "cpu_baseline": None}))
     return 0
 
 
