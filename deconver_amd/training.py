@@ -23,6 +23,17 @@ __all__ = ["dice_bce_loss", "make_optimizer", "smoothed_noise_masks", "ellipsoid
            "train_step"]
 
 
+def _voxel_sum(t: Tensor) -> Tensor:
+    """``t.sum(-1)`` of a ``(B, C, n)`` tensor in two stages when ``n`` is long: a reduction to
+    B*C outputs runs on B*C workgroups (two, for a batch of two one-channel volumes: 0.27 ms
+    per sum of 2 M voxels on an MI355X), 1 024 partial sums per row fill the device."""
+    n = t.shape[-1]
+    for chunks in (1024, 256, 64):
+        if n % chunks == 0 and n // chunks >= 256:
+            return t.view(*t.shape[:-1], chunks, n // chunks).sum(-1).sum(-1)
+    return t.sum(-1)
+
+
 def dice_bce_loss(logits: Tensor, target: Tensor) -> Tensor:
     """Binary cross-entropy on the logits plus soft Dice loss with +1 smoothing, float32."""
     logits = logits.float()
@@ -30,7 +41,7 @@ def dice_bce_loss(logits: Tensor, target: Tensor) -> Tensor:
     bce = F.binary_cross_entropy_with_logits(logits, target)
     p = torch.sigmoid(logits).flatten(2)
     y = target.flatten(2)
-    dice = (2 * (p * y).sum(-1) + 1) / (p.sum(-1) + y.sum(-1) + 1)
+    dice = (2 * _voxel_sum(p * y) + 1) / (_voxel_sum(p) + _voxel_sum(y) + 1)
     return bce + (1 - dice).mean()
 
 
