@@ -1130,14 +1130,14 @@ def main() -> int:
         x = z = g = None
         result["sweep"] = {"workload": "config 5: forward-only NDC update, 3x3x3, ratio 4, bf16, inference "
                                        "form; hbm_frac on 9 U e",
-                           "shapes": sweep_rows(torch, lib, ops, dev, 3, 10)}
+                           "shapes": sweep_rows(torch, lib, ops, dev, 10, 50)}
         result["layers_2d"] = {"workload": "2-D 5x5 update node, depthwise, ratio 4, float32, forward + "
                                            "backward; hbm_frac on 23 U e",
-                               "layers": layers_2d_rows(torch, lib, ops, dev, 3, 10)}
+                               "layers": layers_2d_rows(torch, lib, ops, dev, 10, 50)}
         result["block_kernels"] = {"workload": "InstanceNorm and bias / GELU / residual passes of a Deconver block "
                                                "at config 4's levels, bf16, HIP kernels next to PyTorch's; GB/s on "
                                                "whole passes over the tensor",
-                                   "shapes": block_rows(torch, 10, 3)}
+                                   "shapes": block_rows(torch, 20, 5)}
         _progress("config-5 sweep, 2-D layers and block kernels done")
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(torch)
