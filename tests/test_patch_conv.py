@@ -219,3 +219,26 @@ def test_full_size_regrouping_round_trip():
             for kh in (0, 1):
                 for kw in (0, 1):
                     assert cols[b, c * 8 + (kd * 2 + kh) * 2 + kw, d, h, w] == x[b, c, 2 * d + kd, 2 * h + kh, 2 * w + kw]
+
+
+def test_host_regroup_on_random_grids():
+    """Random even grids (hypothesis): the host build's regrouping equals the strided view in
+    both directions, 2-D and 3-D, float32 and bfloat16."""
+    from hypothesis import given, settings, strategies as st
+
+    lib = hostcheck_library()
+
+    @settings(max_examples=40, deadline=None)
+    @given(st.integers(1, 2), st.integers(1, 3), st.integers(1, 3), st.integers(1, 4), st.integers(1, 3),
+           st.booleans(), st.booleans())
+    def check(B, C, d2, h2, w8, three_d, bf16):
+        dtype = torch.bfloat16 if bf16 else torch.float32
+        W = w8 * (8 if bf16 else 4)
+        shape = (B, C, 2 * d2, 2 * h2, W) if three_d else (B, C, 2 * h2, W)
+        x = torch.randn(*shape).to(dtype)
+        nd = len(shape) - 2
+        cols = ops.windows_to_channels(lib, x)
+        assert torch.equal(cols.flatten(2), layers.patches_to_channels(x, (2,) * nd))
+        assert torch.equal(ops.channels_to_windows(lib, cols), x)
+
+    check()
