@@ -109,7 +109,9 @@ class Stem(nn.Sequential):
 
     def __init__(self, in_channels: int, out_channels: int, patch_size: Sequence[int] = (4, 4),
                  norm: Any = LayerNorm):
-        conv = getattr(nn, f"Conv{len(patch_size)}d")
+        # (a convolution whose windows tile the input: same module and parameters, regrouping +
+        # GEMMs on the GPU)
+        conv = getattr(layers, f"PatchConv{len(patch_size)}d")
         super().__init__(conv(in_channels, out_channels, patch_size, stride=patch_size),
                          build(native_norm(norm), out_channels))
 

@@ -242,3 +242,30 @@ def test_host_regroup_on_random_grids():
         assert torch.equal(ops.channels_to_windows(lib, cols), x)
 
     check()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("regime", ["bf16 autocast", "float32"])
+def test_patchifying_stem_on_the_gpu(regime):
+    """``Stem`` (deconver.py:106-114: a 4 x 4 patchifying convolution + norm) on the GPU: windows
+    other than 2 x 2 are regrouped by a strided view; values and weight gradient against
+    torch's convolution in float64."""
+    import contextlib
+    torch.manual_seed(9)
+    bf16 = regime == "bf16 autocast"
+    stem = dc.Stem(3, 16, patch_size=(4, 4)).cuda()
+    conv = stem[0]
+    assert isinstance(conv, layers.PatchConv2d)
+    x = torch.randn(2, 3, 32, 40, device="cuda")
+    with (torch.autocast("cuda", dtype=torch.bfloat16) if bf16 else contextlib.nullcontext()):
+        y = conv(x)
+    w64 = conv.weight.detach().double().requires_grad_(True)
+    ref = F.conv2d(x.double(), w64, conv.bias.detach().double(), stride=4)
+    g = torch.randn_like(y)
+    (gw,) = torch.autograd.grad(y, conv.weight, g)
+    (gw_ref,) = torch.autograd.grad(ref, w64, g.double())
+    tol = 2e-2 if bf16 else 1e-5
+    for a, r in ((y, ref), (gw, gw_ref)):
+        assert a.shape == r.shape
+        assert float((a.detach().double() - r.detach()).abs().max() / r.detach().abs().max()) <= tol
+    assert stem(x).shape == (2, 16, 8, 10)
