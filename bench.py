@@ -860,7 +860,8 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     # defaults: 200 timed steps after 50 for the headline workload (0.45 s in all: a 20-step region
     # of 36 ms ends before the clocks have settled and reads 2-3 % slow and noisy: 1.81-1.83 against
-    # 1.772 +- 0.001 ms), 20 after 5 for the others
+    # 1.772 +- 0.001 ms), 50 after 10 for the other kernel-level workloads, 20 after 5 for the
+    # model-level ones
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
     ap.add_argument("--dtype", choices=("bf16", "fp32"), default="bf16")
@@ -887,9 +888,9 @@ def main() -> int:
                     help="model-level workloads: which route the NDC layers take")
     args = ap.parse_args()
     if args.steps is None:
-        args.steps = 200 if args.workload == "ndc" else 20
+        args.steps = {"ndc": 200, "sweep": 50, "block": 50, "mixer": 50}.get(args.workload, 20)
     if args.warmup is None:
-        args.warmup = 50 if args.workload == "ndc" else 5
+        args.warmup = {"ndc": 50, "sweep": 10, "block": 10, "mixer": 10}.get(args.workload, 5)
     if args.gpus != 1:
         print("bench.py measures the one-GPU hot path only: this build has no multi-GPU code "
               "path (every box has one GPU); run with --gpus 1", file=sys.stderr)
