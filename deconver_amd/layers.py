@@ -1,7 +1,11 @@
 """Channel-first helper layers around the NDC update (``deconver/layers`` of the reference):
 ``Linear`` (1x1 projection, parameters held by an ``nn.Conv1d`` as there), ``MLP``,
-``LayerNorm``.  They stay on PyTorch-ROCm GEMMs / library kernels; parameter names match the
-reference so that its checkpoints load unchanged."""
+``LayerNorm``, and the network's resampling convolutions, head and stem as subclasses of the
+``torch.nn`` convolutions.  On the GPU the projections are batched channel-first GEMMs
+(hipBLASLt through ``torch.bmm``) followed by one pass of the HIP library for bias, activation
+and residual sum; the strided convolutions are a regrouping copy in front of the same
+projection.  Parameter names and shapes match the reference, so its checkpoints load
+unchanged."""
 
 from __future__ import annotations
 
@@ -30,9 +34,9 @@ def _wgrad_chunks(batch: int, n: int) -> int:
 
 class _PointwiseLinear(torch.autograd.Function):
     """``y[b] = act(W x[b] + bias) + residual[b]`` for ``x`` of shape ``(B, Cin, N)``: the 1x1
-    projection as plain GEMMs on the channel-first layout (hipBLASLt through ``torch.mm`` /
-    ``bmm``), then ONE pass of the HIP library over the result for bias, activation and
-    residual sum (``ndc_bias_act``).
+    projection as plain GEMMs on the channel-first layout (hipBLASLt through ``torch.bmm``),
+    then ONE pass of the HIP library over the result for bias, activation and residual sum
+    (``ndc_bias_act``).
 
     The same map as ``nn.Conv1d(kernel_size=1)`` (layers/linear.py:53-58) followed by the
     activation and the ``x + ...`` of the block (layers/mlp.py:40-63, deconver.py:60-64).  The
