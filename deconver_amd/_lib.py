@@ -47,6 +47,9 @@ EXPORTS = (
     "ndc_bias_act_backward",
     "ndc_regroup",
     "ndc_row_sums",
+    "ndc_chnorm_parts",
+    "ndc_chnorm_forward",
+    "ndc_chnorm_backward",
 )
 
 
@@ -126,6 +129,12 @@ class NdcLibrary:
                                    ctypes.c_int, ctypes.c_int, vp]
         d.ndc_bias_act_backward.argtypes = [vp, vp, vp, vp, vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                                             ctypes.c_int, ctypes.c_int, vp]
+        d.ndc_chnorm_parts.restype = ctypes.c_int64
+        d.ndc_chnorm_parts.argtypes = [ctypes.c_int64, ctypes.c_int64, ctypes.c_int]
+        d.ndc_chnorm_forward.argtypes = [vp, vp, vp, vp, vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                                         ctypes.c_int, ctypes.c_float, vp]
+        d.ndc_chnorm_backward.argtypes = [vp, vp, vp, vp, vp, vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                                          ctypes.c_int, vp]
         d.ndc_row_sums.argtypes = [vp, vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int, vp]
         d.ndc_regroup.argtypes = [vp, vp, vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                                    ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp]
@@ -280,6 +289,20 @@ class NdcLibrary:
                           batch: int, channels: int, n: int, act: int, dtype: int, stream) -> None:
         self._check(self._dll.ndc_bias_act_backward(gy, z, bias, gz, gpart, batch, channels, n, act, dtype,
                                                     stream), "ndc_bias_act_backward")
+
+    def chnorm_parts(self, batch: int, n: int, dtype: int) -> int:
+        return int(self._dll.ndc_chnorm_parts(batch, n, dtype))
+
+    def chnorm_forward(self, x: int, weight: Optional[int], bias: Optional[int], y: int, stats: int,
+                       batch: int, channels: int, n: int, dtype: int, eps: float, stream) -> None:
+        """Normalisation over the channels of a channel-first ``(batch, channels, n)`` tensor."""
+        self._check(self._dll.ndc_chnorm_forward(x, weight, bias, y, stats, batch, channels, n, dtype, eps,
+                                                 stream), "ndc_chnorm_forward")
+
+    def chnorm_backward(self, gy: int, x: int, stats: int, weight: Optional[int], gx: int,
+                        partial: Optional[int], batch: int, channels: int, n: int, dtype: int, stream) -> None:
+        self._check(self._dll.ndc_chnorm_backward(gy, x, stats, weight, gx, partial, batch, channels, n, dtype,
+                                                  stream), "ndc_chnorm_backward")
 
     def row_sums(self, x: int, partial: int, rows: int, n: int, dtype: int, stream) -> None:
         self._check(self._dll.ndc_row_sums(x, partial, rows, n, dtype, stream), "ndc_row_sums")

@@ -518,6 +518,54 @@ int ndc_bias_act_backward(const void *gy, const void *z, const float *bias, void
                                            chunk, act, esz, vec, stream);
 }
 
+static int chnorm_check(long long B, long long C, long long n, int dtype)
+{
+    if (dtype != NDC_F32 && dtype != NDC_BF16) return NDC_ERR_DTYPE;
+    if (B < 1 || C < 1 || C > 0x7fffffffLL || n < 1 || (long double)B * C * n > 9.0e15L) return NDC_ERR_GEOMETRY;
+    return NDC_OK;
+}
+
+int64_t ndc_chnorm_parts(int64_t batch, int64_t n, int dtype)
+{
+    if (batch < 1 || n < 1 || (dtype != NDC_F32 && dtype != NDC_BF16)) return 0;
+    const int esz = dtype == NDC_BF16 ? 2 : 4;
+    // (the count for the vector path if n allows it, which is what the entry points then use
+    // when the buffers are aligned; an unaligned call needs more rows and is refused)
+    const bool vec = n % (16 / esz) == 0;
+    return batch * ndc::Backend::chnorm_blocks(n, esz, vec) * ndc::Backend::kChnormWaves;
+}
+
+int ndc_chnorm_forward(const void *x, const float *weight, const float *bias, void *y, float *stats,
+                       int64_t batch, int64_t channels, int64_t n, int dtype, float eps, void *stream)
+{
+    if (!x || !y || !stats) return NDC_ERR_NULL;
+    int st = chnorm_check(batch, channels, n, dtype);
+    if (st) return st;
+    if (x == (const void *)y || !(eps >= 0.f)) return NDC_ERR_GEOMETRY;
+    const int esz = dtype == NDC_BF16 ? 2 : 4;
+    const bool vec = n % (16 / esz) == 0 && aligned16(x) && aligned16(y);
+    st = ndc::Backend::chnorm(false, nullptr, x, stats, weight, bias, y, nullptr, batch, (int)channels, n, esz, vec,
+                              eps, stream);
+    return st == -2 ? (int)NDC_ERR_GEOMETRY : st;
+}
+
+int ndc_chnorm_backward(const void *gy, const void *x, const float *stats, const float *weight, void *gx,
+                        float *partial, int64_t batch, int64_t channels, int64_t n, int dtype, void *stream)
+{
+    if (!gy || !x || !stats || !gx) return NDC_ERR_NULL;
+    int st = chnorm_check(batch, channels, n, dtype);
+    if (st) return st;
+    if (gx == x) return NDC_ERR_GEOMETRY;
+    const int esz = dtype == NDC_BF16 ? 2 : 4;
+    const bool fits = n % (16 / esz) == 0;
+    const bool vec = fits && aligned16(gy) && aligned16(x) && aligned16(gx);
+    // the partial rows are laid out for the path ndc_chnorm_parts counted
+    if (partial && fits && !vec) return NDC_ERR_WORKSPACE;
+    st = ndc::Backend::chnorm(true, gy, x, stats, weight, nullptr, gx, partial, batch, (int)channels, n, esz, vec,
+                              0.f, stream);
+    return st == -2 ? (int)NDC_ERR_GEOMETRY : st;
+}
+
 int ndc_row_sums(const void *x, float *partial, int64_t rows, int64_t n, int dtype, void *stream)
 {
     if (!x || !partial) return NDC_ERR_NULL;

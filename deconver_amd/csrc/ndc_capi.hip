@@ -6,6 +6,7 @@
 #include "ndc_rownorm.h"
 #include "ndc_epilogue.h"
 #include "ndc_regroup.h"
+#include "ndc_chnorm.h"
 
 #define NDC_LAMBDA __host__ __device__
 
@@ -290,6 +291,43 @@ struct Backend {
         const rownorm::Split sp = {n, chunk, nsplit};
         if (esz == 2) rownorm_t<bf16_t>(bwd, a, b, addend, partial, stats, out, rows, sp, vec, eps, stream);
         else rownorm_t<float>(bwd, a, b, addend, partial, stats, out, rows, sp, vec, eps, stream);
+        return check();
+    }
+
+    // normalisation over the channels of a channel-first (B, C, n) tensor; see ndc_chnorm.h
+    static constexpr int kChnormWaves = rownorm::kThreads / 64;   // partial rows per workgroup
+    static long long chnorm_blocks(long long n, int esz, bool vec)
+    {
+        const long long per = vec ? 16 / esz : 1;
+        return (n / per + rownorm::kThreads - 1) / rownorm::kThreads;
+    }
+    template <typename T, bool VEC>
+    static void chnorm_launch(bool bwd, const void *a, const void *x, const float *stats, const float *weight,
+                              const float *bias, void *out, float *partial, long long B, int C, long long n,
+                              float eps, void *stream)
+    {
+        const chnorm::Shape sh = {n, C, (int)chnorm_blocks(n, (int)sizeof(T), VEC)};
+        const dim3 grid((unsigned)(B * sh.blocks)), block(rownorm::kThreads);
+        if (bwd)
+            hipLaunchKernelGGL((chnorm::backward_kernel<T, VEC>), grid, block, 0, (hipStream_t)stream, (const T *)a,
+                               (const T *)x, stats, weight, (T *)out, partial, sh);
+        else
+            hipLaunchKernelGGL((chnorm::forward_kernel<T, VEC>), grid, block, 0, (hipStream_t)stream, (const T *)x,
+                               weight, bias, (T *)out, const_cast<float *>(stats), sh, eps);
+    }
+    static int chnorm(bool bwd, const void *a, const void *x, const float *stats, const float *weight,
+                      const float *bias, void *out, float *partial, long long B, int C, long long n, int esz,
+                      bool vec, float eps, void *stream)
+    {
+        if (B <= 0 || C <= 0 || n <= 0) return 0;
+        if (B * chnorm_blocks(n, esz, vec) > 0x7fffffffLL) return -2;
+        if (esz == 2) {
+            if (vec) chnorm_launch<bf16_t, true>(bwd, a, x, stats, weight, bias, out, partial, B, C, n, eps, stream);
+            else chnorm_launch<bf16_t, false>(bwd, a, x, stats, weight, bias, out, partial, B, C, n, eps, stream);
+        } else {
+            if (vec) chnorm_launch<float, true>(bwd, a, x, stats, weight, bias, out, partial, B, C, n, eps, stream);
+            else chnorm_launch<float, false>(bwd, a, x, stats, weight, bias, out, partial, B, C, n, eps, stream);
+        }
         return check();
     }
 

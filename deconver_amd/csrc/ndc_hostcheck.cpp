@@ -157,6 +157,78 @@ struct Backend {
         return 0;
     }
 
+    // normalisation over channels, sequentially, with the HIP build's partial-sum layout (one
+    // partial row per wavefront of 64 x (16 / esz or 1) voxels)
+    static constexpr int kChnormWaves = 4;
+    static long long chnorm_blocks(long long n, int esz, bool vec)
+    {
+        const long long per = vec ? 16 / esz : 1;
+        return (n / per + 255) / 256;
+    }
+    template <typename T>
+    static void chnorm_t(bool bwd, const T *a, const T *x, float *stats, const float *weight, const float *bias,
+                         T *out, float *partial, long long B, int C, long long n, bool vec, float eps)
+    {
+        const long long per = vec ? 16 / (long long)sizeof(T) : 1, blocks = chnorm_blocks(n, (int)sizeof(T), vec);
+        if (bwd && partial)
+            for (long long k = 0; k < B * blocks * kChnormWaves * C * 2; ++k) partial[k] = 0.f;
+        for (long long b = 0; b < B; ++b)
+            for (long long i = 0; i < n; ++i) {
+                const T *xb = x + b * C * n + i;
+                if (!bwd) {
+                    const float p = Elem<T>::load(xb);
+                    float s1 = 0.f, s2 = 0.f;
+                    for (int c = 0; c < C; ++c) {
+                        const float d = Elem<T>::load(xb + c * n) - p;
+                        s1 += d;
+                        s2 += d * d;
+                    }
+                    const float m = s1 / (float)C;
+                    float var = s2 / (float)C - m * m;
+                    var = var > 0.f ? var : 0.f;
+                    const float mean = p + m, rstd = 1.f / std::sqrt(var + eps);
+                    stats[(b * 2 + 0) * n + i] = mean;
+                    stats[(b * 2 + 1) * n + i] = rstd;
+                    for (int c = 0; c < C; ++c)
+                        Elem<T>::store(out + b * C * n + c * n + i,
+                                       (Elem<T>::load(xb + c * n) - mean) * rstd * (weight ? weight[c] : 1.f) +
+                                           (bias ? bias[c] : 0.f));
+                } else {
+                    const T *gb = a + b * C * n + i;
+                    const float mean = stats[(b * 2 + 0) * n + i], rstd = stats[(b * 2 + 1) * n + i];
+                    const long long wave = (b * blocks + i / per / 256) * kChnormWaves + (i / per % 256) / 64;
+                    float s1 = 0.f, s2 = 0.f;
+                    for (int c = 0; c < C; ++c) {
+                        const float g = Elem<T>::load(gb + c * n), w = weight ? weight[c] : 1.f;
+                        const float xh = (Elem<T>::load(xb + c * n) - mean) * rstd;
+                        s1 += g * w;
+                        s2 += g * w * xh;
+                        if (partial) {
+                            partial[(wave * C + c) * 2] += g * xh;
+                            partial[(wave * C + c) * 2 + 1] += g;
+                        }
+                    }
+                    for (int c = 0; c < C; ++c) {
+                        const float g = Elem<T>::load(gb + c * n), w = weight ? weight[c] : 1.f;
+                        const float xh = (Elem<T>::load(xb + c * n) - mean) * rstd;
+                        Elem<T>::store(out + b * C * n + c * n + i, rstd * (g * w - s1 / (float)C - xh * s2 / (float)C));
+                    }
+                }
+            }
+    }
+    static int chnorm(bool bwd, const void *a, const void *x, const float *stats, const float *weight,
+                      const float *bias, void *out, float *partial, long long B, int C, long long n, int esz,
+                      bool vec, float eps, void *)
+    {
+        if (esz == 2)
+            chnorm_t<bf16_t>(bwd, (const bf16_t *)a, (const bf16_t *)x, const_cast<float *>(stats), weight, bias,
+                             (bf16_t *)out, partial, B, C, n, vec, eps);
+        else
+            chnorm_t<float>(bwd, (const float *)a, (const float *)x, const_cast<float *>(stats), weight, bias,
+                            (float *)out, partial, B, C, n, vec, eps);
+        return 0;
+    }
+
     static int row_sums(const void *a, float *partial, long long rows, long long n, int nsplit, long long chunk,
                         int esz, bool, void *)
     {

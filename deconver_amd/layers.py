@@ -415,44 +415,56 @@ class MLP(nn.Module):
         return y if residual is None else residual + y
 
 
-class _Transpose(torch.autograd.Function):
-    """``(B, R, K) -> (B, K, R)`` contiguous, by the library's tiled transposition
-    (``ndc_relayout``); the gradient is the transposition back."""
+class _ChannelNorm(torch.autograd.Function):
+    """``nn.LayerNorm`` over the channel axis of a channel-first ``(B, C, n)`` tensor on the HIP
+    kernels (``ndc_chnorm_forward`` / ``_backward``): lanes along the voxels, a loop over the
+    channels, nothing transposed."""
 
     @staticmethod
-    def forward(ctx, x):
+    def forward(ctx, x, weight, bias, eps):
+        lib = _lib.get_library()
         x = x.contiguous()
-        B, R, K = x.shape
-        out = x.new_empty(B, K, R)
+        w32 = None if weight is None else weight.detach().float().contiguous()
+        b32 = None if bias is None else bias.detach().float().contiguous()
         with torch.cuda.device(x.device):
-            # as a (B, C = R, S = K) channel-first tensor going channels-last
-            _lib.get_library().relayout(x.data_ptr(), out.data_ptr(), B, R, K, ops.dtype_tag(x.dtype), True,
-                                        torch.cuda.current_stream(x.device).cuda_stream)
-        return out
+            y, stats = ops.chnorm_forward(lib, x, w32, b32, eps)
+        ctx.save_for_backward(x, stats, w32)
+        ctx.dtypes = (None if weight is None else weight.dtype, None if bias is None else bias.dtype)
+        return y
 
     @staticmethod
     @torch.autograd.function.once_differentiable
-    def backward(ctx, g):
-        return _Transpose.apply(g)
+    def backward(ctx, gy):
+        x, stats, w32 = ctx.saved_tensors
+        gy = gy.to(x.dtype).contiguous()
+        affine = any(ctx.needs_input_grad[1:3])
+        with torch.cuda.device(x.device):
+            gx, gw, gb = ops.chnorm_backward(_lib.get_library(), gy, x, stats, w32, need_affine_grads=affine)
+        wd, bd = ctx.dtypes
+        return (gx if ctx.needs_input_grad[0] else None,
+                gw.to(wd) if affine and ctx.needs_input_grad[1] and wd is not None else None,
+                gb.to(bd) if affine and ctx.needs_input_grad[2] and bd is not None else None, None)
 
 
 class LayerNorm(nn.Module):
     """``nn.LayerNorm`` over the channel axis of a ``(B, C, *S)`` tensor (layers/norm.py:25-34).
 
-    The reference moves the channel axis last, normalises and moves it back, which leaves the
-    two layout changes to generic strided copies (the norm's own and the next projection's
-    ``contiguous()``).  On the GPU (float32 / bfloat16) the two copies here are the library's
-    tiled transposition, 4 TB/s against 0.2-1 TB/s, around the same ``nn.LayerNorm``; the
-    arithmetic, the parameters and (under autocast) the float32 result are the reference's."""
+    The reference moves the channel axis last, normalises and moves it back, which costs two
+    generic strided copies (the norm's own and the next projection's ``contiguous()``).  On the
+    GPU (float32 / bfloat16 tensors) the HIP kernels normalise over the channel axis where it
+    is; parameters and state dict are ``nn.LayerNorm``'s, and under autocast the arithmetic and
+    the result are float32, as PyTorch's autocast rules make them for the reference."""
 
     def __init__(self, dim: int, **kwargs):
         super().__init__()
         self.norm = nn.LayerNorm(dim, **kwargs)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        if x.is_cuda and x.dim() >= 3 and x.dtype in (torch.float32, torch.bfloat16) and x.numel() > 0:
-            y = self.norm(_Transpose.apply(x.flatten(2)))        # (B, N, C), normalised over C
-            if y.dtype in (torch.float32, torch.bfloat16):
-                return _Transpose.apply(y).view(x.shape[0], -1, *x.shape[2:])
-            return y.movedim(-1, 1).reshape(x.shape[0], -1, *x.shape[2:])
+        if (x.is_cuda and x.dim() >= 3 and x.numel() > 0 and len(self.norm.normalized_shape) == 1
+                and x.shape[1] == self.norm.normalized_shape[0]):
+            t = x.float() if torch.is_autocast_enabled(x.device.type) else x
+            if t.dtype in (torch.float32, torch.bfloat16):
+                with torch.autocast(x.device.type, enabled=False):
+                    y = _ChannelNorm.apply(t.flatten(2), self.norm.weight, self.norm.bias, float(self.norm.eps))
+                return y.view(x.shape)
         return self.norm(x.movedim(1, -1)).movedim(-1, 1)

@@ -326,3 +326,43 @@ def channel_sums(lib: _lib.NdcLibrary, g: Tensor) -> Tensor:
     partial = torch.empty(B, C, parts, dtype=torch.float32, device=g.device)
     lib.row_sums(_ptr(g), _ptr(partial), B * C, n, dtype_tag(g.dtype), _stream_of(g))
     return partial.sum((0, 2))
+
+
+def chnorm_forward(lib: _lib.NdcLibrary, x: Tensor, weight: Optional[Tensor], bias: Optional[Tensor],
+                   eps: float):
+    """Normalises a contiguous channel-first ``(B, C, n)`` tensor over its channel axis (per
+    voxel), with float32 ``weight`` / ``bias`` of C entries or None.  Returns ``(y, stats)``;
+    ``stats`` (B, 2, n) holds mean and rstd per voxel."""
+    if x.dim() != 3 or not x.is_contiguous():
+        raise ValueError("chnorm_forward wants a contiguous (B, C, n) tensor")
+    for p in (weight, bias):
+        if p is not None and (p.dtype != torch.float32 or p.numel() != x.shape[1] or not p.is_contiguous()):
+            raise ValueError("weight and bias must be float32 with one entry per channel")
+    B, C, n = x.shape
+    y = torch.empty_like(x)
+    stats = torch.empty(B, 2, n, dtype=torch.float32, device=x.device)
+    lib.chnorm_forward(_ptr(x), _ptr(weight), _ptr(bias), _ptr(y), _ptr(stats), B, C, n, dtype_tag(x.dtype), eps,
+                       _stream_of(x))
+    return y, stats
+
+
+def chnorm_backward(lib: _lib.NdcLibrary, gy: Tensor, x: Tensor, stats: Tensor, weight: Optional[Tensor],
+                    need_affine_grads: bool = True):
+    """``(gx, gweight, gbias)`` of :func:`chnorm_forward`; the last two float32, or None."""
+    if gy.shape != x.shape or gy.dtype != x.dtype or not (gy.is_contiguous() and x.is_contiguous()):
+        raise ValueError("chnorm_backward wants gy and x contiguous, of one shape and dtype")
+    B, C, n = x.shape
+    gx = torch.empty_like(x)
+    partial = None
+    if need_affine_grads:
+        parts = lib.chnorm_parts(B, n, dtype_tag(x.dtype))
+        aligned = all(t.data_ptr() % 16 == 0 for t in (gy, x, gx))
+        if not aligned and n % (16 // x.element_size()) == 0:
+            raise ValueError("chnorm_backward wants 16-byte aligned tensors")
+        partial = torch.empty(parts, C, 2, dtype=torch.float32, device=x.device)
+    lib.chnorm_backward(_ptr(gy), _ptr(x), _ptr(stats), _ptr(weight), _ptr(gx), _ptr(partial), B, C, n,
+                        dtype_tag(x.dtype), _stream_of(x))
+    if partial is None:
+        return gx, None, None
+    sums = partial.sum(0)
+    return gx, sums[:, 0].contiguous(), sums[:, 1].contiguous()

@@ -314,6 +314,28 @@ int ndc_bias_act_backward(const void *gy, const void *z, const float *bias, void
                           int64_t batch, int64_t channels, int64_t n, int act, int dtype, void *stream);
 
 /*
+ * Normalisation over the CHANNEL axis of a channel-first tensor (batch, channels, n):
+ *   y[b][c][i] = (x[b][c][i] - mean[b][i]) * rstd[b][i] * weight[c] + bias[c],
+ * mean and biased variance over c.  The reference's LayerNorm (deconver/layers/norm.py:25-34:
+ * nn.LayerNorm with the channel axis moved last and back), the default norm of its blocks and
+ * stem (deconver/deconver.py:52, 103), on the layout the tensors already have: nothing is
+ * transposed.
+ *   weight, bias   `channels` floats each, or NULL (1 and 0)
+ *   stats          batch * 2 * n floats: mean then rstd per voxel; written by the forward, read
+ *                  by the backward
+ *   partial        NULL, or ndc_chnorm_parts(batch, n, dtype) * channels * 2 floats: per part
+ *                  and channel (sum of gy * xhat, sum of gy); the gradients of weight and bias
+ *                  are the sums over the parts
+ *   x, y / gy, gx  distinct buffers; gx may be gy.  16-byte aligned buffers take 16-byte
+ *                  accesses when n is a multiple of 16 bytes of elements.
+ */
+int64_t ndc_chnorm_parts(int64_t batch, int64_t n, int dtype);
+int ndc_chnorm_forward(const void *x, const float *weight, const float *bias, void *y, float *stats,
+                       int64_t batch, int64_t channels, int64_t n, int dtype, float eps, void *stream);
+int ndc_chnorm_backward(const void *gy, const void *x, const float *stats, const float *weight, void *gx,
+                        float *partial, int64_t batch, int64_t channels, int64_t n, int dtype, void *stream);
+
+/*
  * Regrouping of a grid by 2 x 2 (depth2 = 0) or 2 x 2 x 2 (depth2 = 1) windows: the data
  * movement of the reference's 2-tap, stride-2 resampling convolutions (nn.ConvNd(kernel_size=2,
  * stride=2), nn.ConvTransposeNd(kernel_size=2, stride=2), deconver/unet.py:36-60, 108-131) once

@@ -87,6 +87,14 @@ static int run_block_level(int dtype)
     if (!st) st = ndc_bias_act_backward(g, x, bias, gx, gpart, B, C, n, NDC_ACT_GELU, dtype, nullptr);
     if (!st) st = ndc_row_sums(g, gpart, rows, n, dtype, nullptr);
     if (!st) st = ndc_relayout(x, y, B, C, n, dtype, 1, nullptr);
+    {
+        float *cstats = (float *)malloc(sizeof(float) * 2 * B * n);
+        const long long cparts = ndc_chnorm_parts(B, n, dtype);
+        float *cpart = (float *)malloc(sizeof(float) * cparts * C * 2);
+        if (!st) st = ndc_chnorm_forward(x, bias, bias, y, cstats, B, C, n, dtype, 1e-5f, nullptr);
+        if (!st) st = ndc_chnorm_backward(g, x, cstats, bias, gx, cpart, B, C, n, dtype, nullptr);
+        free(cstats); free(cpart);
+    }
     free(gpart); free(ws); free(stats); free(x); free(y); free(g); free(gx);
     // 2 x 2 x 2 windows of a (rows, 4, 6, 16) grid and back
     const long long D = 4, H = 6, W = 16, m = rows * D * H * W;
