@@ -5,7 +5,7 @@
 // layout the tensors already have: lanes run along the voxels (16 bytes each), a loop runs over
 // the channels, so every access is a contiguous run and nothing is transposed.
 //
-//   forward : loop 1 sums x - p and (x - p)^2 per voxel (p = the voxel's first-channel value);
+//   forward : loop 1 keeps a running mean and sum of squared deviations per voxel (Welford);
 //             loop 2 reads x again and writes y.  stats[b][0][i] = mean, stats[b][1][i] = rstd.
 //   backward: loop 1 sums g w and g w xhat per voxel and, per channel, g xhat and g over the
 //             wavefront's voxels (partial[wave][c] = (sum g xhat, sum g): the affine gradients
@@ -71,29 +71,27 @@ forward_kernel(const T *x, const float *weight, const float *bias, T *y, float *
     if (i >= s.n) return;
     const T *xb = x + b * s.channels * s.n + i;
     T *yb = y + b * s.channels * s.n + i;
-    L p, t;
-    p.load(xb);
-    float s1[L::N], s2[L::N];
+    L t;
+    // running mean and squared deviations per voxel (Welford): no cancellation whatever the
+    // offset of the values
+    float mean[L::N], m2[L::N];
 #pragma unroll
-    for (int e = 0; e < L::N; ++e) s1[e] = s2[e] = 0.f;
+    for (int e = 0; e < L::N; ++e) mean[e] = m2[e] = 0.f;
     for (int c = 0; c < s.channels; ++c) {
         t.load(xb + c * s.n);
+        const float rk = 1.f / (float)(c + 1);
 #pragma unroll
         for (int e = 0; e < L::N; ++e) {
-            const float d = t.v[e] - p.v[e];
-            s1[e] += d;
-            s2[e] += d * d;
+            const float d = t.v[e] - mean[e];
+            mean[e] += d * rk;
+            m2[e] += d * (t.v[e] - mean[e]);
         }
     }
     const float inv_c = 1.f / (float)s.channels;
-    float mean[L::N], rstd[L::N];
+    float rstd[L::N];
 #pragma unroll
     for (int e = 0; e < L::N; ++e) {
-        const float m = s1[e] * inv_c;
-        float var = s2[e] * inv_c - m * m;
-        var = var > 0.f ? var : 0.f;
-        mean[e] = p.v[e] + m;
-        rstd[e] = 1.f / sqrtf(var + eps);
+        rstd[e] = 1.f / sqrtf(m2[e] * inv_c + eps);
         stats[(b * 2 + 0) * s.n + i + e] = mean[e];
         stats[(b * 2 + 1) * s.n + i + e] = rstd[e];
     }

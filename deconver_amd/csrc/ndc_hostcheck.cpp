@@ -176,17 +176,13 @@ struct Backend {
             for (long long i = 0; i < n; ++i) {
                 const T *xb = x + b * C * n + i;
                 if (!bwd) {
-                    const float p = Elem<T>::load(xb);
-                    float s1 = 0.f, s2 = 0.f;
+                    float mean = 0.f, m2 = 0.f;
                     for (int c = 0; c < C; ++c) {
-                        const float d = Elem<T>::load(xb + c * n) - p;
-                        s1 += d;
-                        s2 += d * d;
+                        const float v = Elem<T>::load(xb + c * n), d = v - mean;
+                        mean += d * (1.f / (float)(c + 1));
+                        m2 += d * (v - mean);
                     }
-                    const float m = s1 / (float)C;
-                    float var = s2 / (float)C - m * m;
-                    var = var > 0.f ? var : 0.f;
-                    const float mean = p + m, rstd = 1.f / std::sqrt(var + eps);
+                    const float rstd = 1.f / std::sqrt(m2 / (float)C + eps);
                     stats[(b * 2 + 0) * n + i] = mean;
                     stats[(b * 2 + 1) * n + i] = rstd;
                     for (int c = 0; c < C; ++c)
