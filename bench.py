@@ -808,6 +808,21 @@ def block_rows(torch, steps: int, warmup: int) -> list:
         put("norm_forward_pytorch", timed(lambda: F.instance_norm(x3)), 3 * U)
         put("norm_backward_pytorch", timed(lambda: torch.autograd.grad(y3, x3, g3, retain_graph=True)), 5 * U)
         del x, g, y, x3, y3, g3
+        # LayerNorm over the channel axis (the blocks' default norm in the reference), HIP kernels
+        # next to the reference's moved-axis form on PyTorch's kernels
+        xc = torch.randn(B, C, n, device=dev).bfloat16()
+        gc = torch.randn(B, C, n, device=dev).bfloat16()
+        wln, bln = torch.rand(C, device=dev) + 0.5, torch.rand(C, device=dev)
+        yc, sc_ = ops.chnorm_forward(lib, xc, wln, bln, 1e-5)
+        put("layernorm_forward", timed(lambda: ops.chnorm_forward(lib, xc, wln, bln, 1e-5)), 3 * U)
+        put("layernorm_backward", timed(lambda: ops.chnorm_backward(lib, gc, xc, sc_, wln)), 5 * U)
+        xr = xc.clone().requires_grad_(True)
+        w16, b16_ = wln.bfloat16(), bln.bfloat16()
+        put("layernorm_forward_pytorch",
+            timed(lambda: F.layer_norm(xr.movedim(1, -1), (C,), w16, b16_, 1e-5).movedim(-1, 1).contiguous()), 3 * U)
+        yr = F.layer_norm(xr.movedim(1, -1), (C,), w16, b16_, 1e-5).movedim(-1, 1)
+        put("layernorm_backward_pytorch", timed(lambda: torch.autograd.grad(yr, xr, gc, retain_graph=True)), 5 * U)
+        del xc, gc, yc, sc_, xr, yr
         z = torch.randn(B, 4 * C, n, device=dev).bfloat16()
         gz = torch.randn(B, 4 * C, n, device=dev).bfloat16()
         bias = torch.randn(4 * C, device=dev)

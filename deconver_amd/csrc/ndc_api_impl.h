@@ -525,14 +525,20 @@ static int chnorm_check(long long B, long long C, long long n, int dtype)
     return NDC_OK;
 }
 
+// 16-byte accesses (8 or 4 voxels per thread) where that still leaves a few hundred workgroups;
+// on small grids one voxel per thread, so that the launch spreads over the chip
+static bool chnorm_wide(long long batch, long long n, int esz)
+{
+    return n % (16 / esz) == 0 && batch * ndc::Backend::chnorm_blocks(n, esz, true) >= 256;
+}
+
 int64_t ndc_chnorm_parts(int64_t batch, int64_t n, int dtype)
 {
     if (batch < 1 || n < 1 || (dtype != NDC_F32 && dtype != NDC_BF16)) return 0;
     const int esz = dtype == NDC_BF16 ? 2 : 4;
-    // (the count for the vector path if n allows it, which is what the entry points then use
-    // when the buffers are aligned; an unaligned call needs more rows and is refused)
-    const bool vec = n % (16 / esz) == 0;
-    return batch * ndc::Backend::chnorm_blocks(n, esz, vec) * ndc::Backend::kChnormWaves;
+    // (the count for the access width the entry points use when the buffers are aligned; an
+    // unaligned call where the wide form applies needs more rows and is refused)
+    return batch * ndc::Backend::chnorm_blocks(n, esz, chnorm_wide(batch, n, esz)) * ndc::Backend::kChnormWaves;
 }
 
 int ndc_chnorm_forward(const void *x, const float *weight, const float *bias, void *y, float *stats,
@@ -543,7 +549,7 @@ int ndc_chnorm_forward(const void *x, const float *weight, const float *bias, vo
     if (st) return st;
     if (x == (const void *)y || !(eps >= 0.f)) return NDC_ERR_GEOMETRY;
     const int esz = dtype == NDC_BF16 ? 2 : 4;
-    const bool vec = n % (16 / esz) == 0 && aligned16(x) && aligned16(y);
+    const bool vec = chnorm_wide(batch, n, esz) && aligned16(x) && aligned16(y);
     st = ndc::Backend::chnorm(false, nullptr, x, stats, weight, bias, y, nullptr, batch, (int)channels, n, esz, vec,
                               eps, stream);
     return st == -2 ? (int)NDC_ERR_GEOMETRY : st;
@@ -557,7 +563,7 @@ int ndc_chnorm_backward(const void *gy, const void *x, const float *stats, const
     if (st) return st;
     if (gx == x) return NDC_ERR_GEOMETRY;
     const int esz = dtype == NDC_BF16 ? 2 : 4;
-    const bool fits = n % (16 / esz) == 0;
+    const bool fits = chnorm_wide(batch, n, esz);
     const bool vec = fits && aligned16(gy) && aligned16(x) && aligned16(gx);
     // the partial rows are laid out for the path ndc_chnorm_parts counted
     if (partial && fits && !vec) return NDC_ERR_WORKSPACE;

@@ -356,9 +356,6 @@ def chnorm_backward(lib: _lib.NdcLibrary, gy: Tensor, x: Tensor, stats: Tensor, 
     partial = None
     if need_affine_grads:
         parts = lib.chnorm_parts(B, n, dtype_tag(x.dtype))
-        aligned = all(t.data_ptr() % 16 == 0 for t in (gy, x, gx))
-        if not aligned and n % (16 // x.element_size()) == 0:
-            raise ValueError("chnorm_backward wants 16-byte aligned tensors")
         partial = torch.empty(parts, C, 2, dtype=torch.float32, device=x.device)
     lib.chnorm_backward(_ptr(gy), _ptr(x), _ptr(stats), _ptr(weight), _ptr(gx), _ptr(partial), B, C, n,
                         dtype_tag(x.dtype), _stream_of(x))

@@ -75,7 +75,8 @@ def test_one_channel_and_bad_arguments():
     b = torch.tensor([0.25])
     y, stats = ops.chnorm_forward(lib, x, torch.ones(1), b, 1e-5)
     assert torch.allclose(y, torch.full_like(y, 0.25)) and torch.allclose(stats[:, 0], x[:, 0])
-    assert lib.chnorm_parts(2, 128 ** 3, _lib.NDC_BF16) == 2 * (128 ** 3 // 8 // 256) * 4
+    assert lib.chnorm_parts(2, 128 ** 3, _lib.NDC_BF16) == 2 * (128 ** 3 // 8 // 256) * 4   # 16-byte accesses
+    assert lib.chnorm_parts(2, 4096, _lib.NDC_BF16) == 2 * (4096 // 256) * 4                # a small grid: one voxel per thread
     assert lib.chnorm_parts(1, 7, _lib.NDC_F32) == 4
     with pytest.raises(_lib.NdcError):   # in place
         lib.chnorm_forward(x.data_ptr(), None, None, x.data_ptr(), stats.data_ptr(), 3, 1, 16, _lib.NDC_F32, 1e-5, None)
@@ -97,7 +98,8 @@ def test_module_is_the_reference_form_off_the_gpu():
     assert set(ln.state_dict()) == {"norm.weight", "norm.bias"}
 
 
-GPU_SHAPES = [(2, 8, 6, 10), (2, 64, 8, 12, 16), (1, 5, 7, 9), (2, 32, 64, 64), (1, 130, 4, 6, 8)]
+GPU_SHAPES = [(2, 8, 6, 10), (2, 64, 8, 12, 16), (1, 5, 7, 9), (2, 32, 64, 64), (1, 130, 4, 6, 8),
+              (2, 16, 64, 64, 64)]   # the last one large enough for 16-byte accesses
 
 
 @pytest.mark.gpu
@@ -111,7 +113,7 @@ def test_hip_kernels_match_layer_norm(shape, dtype, affine):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("regime", ["float32", "bfloat16", "bf16 autocast"])
-@pytest.mark.parametrize("shape", [(2, 8, 6, 10), (2, 64, 8, 12, 16), (1, 5, 7, 9)])
+@pytest.mark.parametrize("shape", [(2, 8, 6, 10), (2, 64, 16, 24, 48), (1, 5, 7, 9), (2, 16, 64, 64, 64)])
 def test_module_matches_the_reference_form_on_the_gpu(regime, shape):
     """``dc.LayerNorm`` on the GPU against the reference's movedim form around the same
     ``nn.LayerNorm`` (PyTorch's kernels): values, input gradient and parameter gradients; under
@@ -131,7 +133,9 @@ def test_module_matches_the_reference_form_on_the_gpu(regime, shape):
     with ctx():
         y = ln(x)
         ref = ln.norm(x.movedim(1, -1)).movedim(-1, 1)
-    assert y.shape == x.shape and y.dtype == ref.dtype and y.is_contiguous()
+    assert y.shape == x.shape and y.dtype == ref.dtype
+    on_kernels = shape[0] * int(torch.tensor(shape[2:]).prod()) >= 32768   # smaller grids keep the reference form
+    assert y.is_contiguous() == on_kernels
     params = (x, ln.norm.weight, ln.norm.bias)
     got = torch.autograd.grad(y, params, g.to(y.dtype))
     want = torch.autograd.grad(ref, params, g.to(y.dtype))
@@ -148,7 +152,7 @@ def test_default_norm_block_on_the_gpu_matches_its_float64_general_route():
     torch.manual_seed(6)
     blk = dc.DeconverBlock(16, kernel_size=(3, 3, 3), ratio=4)
     assert isinstance(blk.norm1, dc.LayerNorm)
-    x = torch.rand(2, 16, 12, 12, 16)
+    x = torch.rand(2, 16, 24, 32, 32)      # enough voxels for the module to take the kernels
     ref = blk.double()(x.double())
     blk = blk.float().cuda()
     with torch.autocast("cuda", dtype=torch.bfloat16):
