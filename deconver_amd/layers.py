@@ -336,6 +336,10 @@ class _UnfoldConvMixin:
         return super().forward(x)
 
 
+class UnfoldConv1d(_UnfoldConvMixin, nn.Conv1d):
+    pass
+
+
 class UnfoldConv2d(_UnfoldConvMixin, nn.Conv2d):
     pass
 
@@ -344,11 +348,19 @@ class UnfoldConv3d(_UnfoldConvMixin, nn.Conv3d):
     pass
 
 
+class PatchConv1d(_PatchConvMixin, nn.Conv1d):
+    pass
+
+
 class PatchConv2d(_PatchConvMixin, nn.Conv2d):
     pass
 
 
 class PatchConv3d(_PatchConvMixin, nn.Conv3d):
+    pass
+
+
+class PatchConvTranspose1d(_PatchConvTransposeMixin, nn.ConvTranspose1d):
     pass
 
 

@@ -120,6 +120,25 @@ def test_hip_regroup_is_the_strided_regrouping(shape, dtype):
     assert torch.equal(ops.channels_to_windows(lib, cols, bias), want)
 
 
+def test_one_dimensional_network_builds_and_runs():
+    """spatial_dims = 1: the same subclasses exist for 1-D convolutions (the regrouping is then
+    the strided view; the kernel takes 2-D and 3-D grids)."""
+    torch.manual_seed(4)
+    net = dc.Deconver(in_channels=1, out_channels=2, spatial_dims=1, encoder_depth=(1, 1), encoder_width=(4, 8),
+                      strides=(1, 2), decoder_depth=(1,), kernel_size=(3,), ratio=2)
+    assert isinstance(net.stem, layers.UnfoldConv1d) and isinstance(net.head, layers.PatchConv1d)
+    assert isinstance(net.encoder.blocks[1].downsample, layers.PatchConv1d)
+    assert isinstance(net.decoder.blocks[0].upsample, layers.PatchConvTranspose1d)
+    x = torch.rand(2, 1, 16)
+    y = net(x)
+    assert y.shape == (2, 2, 16)
+    y.sum().backward()
+    k = (2,)
+    w = torch.randn(5, 3, 2, dtype=torch.float64)
+    xx = torch.randn(2, 3, 10, dtype=torch.float64)
+    torch.testing.assert_close(layers.patch_conv(xx, w, None), F.conv1d(xx, w, None, stride=k), rtol=1e-12, atol=1e-12)
+
+
 def test_regrouping_round_trip():
     x = torch.arange(2 * 3 * 4 * 6 * 8, dtype=torch.float32).view(2, 3, 4, 6, 8)
     cols = layers.patches_to_channels(x, (2, 2, 2))
@@ -269,3 +288,18 @@ def test_patchifying_stem_on_the_gpu(regime):
         assert a.shape == r.shape
         assert float((a.detach().double() - r.detach()).abs().max() / r.detach().abs().max()) <= tol
     assert stem(x).shape == (2, 16, 8, 10)
+
+
+@pytest.mark.gpu
+def test_one_dimensional_network_on_the_gpu_matches_float64():
+    """A 1-D network in float32 on the GPU (1-D resampling convolutions regrouped by the strided
+    view, InstanceNorm1d and projection tails on the kernels, NDC layers on the direct kernels)
+    against the same network in float64 on the CPU."""
+    import copy
+    torch.manual_seed(5)
+    net = dc.Deconver(in_channels=2, out_channels=1, spatial_dims=1, encoder_depth=(1, 1), encoder_width=(8, 16),
+                      strides=(1, 2), decoder_depth=(1,), kernel_size=(5,), ratio=4, norm=nn.InstanceNorm1d)
+    x = torch.rand(2, 2, 4096)
+    ref = copy.deepcopy(net).double()(x.double())
+    y = net.cuda()(x.cuda())
+    assert float((y.cpu().double() - ref).abs().max() / ref.abs().max()) <= 1e-4
