@@ -20,7 +20,8 @@ from torch import Tensor
 
 from . import _lib, ops
 
-__all__ = ["deconv_update", "hip_kernels_apply", "DeconvUpdate", "save_ratio", "matrix_kernels"]
+__all__ = ["deconv_update", "projected_update", "hip_kernels_apply", "DeconvUpdate", "ProjectedUpdate",
+           "save_ratio", "matrix_kernels"]
 
 _SAVE_RATIO = os.environ.get("DECONVER_NDC_SAVE_RATIO", "1") != "0"
 
@@ -71,81 +72,136 @@ def hip_kernels_apply(x: Tensor, m: int, sc: int, kernel_size, dtype=None) -> bo
     return lib.check_geometry(g) == 0
 
 
+def _node_forward(ctx, needs, x, z, h, bias, groups, m, sc, eps, relu_input, taps):
+    """Forward of an update node: runs the kernels, records on ``ctx`` what backward needs
+    besides tensors and returns ``(out, tensors to save)``.  ``needs``: whether a gradient is
+    wanted for ``(x, z, h, bias)``."""
+    if not x.is_cuda:
+        raise RuntimeError("deconv_update runs on the GPU only (HIP kernels); "
+                           "CPU tensors take the layer's general PyTorch path")
+    lib = _lib.get_library()
+    # channels-last tensors (torch.channels_last / channels_last_3d) come in through the
+    # library's tiled transposition, and the results go back out the same way, in the
+    # layout of the tensor they belong to
+    ctx.cl = (ops.is_channels_last(x), ops.is_channels_last(z))
+    with torch.cuda.device(x.device):
+        x = ops.to_channel_first(lib, x)
+        z = ops.to_channel_first(lib, z)
+    hc = h.contiguous()
+    need_t1 = any(needs)
+    keep = need_t1 and _SAVE_RATIO
+    # The kernel family is read once, here, and named in both calls of this node: backward
+    # runs on an autograd thread, possibly after the process default has changed.
+    path = _lib.PATH_AUTO
+    if lib.fused_supported(ops.make_geom_for(x, hc, groups, m, sc, eps, relu_input)):
+        path = _lib.PATH_FUSED_MATRIX if lib.matrix_kernels() else _lib.PATH_FUSED_VECTOR
+    if keep:
+        # only where the backward kernels for this geometry read them
+        keep = lib.backward_uses_saved(
+            ops.make_geom_for(x, hc, groups, m, sc, eps, relu_input, path))
+    with torch.cuda.device(x.device):
+        if taps is None:
+            # packed once here, used by the forward kernel and again by the backward's
+            taps = ops.prepare_taps(lib, x, hc, groups=groups, m=m, sc=sc)
+        res = ops.update_forward(lib, x, z, hc, bias, groups=groups, m=m, sc=sc, eps=eps,
+                                 relu_input=relu_input, need_t1=need_t1, save_ratio=keep,
+                                 taps=taps, path=path)
+    out, t1 = res[0], res[1]
+    s_over_den, ratio = res[2] if keep else (None, None)
+    ctx.cfg = (groups, m, sc, eps, relu_input)
+    ctx.path = path
+    ctx.taps = taps if need_t1 else None   # a function of h alone; h is saved
+    if ctx.cl[1]:
+        with torch.cuda.device(x.device):
+            out = ops.to_channels_last(lib, out)
+    return out, (x, z, t1, hc, bias, s_over_den, ratio)
+
+
+def _node_backward(ctx, saved, gout, need_x, need_z, need_h, need_b):
+    """``(gx, gz, gh, gb)`` of an update node from the tensors its forward saved."""
+    # The gradients come from kernels autograd cannot see through, so a second
+    # differentiation would silently drop terms: refuse it, as the reference does.
+    if torch.is_grad_enabled():
+        raise RuntimeError(
+            "double backward through the fused Deconv update is not supported; "
+            "construct the layer with a convolution keyword argument (e.g. stride=1) "
+            "to force the general path, which is plain PyTorch and doubly differentiable")
+    x, z, t1, h, bias, s_over_den, ratio = saved
+    groups, m, sc, eps, relu_input = ctx.cfg
+    if t1 is None:
+        raise RuntimeError("backward called on an update that was run without gradients")
+    lib = _lib.get_library()
+    if gout.dtype != z.dtype:
+        gout = gout.to(z.dtype)
+    with torch.cuda.device(x.device):
+        gout = ops.to_channel_first(lib, gout)
+        gx, gz, gh, gb = ops.update_backward(
+            lib, x, z, t1, h, bias, gout, groups=groups, m=m, sc=sc, eps=eps,
+            relu_input=relu_input, need_x=need_x, need_z=need_z, need_h=need_h,
+            need_b=need_b and bias is not None, path=ctx.path,
+            saved=None if s_over_den is None else (s_over_den, ratio), taps=ctx.taps)
+        if ctx.cl[0] and gx is not None:
+            gx = ops.to_channels_last(lib, gx)
+        if ctx.cl[1] and gz is not None:
+            gz = ops.to_channels_last(lib, gz)
+    return gx, gz, gh, gb
+
+
 class DeconvUpdate(torch.autograd.Function):
     """``out = relu(z + b) * (A(x) + eps) / (A(K(relu(z + b))) + eps)``."""
 
     @staticmethod
     def forward(ctx, x, z, h, bias, groups, m, sc, eps, relu_input, taps=None):
-        if not x.is_cuda:
-            raise RuntimeError("deconv_update runs on the GPU only (HIP kernels); "
-                               "CPU tensors take the layer's general PyTorch path")
-        lib = _lib.get_library()
-        # channels-last tensors (torch.channels_last / channels_last_3d) come in through the
-        # library's tiled transposition, and the results go back out the same way, in the
-        # layout of the tensor they belong to
-        ctx.cl = (ops.is_channels_last(x), ops.is_channels_last(z))
-        with torch.cuda.device(x.device):
-            x = ops.to_channel_first(lib, x)
-            z = ops.to_channel_first(lib, z)
-        hc = h.contiguous()
-        need_t1 = any(ctx.needs_input_grad[:4])
-        keep = need_t1 and _SAVE_RATIO
-        # The kernel family is read once, here, and named in both calls of this node: backward
-        # runs on an autograd thread, possibly after the process default has changed.
-        path = _lib.PATH_AUTO
-        if lib.fused_supported(ops.make_geom_for(x, hc, groups, m, sc, eps, relu_input)):
-            path = _lib.PATH_FUSED_MATRIX if lib.matrix_kernels() else _lib.PATH_FUSED_VECTOR
-        if keep:
-            # only where the backward kernels for this geometry read them
-            keep = lib.backward_uses_saved(
-                ops.make_geom_for(x, hc, groups, m, sc, eps, relu_input, path))
-        with torch.cuda.device(x.device):
-            if taps is None:
-                # packed once here, used by the forward kernel and again by the backward's
-                taps = ops.prepare_taps(lib, x, hc, groups=groups, m=m, sc=sc)
-            res = ops.update_forward(lib, x, z, hc, bias, groups=groups, m=m, sc=sc, eps=eps,
-                                     relu_input=relu_input, need_t1=need_t1, save_ratio=keep,
-                                     taps=taps, path=path)
-        out, t1 = res[0], res[1]
-        s_over_den, ratio = res[2] if keep else (None, None)
-        ctx.cfg = (groups, m, sc, eps, relu_input)
-        ctx.path = path
-        ctx.taps = taps if need_t1 else None   # a function of h alone; h is saved below
-        ctx.save_for_backward(x, z, t1, hc, bias, s_over_den, ratio)
-        if ctx.cl[1]:
-            with torch.cuda.device(x.device):
-                out = ops.to_channels_last(lib, out)
+        out, saved = _node_forward(ctx, ctx.needs_input_grad[:4], x, z, h, bias, groups, m, sc,
+                                   eps, relu_input, taps)
+        ctx.save_for_backward(*saved)
         return out
 
     @staticmethod
     def backward(ctx, gout):
-        # The gradients come from kernels autograd cannot see through, so a second
-        # differentiation would silently drop terms: refuse it, as the reference does.
-        if torch.is_grad_enabled():
-            raise RuntimeError(
-                "double backward through the fused Deconv update is not supported; "
-                "construct the layer with a convolution keyword argument (e.g. stride=1) "
-                "to force the general path, which is plain PyTorch and doubly differentiable")
-        x, z, t1, h, bias, s_over_den, ratio = ctx.saved_tensors
-        groups, m, sc, eps, relu_input = ctx.cfg
-        need_x, need_z, need_h, need_b = ctx.needs_input_grad[:4]
-        if t1 is None:
-            raise RuntimeError("backward called on an update that was run without gradients")
-        lib = _lib.get_library()
-        if gout.dtype != z.dtype:
-            gout = gout.to(z.dtype)
-        with torch.cuda.device(x.device):
-            gout = ops.to_channel_first(lib, gout)
-            gx, gz, gh, gb = ops.update_backward(
-                lib, x, z, t1, h, bias, gout, groups=groups, m=m, sc=sc, eps=eps,
-                relu_input=relu_input, need_x=need_x, need_z=need_z, need_h=need_h,
-                need_b=need_b and bias is not None, path=ctx.path,
-                saved=None if s_over_den is None else (s_over_den, ratio), taps=ctx.taps)
-            if ctx.cl[0] and gx is not None:
-                gx = ops.to_channels_last(lib, gx)
-            if ctx.cl[1] and gz is not None:
-                gz = ops.to_channels_last(lib, gz)
+        gx, gz, gh, gb = _node_backward(ctx, ctx.saved_tensors, gout, *ctx.needs_input_grad[:4])
         return gx, gz, gh, gb, None, None, None, None, None, None
+
+
+class ProjectedUpdate(torch.autograd.Function):
+    """The layer's first update together with the 1x1 projection that makes its source
+    (deconv.py:157-165 with layers/linear.py:53-58 of the reference):
+    ``z = W x`` per sample, then ``DeconvUpdate`` on ``(x, z)`` with the projection's bias and
+    the ReLU applied where the kernels load ``z``.
+
+    One node instead of two because ``x`` feeds both the projection and the update: as two
+    nodes their input gradients are two tensors that autograd adds in a pass of its own;
+    here the projection's input-gradient GEMM accumulates onto the update's ``gx``
+    (``gx += W^T gz``, one rounding instead of two in bfloat16).  The GEMMs are the ones of
+    ``layers.pointwise_linear``: one batched launch over the samples on the channel-first
+    tensors, the weight gradient summed in float32."""
+
+    @staticmethod
+    def forward(ctx, x, weight, h, bias, groups, m, sc, eps, taps=None):
+        B = x.shape[0]
+        w = weight.detach().to(x.dtype)
+        z = x.new_empty(B, w.shape[0], *x.shape[2:])
+        torch.bmm(w.unsqueeze(0).expand(B, -1, -1), x.flatten(2), out=z.flatten(2))
+        need_x, need_w, need_h, need_b = ctx.needs_input_grad[:4]
+        out, saved = _node_forward(ctx, (need_x, need_x or need_w, need_h, need_b), x, z, h,
+                                   bias, groups, m, sc, eps, True, taps)
+        ctx.save_for_backward(*saved, w)
+        ctx.weight_dtype = weight.dtype
+        return out
+
+    @staticmethod
+    def backward(ctx, gout):
+        from .layers import projection_weight_grad
+        *saved, w = ctx.saved_tensors
+        need_x, need_w, need_h, need_b = ctx.needs_input_grad[:4]
+        gx, gz, gh, gb = _node_backward(ctx, saved, gout, need_x, need_x or need_w, need_h, need_b)
+        x = saved[0]
+        gw = None
+        if need_w:
+            gw = projection_weight_grad(gz.flatten(2), x.flatten(2), ctx.weight_dtype)
+        if need_x:
+            gx.flatten(2).baddbmm_(w.t().unsqueeze(0).expand(x.shape[0], -1, -1), gz.flatten(2))
+        return gx, gw, gh, gb, None, None, None, None, None
 
 
 def deconv_update(x: Tensor, z: Tensor, h: Tensor, bias: Optional[Tensor], *, groups: int,
@@ -164,3 +220,18 @@ def deconv_update(x: Tensor, z: Tensor, h: Tensor, bias: Optional[Tensor], *, gr
             ``h``, for callers that run several updates with one filter; made here otherwise.
     """
     return DeconvUpdate.apply(x, z, h, bias, groups, m, sc, eps, relu_input, taps)
+
+
+def projected_update(x: Tensor, weight: Tensor, h: Tensor, bias: Optional[Tensor], *, groups: int,
+                     m: int, sc: int, eps: float, taps: Optional[Tensor] = None) -> Tensor:
+    """``deconv_update(x, W x, h, bias, relu_input=True)`` as one autograd node (not in the
+    reference, which records the projection and the update separately).
+
+    Args:
+        x: input ``(B, C, *S)``, contiguous, float32 or bfloat16 on the GPU.
+        weight: the projection's weight ``(groups*sc, C)``, any floating dtype (cast to ``x``'s
+            for the GEMMs; its gradient comes back in its own dtype).
+        h, bias, groups, m, sc, eps, taps: as for ``deconv_update``.
+    """
+    with torch.autocast(x.device.type, enabled=False):
+        return ProjectedUpdate.apply(x, weight, h, bias, groups, m, sc, eps, taps)

@@ -32,6 +32,26 @@ def _wgrad_chunks(batch: int, n: int) -> int:
     return s
 
 
+def projection_weight_grad(gz: torch.Tensor, x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """``sum_b gz[b] x[b]^T`` for ``gz`` of shape ``(B, Cout, N)`` and ``x`` of shape
+    ``(B, Cin, N)``: the weight gradient of a 1x1 projection, a ``Cout x Cin`` result summed
+    over all voxels.  Short rows (the 2-D network's levels) take one batched GEMM and a sum over
+    the batch; long rows are cut into equal chunks of the voxel axis that become batch entries
+    (strided views, no copies).  The partial results are added in float32, in one reduction."""
+    B, cout, n = gz.shape
+    cin = x.shape[1]
+    s = _wgrad_chunks(B, n) if n >= _CHUNKED_WGRAD_FROM else 1
+    if s == 1:
+        parts = torch.bmm(gz, x.transpose(1, 2))
+    else:
+        parts = gz.new_empty(B * s, cout, cin)
+        for b in range(B):
+            a = gz[b].view(cout, s, n // s).transpose(0, 1)
+            c = x[b].view(cin, s, n // s).permute(1, 2, 0)
+            torch.bmm(a, c, out=parts[b * s:(b + 1) * s])
+    return parts.sum(0, dtype=torch.float32).to(dtype)
+
+
 class _PointwiseLinear(torch.autograd.Function):
     """``y[b] = act(W x[b] + bias) + residual[b]`` for ``x`` of shape ``(B, Cin, N)``: the 1x1
     projection as plain GEMMs on the channel-first layout (hipBLASLt through ``torch.bmm``),
@@ -96,22 +116,7 @@ class _PointwiseLinear(torch.autograd.Function):
             gx = torch.empty_like(x)
             torch.bmm(weight.t().unsqueeze(0).expand(x.shape[0], -1, -1), gz, out=gx)
         if ctx.needs_input_grad[1]:
-            B, cout, n = gz.shape
-            cin = x.shape[1]
-            # short rows (the 2-D network's levels): one batched GEMM and a sum over the batch
-            # (two launches); long rows: chunks of the voxel axis as batch entries
-            s = _wgrad_chunks(B, n) if n >= _CHUNKED_WGRAD_FROM else 1
-            if s == 1:
-                parts = torch.bmm(gz, x.transpose(1, 2))
-            else:
-                parts = gz.new_empty(B * s, cout, cin)
-                for b in range(B):
-                    # chunk c of the voxel axis as batch entry c: strided views, no copies
-                    a = gz[b].view(cout, s, n // s).transpose(0, 1)
-                    c = x[b].view(cin, s, n // s).permute(1, 2, 0)
-                    torch.bmm(a, c, out=parts[b * s:(b + 1) * s])
-            # the partial results are added in float32, in one reduction
-            gw = parts.sum(0, dtype=torch.float32).to(ctx.weight_dtype)
+            gw = projection_weight_grad(gz, x, ctx.weight_dtype)
         return gx, gw, gb, None, gres
 
 

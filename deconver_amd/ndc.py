@@ -12,8 +12,9 @@ Execution
 ``forward`` asks ``fast_path_applicable(x)`` and then runs one of two routes:
 
 HIP route
-    One ``functional.deconv_update`` autograd node per iteration, on
-    ``libdeconver_ndc.so``.  Taken for GPU tensors in float32 or bfloat16 (bfloat16 also
+    One autograd node per iteration, on ``libdeconver_ndc.so``
+    (``functional.projected_update``, which holds the projection too, then
+    ``functional.deconv_update``).  Taken for GPU tensors in float32 or bfloat16 (bfloat16 also
     under autocast, which the reference declines at deconv.py:139-147) when the layer is in
     its default regime: source updates only, odd kernel, no extra convolution arguments, no
     overridden update methods.  The projection runs as a bias-free 1x1 GEMM; its bias and
@@ -37,8 +38,8 @@ from torch import Tensor, nn
 from . import operations as ops_general
 from . import ops
 from ._lib import get_library
-from .functional import deconv_update, hip_kernels_apply
-from .layers import Linear, pointwise_linear
+from .functional import deconv_update, hip_kernels_apply, projected_update
+from .layers import Linear
 
 __all__ = ["Initializer", "Deconv", "NDC"]
 
@@ -183,20 +184,25 @@ class Deconv(nn.Module):
         proj = self.init.linear.linear
         h = F.relu(self.init.h0).float()
         # bias-free projection; bias and ReLU are folded into the first update's loads, so
-        # neither relu(Linear(x)) nor the biased projection ever exists in memory
-        s = pointwise_linear(x.flatten(2), proj.weight.to(dtype)).view(x.shape[0], -1, *x.shape[2:])
-        first = dict(bias=None if proj.bias is None else proj.bias.float(), relu_input=True)
-        later = dict(bias=None, relu_input=False)
-        taps = None
+        # neither relu(Linear(x)) nor the biased projection ever exists in memory.  Projection
+        # and first update are one autograd node: both read x, and the node's backward
+        # accumulates the projection's input gradient onto the update's
+        weight = proj.weight.squeeze(-1) if proj.weight.dim() == 3 else proj.weight
+        bias = None if proj.bias is None else proj.bias.float()
+        kwargs = dict(groups=self.groups, m=self.filter_channels, sc=self.source_channels,
+                      eps=self.eps)
         if self.num_iters > 1:   # one filter table for all iterations (a single one makes its own)
             with torch.no_grad(), torch.cuda.device(x.device):
-                taps = ops.prepare_taps(get_library(), x, h.detach().contiguous(), groups=self.groups,
-                                        m=self.filter_channels, sc=self.source_channels)
+                kwargs["taps"] = ops.prepare_taps(
+                    get_library(), x, h.detach().contiguous(), groups=self.groups,
+                    m=self.filter_channels, sc=self.source_channels)
+        s = None
         for it in range(1, self.num_iters + 1):
             with self.context(it):
-                s = deconv_update(x, s, h, groups=self.groups, m=self.filter_channels,
-                                  sc=self.source_channels, eps=self.eps, taps=taps,
-                                  **(first if it == 1 else later))
+                if it == 1:
+                    s = projected_update(x, weight, h, bias, **kwargs)
+                else:
+                    s = deconv_update(x, s, h, None, relu_input=False, **kwargs)
         return s, h
 
     # ------------------------------------------------------------------ general route

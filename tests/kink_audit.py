@@ -68,11 +68,25 @@ def record_patterns(model: nn.Module, run: Callable[[], None], keep_pre: bool = 
             note(current["name"], z.float() + b)
         return original(x, z, h, bias, **kw)
 
+    original_projected = ndc_module.projected_update
+
+    def recording_projected(x, weight, h, bias, **kw):
+        # HIP route, first iteration: projection and update are one node; its z is this GEMM
+        # (the same call on the same operands gives the same bits)
+        w = weight.detach().to(x.dtype)
+        z = torch.bmm(w.unsqueeze(0).expand(x.shape[0], -1, -1), x.flatten(2))
+        z = z.view(x.shape[0], -1, *x.shape[2:])
+        b = 0 if bias is None else bias.view(1, -1, *([1] * (z.dim() - 2)))
+        note(current["name"], z.float() + b)
+        return original_projected(x, weight, h, bias, **kw)
+
     ndc_module.deconv_update = recording_update
+    ndc_module.projected_update = recording_projected
     try:
         run()
     finally:
         ndc_module.deconv_update = original
+        ndc_module.projected_update = original_projected
         for hd in handles:
             hd.remove()
     return (masks, pres) if keep_pre else masks

@@ -357,3 +357,39 @@ def test_headline_size_channel_slices_match_oracle(dtype, tol, saved, matrix):
         assert O.rel_err(gz[:, cs].cpu(), rgz) < tol, f"gz channel {c}"
         assert O.rel_err(gh[c:c + 1].cpu(), rgh) < tol, f"gh channel {c}"
         assert O.rel_err(gb[cs].cpu(), rgb) < tol, f"gb channel {c}"
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-6), (torch.bfloat16, 8e-3)])
+@pytest.mark.parametrize("need", [("x", "w", "h", "b"), ("w",), ("x",), ("h", "b")])
+def test_projection_and_update_as_one_node_equal_the_two_nodes(dtype, tol, need):
+    """``projected_update`` against ``deconv_update`` on ``pointwise_linear``'s output: same
+    forward bits; the input gradient is the sum autograd would form (to the rounding of one
+    bfloat16 addition), the other gradients are the same GEMMs and kernels."""
+    from deconver_amd.functional import deconv_update, projected_update
+    torch.manual_seed(5)
+    B, C, sc, S = 2, 16, 4, (6, 9, 16)
+    x0 = torch.rand(B, C, *S, device="cuda").to(dtype)
+    w0 = torch.randn(C * sc, C, device="cuda") / C ** 0.5
+    h0 = torch.rand(C, sc, 3, 3, 3, device="cuda")
+    b0 = torch.rand(C * sc, device="cuda") * 0.2
+    g = torch.randn(B, C * sc, *S, device="cuda").to(dtype)
+    kw = dict(groups=C, m=1, sc=sc, eps=1e-8)
+
+    def leaves():
+        return dict(x=x0.clone().requires_grad_("x" in need), w=w0.clone().requires_grad_("w" in need),
+                    h=h0.clone().requires_grad_("h" in need), b=b0.clone().requires_grad_("b" in need))
+
+    one, two = leaves(), leaves()
+    y1 = projected_update(one["x"], one["w"], one["h"], one["b"], **kw)
+    z = pointwise_linear(two["x"].flatten(2), two["w"].to(dtype)).view(B, C * sc, *S)
+    y2 = deconv_update(two["x"], z, two["h"], two["b"], relu_input=True, **kw)
+    assert torch.equal(y1, y2)
+    y1.backward(g)
+    y2.backward(g)
+    for name in ("x", "w", "h", "b"):
+        if name not in need:
+            assert one[name].grad is None
+            continue
+        a, b = one[name].grad.double(), two[name].grad.double()
+        assert one[name].grad.dtype == two[name].grad.dtype == one[name].dtype
+        assert (a - b).norm() <= tol * b.norm(), name
