@@ -50,6 +50,10 @@ EXPORTS = (
     "ndc_chnorm_parts",
     "ndc_chnorm_forward",
     "ndc_chnorm_backward",
+    "ndc_pointwise_gemm_supported",
+    "ndc_pointwise_weight_bytes",
+    "ndc_pointwise_pack",
+    "ndc_pointwise_gemm",
 )
 
 
@@ -136,6 +140,12 @@ class NdcLibrary:
         d.ndc_chnorm_backward.argtypes = [vp, vp, vp, vp, vp, vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                                           ctypes.c_int, vp]
         d.ndc_row_sums.argtypes = [vp, vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int, vp]
+        d.ndc_pointwise_gemm_supported.argtypes = [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int]
+        d.ndc_pointwise_weight_bytes.restype = ctypes.c_size_t
+        d.ndc_pointwise_weight_bytes.argtypes = [ctypes.c_int64, ctypes.c_int64]
+        d.ndc_pointwise_pack.argtypes = [vp, ctypes.c_int, ctypes.c_int, vp, ctypes.c_int64, ctypes.c_int64, vp]
+        d.ndc_pointwise_gemm.argtypes = [vp, vp, vp, vp, vp, vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                                         ctypes.c_int64, ctypes.c_int, ctypes.c_int, vp]
         d.ndc_regroup.argtypes = [vp, vp, vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                                    ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp]
         d.ndc_taps_bytes.restype = ctypes.c_size_t
@@ -289,6 +299,24 @@ class NdcLibrary:
                           batch: int, channels: int, n: int, act: int, dtype: int, stream) -> None:
         self._check(self._dll.ndc_bias_act_backward(gy, z, bias, gz, gpart, batch, channels, n, act, dtype,
                                                     stream), "ndc_bias_act_backward")
+
+    def pointwise_gemm_supported(self, cin: int, cout: int, n: int, dtype: int) -> bool:
+        return bool(self._dll.ndc_pointwise_gemm_supported(cin, cout, n, dtype))
+
+    def pointwise_weight_bytes(self, cin: int, cout: int) -> int:
+        return int(self._dll.ndc_pointwise_weight_bytes(cin, cout))
+
+    def pointwise_pack(self, w: int, w_dtype: int, transposed: bool, wfrag: int, cin: int, cout: int,
+                       stream) -> None:
+        self._check(self._dll.ndc_pointwise_pack(w, w_dtype, int(transposed), wfrag, cin, cout, stream),
+                    "ndc_pointwise_pack")
+
+    def pointwise_gemm(self, x: int, wfrag: int, bias: Optional[int], residual: Optional[int], y: int,
+                       zkeep: Optional[int], batch: int, cin: int, cout: int, n: int, act: int, dtype: int,
+                       stream) -> None:
+        """``y = act(W x + bias) + residual`` on channel-first bf16 ``(batch, c, n)`` tensors."""
+        self._check(self._dll.ndc_pointwise_gemm(x, wfrag, bias, residual, y, zkeep, batch, cin, cout, n, act,
+                                                 dtype, stream), "ndc_pointwise_gemm")
 
     def chnorm_parts(self, batch: int, n: int, dtype: int) -> int:
         return int(self._dll.ndc_chnorm_parts(batch, n, dtype))

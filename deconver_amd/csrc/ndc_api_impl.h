@@ -518,6 +518,51 @@ int ndc_bias_act_backward(const void *gy, const void *z, const float *bias, void
                                            chunk, act, esz, vec, stream);
 }
 
+// ---- streaming GEMM of the 1x1 projections (ndc_pwgemm.h)
+
+int ndc_pointwise_gemm_supported(int64_t cin, int64_t cout, int64_t n, int dtype)
+{
+    if (dtype != NDC_BF16) return 0;
+    if (cin != 64 && cin != 128 && cin != 256) return 0;
+    if (cout < 32 || cout % 32 || cout > 4096) return 0;
+    if (cin * cout * 2 > 128 * 1024) return 0;        // the packed weights stay in LDS
+    if (n < 64 || n % 64) return 0;
+    return 1;
+}
+
+size_t ndc_pointwise_weight_bytes(int64_t cin, int64_t cout)
+{
+    return cin > 0 && cout > 0 ? (size_t)cin * (size_t)cout * 2 : 0;
+}
+
+int ndc_pointwise_pack(const void *w, int w_dtype, int transposed, void *wfrag, int64_t cin, int64_t cout,
+                       void *stream)
+{
+    if (!w || !wfrag) return NDC_ERR_NULL;
+    if (w_dtype != NDC_F32 && w_dtype != NDC_BF16) return NDC_ERR_DTYPE;
+    if (cin < 16 || cin % 16 || cout < 32 || cout % 32 || cin > 4096 || cout > 4096) return NDC_ERR_GEOMETRY;
+    if ((uintptr_t)wfrag & 15u) return NDC_ERR_WORKSPACE;
+    return ndc::Backend::pwgemm_pack(w, w_dtype == NDC_BF16, transposed != 0, wfrag, (int)cout, (int)cin, stream);
+}
+
+int ndc_pointwise_gemm(const void *x, const void *wfrag, const float *bias, const void *residual, void *y,
+                       void *zkeep, int64_t batch, int64_t cin, int64_t cout, int64_t n, int act, int dtype,
+                       void *stream)
+{
+    if (!x || !wfrag || !y) return NDC_ERR_NULL;
+    if (dtype != NDC_BF16) return NDC_ERR_DTYPE;
+    if (batch < 1 || act < NDC_ACT_NONE || act > NDC_ACT_GELU) return NDC_ERR_GEOMETRY;
+    if (!ndc_pointwise_gemm_supported(cin, cout, n, dtype)) return NDC_ERR_GEOMETRY;
+    if ((long double)batch * (cin > cout ? cin : cout) * n > 9.0e15L) return NDC_ERR_GEOMETRY;
+    if (batch * (n / 64) > 0x7fffff00LL || n > 0x3fffffffLL) return NDC_ERR_GEOMETRY;   // 32-bit tile count and lane offsets
+    // word accesses on voxel pairs, 16-byte reads of the weights
+    if (((uintptr_t)x & 3u) || ((uintptr_t)y & 3u) || (residual && ((uintptr_t)residual & 3u)) ||
+        (zkeep && ((uintptr_t)zkeep & 3u)) || ((uintptr_t)wfrag & 15u) || (bias && ((uintptr_t)bias & 3u)))
+        return NDC_ERR_WORKSPACE;
+    if (y == x || zkeep == x || (zkeep && zkeep == y)) return NDC_ERR_GEOMETRY;
+    return ndc::Backend::pwgemm(x, wfrag, bias, residual, y, zkeep, batch, (int)cin, (int)cout, n, act, stream);
+}
+
 static int chnorm_check(long long B, long long C, long long n, int dtype)
 {
     if (dtype != NDC_F32 && dtype != NDC_BF16) return NDC_ERR_DTYPE;

@@ -1,12 +1,15 @@
 // HIP (gfx950) build of the NDC C ABI: launch primitives + the shared host logic.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include "ndc_common.h"
 #include "ndc_exec.h"
 #include "ndc_rownorm.h"
 #include "ndc_epilogue.h"
 #include "ndc_regroup.h"
 #include "ndc_chnorm.h"
+#include "ndc_pwgemm.h"
 
 #define NDC_LAMBDA __host__ __device__
 
@@ -433,6 +436,94 @@ struct Backend {
             else hipLaunchKernelGGL((regroup::kernel<4, false>), grid, block, 0, (hipStream_t)stream, src, dst, bias, sh, nvec);
         }
         return check();
+    }
+
+    // weights (cout x cin, or the transpose stored as cin x cout) -> fragment order; see ndc_pwgemm.h
+    static int pwgemm_pack(const void *w, int w_is_bf16, int transposed, void *wfrag, int cout, int cin, void *stream)
+    {
+        const long long n = (long long)(cout / 32) * (cin / 16) * 64;
+        const dim3 grid((unsigned)((n + 255) / 256)), block(256);
+        uint16_t *o = (uint16_t *)wfrag;
+        if (w_is_bf16) {
+            if (transposed) hipLaunchKernelGGL((pwgemm::pack_kernel<bf16_t, true>), grid, block, 0, (hipStream_t)stream, (const bf16_t *)w, o, cout, cin);
+            else hipLaunchKernelGGL((pwgemm::pack_kernel<bf16_t, false>), grid, block, 0, (hipStream_t)stream, (const bf16_t *)w, o, cout, cin);
+        } else {
+            if (transposed) hipLaunchKernelGGL((pwgemm::pack_kernel<float, true>), grid, block, 0, (hipStream_t)stream, (const float *)w, o, cout, cin);
+            else hipLaunchKernelGGL((pwgemm::pack_kernel<float, false>), grid, block, 0, (hipStream_t)stream, (const float *)w, o, cout, cin);
+        }
+        return check();
+    }
+
+    // persistent workgroups: as many as are resident at once (asked of the runtime once per
+    // kernel and LDS size), so that every wavefront walks the same number of tiles
+    template <int CIN, int ACT, bool RES, int THREADS>
+    static int pwgemm_launch(const pwgemm::Params &p, size_t lds, void *stream)
+    {
+        void (*entry)(pwgemm::Params) = pwgemm::gemm_kernel<CIN, ACT, RES, THREADS>;
+        static std::atomic<int> resident[3] = {{0}, {0}, {0}};   // by LDS size class
+        const int cls = lds <= 40 * 1024 ? 0 : lds <= 80 * 1024 ? 1 : 2;
+        int per_cu = resident[cls].load(std::memory_order_relaxed);
+        if (per_cu == 0) {
+            // (asked for the largest LDS size of the class, so that the answer holds for all of it)
+            const size_t worst = cls == 0 ? 40 * 1024 : cls == 1 ? 80 * 1024 : 136 * 1024;
+            if (worst > 64 * 1024 &&
+                hipFuncSetAttribute((const void *)entry, hipFuncAttributeMaxDynamicSharedMemorySize, (int)worst) != hipSuccess)
+                return -5;
+            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void *)entry, THREADS, worst) != hipSuccess ||
+                per_cu < 1)
+                per_cu = 1;
+            resident[cls].store(per_cu, std::memory_order_relaxed);
+        }
+        int dev = 0, cus = 256;
+        if (hipGetDevice(&dev) == hipSuccess) {
+            static std::atomic<int> cu_count{0};
+            cus = cu_count.load(std::memory_order_relaxed);
+            if (cus == 0) {
+                if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) cus = 256;
+                cu_count.store(cus, std::memory_order_relaxed);
+            }
+        }
+        long long blocks = (long long)cus * per_cu;
+        const long long need = ((long long)p.tiles + THREADS / 64 - 1) / (THREADS / 64);
+        if (blocks > need) blocks = need;
+        hipLaunchKernelGGL(entry, dim3((unsigned)blocks), dim3(THREADS), lds, (hipStream_t)stream, p);
+        return check();
+    }
+
+    template <int CIN, int THREADS>
+    static int pwgemm_act(const pwgemm::Params &p, size_t lds, int act, void *stream)
+    {
+#define NDC_PWGEMM_RES(ACT)                                                                 \
+    (p.res ? pwgemm_launch<CIN, ACT, true, THREADS>(p, lds, stream)                         \
+           : pwgemm_launch<CIN, ACT, false, THREADS>(p, lds, stream))
+        if (act == epilogue::kRelu) return NDC_PWGEMM_RES(epilogue::kRelu);
+        if (act == epilogue::kGelu) return NDC_PWGEMM_RES(epilogue::kGelu);
+        return NDC_PWGEMM_RES(epilogue::kNone);
+#undef NDC_PWGEMM_RES
+    }
+
+    // y = act(W x + bias) + residual on persistent workgroups; the caller has checked the shape
+    // (cin in {64, 128, 256}, cout a multiple of 32, n a multiple of 64, packed weights <= 128 KB)
+    static int pwgemm(const void *x, const void *wfrag, const float *bias, const void *res, void *y, void *zkeep,
+                      long long batch, int cin, int cout, long long n, int act, void *stream)
+    {
+        pwgemm::Params p;
+        p.x = (const uint16_t *)x, p.wfrag = (const uint16_t *)wfrag, p.bias = bias;
+        p.res = (const uint16_t *)res, p.y = (uint16_t *)y, p.zkeep = (uint16_t *)zkeep;
+        p.n = n, p.tiles_per_sample = (int)(n / pwgemm::kTileVoxels), p.tiles = (int)(batch * (n / pwgemm::kTileVoxels)), p.cout = cout;
+        if (p.tiles <= 0) return 0;
+        const size_t wbytes = (size_t)cin * cout * 2;
+        const size_t lds = wbytes + (size_t)cout * 4;   // packed weights, bias
+        // small weight tables: several workgroups per CU; large ones: one, of more wavefronts
+        const int threads = wbytes <= 32 * 1024 ? 256 : wbytes <= 64 * 1024 || cin == 256 ? 512 : 1024;
+#define NDC_PWGEMM(CIN)                                                                            \
+    (threads == 256 ? pwgemm_act<CIN, 256>(p, lds, act, stream)                                     \
+     : threads == 512 ? pwgemm_act<CIN, 512>(p, lds, act, stream)                                   \
+                      : pwgemm_act<CIN, 1024>(p, lds, act, stream))
+        if (cin == 64) return NDC_PWGEMM(64);
+        if (cin == 128) return NDC_PWGEMM(128);
+        return threads == 256 ? pwgemm_act<256, 256>(p, lds, act, stream) : pwgemm_act<256, 512>(p, lds, act, stream);
+#undef NDC_PWGEMM
     }
 
     static constexpr int kSumSlices = 8;

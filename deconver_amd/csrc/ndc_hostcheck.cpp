@@ -247,6 +247,47 @@ struct Backend {
         return grad ? 1.f : u;
     }
 
+    // the packed weights of the streaming GEMM: fragment (c, s), lane l, element e holds
+    // W[32 c + l % 32][16 s + 8 (l / 32) + e] as bf16
+    static int pwgemm_pack(const void *w, int w_is_bf16, int transposed, void *wfrag, int cout, int cin, void *)
+    {
+        const int S = cin / 16;
+        bf16_t *o = (bf16_t *)wfrag;
+        for (int c = 0; c < cout / 32; ++c)
+            for (int s = 0; s < S; ++s)
+                for (int l = 0; l < 64; ++l)
+                    for (int e = 0; e < 8; ++e) {
+                        const int row = 32 * c + l % 32, k = 16 * s + 8 * (l / 32) + e;
+                        const long long at = transposed ? (long long)k * cout + row : (long long)row * cin + k;
+                        const float v = w_is_bf16 ? Elem<bf16_t>::load((const bf16_t *)w + at) : ((const float *)w)[at];
+                        o[(((long long)c * S + s) * 64 + l) * 8 + e] = float_to_bf16(v);
+                    }
+        return 0;
+    }
+
+    static int pwgemm(const void *x, const void *wfrag, const float *bias, const void *res, void *y, void *zkeep,
+                      long long batch, int cin, int cout, long long n, int act, void *)
+    {
+        const int S = cin / 16;
+        const bf16_t *xs = (const bf16_t *)x, *wf = (const bf16_t *)wfrag, *rs = (const bf16_t *)res;
+        bf16_t *ys = (bf16_t *)y, *zs = (bf16_t *)zkeep;
+        for (long long b = 0; b < batch; ++b)
+            for (int co = 0; co < cout; ++co)
+                for (long long v = 0; v < n; ++v) {
+                    float acc = 0.f;
+                    for (int k = 0; k < cin; ++k) {
+                        const long long f = ((long long)(co / 32) * S + k / 16) * 64 + (k % 16 / 8) * 32 + co % 32;
+                        acc += Elem<bf16_t>::load(wf + f * 8 + k % 8) * Elem<bf16_t>::load(xs + (b * cin + k) * n + v);
+                    }
+                    const long long at = (b * cout + co) * n + v;
+                    if (zs) zs[at] = float_to_bf16(acc);
+                    float out = act_value(act, acc + (bias ? bias[co] : 0.f), false);
+                    if (rs) out += Elem<bf16_t>::load(rs + at);
+                    ys[at] = float_to_bf16(out);
+                }
+        return 0;
+    }
+
     template <typename T>
     static void bias_act_t(const T *z, const float *bias, const T *res, T *y, long long rows, int channels,
                            long long n, int act)

@@ -178,10 +178,9 @@ class ProjectedUpdate(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, weight, h, bias, groups, m, sc, eps, taps=None):
-        B = x.shape[0]
+        from .layers import project
         w = weight.detach().to(x.dtype)
-        z = x.new_empty(B, w.shape[0], *x.shape[2:])
-        torch.bmm(w.unsqueeze(0).expand(B, -1, -1), x.flatten(2), out=z.flatten(2))
+        z = project(weight.detach(), x.flatten(2)).view(x.shape[0], w.shape[0], *x.shape[2:])
         need_x, need_w, need_h, need_b = ctx.needs_input_grad[:4]
         out, saved = _node_forward(ctx, (need_x, need_x or need_w, need_h, need_b), x, z, h,
                                    bias, groups, m, sc, eps, True, taps)
@@ -191,7 +190,7 @@ class ProjectedUpdate(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, gout):
-        from .layers import projection_weight_grad
+        from .layers import project_back, projection_weight_grad
         *saved, w = ctx.saved_tensors
         need_x, need_w, need_h, need_b = ctx.needs_input_grad[:4]
         gx, gz, gh, gb = _node_backward(ctx, saved, gout, need_x, need_x or need_w, need_h, need_b)
@@ -200,7 +199,7 @@ class ProjectedUpdate(torch.autograd.Function):
         if need_w:
             gw = projection_weight_grad(gz.flatten(2), x.flatten(2), ctx.weight_dtype)
         if need_x:
-            gx.flatten(2).baddbmm_(w.t().unsqueeze(0).expand(x.shape[0], -1, -1), gz.flatten(2))
+            gx = project_back(w, gz.flatten(2), accumulate=gx.flatten(2)).view_as(x)
         return gx, gw, gh, gb, None, None, None, None, None
 
 

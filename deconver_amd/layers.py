@@ -52,6 +52,38 @@ def projection_weight_grad(gz: torch.Tensor, x: torch.Tensor, dtype: torch.dtype
     return parts.sum(0, dtype=torch.float32).to(dtype)
 
 
+def project(weight: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+    """``W x`` per sample for contiguous ``x`` of shape ``(B, Cin, N)`` and ``weight`` of shape
+    ``(Cout, Cin)`` in any floating dtype (used in ``x``'s): the library's streaming GEMM where
+    it applies, else one batched hipBLASLt GEMM with the weight shared through a zero stride."""
+    lib = _lib.get_library()
+    if ops.pointwise_gemm_applies(lib, x, weight.shape[0]):
+        with torch.cuda.device(x.device):
+            return ops.pointwise_gemm(lib, x, ops.pointwise_pack(lib, weight.contiguous()), weight.shape[0])[0]
+    z = x.new_empty(x.shape[0], weight.shape[0], x.shape[2])
+    torch.bmm(weight.to(x.dtype).unsqueeze(0).expand(x.shape[0], -1, -1), x, out=z)
+    return z
+
+
+def project_back(weight: torch.Tensor, gz: torch.Tensor, accumulate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``W^T gz`` per sample (the input gradient of a 1x1 projection with ``weight`` of shape
+    ``(Cout, Cin)``), plus ``accumulate`` if given (a tensor of the result's shape, which may
+    be overwritten).  The library's streaming GEMM where it applies -- the weight is packed as
+    it lies, no transposed copy --, else one batched hipBLASLt GEMM."""
+    B, cout, n = gz.shape
+    lib = _lib.get_library()
+    if gz.is_contiguous() and ops.pointwise_gemm_applies(lib, gz, weight.shape[1]):
+        with torch.cuda.device(gz.device):
+            wfrag = ops.pointwise_pack(lib, weight.contiguous(), transposed=True)
+            return ops.pointwise_gemm(lib, gz, wfrag, weight.shape[1], residual=accumulate)[0]
+    wt = weight.t().unsqueeze(0).expand(B, -1, -1)
+    if accumulate is not None:
+        return accumulate.baddbmm_(wt, gz)
+    gx = gz.new_empty(B, weight.shape[1], n)
+    torch.bmm(wt, gz, out=gx)
+    return gx
+
+
 class _PointwiseLinear(torch.autograd.Function):
     """``y[b] = act(W x[b] + bias) + residual[b]`` for ``x`` of shape ``(B, Cin, N)``: the 1x1
     projection as plain GEMMs on the channel-first layout (hipBLASLt through ``torch.bmm``),
@@ -76,16 +108,23 @@ class _PointwiseLinear(torch.autograd.Function):
         # that its gradient leaves backward as the float32 sum it is, not rounded to bf16 first)
         B = x.shape[0]
         w = weight.detach().to(x.dtype)
-        z = x.new_empty(B, w.shape[0], x.shape[2])
-        torch.bmm(w.unsqueeze(0).expand(B, -1, -1), x, out=z)
         bias32 = None if bias is None else bias.detach().float().contiguous()
-        y = z
         # the activation's gradient needs z + bias: gelu keeps z; relu alone needs only the
         # sign of its output, which may then overwrite z
         keep_z = act == "gelu" or (act == "relu" and residual is not None)
-        if bias is not None or act is not None or residual is not None:
+        if ops.pointwise_gemm_applies(lib, x, w.shape[0]):
+            # the library's streaming GEMM: product, bias, activation and residual in one
+            # kernel that reads x once and writes the result (and z where it is kept) once
             with torch.cuda.device(x.device):
-                y = ops.bias_act(lib, z, bias32, residual, act, inplace=not keep_z)
+                y, z = ops.pointwise_gemm(lib, x, ops.pointwise_pack(lib, weight.detach().contiguous()),
+                                          w.shape[0], bias32, residual, act, keep_z=keep_z)
+        else:
+            z = x.new_empty(B, w.shape[0], x.shape[2])
+            torch.bmm(w.unsqueeze(0).expand(B, -1, -1), x, out=z)
+            y = z
+            if bias is not None or act is not None or residual is not None:
+                with torch.cuda.device(x.device):
+                    y = ops.bias_act(lib, z, bias32, residual, act, inplace=not keep_z)
         kept = z if keep_z else y if act == "relu" else None
         ctx.save_for_backward(x, w, kept, bias32 if keep_z else None)
         ctx.weight_dtype = weight.dtype
@@ -113,8 +152,7 @@ class _PointwiseLinear(torch.autograd.Function):
             with torch.cuda.device(gy.device):
                 gb = ops.channel_sums(_lib.get_library(), gy)
         if ctx.needs_input_grad[0]:
-            gx = torch.empty_like(x)
-            torch.bmm(weight.t().unsqueeze(0).expand(x.shape[0], -1, -1), gz, out=gx)
+            gx = project_back(weight, gz)
         if ctx.needs_input_grad[1]:
             gw = projection_weight_grad(gz, x, ctx.weight_dtype)
         return gx, gw, gb, None, gres

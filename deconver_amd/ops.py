@@ -279,6 +279,47 @@ def bias_act_backward(lib: _lib.NdcLibrary, gy: Tensor, z: Tensor, bias: Optiona
     return gz, (gpart.sum((0, 2)) if need_bias_grad else None)
 
 
+def pointwise_gemm_applies(lib: _lib.NdcLibrary, x: Tensor, cout: int) -> bool:
+    """Whether ``pointwise_gemm`` takes the projection of ``x`` (B, cin, n) to ``cout`` channels:
+    contiguous bfloat16 on the GPU in the shapes ``ndc_pointwise_gemm_supported`` lists."""
+    return (x.is_cuda and x.dtype == torch.bfloat16 and x.dim() == 3 and x.is_contiguous()
+            and lib.pointwise_gemm_supported(x.shape[1], cout, x.shape[2], _lib.NDC_BF16))
+
+
+def pointwise_pack(lib: _lib.NdcLibrary, weight: Tensor, transposed: bool = False) -> Tensor:
+    """The weight of a 1x1 projection in the order ``pointwise_gemm`` reads it (bf16).
+    ``weight``: ``(cout, cin)``, float32 or bfloat16, contiguous; with ``transposed`` it is
+    taken as the ``(cin, cout)`` storage of the matrix to apply (the input gradient's ``W^T``
+    from ``W`` as it lies)."""
+    if weight.dim() != 2 or not weight.is_contiguous() or weight.dtype not in _DTYPES:
+        raise ValueError("pointwise_pack wants a contiguous float32 or bfloat16 matrix")
+    cout, cin = (weight.shape[1], weight.shape[0]) if transposed else weight.shape
+    wfrag = torch.empty(cout * cin, dtype=torch.bfloat16, device=weight.device)
+    lib.pointwise_pack(_ptr(weight), dtype_tag(weight.dtype), transposed, _ptr(wfrag), cin, cout,
+                       _stream_of(weight))
+    return wfrag
+
+
+def pointwise_gemm(lib: _lib.NdcLibrary, x: Tensor, wfrag: Tensor, cout: int, bias: Optional[Tensor] = None,
+                   residual: Optional[Tensor] = None, act: Optional[str] = None, keep_z: bool = False):
+    """``y = act(W x + bias) + residual`` for contiguous bfloat16 ``x`` (B, cin, n) and packed
+    ``W`` (``pointwise_pack``); returns ``(y, z)`` with ``z`` the product before bias and
+    activation when ``keep_z``, else None."""
+    B, cin, n = x.shape
+    if wfrag.numel() != cin * cout or wfrag.dtype != torch.bfloat16:
+        raise ValueError("wfrag does not belong to this projection")
+    if bias is not None and (bias.dtype != torch.float32 or bias.numel() != cout or not bias.is_contiguous()):
+        raise ValueError("bias must be float32 with one entry per output channel")
+    if residual is not None and (residual.shape != (B, cout, n) or residual.dtype != x.dtype
+                                 or not residual.is_contiguous()):
+        raise ValueError("residual must be contiguous, of the output's shape and dtype")
+    y = x.new_empty(B, cout, n)
+    z = x.new_empty(B, cout, n) if keep_z else None
+    lib.pointwise_gemm(_ptr(x), _ptr(wfrag), _ptr(bias), _ptr(residual), _ptr(y), _ptr(z), B, cin, cout, n,
+                       ACTS[act], _lib.NDC_BF16, _stream_of(x))
+    return y, z
+
+
 def regroup2_applies(fine_shape, dtype, *ptrs) -> bool:
     """Whether ``ndc_regroup`` takes a fine-grid tensor ``(B, C, [D,] H, W)``: float32 or
     bfloat16, even extents, rows of whole 16-byte vectors, 16-byte aligned buffers."""

@@ -314,6 +314,35 @@ int ndc_bias_act_backward(const void *gy, const void *z, const float *bias, void
                           int64_t batch, int64_t channels, int64_t n, int act, int dtype, void *stream);
 
 /*
+ * The 1x1 projection itself, with its tail, for bfloat16 channel-first tensors:
+ *   y[b][co][i] = act( sum_ci W[co][ci] * x[b][ci][i] + bias[co] ) + residual[b][co][i]
+ * (nn.Conv1d with kernel size 1 in deconver/layers/linear.py:53-58, followed by what
+ * deconver/deconver.py:41-46, 60-64 and deconver/layers/mlp.py:40-63 apply to its output).
+ * A streaming kernel on the matrix units: x is read once, y written once, float32 accumulation,
+ * one rounding of the result.
+ *   ndc_pointwise_gemm_supported  1 where the kernel applies: NDC_BF16, cin 64, 128 or 256,
+ *                  cout a multiple of 32, cin * cout * 2 <= 128 KiB, n a multiple of 64; else 0
+ *                  (callers then use a library GEMM and ndc_bias_act)
+ *   ndc_pointwise_pack  writes W in the order the kernel reads it into wfrag
+ *                  (ndc_pointwise_weight_bytes(cin, cout) bytes, 16-byte aligned): the 8 values
+ *                  W[32 c + l % 32][16 s + 8 (l / 32) + 0..7], as bf16, at element
+ *                  (((c * cin / 16) + s) * 64 + l) * 8.  w: cout x cin row-major, float32 or
+ *                  bf16; with transposed != 0 the same matrix stored as cin x cout (so that the
+ *                  input gradient, W^T gy, packs the weight as it lies).
+ *   x              (batch, cin, n); y, residual, zkeep: (batch, cout, n); all bf16, 4-byte aligned
+ *   bias           cout floats or NULL; residual NULL or a tensor added to the result
+ *   zkeep          NULL, or receives the product before bias and activation (what
+ *                  ndc_bias_act_backward reads as z)
+ */
+int ndc_pointwise_gemm_supported(int64_t cin, int64_t cout, int64_t n, int dtype);
+size_t ndc_pointwise_weight_bytes(int64_t cin, int64_t cout);
+int ndc_pointwise_pack(const void *w, int w_dtype, int transposed, void *wfrag, int64_t cin, int64_t cout,
+                       void *stream);
+int ndc_pointwise_gemm(const void *x, const void *wfrag, const float *bias, const void *residual, void *y,
+                       void *zkeep, int64_t batch, int64_t cin, int64_t cout, int64_t n, int act, int dtype,
+                       void *stream);
+
+/*
  * Normalisation over the CHANNEL axis of a channel-first tensor (batch, channels, n):
  *   y[b][c][i] = (x[b][c][i] - mean[b][i]) * rstd[b][i] * weight[c] + bias[c],
  * mean and biased variance over c.  The reference's LayerNorm (deconver/layers/norm.py:25-34:

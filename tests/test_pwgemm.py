@@ -1,0 +1,119 @@
+"""The streaming GEMM of the 1x1 projections (``ndc_pointwise_gemm``) against ``conv1d`` in
+float64 (the map of the reference's ``Linear``, layers/linear.py:53-58, with the tail its callers
+apply, deconver.py:41-46, 60-64, layers/mlp.py:40-63)."""
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from deconver_amd import _lib, ops
+from tests.helpers import hostcheck_library
+
+
+def _case(B, cin, cout, n, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(B, cin, n, generator=g).bfloat16()
+    w = torch.randn(cout, cin, generator=g) / cin ** 0.5
+    bias = torch.randn(cout, generator=g)
+    res = torch.randn(B, cout, n, generator=g).bfloat16()
+    return x, w, bias, res
+
+
+def _reference(x, w, bias, res, act):
+    """float64 on the bf16-rounded operands (the kernel rounds W to bf16 when packing)."""
+    z = F.conv1d(x.double(), w.bfloat16().double().unsqueeze(-1))
+    u = z if bias is None else z + bias.double().view(1, -1, 1)
+    y = {None: lambda t: t, "relu": torch.relu, "gelu": F.gelu}[act](u)
+    return z, (y if res is None else y + res.double())
+
+
+def _rel(a, ref):
+    return float((a.double().cpu() - ref).abs().max() / ref.abs().max())
+
+
+def test_support_predicate():
+    lib = hostcheck_library()
+    bf, f32 = _lib.NDC_BF16, _lib.NDC_F32
+    assert lib.pointwise_gemm_supported(64, 256, 128 ** 3, bf)
+    assert lib.pointwise_gemm_supported(256, 64, 64, bf) and lib.pointwise_gemm_supported(128, 512, 4096, bf)
+    assert not lib.pointwise_gemm_supported(64, 256, 128 ** 3, f32)       # bfloat16 only
+    assert not lib.pointwise_gemm_supported(512, 128, 4096, bf)           # 512 input channels
+    assert not lib.pointwise_gemm_supported(256, 512, 4096, bf)           # weights beyond 128 KiB
+    assert not lib.pointwise_gemm_supported(64, 48, 4096, bf)             # cout not a multiple of 32
+    assert not lib.pointwise_gemm_supported(64, 64, 100, bf)              # n not a multiple of 64
+    assert lib.pointwise_weight_bytes(64, 256) == 64 * 256 * 2
+
+
+@pytest.mark.parametrize("transposed", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_pack_order_on_the_host_build(transposed, dtype):
+    lib = hostcheck_library()
+    cout, cin = 64, 128
+    w = (torch.arange(cout * cin, dtype=torch.float32).view(cout, cin) % 251 - 125).to(dtype)
+    stored = w.t().contiguous() if transposed else w
+    frag = ops.pointwise_pack(lib, stored, transposed=transposed).view(cout // 32, cin // 16, 2, 32, 8)
+    # fragment (c, s), lane (kb, i), element e  <->  W[32 c + i][16 s + 8 kb + e]
+    want = w.bfloat16().view(cout // 32, 32, cin // 16, 2, 8).permute(0, 2, 3, 1, 4)
+    assert torch.equal(frag, want)
+
+
+@pytest.mark.parametrize("B,cin,cout,n", [(2, 64, 96, 128), (1, 128, 32, 64), (1, 256, 64, 64)])
+@pytest.mark.parametrize("act,with_bias,with_res,keep", [(None, False, False, False), (None, True, True, False),
+                                                          ("gelu", True, False, True), ("relu", False, True, True)])
+def test_host_build_matches_float64(B, cin, cout, n, act, with_bias, with_res, keep):
+    lib = hostcheck_library()
+    x, w, bias, res = _case(B, cin, cout, n)
+    bias, res = (bias if with_bias else None), (res if with_res else None)
+    y, z = ops.pointwise_gemm(lib, x, ops.pointwise_pack(lib, w), cout, bias, res, act, keep_z=keep)
+    zr, yr = _reference(x, w, bias, res, act)
+    assert y.dtype == torch.bfloat16 and _rel(y, yr) < 1e-2
+    assert (z is not None) == keep
+    if keep:
+        assert _rel(z, zr) < 1e-2
+
+
+def test_bad_arguments_are_refused():
+    lib = hostcheck_library()
+    x, w, bias, res = _case(1, 64, 32, 64)
+    wf = ops.pointwise_pack(lib, w)
+    with pytest.raises(ValueError):
+        ops.pointwise_gemm(lib, x, wf, 64)                      # not this projection's weights
+    with pytest.raises(ValueError):
+        ops.pointwise_gemm(lib, x, wf, 32, bias=bias.double())
+    with pytest.raises(_lib.NdcError):
+        ops.pointwise_gemm(lib, x[:, :, :32].contiguous(), wf, 32)   # n = 32
+    with pytest.raises(ValueError):
+        ops.pointwise_pack(lib, w.t())                          # not contiguous
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("B,cin,cout,n", [
+    (2, 64, 256, 64 * 64 * 8), (2, 256, 64, 64 * 64 * 8), (1, 64, 64, 4096), (2, 128, 512, 32 ** 3),
+    (3, 128, 128, 64 * 33), (1, 256, 256, 64 * 7), (2, 64, 32, 64)])
+@pytest.mark.parametrize("act,with_bias,with_res,keep", [(None, False, False, False), (None, True, True, False),
+                                                          ("gelu", True, False, True), ("relu", False, False, False)])
+def test_gpu_matches_float64(B, cin, cout, n, act, with_bias, with_res, keep):
+    lib = _lib.get_library()
+    x, w, bias, res = _case(B, cin, cout, n, seed=1)
+    bias, res = (bias if with_bias else None), (res if with_res else None)
+    dev = [t.cuda() if t is not None else None for t in (x, w, bias, res)]
+    assert ops.pointwise_gemm_applies(lib, dev[0], cout)
+    y, z = ops.pointwise_gemm(lib, dev[0], ops.pointwise_pack(lib, dev[1]), cout, dev[2], dev[3], act, keep_z=keep)
+    zr, yr = _reference(x, w, bias, res, act)
+    assert _rel(y, yr) < 1e-2
+    if keep:
+        assert _rel(z, zr) < 1e-2
+    # the same product through the transposed packing (what the input gradient uses)
+    y2, _ = ops.pointwise_gemm(lib, dev[0], ops.pointwise_pack(lib, dev[1].t().contiguous(), transposed=True),
+                               cout, dev[2], dev[3], act)
+    assert torch.equal(y, y2)
+
+
+@pytest.mark.gpu
+def test_gpu_equals_the_host_build_bit_for_bit_up_to_summation_order():
+    """Device (matrix instruction, float32 accumulation in its own order) against the host loops."""
+    x, w, bias, res = _case(2, 64, 64, 256, seed=2)
+    host, _ = ops.pointwise_gemm(hostcheck_library(), x, ops.pointwise_pack(hostcheck_library(), w), 64, bias, res)
+    lib = _lib.get_library()
+    dev, _ = ops.pointwise_gemm(lib, x.cuda(), ops.pointwise_pack(lib, w.cuda()), 64, bias.cuda(), res.cuda())
+    assert _rel(dev, host.double()) < 8e-3
