@@ -54,6 +54,8 @@ EXPORTS = (
     "ndc_pointwise_weight_bytes",
     "ndc_pointwise_pack",
     "ndc_pointwise_gemm",
+    "ndc_pointwise_gemm_parts",
+    "ndc_pointwise_gemm_actgrad",
 )
 
 
@@ -146,6 +148,10 @@ class NdcLibrary:
         d.ndc_pointwise_pack.argtypes = [vp, ctypes.c_int, ctypes.c_int, vp, ctypes.c_int64, ctypes.c_int64, vp]
         d.ndc_pointwise_gemm.argtypes = [vp, vp, vp, vp, vp, vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                                          ctypes.c_int64, ctypes.c_int, ctypes.c_int, vp]
+        d.ndc_pointwise_gemm_parts.restype = ctypes.c_int64
+        d.ndc_pointwise_gemm_parts.argtypes = []
+        d.ndc_pointwise_gemm_actgrad.argtypes = [vp, vp, vp, vp, vp, vp, ctypes.c_int64, ctypes.c_int64,
+                                                 ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_int, vp]
         d.ndc_regroup.argtypes = [vp, vp, vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                                    ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp]
         d.ndc_taps_bytes.restype = ctypes.c_size_t
@@ -317,6 +323,16 @@ class NdcLibrary:
         """``y = act(W x + bias) + residual`` on channel-first bf16 ``(batch, c, n)`` tensors."""
         self._check(self._dll.ndc_pointwise_gemm(x, wfrag, bias, residual, y, zkeep, batch, cin, cout, n, act,
                                                  dtype, stream), "ndc_pointwise_gemm")
+
+    def pointwise_gemm_parts(self) -> int:
+        return int(self._dll.ndc_pointwise_gemm_parts())
+
+    def pointwise_gemm_actgrad(self, gy: int, wfrag: int, bias: Optional[int], z: int, gz: int,
+                               gpart: Optional[int], batch: int, cin: int, cout: int, n: int, act: int,
+                               dtype: int, stream) -> None:
+        """``gz = (W gy) * act'(z + bias)`` with per-wavefront sums of ``gz`` in ``gpart``."""
+        self._check(self._dll.ndc_pointwise_gemm_actgrad(gy, wfrag, bias, z, gz, gpart, batch, cin, cout, n,
+                                                         act, dtype, stream), "ndc_pointwise_gemm_actgrad")
 
     def chnorm_parts(self, batch: int, n: int, dtype: int) -> int:
         return int(self._dll.ndc_chnorm_parts(batch, n, dtype))

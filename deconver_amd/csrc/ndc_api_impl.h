@@ -560,7 +560,29 @@ int ndc_pointwise_gemm(const void *x, const void *wfrag, const float *bias, cons
         (zkeep && ((uintptr_t)zkeep & 3u)) || ((uintptr_t)wfrag & 15u) || (bias && ((uintptr_t)bias & 3u)))
         return NDC_ERR_WORKSPACE;
     if (y == x || zkeep == x || (zkeep && zkeep == y)) return NDC_ERR_GEOMETRY;
-    return ndc::Backend::pwgemm(x, wfrag, bias, residual, y, zkeep, batch, (int)cin, (int)cout, n, act, stream);
+    return ndc::Backend::pwgemm(x, wfrag, bias, residual, y, zkeep, nullptr, batch, (int)cin, (int)cout, n, act, stream);
+}
+
+int64_t ndc_pointwise_gemm_parts(void)
+{
+    return 4096;
+}
+
+int ndc_pointwise_gemm_actgrad(const void *gy, const void *wfrag, const float *bias, const void *z, void *gz,
+                               float *gpart, int64_t batch, int64_t cin, int64_t cout, int64_t n, int act,
+                               int dtype, void *stream)
+{
+    if (!gy || !wfrag || !z || !gz) return NDC_ERR_NULL;
+    if (dtype != NDC_BF16) return NDC_ERR_DTYPE;
+    if (batch < 1 || (act != NDC_ACT_RELU && act != NDC_ACT_GELU)) return NDC_ERR_GEOMETRY;
+    if (!ndc_pointwise_gemm_supported(cin, cout, n, dtype)) return NDC_ERR_GEOMETRY;
+    if ((long double)batch * (cin > cout ? cin : cout) * n > 9.0e15L) return NDC_ERR_GEOMETRY;
+    if (batch * (n / 64) > 0x7fffff00LL || n > 0x3fffffffLL) return NDC_ERR_GEOMETRY;
+    if (((uintptr_t)gy & 3u) || ((uintptr_t)gz & 3u) || ((uintptr_t)z & 3u) || ((uintptr_t)wfrag & 15u) ||
+        (bias && ((uintptr_t)bias & 3u)) || (gpart && ((uintptr_t)gpart & 3u)))
+        return NDC_ERR_WORKSPACE;
+    if (gz == gy || gz == z) return NDC_ERR_GEOMETRY;
+    return ndc::Backend::pwgemm(gy, wfrag, bias, z, gz, nullptr, gpart, batch, (int)cin, (int)cout, n, act + 2, stream);
 }
 
 static int chnorm_check(long long B, long long C, long long n, int dtype)

@@ -486,6 +486,8 @@ struct Backend {
         long long blocks = (long long)cus * per_cu;
         const long long need = ((long long)p.tiles + THREADS / 64 - 1) / (THREADS / 64);
         if (blocks > need) blocks = need;
+        // gradient modes: one row of sums per wavefront (the kernel zeroes the rows nobody owns)
+        if (p.gpart && blocks * (THREADS / 64) > pwgemm::kMaxParts) blocks = pwgemm::kMaxParts / (THREADS / 64);
         hipLaunchKernelGGL(entry, dim3((unsigned)blocks), dim3(THREADS), lds, (hipStream_t)stream, p);
         return check();
     }
@@ -496,6 +498,8 @@ struct Backend {
 #define NDC_PWGEMM_RES(ACT)                                                                 \
     (p.res ? pwgemm_launch<CIN, ACT, true, THREADS>(p, lds, stream)                         \
            : pwgemm_launch<CIN, ACT, false, THREADS>(p, lds, stream))
+        if (act == pwgemm::kGeluGrad) return pwgemm_launch<CIN, pwgemm::kGeluGrad, true, THREADS>(p, lds + (size_t)(THREADS / 64) * p.cout * 4, stream);
+        if (act == pwgemm::kReluGrad) return pwgemm_launch<CIN, pwgemm::kReluGrad, true, THREADS>(p, lds + (size_t)(THREADS / 64) * p.cout * 4, stream);
         if (act == epilogue::kRelu) return NDC_PWGEMM_RES(epilogue::kRelu);
         if (act == epilogue::kGelu) return NDC_PWGEMM_RES(epilogue::kGelu);
         return NDC_PWGEMM_RES(epilogue::kNone);
@@ -504,10 +508,13 @@ struct Backend {
 
     // y = act(W x + bias) + residual on persistent workgroups; the caller has checked the shape
     // (cin in {64, 128, 256}, cout a multiple of 32, n a multiple of 64, packed weights <= 128 KB)
+    // act 3 / 4: y = (W x) * relu' / gelu'(res + bias), gpart (kMaxParts x cout, or null) receives
+    // per-wavefront sums of y whose total over the rows is the bias gradient
     static int pwgemm(const void *x, const void *wfrag, const float *bias, const void *res, void *y, void *zkeep,
-                      long long batch, int cin, int cout, long long n, int act, void *stream)
+                      float *gpart, long long batch, int cin, int cout, long long n, int act, void *stream)
     {
         pwgemm::Params p;
+        p.gpart = gpart;
         p.x = (const uint16_t *)x, p.wfrag = (const uint16_t *)wfrag, p.bias = bias;
         p.res = (const uint16_t *)res, p.y = (uint16_t *)y, p.zkeep = (uint16_t *)zkeep;
         p.n = n, p.tiles_per_sample = (int)(n / pwgemm::kTileVoxels), p.tiles = (int)(batch * (n / pwgemm::kTileVoxels)), p.cout = cout;

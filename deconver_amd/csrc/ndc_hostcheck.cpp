@@ -266,8 +266,10 @@ struct Backend {
     }
 
     static int pwgemm(const void *x, const void *wfrag, const float *bias, const void *res, void *y, void *zkeep,
-                      long long batch, int cin, int cout, long long n, int act, void *)
+                      float *gpart, long long batch, int cin, int cout, long long n, int act, void *)
     {
+        if (gpart)
+            for (long long i = 0; i < 4096LL * cout; ++i) gpart[i] = 0.f;
         const int S = cin / 16;
         const bf16_t *xs = (const bf16_t *)x, *wf = (const bf16_t *)wfrag, *rs = (const bf16_t *)res;
         bf16_t *ys = (bf16_t *)y, *zs = (bf16_t *)zkeep;
@@ -280,6 +282,12 @@ struct Backend {
                         acc += Elem<bf16_t>::load(wf + f * 8 + k % 8) * Elem<bf16_t>::load(xs + (b * cin + k) * n + v);
                     }
                     const long long at = (b * cout + co) * n + v;
+                    if (act >= 3) {   // times the derivative of relu (3) / gelu (4) at aux + bias
+                        const float out = acc * act_value(act - 2, Elem<bf16_t>::load(rs + at) + (bias ? bias[co] : 0.f), true);
+                        if (gpart) gpart[(v / 64 % 7) * cout + co] += out;   // a few rows, as the device uses many
+                        ys[at] = float_to_bf16(out);
+                        continue;
+                    }
                     if (zs) zs[at] = float_to_bf16(acc);
                     float out = act_value(act, acc + (bias ? bias[co] : 0.f), false);
                     if (rs) out += Elem<bf16_t>::load(rs + at);

@@ -44,6 +44,11 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 static const int kTileVoxels = 64;       // voxels a wavefront owns at a time
+static const int kMaxParts = 4096;       // wavefronts of a launch (rows of Params::gpart) at most
+// Epilogue modes beyond epilogue::kNone / kRelu / kGelu: the product times the activation's
+// derivative at (aux + bias), aux read through Params::res -- the input gradient of a
+// projection whose INPUT was act(aux + bias) (the MLP's second projection, layers/mlp.py:40-63)
+enum { kReluGrad = 3, kGeluGrad = 4 };
 static const int kMaxLdsBytes = 128 * 1024;   // packed weights a workgroup may hold
 
 struct Params {
@@ -53,6 +58,7 @@ struct Params {
     const uint16_t *res;     // (B, cout, n) or null
     uint16_t *y;             // (B, cout, n)
     uint16_t *zkeep;         // (B, cout, n) or null: the product before bias and activation
+    float *gpart;            // gradient modes: (gridDim.x * waves, cout) sums of y per wavefront, or null
     long long n;             // voxels per sample, a multiple of 64
     int tiles;               // B * n / 64
     int tiles_per_sample;
@@ -142,6 +148,12 @@ __global__ void __launch_bounds__(THREADS) gemm_kernel(Params p)
         for (int i = threadIdx.x; i < chunks; i += THREADS) wl[i] = src[i];
         for (int i = threadIdx.x; i < p.cout; i += THREADS) bl[i] = p.bias ? p.bias[i] : 0.f;
     }
+    constexpr bool GRAD = ACT == kReluGrad || ACT == kGeluGrad;
+    static_assert(!GRAD || RES, "the gradient modes read aux through the residual pointer");
+    // gradient modes: every wavefront sums y per output channel in a row of its own (LDS)
+    float *gs = bl + p.cout + (threadIdx.x >> 6) * p.cout;
+    if constexpr (GRAD)
+        for (int i = threadIdx.x; i < WAVES * p.cout; i += THREADS) bl[p.cout + i] = 0.f;
     __syncthreads();
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // tile indices stay scalar
@@ -201,12 +213,37 @@ __global__ void __launch_bounds__(THREADS) gemm_kernel(Params p)
                     const int j = 4 * q + jj;
                     const long long at = at0 + (long long)(8 * q + jj) * p.n;
                     const float z0 = acc0[j], z1 = acc1[j];
-                    if (p.zkeep) words(p.zkeep + at)[yw] = pack_bf16x2(z0, z1);
-                    float y0 = epilogue::act_fwd<ACT>(z0 + bq[jj]), y1 = epilogue::act_fwd<ACT>(z1 + bq[jj]);
-                    if constexpr (RES) y0 += lo_bf16(rw[j]), y1 += hi_bf16(rw[j]);
+                    float y0, y1;
+                    if constexpr (GRAD) {
+                        constexpr int A = ACT == kGeluGrad ? epilogue::kGelu : epilogue::kRelu;
+                        y0 = z0 * epilogue::act_grad<A>(lo_bf16(rw[j]) + bq[jj]);
+                        y1 = z1 * epilogue::act_grad<A>(hi_bf16(rw[j]) + bq[jj]);
+                        // the channel's sum over the tile's 64 voxels: the 32 lanes of this half
+                        float t = y0 + y1;
+#pragma unroll
+                        for (int m = 1; m < 32; m <<= 1) t += __shfl_xor(t, m);
+                        if (p.gpart && n32 == 0) gs[32 * c + 8 * q + 4 * kb + jj] += t;
+                    } else {
+                        if (p.zkeep) words(p.zkeep + at)[yw] = pack_bf16x2(z0, z1);
+                        y0 = epilogue::act_fwd<ACT>(z0 + bq[jj]), y1 = epilogue::act_fwd<ACT>(z1 + bq[jj]);
+                        if constexpr (RES) y0 += lo_bf16(rw[j]), y1 += hi_bf16(rw[j]);
+                    }
                     words(p.y + at)[yw] = pack_bf16x2(y0, y1);
                 }
             }
+        }
+    }
+    if constexpr (GRAD) {
+        // (only this wavefront touched its row; lanes 0 and 32 wrote it, all lanes read it)
+        if (p.gpart) {
+            __builtin_amdgcn_wave_barrier();
+            const int g = (int)blockIdx.x * WAVES + wave;
+            float *row = p.gpart + (long long)g * p.cout;
+            for (int i = lane; i < p.cout; i += 64) row[i] = gs[i];
+            // rows beyond the launch's wavefronts read zero (written here, not by a memset, so
+            // that the call can be recorded into a graph)
+            for (int r = g + nwaves; r < kMaxParts; r += nwaves)
+                for (int i = lane; i < p.cout; i += 64) p.gpart[(long long)r * p.cout + i] = 0.f;
         }
     }
 }

@@ -440,6 +440,60 @@ class Linear(nn.Module):
         return y.view(shape[0], -1, *shape[2:])
 
 
+class _FusedMLP(torch.autograd.Function):
+    """``W2 gelu(W1 x + b1) + b2 + residual`` on contiguous bfloat16 ``(B, C, N)`` tensors as ONE
+    autograd node on the library's streaming GEMM (layers/mlp.py:40-63 with the block's sum,
+    deconver.py:60-64): two launches forward (the GELU and the kept pre-activation leave the
+    first, bias and residual ride on the second), and a backward in which the input gradient
+    of the second projection comes out already multiplied by the GELU's derivative, with the
+    first bias's gradient summed in the same kernel -- the hidden tensor's gradient is written
+    once and never read back by an activation pass."""
+
+    @staticmethod
+    def applies(lib, x: torch.Tensor, hidden: int, cout: int) -> bool:
+        B, c, n = x.shape
+        ok = lambda cin, co: lib.pointwise_gemm_supported(cin, co, n, _lib.NDC_BF16)   # noqa: E731
+        return (x.is_cuda and x.dtype == torch.bfloat16 and ok(c, hidden) and ok(hidden, cout)
+                and ok(cout, hidden) and ok(hidden, c))
+
+    @staticmethod
+    def forward(ctx, x, w1, b1, w2, b2, residual):
+        lib = _lib.get_library()
+        hidden, cout = w1.shape[0], w2.shape[0]
+        b1f = None if b1 is None else b1.detach().float().contiguous()
+        b2f = None if b2 is None else b2.detach().float().contiguous()
+        with torch.cuda.device(x.device):
+            a, z = ops.pointwise_gemm(lib, x, ops.pointwise_pack(lib, w1.detach().contiguous()), hidden, b1f,
+                                      None, "gelu", keep_z=True)
+            y, _ = ops.pointwise_gemm(lib, a, ops.pointwise_pack(lib, w2.detach().contiguous()), cout, b2f,
+                                      residual, None)
+        ctx.save_for_backward(x, z, a, w1.detach().to(x.dtype), w2.detach().to(x.dtype), b1f)
+        ctx.dtypes = (w1.dtype, w2.dtype)
+        return y
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, gy):
+        x, z, a, w1, w2, b1f = ctx.saved_tensors
+        lib = _lib.get_library()
+        gy = gy.contiguous()
+        need_x, need_w1, need_b1, need_w2, need_b2, need_res = ctx.needs_input_grad
+        gx = gw1 = gb1 = gw2 = gb2 = None
+        with torch.cuda.device(gy.device):
+            if need_b2:
+                gb2 = ops.channel_sums(lib, gy)
+            if need_w2:
+                gw2 = projection_weight_grad(gy, a, ctx.dtypes[1])
+            if need_x or need_w1 or need_b1:
+                gz, gb1 = ops.pointwise_gemm_actgrad(lib, gy, ops.pointwise_pack(lib, w2, transposed=True),
+                                                     w2.shape[1], z, b1f, "gelu", need_bias_grad=need_b1)
+                if need_w1:
+                    gw1 = projection_weight_grad(gz, x, ctx.dtypes[0])
+                if need_x:
+                    gx = project_back(w1, gz)
+        return gx, gw1, gb1, gw2, gb2, (gy if need_res else None)
+
+
 class MLP(nn.Module):
     """Linear - GELU - Linear on channels, with dropout after each (layers/mlp.py:40-63)."""
 
@@ -465,9 +519,28 @@ class MLP(nn.Module):
         idle = lambda d: d.p == 0 or not d.training   # noqa: E731
         if (isinstance(first, Linear) and isinstance(second, Linear) and type(act) is nn.GELU
                 and act.approximate == "none" and idle(drop1) and idle(drop2)):
-            return second(first(x, act="gelu"), residual=residual)
+            fused = self._fused(first, second, x, residual)
+            return second(first(x, act="gelu"), residual=residual) if fused is None else fused
         y = self.block(x)
         return y if residual is None else residual + y
+
+    @staticmethod
+    def _fused(first: "Linear", second: "Linear", x: torch.Tensor, residual: Optional[torch.Tensor]):
+        """The block as one node on the streaming GEMM where all four of its products fit it
+        (bfloat16, stored or under autocast; e.g. 64 -> 256 -> 64 channels), else None."""
+        if not _gemm_route(x):
+            return None
+        dtype = torch.get_autocast_dtype(x.device.type) if torch.is_autocast_enabled(x.device.type) else x.dtype
+        if dtype != torch.bfloat16:
+            return None
+        flat = x.flatten(2).to(dtype).contiguous()
+        w1, w2 = first.linear.weight.squeeze(-1), second.linear.weight.squeeze(-1)
+        if not _FusedMLP.applies(_lib.get_library(), flat, w1.shape[0], w2.shape[0]):
+            return None
+        res = None if residual is None else residual.flatten(2).to(dtype).contiguous()
+        with torch.autocast(x.device.type, enabled=False):
+            y = _FusedMLP.apply(flat, w1, first.linear.bias, w2, second.linear.bias, res)
+        return y.view(x.shape[0], -1, *x.shape[2:])
 
 
 class _ChannelNorm(torch.autograd.Function):

@@ -57,7 +57,13 @@ class DeconvMixer(nn.Module):
     def forward(self, x: Tensor, residual: Optional[Tensor] = None) -> Tensor:
         """The mixer's output, plus ``residual`` if given (the block's ``x + dcm(...)``, which
         then rides on ``out_proj`` unless dropout is active)."""
-        sources = self.deconv(self.act(self.in_proj(x)))
+        if type(self.act) is nn.ReLU and not self.act._forward_hooks and layers._gemm_route(x):
+            # the rectifier rides on the projection (one kernel, or one pass over its output);
+            # a hooked activation module is still called as a module
+            h = self.in_proj(x, act="relu")
+        else:
+            h = self.act(self.in_proj(x))
+        sources = self.deconv(h)
         if self.dropout.p == 0 or not self.training:
             return self.out_proj(sources, residual=residual)
         y = self.dropout(self.out_proj(sources))

@@ -320,6 +320,29 @@ def pointwise_gemm(lib: _lib.NdcLibrary, x: Tensor, wfrag: Tensor, cout: int, bi
     return y, z
 
 
+def pointwise_gemm_actgrad(lib: _lib.NdcLibrary, gy: Tensor, wfrag: Tensor, cout: int, z: Tensor,
+                           bias: Optional[Tensor], act: str, need_bias_grad: bool = True):
+    """``(gz, gbias)`` with ``gz = (W gy) * act'(z + bias)`` for contiguous bfloat16 ``gy``
+    (B, cin, n), packed ``W`` (cout x cin) and ``z`` (B, cout, n): the input gradient of a
+    projection taken through the activation that made its input.  ``gbias``: the sum of ``gz``
+    over batch and voxels, float32 (None unless ``need_bias_grad``)."""
+    B, cin, n = gy.shape
+    if wfrag.numel() != cin * cout or wfrag.dtype != torch.bfloat16:
+        raise ValueError("wfrag does not belong to this projection")
+    if z.shape != (B, cout, n) or z.dtype != gy.dtype or not z.is_contiguous():
+        raise ValueError("z must be contiguous, of the output's shape and dtype")
+    if bias is not None and (bias.dtype != torch.float32 or bias.numel() != cout or not bias.is_contiguous()):
+        raise ValueError("bias must be float32 with one entry per output channel")
+    if act not in ("relu", "gelu"):
+        raise ValueError("act must be 'relu' or 'gelu'")
+    gz = torch.empty_like(z)
+    gpart = (torch.empty(lib.pointwise_gemm_parts(), cout, dtype=torch.float32, device=gy.device)
+             if need_bias_grad else None)
+    lib.pointwise_gemm_actgrad(_ptr(gy), _ptr(wfrag), _ptr(bias), _ptr(z), _ptr(gz), _ptr(gpart), B, cin, cout,
+                               n, ACTS[act], _lib.NDC_BF16, _stream_of(gy))
+    return gz, (gpart.sum(0) if need_bias_grad else None)
+
+
 def regroup2_applies(fine_shape, dtype, *ptrs) -> bool:
     """Whether ``ndc_regroup`` takes a fine-grid tensor ``(B, C, [D,] H, W)``: float32 or
     bfloat16, even extents, rows of whole 16-byte vectors, 16-byte aligned buffers."""

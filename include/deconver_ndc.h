@@ -341,6 +341,20 @@ int ndc_pointwise_pack(const void *w, int w_dtype, int transposed, void *wfrag, 
 int ndc_pointwise_gemm(const void *x, const void *wfrag, const float *bias, const void *residual, void *y,
                        void *zkeep, int64_t batch, int64_t cin, int64_t cout, int64_t n, int act, int dtype,
                        void *stream);
+/*
+ * The input gradient of a projection whose INPUT was act(z + bias) (the second projection of
+ * the MLP, deconver/layers/mlp.py:40-63, whose input is the GELU of the first one's output),
+ * taken through that activation in the same kernel:
+ *   gz[b][co][i] = ( sum_ci W[co][ci] * gy[b][ci][i] ) * act'(z[b][co][i] + bias[co])
+ * with wfrag the packed TRANSPOSE of the projection's weight (ndc_pointwise_pack with
+ * transposed != 0), act NDC_ACT_RELU or NDC_ACT_GELU, shapes as for ndc_pointwise_gemm.
+ *   gpart          NULL, or ndc_pointwise_gemm_parts() * cout floats: per-wavefront sums of gz
+ *                  (unused rows are zeroed); the gradient of `bias` is the sum over the rows
+ */
+int64_t ndc_pointwise_gemm_parts(void);
+int ndc_pointwise_gemm_actgrad(const void *gy, const void *wfrag, const float *bias, const void *z, void *gz,
+                               float *gpart, int64_t batch, int64_t cin, int64_t cout, int64_t n, int act,
+                               int dtype, void *stream);
 
 /*
  * Normalisation over the CHANNEL axis of a channel-first tensor (batch, channels, n):

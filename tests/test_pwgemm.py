@@ -117,3 +117,79 @@ def test_gpu_equals_the_host_build_bit_for_bit_up_to_summation_order():
     lib = _lib.get_library()
     dev, _ = ops.pointwise_gemm(lib, x.cuda(), ops.pointwise_pack(lib, w.cuda()), 64, bias.cuda(), res.cuda())
     assert _rel(dev, host.double()) < 8e-3
+
+
+def _actgrad_reference(gy, w, z, bias, act):
+    """float64: (W gy) * act'(z + bias) and its sum over batch and voxels."""
+    prod = F.conv1d(gy.double(), w.bfloat16().double().unsqueeze(-1))
+    u = (z.double() + bias.double().view(1, -1, 1)).requires_grad_(True)
+    {"relu": torch.relu, "gelu": F.gelu}[act](u).sum().backward()
+    gz = prod * u.grad
+    return gz, gz.sum((0, 2))
+
+
+@pytest.mark.parametrize("act", ["gelu", "relu"])
+def test_activation_gradient_epilogue_on_the_host_build(act):
+    lib = hostcheck_library()
+    g = torch.Generator().manual_seed(4)
+    B, cin, cout, n = 2, 64, 96, 128
+    gy = torch.randn(B, cin, n, generator=g).bfloat16()
+    w = torch.randn(cout, cin, generator=g) / 8
+    z = torch.randn(B, cout, n, generator=g).bfloat16()
+    bias = torch.randn(cout, generator=g)
+    gz, gb = ops.pointwise_gemm_actgrad(lib, gy, ops.pointwise_pack(lib, w), cout, z, bias, act)
+    rz, rb = _actgrad_reference(gy, w, z, bias, act)
+    assert _rel(gz, rz) < 1e-2 and _rel(gb, rb) < 1e-2
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("act", ["gelu", "relu"])
+@pytest.mark.parametrize("B,cin,cout,n", [(2, 64, 256, 64 * 64 * 4), (1, 128, 128, 64 * 9), (2, 256, 64, 4096)])
+def test_gpu_activation_gradient_epilogue(act, B, cin, cout, n):
+    lib = _lib.get_library()
+    g = torch.Generator().manual_seed(5)
+    gy = torch.randn(B, cin, n, generator=g).bfloat16()
+    w = torch.randn(cout, cin, generator=g) / cin ** 0.5
+    z = torch.randn(B, cout, n, generator=g).bfloat16()
+    bias = torch.randn(cout, generator=g)
+    gz, gb = ops.pointwise_gemm_actgrad(lib, gy.cuda(), ops.pointwise_pack(lib, w.cuda()), cout, z.cuda(),
+                                        bias.cuda(), act)
+    rz, rb = _actgrad_reference(gy, w, z, bias, act)
+    assert _rel(gz, rz) < 1e-2
+    assert gb.dtype == torch.float32 and _rel(gb, rb) < 2e-3
+    gz2, none = ops.pointwise_gemm_actgrad(lib, gy.cuda(), ops.pointwise_pack(lib, w.cuda()), cout, z.cuda(),
+                                           bias.cuda(), act, need_bias_grad=False)
+    assert none is None and torch.equal(gz, gz2)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("with_residual", [False, True])
+def test_mlp_as_one_node_matches_float64(with_residual):
+    """The 64 -> 256 -> 64 MLP of the network's first level under bf16 autocast: forward, input,
+    residual and parameter gradients against the same module in float64 on the CPU."""
+    import copy
+    from deconver_amd.layers import MLP, _FusedMLP
+    torch.manual_seed(6)
+    mlp = MLP(64)
+    ref = copy.deepcopy(mlp).double()
+    mlp = mlp.cuda()
+    x0, r0 = torch.randn(2, 64, 8, 8, 64), torch.randn(2, 64, 8, 8, 64)
+    g0 = torch.randn(2, 64, 8, 8, 64)
+    x = x0.cuda().bfloat16().requires_grad_(True)
+    r = r0.cuda().bfloat16().requires_grad_(True) if with_residual else None
+    assert _FusedMLP.applies(_lib.get_library(), x.flatten(2), 256, 64)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        y = mlp(x, residual=r)
+    assert y.dtype == torch.bfloat16
+    assert "_FusedMLP" in type(y.grad_fn.next_functions[0][0]).__name__   # (under the final view)
+    y.backward(g0.cuda().bfloat16())
+    xr = x.detach().double().cpu().requires_grad_(True)
+    rr = r.detach().double().cpu().requires_grad_(True) if with_residual else None
+    yr = ref(xr, residual=rr)
+    yr.backward(g0.bfloat16().double())
+    assert _rel(y.detach(), yr.detach()) < 1e-2
+    assert _rel(x.grad, xr.grad) < 2e-2
+    if with_residual:
+        assert _rel(r.grad, rr.grad) < 1e-2
+    for (name, p), (_, q) in zip(mlp.named_parameters(), ref.named_parameters()):
+        assert p.grad.dtype == torch.float32 and _rel(p.grad, q.grad) < 2e-2, name
