@@ -523,9 +523,14 @@ int ndc_bias_act_backward(const void *gy, const void *z, const float *bias, void
 int ndc_pointwise_gemm_supported(int64_t cin, int64_t cout, int64_t n, int dtype)
 {
     if (dtype != NDC_BF16) return 0;
-    if (cin != 64 && cin != 128 && cin != 256) return 0;
+    // up to 256 input channels held whole in registers, any width of output; or many input
+    // channels in chunks of 128 with the accumulators of at most 128 output channels
+    const bool whole = cin == 64 || cin == 128 || cin == 256;
+    const bool deep = cin > 256 && cin % 128 == 0 && cin <= 4096 && cout <= 128;
+    if (!whole && !deep) return 0;
     if (cout < 32 || cout % 32 || cout > 4096) return 0;
-    if (cin * cout * 2 > 128 * 1024) return 0;        // the packed weights stay in LDS
+    if (cin * cout * 2 > 128 * 1024) return 0;        // the packed weights stay in LDS,
+    if (cin * cout * 2 + cout * 36 > 160 * 1024) return 0;   // with the bias and eight rows of sums
     if (n < 64 || n % 64) return 0;
     return 1;
 }
@@ -575,7 +580,7 @@ int ndc_pointwise_gemm_actgrad(const void *gy, const void *wfrag, const float *b
     if (!gy || !wfrag || !z || !gz) return NDC_ERR_NULL;
     if (dtype != NDC_BF16) return NDC_ERR_DTYPE;
     if (batch < 1 || (act != NDC_ACT_RELU && act != NDC_ACT_GELU)) return NDC_ERR_GEOMETRY;
-    if (!ndc_pointwise_gemm_supported(cin, cout, n, dtype)) return NDC_ERR_GEOMETRY;
+    if (!ndc_pointwise_gemm_supported(cin, cout, n, dtype) || cin > 256) return NDC_ERR_GEOMETRY;
     if ((long double)batch * (cin > cout ? cin : cout) * n > 9.0e15L) return NDC_ERR_GEOMETRY;
     if (batch * (n / 64) > 0x7fffff00LL || n > 0x3fffffffLL) return NDC_ERR_GEOMETRY;
     if (((uintptr_t)gy & 3u) || ((uintptr_t)gz & 3u) || ((uintptr_t)z & 3u) || ((uintptr_t)wfrag & 15u) ||

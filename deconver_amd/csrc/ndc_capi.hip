@@ -465,7 +465,7 @@ struct Backend {
         int per_cu = resident[cls].load(std::memory_order_relaxed);
         if (per_cu == 0) {
             // (asked for the largest LDS size of the class, so that the answer holds for all of it)
-            const size_t worst = cls == 0 ? 40 * 1024 : cls == 1 ? 80 * 1024 : 136 * 1024;
+            const size_t worst = cls == 0 ? 40 * 1024 : cls == 1 ? 80 * 1024 : 160 * 1024;
             if (worst > 64 * 1024 &&
                 hipFuncSetAttribute((const void *)entry, hipFuncAttributeMaxDynamicSharedMemorySize, (int)worst) != hipSuccess)
                 return -5;
@@ -498,8 +498,11 @@ struct Backend {
 #define NDC_PWGEMM_RES(ACT)                                                                 \
     (p.res ? pwgemm_launch<CIN, ACT, true, THREADS>(p, lds, stream)                         \
            : pwgemm_launch<CIN, ACT, false, THREADS>(p, lds, stream))
-        if (act == pwgemm::kGeluGrad) return pwgemm_launch<CIN, pwgemm::kGeluGrad, true, THREADS>(p, lds + (size_t)(THREADS / 64) * p.cout * 4, stream);
-        if (act == pwgemm::kReluGrad) return pwgemm_launch<CIN, pwgemm::kReluGrad, true, THREADS>(p, lds + (size_t)(THREADS / 64) * p.cout * 4, stream);
+        // gradient modes hold a row of sums per wavefront in LDS as well
+        const size_t glds = lds + (size_t)(THREADS / 64) * p.cout * 4;
+        if (act >= pwgemm::kReluGrad && glds > 160 * 1024) return -2;
+        if (act == pwgemm::kGeluGrad) return pwgemm_launch<CIN, pwgemm::kGeluGrad, true, THREADS>(p, glds, stream);
+        if (act == pwgemm::kReluGrad) return pwgemm_launch<CIN, pwgemm::kReluGrad, true, THREADS>(p, glds, stream);
         if (act == epilogue::kRelu) return NDC_PWGEMM_RES(epilogue::kRelu);
         if (act == epilogue::kGelu) return NDC_PWGEMM_RES(epilogue::kGelu);
         return NDC_PWGEMM_RES(epilogue::kNone);
@@ -508,6 +511,46 @@ struct Backend {
 
     // y = act(W x + bias) + residual on persistent workgroups; the caller has checked the shape
     // (cin in {64, 128, 256}, cout a multiple of 32, n a multiple of 64, packed weights <= 128 KB)
+    template <int CT, int ACT, bool RES>
+    static int pwgemm_deep_launch(const pwgemm::Params &p, int cin, size_t lds, void *stream)
+    {
+        constexpr int THREADS = 512;
+        void (*entry)(pwgemm::Params, int) = pwgemm::gemm_kernel_deep<CT, ACT, RES, THREADS>;
+        static std::atomic<int> resident[2] = {{0}, {0}};
+        const int cls = lds <= 72 * 1024 ? 0 : 1;
+        int per_cu = resident[cls].load(std::memory_order_relaxed);
+        if (per_cu == 0) {
+            const size_t worst = cls == 0 ? 72 * 1024 : 160 * 1024;
+            if (hipFuncSetAttribute((const void *)entry, hipFuncAttributeMaxDynamicSharedMemorySize, (int)worst) != hipSuccess)
+                return -5;
+            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void *)entry, THREADS, worst) != hipSuccess ||
+                per_cu < 1)
+                per_cu = 1;
+            resident[cls].store(per_cu, std::memory_order_relaxed);
+        }
+        int dev = 0, cus = 256;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1)
+            cus = 256;
+        long long blocks = (long long)cus * per_cu;
+        const long long need = ((long long)p.tiles + THREADS / 64 - 1) / (THREADS / 64);
+        if (blocks > need) blocks = need;
+        hipLaunchKernelGGL(entry, dim3((unsigned)blocks), dim3(THREADS), lds, (hipStream_t)stream, p, cin);
+        return check();
+    }
+
+    template <int CT>
+    static int pwgemm_deep(const pwgemm::Params &p, int cin, size_t lds, int act, void *stream)
+    {
+#define NDC_PWGEMM_DEEP(ACT)                                                             \
+    (p.res ? pwgemm_deep_launch<CT, ACT, true>(p, cin, lds, stream)                      \
+           : pwgemm_deep_launch<CT, ACT, false>(p, cin, lds, stream))
+        if (act == epilogue::kRelu) return NDC_PWGEMM_DEEP(epilogue::kRelu);
+        if (act == epilogue::kGelu) return NDC_PWGEMM_DEEP(epilogue::kGelu);
+        return NDC_PWGEMM_DEEP(epilogue::kNone);
+#undef NDC_PWGEMM_DEEP
+    }
+
     // act 3 / 4: y = (W x) * relu' / gelu'(res + bias), gpart (kMaxParts x cout, or null) receives
     // per-wavefront sums of y whose total over the rows is the bias gradient
     static int pwgemm(const void *x, const void *wfrag, const float *bias, const void *res, void *y, void *zkeep,
@@ -521,8 +564,18 @@ struct Backend {
         if (p.tiles <= 0) return 0;
         const size_t wbytes = (size_t)cin * cout * 2;
         const size_t lds = wbytes + (size_t)cout * 4;   // packed weights, bias
+        if (cin > 256) {   // many input channels, at most 128 output channels (checked by the caller)
+            if (act > epilogue::kGelu) return -2;
+            switch (cout / 32) {
+            case 1: return pwgemm_deep<1>(p, cin, lds, act, stream);
+            case 2: return pwgemm_deep<2>(p, cin, lds, act, stream);
+            case 3: return pwgemm_deep<3>(p, cin, lds, act, stream);
+            default: return pwgemm_deep<4>(p, cin, lds, act, stream);
+            }
+        }
         // small weight tables: several workgroups per CU; large ones: one, of more wavefronts
-        const int threads = wbytes <= 32 * 1024 ? 256 : wbytes <= 64 * 1024 || cin == 256 ? 512 : 1024;
+        int threads = wbytes <= 32 * 1024 ? 256 : wbytes <= 64 * 1024 || cin == 256 ? 512 : 1024;
+        if (act >= pwgemm::kReluGrad && lds + (size_t)(threads / 64) * cout * 4 > 160 * 1024) threads = 512;
 #define NDC_PWGEMM(CIN)                                                                            \
     (threads == 256 ? pwgemm_act<CIN, 256>(p, lds, act, stream)                                     \
      : threads == 512 ? pwgemm_act<CIN, 512>(p, lds, act, stream)                                   \

@@ -103,7 +103,7 @@ __device__ inline uint32_t *words(uint16_t *p) { return reinterpret_cast<uint32_
 
 // the 8 words (voxel 2n, voxel 2n + 1) of every k-step of a tile; xw: lane offset 4 kb n + n32
 template <int S>
-__device__ inline void request_x(const Params &p, int tile, int cin, uint32_t xw, uint32_t (&raw)[S][8])
+__device__ inline void request_x(const Params &p, int tile, int cin, uint32_t xw, uint32_t (&raw)[S][8], int k0 = 0)
 {
     // (the quotient comes out of vector arithmetic; as a scalar again it keeps the pointers scalar)
     const int b = __builtin_amdgcn_readfirstlane(tile / p.tiles_per_sample);
@@ -111,7 +111,7 @@ __device__ inline void request_x(const Params &p, int tile, int cin, uint32_t xw
 #pragma unroll
     for (int s = 0; s < S; ++s)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) raw[s][e] = words(xb + (long long)(16 * s + e) * p.n)[xw];
+        for (int e = 0; e < 8; ++e) raw[s][e] = words(xb + (long long)(k0 + 16 * s + e) * p.n)[xw];
 }
 
 // ... into the fragments of the even-voxel tile and the odd-voxel tile
@@ -128,6 +128,30 @@ __device__ inline void split_x(const uint32_t (&raw)[S][8], bf16x8 (&xf)[S][2])
         }
         xf[s][0] = __builtin_bit_cast(bf16x8, even);
         xf[s][1] = __builtin_bit_cast(bf16x8, odd);
+    }
+}
+
+// The epilogue of one 32-channel output tile (forward modes).  Register j of a lane holds output
+// row 8 * (j / 4) + 4 * kb + j % 4, column n32, of the even-voxel tile (acc0) and the odd-voxel
+// tile (acc1): one output word.  rw: the residual words, requested by the caller.
+template <int ACT, bool RES>
+__device__ inline void finish_tile(const Params &p, const f32x16 &acc0, const f32x16 &acc1, const uint32_t (&rw)[16],
+                                   const float *bl, int c, long long at0, uint32_t yw, int kb)
+{
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const float4 t4 = *reinterpret_cast<const float4 *>(bl + 32 * c + 8 * q + 4 * kb);
+        const float bq[4] = {t4.x, t4.y, t4.z, t4.w};
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+            const int j = 4 * q + jj;
+            const long long at = at0 + (long long)(8 * q + jj) * p.n;
+            const float z0 = acc0[j], z1 = acc1[j];
+            if (p.zkeep) words(p.zkeep + at)[yw] = pack_bf16x2(z0, z1);
+            float y0 = epilogue::act_fwd<ACT>(z0 + bq[jj]), y1 = epilogue::act_fwd<ACT>(z1 + bq[jj]);
+            if constexpr (RES) y0 += lo_bf16(rw[j]), y1 += hi_bf16(rw[j]);
+            words(p.y + at)[yw] = pack_bf16x2(y0, y1);
+        }
     }
 }
 
@@ -206,8 +230,8 @@ __global__ void __launch_bounds__(THREADS) gemm_kernel(Params p)
             }
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const float4 t = *reinterpret_cast<const float4 *>(bl + 32 * c + 8 * q + 4 * kb);
-                const float bq[4] = {t.x, t.y, t.z, t.w};
+                const float4 t4 = *reinterpret_cast<const float4 *>(bl + 32 * c + 8 * q + 4 * kb);
+                const float bq[4] = {t4.x, t4.y, t4.z, t4.w};
 #pragma unroll
                 for (int jj = 0; jj < 4; ++jj) {
                     const int j = 4 * q + jj;
@@ -244,6 +268,69 @@ __global__ void __launch_bounds__(THREADS) gemm_kernel(Params p)
             // that the call can be recorded into a graph)
             for (int r = g + nwaves; r < kMaxParts; r += nwaves)
                 for (int i = lane; i < p.cout; i += 64) p.gpart[(long long)r * p.cout + i] = 0.f;
+        }
+    }
+}
+
+// Many input channels, at most 128 output channels (the projections back from the widened
+// tensors: 512 -> 128): the accumulators of ALL CT output tiles stay in registers while the
+// input channels go by in chunks of 128, so that x is still read once.  p.cin: a multiple of 128.
+template <int CT, int ACT, bool RES, int THREADS>
+__global__ void __launch_bounds__(THREADS) gemm_kernel_deep(Params p, int cin)
+{
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    constexpr int WAVES = THREADS / 64;
+    constexpr int SC = 8;                    // k-steps per chunk of 128 input channels
+    static_assert(ACT <= epilogue::kGelu, "no gradient modes here");
+    const int S = cin / 16, chunks_k = cin / 128;
+    u32x4 *wl = reinterpret_cast<u32x4 *>(smem);
+    float *bl = reinterpret_cast<float *>(smem + (size_t)CT * S * 64 * 16);
+    {
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(p.wfrag);
+        const int chunks = CT * S * 64;
+        for (int i = threadIdx.x; i < chunks; i += THREADS) wl[i] = src[i];
+        for (int i = threadIdx.x; i < 32 * CT; i += THREADS) bl[i] = p.bias ? p.bias[i] : 0.f;
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n32 = lane & 31, kb = lane >> 5;
+    const uint32_t xw = (uint32_t)(4 * kb) * (uint32_t)p.n + n32;
+    const uint32_t yw = (uint32_t)(2 * kb) * (uint32_t)p.n + n32;
+    const int nwaves = (int)gridDim.x * WAVES;
+    for (int tile = (int)blockIdx.x * WAVES + wave; tile < p.tiles; tile += nwaves) {
+        const int b = __builtin_amdgcn_readfirstlane(tile / p.tiles_per_sample);
+        f32x16 acc[CT][2];
+#pragma unroll
+        for (int c = 0; c < CT; ++c) acc[c][0] = f32x16{}, acc[c][1] = f32x16{};
+#pragma unroll 1
+        for (int kc = 0; kc < chunks_k; ++kc) {
+            uint32_t raw[SC][8];
+            request_x<SC>(p, tile, cin, xw, raw, 128 * kc);
+            bf16x8 xf[SC][2];
+            split_x<SC>(raw, xf);
+#pragma unroll
+            for (int c = 0; c < CT; ++c) {
+                const u32x4 *wt = wl + (c * S + kc * SC) * 64 + lane;
+#pragma unroll
+                for (int s = 0; s < SC; ++s) {
+                    const bf16x8 wf = __builtin_bit_cast(bf16x8, wt[s * 64]);
+                    acc[c][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf, xf[s][0], acc[c][0], 0, 0, 0);
+                    acc[c][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf, xf[s][1], acc[c][1], 0, 0, 0);
+                }
+            }
+        }
+        const long long out0 = (long long)b * p.cout * p.n + (long long)(tile - b * p.tiles_per_sample) * kTileVoxels;
+#pragma unroll
+        for (int c = 0; c < CT; ++c) {
+            const long long at0 = out0 + (long long)(32 * c) * p.n;
+            uint32_t rw[16];
+            if constexpr (RES) {
+#pragma unroll
+                for (int j = 0; j < 16; ++j)
+                    rw[j] = words(p.res + at0 + (long long)(8 * (j / 4) + j % 4) * p.n)[yw];
+            }
+            finish_tile<ACT, RES>(p, acc[c][0], acc[c][1], rw, bl, c, at0, yw, kb);
         }
     }
 }

@@ -320,9 +320,10 @@ int ndc_bias_act_backward(const void *gy, const void *z, const float *bias, void
  * deconver/deconver.py:41-46, 60-64 and deconver/layers/mlp.py:40-63 apply to its output).
  * A streaming kernel on the matrix units: x is read once, y written once, float32 accumulation,
  * one rounding of the result.
- *   ndc_pointwise_gemm_supported  1 where the kernel applies: NDC_BF16, cin 64, 128 or 256,
- *                  cout a multiple of 32, cin * cout * 2 <= 128 KiB, n a multiple of 64; else 0
- *                  (callers then use a library GEMM and ndc_bias_act)
+ *   ndc_pointwise_gemm_supported  1 where the kernel applies: NDC_BF16; cin 64, 128 or 256, or a
+ *                  larger multiple of 128 with cout <= 128; cout a multiple of 32;
+ *                  cin * cout * 2 <= 128 KiB; n a multiple of 64; else 0 (callers then use a
+ *                  library GEMM and ndc_bias_act)
  *   ndc_pointwise_pack  writes W in the order the kernel reads it into wfrag
  *                  (ndc_pointwise_weight_bytes(cin, cout) bytes, 16-byte aligned): the 8 values
  *                  W[32 c + l % 32][16 s + 8 (l / 32) + 0..7], as bf16, at element
@@ -347,7 +348,8 @@ int ndc_pointwise_gemm(const void *x, const void *wfrag, const float *bias, cons
  * taken through that activation in the same kernel:
  *   gz[b][co][i] = ( sum_ci W[co][ci] * gy[b][ci][i] ) * act'(z[b][co][i] + bias[co])
  * with wfrag the packed TRANSPOSE of the projection's weight (ndc_pointwise_pack with
- * transposed != 0), act NDC_ACT_RELU or NDC_ACT_GELU, shapes as for ndc_pointwise_gemm.
+ * transposed != 0), act NDC_ACT_RELU or NDC_ACT_GELU, shapes as for ndc_pointwise_gemm with
+ * cin <= 256.
  *   gpart          NULL, or ndc_pointwise_gemm_parts() * cout floats: per-wavefront sums of gz
  *                  (unused rows are zeroed); the gradient of `bias` is the sum over the rows
  */

@@ -37,7 +37,8 @@ def test_support_predicate():
     assert lib.pointwise_gemm_supported(64, 256, 128 ** 3, bf)
     assert lib.pointwise_gemm_supported(256, 64, 64, bf) and lib.pointwise_gemm_supported(128, 512, 4096, bf)
     assert not lib.pointwise_gemm_supported(64, 256, 128 ** 3, f32)       # bfloat16 only
-    assert not lib.pointwise_gemm_supported(512, 128, 4096, bf)           # 512 input channels
+    assert lib.pointwise_gemm_supported(512, 128, 4096, bf)               # many input channels: up to 128 out
+    assert not lib.pointwise_gemm_supported(512, 256, 4096, bf) and not lib.pointwise_gemm_supported(320, 64, 4096, bf)
     assert not lib.pointwise_gemm_supported(256, 512, 4096, bf)           # weights beyond 128 KiB
     assert not lib.pointwise_gemm_supported(64, 48, 4096, bf)             # cout not a multiple of 32
     assert not lib.pointwise_gemm_supported(64, 64, 100, bf)              # n not a multiple of 64
@@ -57,7 +58,7 @@ def test_pack_order_on_the_host_build(transposed, dtype):
     assert torch.equal(frag, want)
 
 
-@pytest.mark.parametrize("B,cin,cout,n", [(2, 64, 96, 128), (1, 128, 32, 64), (1, 256, 64, 64)])
+@pytest.mark.parametrize("B,cin,cout,n", [(2, 64, 96, 128), (1, 128, 32, 64), (1, 256, 64, 64), (1, 384, 64, 64)])
 @pytest.mark.parametrize("act,with_bias,with_res,keep", [(None, False, False, False), (None, True, True, False),
                                                           ("gelu", True, False, True), ("relu", False, True, True)])
 def test_host_build_matches_float64(B, cin, cout, n, act, with_bias, with_res, keep):
@@ -89,7 +90,8 @@ def test_bad_arguments_are_refused():
 @pytest.mark.gpu
 @pytest.mark.parametrize("B,cin,cout,n", [
     (2, 64, 256, 64 * 64 * 8), (2, 256, 64, 64 * 64 * 8), (1, 64, 64, 4096), (2, 128, 512, 32 ** 3),
-    (3, 128, 128, 64 * 33), (1, 256, 256, 64 * 7), (2, 64, 32, 64)])
+    (3, 128, 128, 64 * 33), (1, 256, 256, 64 * 7), (2, 64, 32, 64),
+    (2, 512, 128, 64 * 64 * 4), (1, 512, 64, 64 * 5), (1, 1024, 32, 128), (2, 384, 96, 64 * 3)])
 @pytest.mark.parametrize("act,with_bias,with_res,keep", [(None, False, False, False), (None, True, True, False),
                                                           ("gelu", True, False, True), ("relu", False, False, False)])
 def test_gpu_matches_float64(B, cin, cout, n, act, with_bias, with_res, keep):
