@@ -766,7 +766,8 @@ BLOCK_SHAPES = [("config 4, level 0: B 2, 64 ch, 128^3", 2, 64, 128 ** 3),
 
 def block_rows(torch, steps: int, warmup: int) -> list:
     """The HBM-bound kernels between the NDC layers of a Deconver block (InstanceNorm as row
-    normalisation, and the bias / GELU / residual pass after a 1x1 projection), bf16, forward and
+    normalisation, the bias / GELU / residual pass after a 1x1 projection, and the projections
+    themselves on the streaming GEMM), bf16, forward and
     backward, next to PyTorch's own kernels for the same arithmetic: ms and achieved GB/s on
     the bytes each must move (U = B*C*N elements of 2 bytes: norm forward 3 U, backward 5 U;
     bias + GELU on the 4C hidden tensor forward 8 U, backward 12 U; bias + residual 3 U)."""
@@ -841,7 +842,35 @@ def block_rows(torch, steps: int, warmup: int) -> list:
         put("bias_residual", timed(lambda: ops.bias_act(lib, z1, b1, res, None)), 3 * U)
         b1h = b1.bfloat16().view(1, -1, 1)
         put("bias_residual_pytorch", timed(lambda: res + (z1 + b1h)), 3 * U)
-        del z1, res
+        del z1
+        # the 1x1 projections themselves: the library's streaming GEMM next to hipBLASLt (one
+        # batched launch with the weight shared through a zero stride), where the kernel applies
+        if lib.pointwise_gemm_supported(C, 4 * C, n, _lib.NDC_BF16) and lib.pointwise_gemm_supported(4 * C, C, n, _lib.NDC_BF16):
+            xs = torch.randn(B, C, n, device=dev).bfloat16()
+            hs = torch.randn(B, 4 * C, n, device=dev).bfloat16()
+            w_up = torch.randn(4 * C, C, device=dev) / C ** 0.5
+            w_dn = torch.randn(C, 4 * C, device=dev) / (4 * C) ** 0.5
+            f_up, f_dn, f_sq = (ops.pointwise_pack(lib, w) for w in (w_up, w_dn, w_dn[:, :C].contiguous()))
+            f_upT = ops.pointwise_pack(lib, w_dn, transposed=True)     # (C x 4C storage) -> applies 4C x C
+            out_up, out_dn = torch.empty_like(hs), torch.empty_like(xs)
+            up16 = w_up.bfloat16().unsqueeze(0).expand(B, -1, -1)
+            dn16 = w_dn.bfloat16().unsqueeze(0).expand(B, -1, -1)
+            sq16 = w_dn[:, :C].bfloat16().unsqueeze(0).expand(B, -1, -1)
+            put("project_up", timed(lambda: ops.pointwise_gemm(lib, xs, f_up, 4 * C)), 5 * U)
+            put("project_up_hipblaslt", timed(lambda: torch.bmm(up16, xs, out=out_up)), 5 * U)
+            put("project_down", timed(lambda: ops.pointwise_gemm(lib, hs, f_dn, C)), 5 * U)
+            put("project_down_hipblaslt", timed(lambda: torch.bmm(dn16, hs, out=out_dn)), 5 * U)
+            put("project_square", timed(lambda: ops.pointwise_gemm(lib, xs, f_sq, C)), 2 * U)
+            put("project_square_hipblaslt", timed(lambda: torch.bmm(sq16, xs, out=out_dn)), 2 * U)
+            # with their tails: up + bias + GELU keeping the product (1 + 4 + 4 U), down + bias +
+            # residual (4 + 1 + 1 U), and the input gradient of `down` through the GELU with the
+            # bias gradient's sums (1 + 4 + 4 U) -- against GEMM + separate pass above
+            bias4 = torch.randn(4 * C, device=dev)
+            put("project_up_bias_gelu", timed(lambda: ops.pointwise_gemm(lib, xs, f_up, 4 * C, bias4, None, "gelu", keep_z=True)), 9 * U)
+            put("project_down_bias_residual", timed(lambda: ops.pointwise_gemm(lib, hs, f_dn, C, b1, res, None)), 6 * U)
+            put("project_back_through_gelu", timed(lambda: ops.pointwise_gemm_actgrad(lib, xs, f_upT, 4 * C, hs, bias4, "gelu")), 9 * U)
+            del xs, hs, out_up, out_dn
+        del res
         rows.append(r)
         torch.cuda.empty_cache()
     return rows

@@ -185,24 +185,12 @@ __global__ void __launch_bounds__(THREADS) gemm_kernel(Params p)
     const uint32_t xw = (uint32_t)(4 * kb) * (uint32_t)p.n + n32;   // lane offsets in words:
     const uint32_t yw = (uint32_t)(2 * kb) * (uint32_t)p.n + n32;   // 8 kb rows of x, 4 kb rows of y
     const int nwaves = (int)gridDim.x * WAVES;
-    // The x words of a tile are requested one tile ahead where the registers allow it (up to 128
-    // input channels): they then arrive during the previous tile's arithmetic, and -- loads and
-    // stores being counted by one in-order counter -- waiting for them does not wait for the
-    // stores issued after them.  No condition around the requests: past the last tile the
-    // current one is requested again.
-    constexpr bool AHEAD = false;
-    int tile = (int)blockIdx.x * WAVES + wave;
-    uint32_t ahead[AHEAD ? S : 1][8];
-    if constexpr (AHEAD) {
-        if (tile < p.tiles) request_x<S>(p, tile, CIN, xw, ahead);
-    }
-    for (; tile < p.tiles; tile += nwaves) {
+    // (Requesting a tile's words one tile ahead was measured, with 64 and 128 input channels:
+    // no gain at 64, a loss at 128 -- the resident wavefronts already cover the latency.)
+    for (int tile = (int)blockIdx.x * WAVES + wave; tile < p.tiles; tile += nwaves) {
         const int b = __builtin_amdgcn_readfirstlane(tile / p.tiles_per_sample);
         bf16x8 xf[S][2];
-        if constexpr (AHEAD) {
-            split_x<S>(ahead, xf);
-            request_x<S>(p, tile + nwaves < p.tiles ? tile + nwaves : tile, CIN, xw, ahead);
-        } else {
+        {
             uint32_t raw[S][8];
             request_x<S>(p, tile, CIN, xw, raw);
             split_x<S>(raw, xf);
