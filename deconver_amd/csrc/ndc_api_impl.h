@@ -167,7 +167,7 @@ static int direct_gconv(const KGeom &q, const TI *in, const float *h, const floa
 
 extern "C" {
 
-int ndc_version(void) { return 200; }   // 0.2.0: row normalisation, projection tails, regrouping
+int ndc_version(void) { return 300; }   // 0.3.0: the projections themselves (streaming GEMM)
 
 const char *ndc_status_string(int status)
 {
