@@ -102,6 +102,26 @@ static int run_block_level(int dtype)
     if (!st) st = ndc_regroup(fine, coarse, nullptr, rows, C, D, H, W, 1, dtype, 1, nullptr);
     if (!st) st = ndc_regroup(coarse, back, bias, rows, C, D, H, W, 1, dtype, 0, nullptr);
     free(fine); free(coarse); free(back);
+    if (dtype == NDC_BF16) {
+        // the streaming GEMM's host loops: 128 -> 64 channels of 2 x 128 voxels, every tail, the
+        // transposed packing and the gradient mode with its rows of sums
+        const long long cin = 128, cout = 64, nv = 128;
+        void *px = calloc(1, (size_t)(B * cin * nv * 2)), *py = malloc((size_t)(B * cout * nv * 2));
+        void *pz = malloc((size_t)(B * cout * nv * 2)), *pr = calloc(1, (size_t)(B * cout * nv * 2));
+        void *pg = malloc((size_t)(B * cin * nv * 2));
+        float *w = (float *)calloc((size_t)(cin * cout), sizeof(float)), *b64 = (float *)calloc((size_t)cout, sizeof(float));
+        float *b128 = (float *)calloc((size_t)cin, sizeof(float));
+        void *wf = aligned_alloc(16, ndc_pointwise_weight_bytes(cin, cout));
+        void *wft = aligned_alloc(16, ndc_pointwise_weight_bytes(cout, cin));
+        float *sums = (float *)malloc(sizeof(float) * (size_t)(ndc_pointwise_gemm_parts() * cin));
+        if (!st) st = ndc_pointwise_gemm_supported(cin, cout, nv, dtype) ? 0 : -2;
+        if (!st) st = ndc_pointwise_pack(w, NDC_F32, 0, wf, cin, cout, nullptr);
+        if (!st) st = ndc_pointwise_pack(w, NDC_F32, 1, wft, cout, cin, nullptr);   // W^T from W as it lies
+        if (!st) st = ndc_pointwise_gemm(px, wf, b64, pr, py, pz, B, cin, cout, nv, NDC_ACT_GELU, dtype, nullptr);
+        if (!st) st = ndc_pointwise_gemm(px, wf, nullptr, nullptr, py, nullptr, B, cin, cout, nv, NDC_ACT_NONE, dtype, nullptr);
+        if (!st) st = ndc_pointwise_gemm_actgrad(py, wft, b128, px, pg, sums, B, cout, cin, nv, NDC_ACT_GELU, dtype, nullptr);
+        free(px); free(py); free(pz); free(pr); free(pg); free(w); free(b64); free(b128); free(wf); free(wft); free(sums);
+    }
     printf("block-level entry points dtype%d -> status %d\n", dtype, st);
     return st;
 }
