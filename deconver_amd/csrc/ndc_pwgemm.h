@@ -29,7 +29,11 @@
 //
 // Whatever the instruction's internal order of the 16 k-values is, both operands are filled by
 // the same rule (lane half kb, element e <-> channel 16 s + 8 kb + e), so the products pair up.
-// Device code only; float32 accumulation; the output is rounded to bf16 once.
+// Two kernels: gemm_kernel holds the fragments of up to 256 input channels whole and walks the
+// output tiles one after the other (any number of output channels; also the modes that multiply
+// the product by an activation's derivative and sum the result per channel); gemm_kernel_deep
+// takes more input channels in chunks of 128 with the accumulators of all (at most four) output
+// tiles kept.  Device code only; float32 accumulation; the output is rounded to bf16 once.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -49,7 +53,6 @@ static const int kMaxParts = 4096;       // wavefronts of a launch (rows of Para
 // derivative at (aux + bias), aux read through Params::res -- the input gradient of a
 // projection whose INPUT was act(aux + bias) (the MLP's second projection, layers/mlp.py:40-63)
 enum { kReluGrad = 3, kGeluGrad = 4 };
-static const int kMaxLdsBytes = 128 * 1024;   // packed weights a workgroup may hold
 
 struct Params {
     const uint16_t *x;       // (B, cin, n) bf16
