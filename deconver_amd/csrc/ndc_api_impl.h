@@ -565,6 +565,7 @@ int ndc_pointwise_gemm(const void *x, const void *wfrag, const float *bias, cons
         (zkeep && ((uintptr_t)zkeep & 3u)) || ((uintptr_t)wfrag & 15u) || (bias && ((uintptr_t)bias & 3u)))
         return NDC_ERR_WORKSPACE;
     if (y == x || zkeep == x || (zkeep && zkeep == y)) return NDC_ERR_GEOMETRY;
+    if (cin > 256 && (act != NDC_ACT_NONE || zkeep)) return NDC_ERR_GEOMETRY;   // see the header
     return ndc::Backend::pwgemm(x, wfrag, bias, residual, y, zkeep, nullptr, batch, (int)cin, (int)cout, n, act, stream);
 }
 

@@ -511,11 +511,11 @@ struct Backend {
 
     // y = act(W x + bias) + residual on persistent workgroups; the caller has checked the shape
     // (cin in {64, 128, 256}, cout a multiple of 32, n a multiple of 64, packed weights <= 128 KB)
-    template <int CT, int ACT, bool RES>
+    template <int CT, bool RES>
     static int pwgemm_deep_launch(const pwgemm::Params &p, int cin, size_t lds, void *stream)
     {
         constexpr int THREADS = 512;
-        void (*entry)(pwgemm::Params, int) = pwgemm::gemm_kernel_deep<CT, ACT, RES, THREADS>;
+        void (*entry)(pwgemm::Params, int) = pwgemm::gemm_kernel_deep<CT, RES, THREADS>;
         static std::atomic<int> resident[2] = {{0}, {0}};
         const int cls = lds <= 72 * 1024 ? 0 : 1;
         int per_cu = resident[cls].load(std::memory_order_relaxed);
@@ -540,15 +540,9 @@ struct Backend {
     }
 
     template <int CT>
-    static int pwgemm_deep(const pwgemm::Params &p, int cin, size_t lds, int act, void *stream)
+    static int pwgemm_deep(const pwgemm::Params &p, int cin, size_t lds, void *stream)
     {
-#define NDC_PWGEMM_DEEP(ACT)                                                             \
-    (p.res ? pwgemm_deep_launch<CT, ACT, true>(p, cin, lds, stream)                      \
-           : pwgemm_deep_launch<CT, ACT, false>(p, cin, lds, stream))
-        if (act == epilogue::kRelu) return NDC_PWGEMM_DEEP(epilogue::kRelu);
-        if (act == epilogue::kGelu) return NDC_PWGEMM_DEEP(epilogue::kGelu);
-        return NDC_PWGEMM_DEEP(epilogue::kNone);
-#undef NDC_PWGEMM_DEEP
+        return p.res ? pwgemm_deep_launch<CT, true>(p, cin, lds, stream) : pwgemm_deep_launch<CT, false>(p, cin, lds, stream);
     }
 
     // act 3 / 4: y = (W x) * relu' / gelu'(res + bias), gpart (kMaxParts x cout, or null) receives
@@ -565,12 +559,12 @@ struct Backend {
         const size_t wbytes = (size_t)cin * cout * 2;
         const size_t lds = wbytes + (size_t)cout * 4;   // packed weights, bias
         if (cin > 256) {   // many input channels, at most 128 output channels (checked by the caller)
-            if (act > epilogue::kGelu) return -2;
+            if (act != epilogue::kNone || zkeep) return -2;   // plain product, bias, residual
             switch (cout / 32) {
-            case 1: return pwgemm_deep<1>(p, cin, lds, act, stream);
-            case 2: return pwgemm_deep<2>(p, cin, lds, act, stream);
-            case 3: return pwgemm_deep<3>(p, cin, lds, act, stream);
-            default: return pwgemm_deep<4>(p, cin, lds, act, stream);
+            case 1: return pwgemm_deep<1>(p, cin, lds, stream);
+            case 2: return pwgemm_deep<2>(p, cin, lds, stream);
+            case 3: return pwgemm_deep<3>(p, cin, lds, stream);
+            default: return pwgemm_deep<4>(p, cin, lds, stream);
             }
         }
         // small weight tables: several workgroups per CU; large ones: one, of more wavefronts

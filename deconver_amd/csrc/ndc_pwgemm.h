@@ -33,7 +33,8 @@
 // output tiles one after the other (any number of output channels; also the modes that multiply
 // the product by an activation's derivative and sum the result per channel); gemm_kernel_deep
 // takes more input channels in chunks of 128 with the accumulators of all (at most four) output
-// tiles kept.  Device code only; float32 accumulation; the output is rounded to bf16 once.
+// tiles kept (these are the projections back from a widened tensor: bias and residual only, no
+// activation, nothing kept).  Device code only; float32 accumulation; the output is rounded to bf16 once.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -134,10 +135,10 @@ __device__ inline void split_x(const uint32_t (&raw)[S][8], bf16x8 (&xf)[S][2])
     }
 }
 
-// The epilogue of one 32-channel output tile (forward modes).  Register j of a lane holds output
+// The epilogue of one 32-channel output tile of gemm_kernel_deep (bias and residual only).  Register j of a lane holds output
 // row 8 * (j / 4) + 4 * kb + j % 4, column n32, of the even-voxel tile (acc0) and the odd-voxel
 // tile (acc1): one output word.  rw: the residual words, requested by the caller.
-template <int ACT, bool RES>
+template <bool RES>
 __device__ inline void finish_tile(const Params &p, const f32x16 &acc0, const f32x16 &acc1, const uint32_t (&rw)[16],
                                    const float *bl, int c, long long at0, uint32_t yw, int kb)
 {
@@ -150,8 +151,7 @@ __device__ inline void finish_tile(const Params &p, const f32x16 &acc0, const f3
             const int j = 4 * q + jj;
             const long long at = at0 + (long long)(8 * q + jj) * p.n;
             const float z0 = acc0[j], z1 = acc1[j];
-            if (p.zkeep) words(p.zkeep + at)[yw] = pack_bf16x2(z0, z1);
-            float y0 = epilogue::act_fwd<ACT>(z0 + bq[jj]), y1 = epilogue::act_fwd<ACT>(z1 + bq[jj]);
+            float y0 = z0 + bq[jj], y1 = z1 + bq[jj];
             if constexpr (RES) y0 += lo_bf16(rw[j]), y1 += hi_bf16(rw[j]);
             words(p.y + at)[yw] = pack_bf16x2(y0, y1);
         }
@@ -266,13 +266,12 @@ __global__ void __launch_bounds__(THREADS) gemm_kernel(Params p)
 // Many input channels, at most 128 output channels (the projections back from the widened
 // tensors: 512 -> 128): the accumulators of ALL CT output tiles stay in registers while the
 // input channels go by in chunks of 128, so that x is still read once.  p.cin: a multiple of 128.
-template <int CT, int ACT, bool RES, int THREADS>
+template <int CT, bool RES, int THREADS>
 __global__ void __launch_bounds__(THREADS) gemm_kernel_deep(Params p, int cin)
 {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     constexpr int WAVES = THREADS / 64;
     constexpr int SC = 8;                    // k-steps per chunk of 128 input channels
-    static_assert(ACT <= epilogue::kGelu, "no gradient modes here");
     const int S = cin / 16, chunks_k = cin / 128;
     u32x4 *wl = reinterpret_cast<u32x4 *>(smem);
     float *bl = reinterpret_cast<float *>(smem + (size_t)CT * S * 64 * 16);
@@ -321,7 +320,7 @@ __global__ void __launch_bounds__(THREADS) gemm_kernel_deep(Params p, int cin)
                 for (int j = 0; j < 16; ++j)
                     rw[j] = words(p.res + at0 + (long long)(8 * (j / 4) + j % 4) * p.n)[yw];
             }
-            finish_tile<ACT, RES>(p, acc[c][0], acc[c][1], rw, bl, c, at0, yw, kb);
+            finish_tile<RES>(p, acc[c][0], acc[c][1], rw, bl, c, at0, yw, kb);
         }
     }
 }

@@ -117,7 +117,7 @@ class _PointwiseLinear(torch.autograd.Function):
         # the activation's gradient needs z + bias: gelu keeps z; relu alone needs only the
         # sign of its output, which may then overwrite z
         keep_z = act == "gelu" or (act == "relu" and residual is not None)
-        if ops.pointwise_gemm_applies(lib, x, w.shape[0]):
+        if ops.pointwise_gemm_applies(lib, x, w.shape[0], act, keep_z):
             # the library's streaming GEMM: product, bias, activation and residual in one
             # kernel that reads x once and writes the result (and z where it is kept) once
             with torch.cuda.device(x.device):

@@ -279,9 +279,13 @@ def bias_act_backward(lib: _lib.NdcLibrary, gy: Tensor, z: Tensor, bias: Optiona
     return gz, (gpart.sum((0, 2)) if need_bias_grad else None)
 
 
-def pointwise_gemm_applies(lib: _lib.NdcLibrary, x: Tensor, cout: int) -> bool:
+def pointwise_gemm_applies(lib: _lib.NdcLibrary, x: Tensor, cout: int, act: Optional[str] = None,
+                           keep_z: bool = False) -> bool:
     """Whether ``pointwise_gemm`` takes the projection of ``x`` (B, cin, n) to ``cout`` channels:
-    contiguous bfloat16 on the GPU in the shapes ``ndc_pointwise_gemm_supported`` lists."""
+    contiguous bfloat16 on the GPU in the shapes ``ndc_pointwise_gemm_supported`` lists (with
+    more than 256 input channels: no activation, nothing kept)."""
+    if x.dim() == 3 and x.shape[1] > 256 and (act is not None or keep_z):
+        return False
     return (x.is_cuda and x.dtype == torch.bfloat16 and x.dim() == 3 and x.is_contiguous()
             and lib.pointwise_gemm_supported(x.shape[1], cout, x.shape[2], _lib.NDC_BF16))
 

@@ -334,6 +334,8 @@ int ndc_bias_act_backward(const void *gy, const void *z, const float *bias, void
  *   bias           cout floats or NULL; residual NULL or a tensor added to the result
  *   zkeep          NULL, or receives the product before bias and activation (what
  *                  ndc_bias_act_backward reads as z)
+ * With more than 256 input channels (the projections back from a widened tensor) the call takes
+ * NDC_ACT_NONE and no zkeep: product, bias and residual.
  */
 int ndc_pointwise_gemm_supported(int64_t cin, int64_t cout, int64_t n, int dtype);
 size_t ndc_pointwise_weight_bytes(int64_t cin, int64_t cout);
