@@ -566,6 +566,7 @@ int ndc_pointwise_gemm(const void *x, const void *wfrag, const float *bias, cons
         return NDC_ERR_WORKSPACE;
     if (y == x || zkeep == x || (zkeep && zkeep == y)) return NDC_ERR_GEOMETRY;
     if (cin > 256 && (act != NDC_ACT_NONE || zkeep)) return NDC_ERR_GEOMETRY;   // see the header
+    if (act == NDC_ACT_NONE && zkeep) return NDC_ERR_GEOMETRY;   // without an activation y - bias is the product
     return ndc::Backend::pwgemm(x, wfrag, bias, residual, y, zkeep, nullptr, batch, (int)cin, (int)cout, n, act, stream);
 }
 

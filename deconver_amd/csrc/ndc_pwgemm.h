@@ -239,7 +239,9 @@ __global__ void __launch_bounds__(THREADS) gemm_kernel(Params p)
                         for (int m = 1; m < 32; m <<= 1) t += __shfl_xor(t, m);
                         if (p.gpart && n32 == 0) gs[32 * c + 8 * q + 4 * kb + jj] += t;
                     } else {
-                        if (p.zkeep) words(p.zkeep + at)[yw] = pack_bf16x2(z0, z1);
+                        if constexpr (ACT != epilogue::kNone) {   // (kept only for an activation's gradient)
+                            if (p.zkeep) words(p.zkeep + at)[yw] = pack_bf16x2(z0, z1);
+                        }
                         y0 = epilogue::act_fwd<ACT>(z0 + bq[jj]), y1 = epilogue::act_fwd<ACT>(z1 + bq[jj]);
                         if constexpr (RES) y0 += lo_bf16(rw[j]), y1 += hi_bf16(rw[j]);
                     }

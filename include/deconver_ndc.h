@@ -332,8 +332,8 @@ int ndc_bias_act_backward(const void *gy, const void *z, const float *bias, void
  *                  input gradient, W^T gy, packs the weight as it lies).
  *   x              (batch, cin, n); y, residual, zkeep: (batch, cout, n); all bf16, 4-byte aligned
  *   bias           cout floats or NULL; residual NULL or a tensor added to the result
- *   zkeep          NULL, or receives the product before bias and activation (what
- *                  ndc_bias_act_backward reads as z)
+ *   zkeep          NULL, or (with NDC_ACT_RELU / NDC_ACT_GELU) receives the product before bias
+ *                  and activation (what ndc_bias_act_backward reads as z)
  * With more than 256 input channels (the projections back from a widened tensor) the call takes
  * NDC_ACT_NONE and no zkeep: product, bias and residual.
  */
