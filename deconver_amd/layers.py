@@ -117,6 +117,7 @@ class _PointwiseLinear(torch.autograd.Function):
         # the activation's gradient needs z + bias: gelu keeps z; relu alone needs only the
         # sign of its output, which may then overwrite z
         keep_z = act == "gelu" or (act == "relu" and residual is not None)
+        keep_z = keep_z and any(ctx.needs_input_grad)     # (nothing is kept for a forward-only call)
         if ops.pointwise_gemm_applies(lib, x, w.shape[0], act, keep_z):
             # the library's streaming GEMM: product, bias, activation and residual in one
             # kernel that reads x once and writes the result (and z where it is kept) once
@@ -469,7 +470,7 @@ class _FusedMLP(torch.autograd.Function):
         b2f = None if b2 is None else b2.detach().float().contiguous()
         with torch.cuda.device(x.device):
             a, z = ops.pointwise_gemm(lib, x, ops.pointwise_pack(lib, w1.detach().contiguous()), hidden, b1f,
-                                      None, "gelu", keep_z=True)
+                                      None, "gelu", keep_z=any(ctx.needs_input_grad))
             y, _ = ops.pointwise_gemm(lib, a, ops.pointwise_pack(lib, w2.detach().contiguous()), cout, b2f,
                                       residual, None)
         ctx.save_for_backward(x, z, a, w1.detach().to(x.dtype), w2.detach().to(x.dtype), b1f)
