@@ -10,6 +10,7 @@
     python bench.py --workload block      (norm and projection-tail kernels of a Deconver block)
     python bench.py --workload mixer [--dtype bf16|fp32]                  (one DeconvMixer, fwd+bwd)
     python bench.py --workload layout                                     (channels-last copies around the update)
+    python bench.py --workload graphed    (small batches: the training step eager and replayed from a HIP graph)
 
 One step = one forward + one backward (input-, source-, filter- and bias-gradient) of the
 update node on config 3 of the baseline: batch 2, 128 depthwise channels, 64^3 voxels,
@@ -899,6 +900,56 @@ def block_workload(args) -> int:
     return 0
 
 
+def graphed_workload(args) -> int:
+    """Training steps on ONE small sample (a 3-D step on a 32^3 volume under bf16 autocast, a 2-D
+    step on a 128^2 image in float32): there a step is bound by the rate at which the host
+    launches its ~600 kernels, and replaying it from a HIP graph (training.GraphedTrainStep)
+    removes that bound.  ms per step eager and replayed, same networks as train3d / model2d."""
+    import torch
+    from torch import nn
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    import deconver_amd as dc
+    from deconver_amd import training
+
+    def timed(fn):
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / args.steps * 1e3
+
+    rows = []
+    for name, key, size, autocast in (("3-D, one 32^3 volume, bf16 autocast", "train3d", (32, 32, 32), torch.bfloat16),
+                                      ("2-D, one 128^2 image, float32", "model2d", (128, 128), None)):
+        w = MODEL_WORKLOADS[key]
+        torch.manual_seed(0)
+        norm = nn.InstanceNorm3d if len(size) == 3 else nn.InstanceNorm2d
+        model = dc.Deconver(norm=norm, **w["net"]).cuda()
+        opt = training.make_optimizer(model, capturable=True)
+        make = training.ellipsoid_phantoms if len(size) == 3 else training.smoothed_noise_masks
+        images, targets = make(1, w["net"]["in_channels"], size, seed=0, device="cuda")
+        eager = timed(lambda: training.train_step(model, opt, images, targets, autocast_dtype=autocast))
+        step = training.GraphedTrainStep(model, opt, images, targets, autocast_dtype=autocast)
+        replayed = timed(lambda: step(images, targets))
+        rows.append({"case": name, "eager_ms": eager, "graph_ms": replayed, "speedup": eager / replayed})
+        del model, opt, step
+        torch.cuda.empty_cache()
+    print(json.dumps({
+        "metric": "small-batch training step replayed from a HIP graph, ms", "value": rows[0]["graph_ms"],
+        "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": rows[0]["graph_ms"],
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "Deconver training steps on one small sample, eager and replayed from a HIP graph"},
+        "cases": rows, "roofline": None, "cpu_baseline": None}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -925,7 +976,8 @@ def main() -> int:
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     ap.add_argument("--build-probe", action="store_true",
                     help="with --workload valu: compile the probe (no GPU needed) and exit")
-    ap.add_argument("--workload", choices=("ndc", "sweep", "accuracy", "grid", "valu", "train3d", "model2d", "mixer", "layout", "block"),
+    ap.add_argument("--workload", choices=("ndc", "sweep", "accuracy", "grid", "valu", "train3d", "model2d", "mixer", "layout", "block",
+                                           "graphed"),
                     default="ndc",
                     help="ndc: the headline update node (default); the others are model level")
     ap.add_argument("--ndc", choices=("hip", "pytorch", "both"), default="hip",
@@ -956,6 +1008,8 @@ def main() -> int:
         return layout_workload(args)
     if args.workload == "block":
         return block_workload(args)
+    if args.workload == "graphed":
+        return graphed_workload(args)
     if args.workload != "ndc":
         return model_workload(args)
 
