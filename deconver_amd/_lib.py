@@ -56,6 +56,7 @@ EXPORTS = (
     "ndc_pointwise_gemm",
     "ndc_pointwise_gemm_parts",
     "ndc_pointwise_gemm_actgrad",
+    "ndc_pointwise_gemm_masked",
 )
 
 
@@ -148,6 +149,8 @@ class NdcLibrary:
         d.ndc_pointwise_pack.argtypes = [vp, ctypes.c_int, ctypes.c_int, vp, ctypes.c_int64, ctypes.c_int64, vp]
         d.ndc_pointwise_gemm.argtypes = [vp, vp, vp, vp, vp, vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                                          ctypes.c_int64, ctypes.c_int, ctypes.c_int, vp]
+        d.ndc_pointwise_gemm_masked.argtypes = [vp, vp, vp, vp, vp, vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                                                ctypes.c_int64, ctypes.c_int, vp]
         d.ndc_pointwise_gemm_parts.restype = ctypes.c_int64
         d.ndc_pointwise_gemm_parts.argtypes = []
         d.ndc_pointwise_gemm_actgrad.argtypes = [vp, vp, vp, vp, vp, vp, ctypes.c_int64, ctypes.c_int64,
@@ -323,6 +326,12 @@ class NdcLibrary:
         """``y = act(W x + bias) + residual`` on channel-first bf16 ``(batch, c, n)`` tensors."""
         self._check(self._dll.ndc_pointwise_gemm(x, wfrag, bias, residual, y, zkeep, batch, cin, cout, n, act,
                                                  dtype, stream), "ndc_pointwise_gemm")
+
+    def pointwise_gemm_masked(self, x: int, wfrag: int, bias: Optional[int], residual: Optional[int], mask: int,
+                              y: int, batch: int, cin: int, cout: int, n: int, dtype: int, stream) -> None:
+        """``y = (W x + bias + residual)`` where ``mask > 0``, else 0."""
+        self._check(self._dll.ndc_pointwise_gemm_masked(x, wfrag, bias, residual, mask, y, batch, cin, cout, n,
+                                                        dtype, stream), "ndc_pointwise_gemm_masked")
 
     def pointwise_gemm_parts(self) -> int:
         return int(self._dll.ndc_pointwise_gemm_parts())

@@ -524,9 +524,9 @@ int ndc_pointwise_gemm_supported(int64_t cin, int64_t cout, int64_t n, int dtype
 {
     if (dtype != NDC_BF16) return 0;
     // up to 256 input channels held whole in registers, any width of output; or many input
-    // channels in chunks of 128 with the accumulators of at most 128 output channels
+    // channels in chunks of 64 with the accumulators of at most 128 output channels
     const bool whole = cin == 64 || cin == 128 || cin == 256;
-    const bool deep = cin > 256 && cin % 128 == 0 && cin <= 4096 && cout <= 128;
+    const bool deep = cin > 256 && cin % 64 == 0 && cin <= 4096 && cout <= 128;
     if (!whole && !deep) return 0;
     if (cout < 32 || cout % 32 || cout > 4096) return 0;
     if (cin * cout * 2 > 128 * 1024) return 0;        // the packed weights stay in LDS,
@@ -567,7 +567,24 @@ int ndc_pointwise_gemm(const void *x, const void *wfrag, const float *bias, cons
     if (y == x || zkeep == x || (zkeep && zkeep == y)) return NDC_ERR_GEOMETRY;
     if (cin > 256 && (act != NDC_ACT_NONE || zkeep)) return NDC_ERR_GEOMETRY;   // see the header
     if (act == NDC_ACT_NONE && zkeep) return NDC_ERR_GEOMETRY;   // without an activation y - bias is the product
-    return ndc::Backend::pwgemm(x, wfrag, bias, residual, y, zkeep, nullptr, batch, (int)cin, (int)cout, n, act, stream);
+    return ndc::Backend::pwgemm(x, wfrag, bias, residual, y, zkeep, nullptr, nullptr, batch, (int)cin, (int)cout, n, act,
+                                stream);
+}
+
+int ndc_pointwise_gemm_masked(const void *x, const void *wfrag, const float *bias, const void *residual,
+                              const void *mask, void *y, int64_t batch, int64_t cin, int64_t cout, int64_t n,
+                              int dtype, void *stream)
+{
+    if (!x || !wfrag || !y || !mask) return NDC_ERR_NULL;
+    if (dtype != NDC_BF16) return NDC_ERR_DTYPE;
+    if (batch < 1 || !ndc_pointwise_gemm_supported(cin, cout, n, dtype)) return NDC_ERR_GEOMETRY;
+    if ((long double)batch * (cin > cout ? cin : cout) * n > 9.0e15L) return NDC_ERR_GEOMETRY;
+    if (batch * (n / 64) > 0x7fffff00LL || n > 0x3fffffffLL) return NDC_ERR_GEOMETRY;
+    if (((uintptr_t)x & 3u) || ((uintptr_t)y & 3u) || ((uintptr_t)mask & 3u) || (residual && ((uintptr_t)residual & 3u)) ||
+        ((uintptr_t)wfrag & 15u) || (bias && ((uintptr_t)bias & 3u)))
+        return NDC_ERR_WORKSPACE;
+    if (y == x || y == mask) return NDC_ERR_GEOMETRY;
+    return ndc::Backend::pwgemm(x, wfrag, bias, residual, y, nullptr, nullptr, mask, batch, (int)cin, (int)cout, n, 5, stream);
 }
 
 int64_t ndc_pointwise_gemm_parts(void)
@@ -589,7 +606,7 @@ int ndc_pointwise_gemm_actgrad(const void *gy, const void *wfrag, const float *b
         (bias && ((uintptr_t)bias & 3u)) || (gpart && ((uintptr_t)gpart & 3u)))
         return NDC_ERR_WORKSPACE;
     if (gz == gy || gz == z) return NDC_ERR_GEOMETRY;
-    return ndc::Backend::pwgemm(gy, wfrag, bias, z, gz, nullptr, gpart, batch, (int)cin, (int)cout, n, act + 2, stream);
+    return ndc::Backend::pwgemm(gy, wfrag, bias, z, gz, nullptr, gpart, nullptr, batch, (int)cin, (int)cout, n, act + 2, stream);
 }
 
 static int chnorm_check(long long B, long long C, long long n, int dtype)

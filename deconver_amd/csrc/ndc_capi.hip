@@ -503,6 +503,7 @@ struct Backend {
         if (act >= pwgemm::kReluGrad && glds > 160 * 1024) return -2;
         if (act == pwgemm::kGeluGrad) return pwgemm_launch<CIN, pwgemm::kGeluGrad, true, THREADS>(p, glds, stream);
         if (act == pwgemm::kReluGrad) return pwgemm_launch<CIN, pwgemm::kReluGrad, true, THREADS>(p, glds, stream);
+        if (act == pwgemm::kMasked) return NDC_PWGEMM_RES(pwgemm::kMasked);
         if (act == epilogue::kRelu) return NDC_PWGEMM_RES(epilogue::kRelu);
         if (act == epilogue::kGelu) return NDC_PWGEMM_RES(epilogue::kGelu);
         return NDC_PWGEMM_RES(epilogue::kNone);
@@ -511,11 +512,11 @@ struct Backend {
 
     // y = act(W x + bias) + residual on persistent workgroups; the caller has checked the shape
     // (cin in {64, 128, 256}, cout a multiple of 32, n a multiple of 64, packed weights <= 128 KB)
-    template <int CT, bool RES>
+    template <int CT, bool RES, bool MASK>
     static int pwgemm_deep_launch(const pwgemm::Params &p, int cin, size_t lds, void *stream)
     {
         constexpr int THREADS = 512;
-        void (*entry)(pwgemm::Params, int) = pwgemm::gemm_kernel_deep<CT, RES, THREADS>;
+        void (*entry)(pwgemm::Params, int) = pwgemm::gemm_kernel_deep<CT, RES, MASK, THREADS>;
         static std::atomic<int> resident[2] = {{0}, {0}};
         const int cls = lds <= 72 * 1024 ? 0 : 1;
         int per_cu = resident[cls].load(std::memory_order_relaxed);
@@ -542,16 +543,23 @@ struct Backend {
     template <int CT>
     static int pwgemm_deep(const pwgemm::Params &p, int cin, size_t lds, void *stream)
     {
-        return p.res ? pwgemm_deep_launch<CT, true>(p, cin, lds, stream) : pwgemm_deep_launch<CT, false>(p, cin, lds, stream);
+        if (p.mask)
+            return p.res ? pwgemm_deep_launch<CT, true, true>(p, cin, lds, stream)
+                         : pwgemm_deep_launch<CT, false, true>(p, cin, lds, stream);
+        return p.res ? pwgemm_deep_launch<CT, true, false>(p, cin, lds, stream)
+                     : pwgemm_deep_launch<CT, false, false>(p, cin, lds, stream);
     }
 
     // act 3 / 4: y = (W x) * relu' / gelu'(res + bias), gpart (kMaxParts x cout, or null) receives
     // per-wavefront sums of y whose total over the rows is the bias gradient
+    // act 5: y = (W x + bias + res) where mask > 0, else 0
     static int pwgemm(const void *x, const void *wfrag, const float *bias, const void *res, void *y, void *zkeep,
-                      float *gpart, long long batch, int cin, int cout, long long n, int act, void *stream)
+                      float *gpart, const void *mask, long long batch, int cin, int cout, long long n, int act,
+                      void *stream)
     {
         pwgemm::Params p;
         p.gpart = gpart;
+        p.mask = (const uint16_t *)mask;
         p.x = (const uint16_t *)x, p.wfrag = (const uint16_t *)wfrag, p.bias = bias;
         p.res = (const uint16_t *)res, p.y = (uint16_t *)y, p.zkeep = (uint16_t *)zkeep;
         p.n = n, p.tiles_per_sample = (int)(n / pwgemm::kTileVoxels), p.tiles = (int)(batch * (n / pwgemm::kTileVoxels)), p.cout = cout;
@@ -559,7 +567,7 @@ struct Backend {
         const size_t wbytes = (size_t)cin * cout * 2;
         const size_t lds = wbytes + (size_t)cout * 4;   // packed weights, bias
         if (cin > 256) {   // many input channels, at most 128 output channels (checked by the caller)
-            if (act != epilogue::kNone || zkeep) return -2;   // plain product, bias, residual
+            if ((act != epilogue::kNone && act != pwgemm::kMasked) || zkeep) return -2;   // product, bias, residual, mask
             switch (cout / 32) {
             case 1: return pwgemm_deep<1>(p, cin, lds, stream);
             case 2: return pwgemm_deep<2>(p, cin, lds, stream);

@@ -266,7 +266,7 @@ struct Backend {
     }
 
     static int pwgemm(const void *x, const void *wfrag, const float *bias, const void *res, void *y, void *zkeep,
-                      float *gpart, long long batch, int cin, int cout, long long n, int act, void *)
+                      float *gpart, const void *mask, long long batch, int cin, int cout, long long n, int act, void *)
     {
         if (gpart)
             for (long long i = 0; i < 4096LL * cout; ++i) gpart[i] = 0.f;
@@ -282,9 +282,15 @@ struct Backend {
                         acc += Elem<bf16_t>::load(wf + f * 8 + k % 8) * Elem<bf16_t>::load(xs + (b * cin + k) * n + v);
                     }
                     const long long at = (b * cout + co) * n + v;
-                    if (act >= 3) {   // times the derivative of relu (3) / gelu (4) at aux + bias
+                    if (act == 3 || act == 4) {   // times the derivative of relu (3) / gelu (4) at aux + bias
                         const float out = acc * act_value(act - 2, Elem<bf16_t>::load(rs + at) + (bias ? bias[co] : 0.f), true);
                         if (gpart) gpart[(v / 64 % 7) * cout + co] += out;   // a few rows, as the device uses many
+                        ys[at] = float_to_bf16(out);
+                        continue;
+                    }
+                    if (act == 5) {   // the sum where mask > 0, else 0
+                        float out = acc + (bias ? bias[co] : 0.f) + (rs ? Elem<bf16_t>::load(rs + at) : 0.f);
+                        if (!(Elem<bf16_t>::load((const bf16_t *)mask + at) > 0.f)) out = 0.f;
                         ys[at] = float_to_bf16(out);
                         continue;
                     }

@@ -32,7 +32,7 @@
 // Two kernels: gemm_kernel holds the fragments of up to 256 input channels whole and walks the
 // output tiles one after the other (any number of output channels; also the modes that multiply
 // the product by an activation's derivative and sum the result per channel); gemm_kernel_deep
-// takes more input channels in chunks of 128 with the accumulators of all (at most four) output
+// takes more input channels in chunks of 64 with the accumulators of all (at most four) output
 // tiles kept (these are the projections back from a widened tensor: bias and residual only, no
 // activation, nothing kept).  Device code only; float32 accumulation; the output is rounded to bf16 once.
 #pragma once
@@ -54,6 +54,10 @@ static const int kMaxParts = 4096;       // wavefronts of a launch (rows of Para
 // derivative at (aux + bias), aux read through Params::res -- the input gradient of a
 // projection whose INPUT was act(aux + bias) (the MLP's second projection, layers/mlp.py:40-63)
 enum { kReluGrad = 3, kGeluGrad = 4 };
+// ... and kMasked: y = (W x + bias + residual) where mask > 0, else 0 -- an input gradient taken
+// through the rectifier that made the projection's input (mask: that rectifier's output), with
+// another gradient of the same tensor accumulated on the way (residual)
+enum { kMasked = 5 };
 
 struct Params {
     const uint16_t *x;       // (B, cin, n) bf16
@@ -63,6 +67,7 @@ struct Params {
     uint16_t *y;             // (B, cout, n)
     uint16_t *zkeep;         // (B, cout, n) or null: the product before bias and activation
     float *gpart;            // gradient modes: (gridDim.x * waves, cout) sums of y per wavefront, or null
+    const uint16_t *mask;    // kMasked: (B, cout, n)
     long long n;             // voxels per sample, a multiple of 64
     int tiles;               // B * n / 64
     int tiles_per_sample;
@@ -138,9 +143,9 @@ __device__ inline void split_x(const uint32_t (&raw)[S][8], bf16x8 (&xf)[S][2])
 // The epilogue of one 32-channel output tile of gemm_kernel_deep (bias and residual only).  Register j of a lane holds output
 // row 8 * (j / 4) + 4 * kb + j % 4, column n32, of the even-voxel tile (acc0) and the odd-voxel
 // tile (acc1): one output word.  rw: the residual words, requested by the caller.
-template <bool RES>
+template <bool RES, bool MASK>
 __device__ inline void finish_tile(const Params &p, const f32x16 &acc0, const f32x16 &acc1, const uint32_t (&rw)[16],
-                                   const float *bl, int c, long long at0, uint32_t yw, int kb)
+                                   const uint32_t (&mw)[16], const float *bl, int c, long long at0, uint32_t yw, int kb)
 {
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
@@ -153,6 +158,7 @@ __device__ inline void finish_tile(const Params &p, const f32x16 &acc0, const f3
             const float z0 = acc0[j], z1 = acc1[j];
             float y0 = z0 + bq[jj], y1 = z1 + bq[jj];
             if constexpr (RES) y0 += lo_bf16(rw[j]), y1 += hi_bf16(rw[j]);
+            if constexpr (MASK) y0 = lo_bf16(mw[j]) > 0.f ? y0 : 0.f, y1 = hi_bf16(mw[j]) > 0.f ? y1 : 0.f;
             words(p.y + at)[yw] = pack_bf16x2(y0, y1);
         }
     }
@@ -205,11 +211,16 @@ __global__ void __launch_bounds__(THREADS) gemm_kernel(Params p)
 #pragma unroll 1
         for (int c = 0; c < CT; ++c) {
             const long long at0 = out0 + (long long)(32 * c) * p.n;
-            uint32_t rw[16];
+            uint32_t rw[16], mw[16];
             if constexpr (RES) {
 #pragma unroll
                 for (int j = 0; j < 16; ++j)
                     rw[j] = words(p.res + at0 + (long long)(8 * (j / 4) + j % 4) * p.n)[yw];
+            }
+            if constexpr (ACT == kMasked) {
+#pragma unroll
+                for (int j = 0; j < 16; ++j)
+                    mw[j] = words(p.mask + at0 + (long long)(8 * (j / 4) + j % 4) * p.n)[yw];
             }
             f32x16 acc0 = {}, acc1 = {};
             const u32x4 *wt = wl + (c * S) * 64 + lane;
@@ -238,6 +249,10 @@ __global__ void __launch_bounds__(THREADS) gemm_kernel(Params p)
 #pragma unroll
                         for (int m = 1; m < 32; m <<= 1) t += __shfl_xor(t, m);
                         if (p.gpart && n32 == 0) gs[32 * c + 8 * q + 4 * kb + jj] += t;
+                    } else if constexpr (ACT == kMasked) {
+                        y0 = z0 + bq[jj], y1 = z1 + bq[jj];
+                        if constexpr (RES) y0 += lo_bf16(rw[j]), y1 += hi_bf16(rw[j]);
+                        y0 = lo_bf16(mw[j]) > 0.f ? y0 : 0.f, y1 = hi_bf16(mw[j]) > 0.f ? y1 : 0.f;
                     } else {
                         if constexpr (ACT != epilogue::kNone) {   // (kept only for an activation's gradient)
                             if (p.zkeep) words(p.zkeep + at)[yw] = pack_bf16x2(z0, z1);
@@ -267,14 +282,14 @@ __global__ void __launch_bounds__(THREADS) gemm_kernel(Params p)
 
 // Many input channels, at most 128 output channels (the projections back from the widened
 // tensors: 512 -> 128): the accumulators of ALL CT output tiles stay in registers while the
-// input channels go by in chunks of 128, so that x is still read once.  p.cin: a multiple of 128.
-template <int CT, bool RES, int THREADS>
+// input channels go by in chunks of 64, so that x is still read once.  cin: a multiple of 64.
+template <int CT, bool RES, bool MASK, int THREADS>
 __global__ void __launch_bounds__(THREADS) gemm_kernel_deep(Params p, int cin)
 {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     constexpr int WAVES = THREADS / 64;
-    constexpr int SC = 8;                    // k-steps per chunk of 128 input channels
-    const int S = cin / 16, chunks_k = cin / 128;
+    constexpr int SC = 4;                    // k-steps per chunk of 64 input channels
+    const int S = cin / 16, chunks_k = cin / 64;
     u32x4 *wl = reinterpret_cast<u32x4 *>(smem);
     float *bl = reinterpret_cast<float *>(smem + (size_t)CT * S * 64 * 16);
     {
@@ -298,7 +313,7 @@ __global__ void __launch_bounds__(THREADS) gemm_kernel_deep(Params p, int cin)
 #pragma unroll 1
         for (int kc = 0; kc < chunks_k; ++kc) {
             uint32_t raw[SC][8];
-            request_x<SC>(p, tile, cin, xw, raw, 128 * kc);
+            request_x<SC>(p, tile, cin, xw, raw, 64 * kc);
             bf16x8 xf[SC][2];
             split_x<SC>(raw, xf);
 #pragma unroll
@@ -316,13 +331,18 @@ __global__ void __launch_bounds__(THREADS) gemm_kernel_deep(Params p, int cin)
 #pragma unroll
         for (int c = 0; c < CT; ++c) {
             const long long at0 = out0 + (long long)(32 * c) * p.n;
-            uint32_t rw[16];
+            uint32_t rw[16], mw[16];
             if constexpr (RES) {
 #pragma unroll
                 for (int j = 0; j < 16; ++j)
                     rw[j] = words(p.res + at0 + (long long)(8 * (j / 4) + j % 4) * p.n)[yw];
             }
-            finish_tile<RES>(p, acc[c][0], acc[c][1], rw, bl, c, at0, yw, kb);
+            if constexpr (MASK) {
+#pragma unroll
+                for (int j = 0; j < 16; ++j)
+                    mw[j] = words(p.mask + at0 + (long long)(8 * (j / 4) + j % 4) * p.n)[yw];
+            }
+            finish_tile<RES, MASK>(p, acc[c][0], acc[c][1], rw, mw, bl, c, at0, yw, kb);
         }
     }
 }

@@ -177,7 +177,7 @@ class ProjectedUpdate(torch.autograd.Function):
     tensors, the weight gradient summed in float32."""
 
     @staticmethod
-    def forward(ctx, x, weight, h, bias, groups, m, sc, eps, taps=None):
+    def forward(ctx, x, weight, h, bias, groups, m, sc, eps, taps=None, rectified_input=False):
         from .layers import project
         w = weight.detach().to(x.dtype)
         z = project(weight.detach(), x.flatten(2)).view(x.shape[0], w.shape[0], *x.shape[2:])
@@ -186,6 +186,9 @@ class ProjectedUpdate(torch.autograd.Function):
                                    bias, groups, m, sc, eps, True, taps)
         ctx.save_for_backward(*saved, w)
         ctx.weight_dtype = weight.dtype
+        # x is a rectifier's output and its producer skips the rectifier's backward pass: the
+        # gradient of x leaves this node already zero where x is
+        ctx.rectified_input = bool(rectified_input)
         return out
 
     @staticmethod
@@ -199,8 +202,9 @@ class ProjectedUpdate(torch.autograd.Function):
         if need_w:
             gw = projection_weight_grad(gz.flatten(2), x.flatten(2), ctx.weight_dtype)
         if need_x:
-            gx = project_back(w, gz.flatten(2), accumulate=gx.flatten(2)).view_as(x)
-        return gx, gw, gh, gb, None, None, None, None, None
+            gx = project_back(w, gz.flatten(2), accumulate=gx.flatten(2),
+                              mask=x.flatten(2) if ctx.rectified_input else None).view_as(x)
+        return gx, gw, gh, gb, None, None, None, None, None, None
 
 
 def deconv_update(x: Tensor, z: Tensor, h: Tensor, bias: Optional[Tensor], *, groups: int,
@@ -222,7 +226,8 @@ def deconv_update(x: Tensor, z: Tensor, h: Tensor, bias: Optional[Tensor], *, gr
 
 
 def projected_update(x: Tensor, weight: Tensor, h: Tensor, bias: Optional[Tensor], *, groups: int,
-                     m: int, sc: int, eps: float, taps: Optional[Tensor] = None) -> Tensor:
+                     m: int, sc: int, eps: float, taps: Optional[Tensor] = None,
+                     rectified_input: bool = False) -> Tensor:
     """``deconv_update(x, W x, h, bias, relu_input=True)`` as one autograd node (not in the
     reference, which records the projection and the update separately).
 
@@ -231,6 +236,9 @@ def projected_update(x: Tensor, weight: Tensor, h: Tensor, bias: Optional[Tensor
         weight: the projection's weight ``(groups*sc, C)``, any floating dtype (cast to ``x``'s
             for the GEMMs; its gradient comes back in its own dtype).
         h, bias, groups, m, sc, eps, taps: as for ``deconv_update``.
+        rectified_input: ``x`` is the output of a rectifier whose backward pass its producer
+            skips (``Linear(..., act="relu", grad_premasked=True)``): the gradient of ``x`` is
+            returned zero where ``x`` is, from the GEMM that forms it.
     """
     with torch.autocast(x.device.type, enabled=False):
-        return ProjectedUpdate.apply(x, weight, h, bias, groups, m, sc, eps, taps)
+        return ProjectedUpdate.apply(x, weight, h, bias, groups, m, sc, eps, taps, rectified_input)

@@ -65,28 +65,33 @@ def project(weight: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
     return z
 
 
-def project_back(weight: torch.Tensor, gz: torch.Tensor, accumulate: Optional[torch.Tensor] = None) -> torch.Tensor:
+def project_back(weight: torch.Tensor, gz: torch.Tensor, accumulate: Optional[torch.Tensor] = None,
+                 mask: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``W^T gz`` per sample (the input gradient of a 1x1 projection with ``weight`` of shape
     ``(Cout, Cin)``), plus ``accumulate`` if given (a tensor of the result's shape, which may
-    be overwritten).  The library's streaming GEMM where it applies -- the weight is packed as
-    it lies, no transposed copy --, else one batched hipBLASLt GEMM."""
+    be overwritten), and zero wherever ``mask <= 0`` if a mask of the result's shape is given
+    (the gradient taken through the rectifier whose output the projection read).  The
+    library's streaming GEMM where it applies -- the weight is packed as it lies, no transposed
+    copy --, else one batched hipBLASLt GEMM."""
     B, cout, n = gz.shape
     if cout == 1:
         # one output channel (the network's head): the product is an outer product, i.e. a
         # broadcast multiplication at the memory rate (as a GEMM it ran at a fifth of it)
         gx = gz * weight.reshape(1, -1, 1).to(gz.dtype)
-        return gx if accumulate is None else accumulate.add_(gx)
-    lib = _lib.get_library()
-    if gz.is_contiguous() and ops.pointwise_gemm_applies(lib, gz, weight.shape[1]):
-        with torch.cuda.device(gz.device):
-            wfrag = ops.pointwise_pack(lib, weight.contiguous(), transposed=True)
-            return ops.pointwise_gemm(lib, gz, wfrag, weight.shape[1], residual=accumulate)[0]
-    wt = weight.t().unsqueeze(0).expand(B, -1, -1)
-    if accumulate is not None:
-        return accumulate.baddbmm_(wt, gz)
-    gx = gz.new_empty(B, weight.shape[1], n)
-    torch.bmm(wt, gz, out=gx)
-    return gx
+        gx = gx if accumulate is None else accumulate.add_(gx)
+    else:
+        lib = _lib.get_library()
+        if gz.is_contiguous() and ops.pointwise_gemm_applies(lib, gz, weight.shape[1]):
+            with torch.cuda.device(gz.device):
+                wfrag = ops.pointwise_pack(lib, weight.contiguous(), transposed=True)
+                return ops.pointwise_gemm(lib, gz, wfrag, weight.shape[1], residual=accumulate, mask=mask)[0]
+        wt = weight.t().unsqueeze(0).expand(B, -1, -1)
+        if accumulate is not None:
+            gx = accumulate.baddbmm_(wt, gz)
+        else:
+            gx = gz.new_empty(B, weight.shape[1], n)
+            torch.bmm(wt, gz, out=gx)
+    return gx if mask is None else gx.mul_(mask > 0)
 
 
 class _PointwiseLinear(torch.autograd.Function):
@@ -105,7 +110,7 @@ class _PointwiseLinear(torch.autograd.Function):
     of the 128 -> 512 projection at 2 x 64^3 in bf16."""
 
     @staticmethod
-    def forward(ctx, x, weight, bias, act, residual):
+    def forward(ctx, x, weight, bias, act, residual, grad_premasked=False):
         lib = _lib.get_library()
         # one batched GEMM on the tensors as they lie, the weight shared by the batch entries
         # through a zero stride (no copy; the same bits as one GEMM per sample, in one launch)
@@ -136,6 +141,9 @@ class _PointwiseLinear(torch.autograd.Function):
         ctx.weight_dtype = weight.dtype
         ctx.has_bias = bias is not None
         ctx.act = act
+        # a ReLU whose consumer hands back a gradient that is already zero where the output is
+        # (``project_back(mask=...)``): the backward then has no pass of its own for it
+        ctx.premasked = bool(grad_premasked) and act == "relu" and residual is None
         return y
 
     @staticmethod
@@ -147,7 +155,11 @@ class _PointwiseLinear(torch.autograd.Function):
         gres = gy if ctx.needs_input_grad[4] else None
         want_gb = ctx.has_bias and ctx.needs_input_grad[2]
         gz = gy
-        if ctx.act is not None:
+        if ctx.premasked:
+            if want_gb:
+                with torch.cuda.device(gy.device):
+                    gb = ops.channel_sums(_lib.get_library(), gy)
+        elif ctx.act is not None:
             with torch.cuda.device(gy.device):
                 gz, gb = ops.bias_act_backward(_lib.get_library(), gy, kept, bias32, ctx.act,
                                                need_bias_grad=want_gb)
@@ -161,20 +173,26 @@ class _PointwiseLinear(torch.autograd.Function):
             gx = project_back(weight, gz)
         if ctx.needs_input_grad[1]:
             gw = projection_weight_grad(gz, x, ctx.weight_dtype)
-        return gx, gw, gb, None, gres
+        return gx, gw, gb, None, gres, None
 
 
 _ACT_FUNCTIONS = {None: lambda t: t, "relu": torch.relu, "gelu": torch.nn.functional.gelu}
 
 
 def pointwise_linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
-                     act: Optional[str] = None, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     act: Optional[str] = None, residual: Optional[torch.Tensor] = None,
+                     grad_premasked: bool = False) -> torch.Tensor:
     """``act(W x + bias) + residual``: the 1x1 projection ``(B, Cin, N) -> (B, Cout, N)`` with
     ``weight`` of shape ``(Cout, Cin)`` or ``(Cout, Cin, 1)``, optionally followed by an
     activation (``"relu"`` or ``"gelu"``, the exact one) and the sum with a tensor of the
     output's shape.  bfloat16 (stored or under autocast) and float32 tensors on the GPU run as
     batched GEMMs on the channel-first layout plus one pass of the HIP library over the result;
-    everything else as the reference's ``conv1d`` followed by PyTorch's activation and sum."""
+    everything else as the reference's ``conv1d`` followed by PyTorch's activation and sum.
+
+    ``grad_premasked`` (GEMM route, ``act="relu"`` without residual only; ignored elsewhere): the
+    caller guarantees that every gradient reaching the result is already zero where the result
+    is -- its only consumer took it through the rectifier (``project_back(mask=...)``) --, so the
+    backward skips the rectifier's pass."""
     w2 = weight.squeeze(-1) if weight.dim() == 3 else weight
     dtype = x.dtype
     if x.is_cuda and torch.is_autocast_enabled(x.device.type):
@@ -188,7 +206,7 @@ def pointwise_linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch
     if residual is not None:
         residual = residual.to(dtype).contiguous()
     with torch.autocast(x.device.type, enabled=False):
-        return _PointwiseLinear.apply(x.contiguous(), w2, bias, act, residual)
+        return _PointwiseLinear.apply(x.contiguous(), w2, bias, act, residual, grad_premasked)
 
 
 def _gemm_route(x: torch.Tensor) -> bool:
@@ -436,13 +454,14 @@ class Linear(nn.Module):
                                 device=device, dtype=dtype)
 
     def forward(self, x: torch.Tensor, act: Optional[str] = None,
-                residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+                residual: Optional[torch.Tensor] = None, grad_premasked: bool = False) -> torch.Tensor:
         """``act(linear(x)) + residual``; ``act`` None, ``"relu"`` or ``"gelu"``; ``residual``
-        of the output's shape."""
+        of the output's shape; ``grad_premasked`` as for ``pointwise_linear``."""
         shape = x.shape
         if residual is not None:
             residual = residual.flatten(2)
-        y = pointwise_linear(self.flatten(x), self.linear.weight, self.linear.bias, act, residual)
+        y = pointwise_linear(self.flatten(x), self.linear.weight, self.linear.bias, act, residual,
+                             grad_premasked)
         return y.view(shape[0], -1, *shape[2:])
 
 

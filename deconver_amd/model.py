@@ -59,11 +59,17 @@ class DeconvMixer(nn.Module):
         then rides on ``out_proj`` unless dropout is active)."""
         if type(self.act) is nn.ReLU and not self.act._forward_hooks and layers._gemm_route(x):
             # the rectifier rides on the projection (one kernel, or one pass over its output);
-            # a hooked activation module is still called as a module
-            h = self.in_proj(x, act="relu")
+            # a hooked activation module is still called as a module.  Its backward rides on the
+            # layer's input gradient where the layer forms that in one GEMM; x stands in for
+            # the projection's output when asking (same batch, grid, device and autocast state,
+            # same channel count for the square in_proj of a block)
+            premasked = (type(self.deconv) is Deconv and x.shape[1] == self.in_proj.linear.out_channels
+                         and not self.deconv._forward_hooks and not self.deconv._forward_pre_hooks
+                         and self.deconv.takes_rectified_input(x))
+            h = self.in_proj(x, act="relu", grad_premasked=premasked)
+            sources = self.deconv(h, rectified_input=True) if premasked else self.deconv(h)
         else:
-            h = self.act(self.in_proj(x))
-        sources = self.deconv(h)
+            sources = self.deconv(self.act(self.in_proj(x)))
         if self.dropout.p == 0 or not self.training:
             return self.out_proj(sources, residual=residual)
         y = self.dropout(self.out_proj(sources))

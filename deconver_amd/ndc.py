@@ -178,7 +178,7 @@ class Deconv(nn.Module):
 
     # ------------------------------------------------------------------ HIP route
 
-    def _fit_fast(self, x: Tensor) -> tuple[Tensor, Tensor]:
+    def _fit_fast(self, x: Tensor, rectified_input: bool = False) -> tuple[Tensor, Tensor]:
         dtype = self._hip_dtype(x)
         x = x.contiguous().to(dtype)
         proj = self.init.linear.linear
@@ -200,7 +200,7 @@ class Deconv(nn.Module):
         for it in range(1, self.num_iters + 1):
             with self.context(it):
                 if it == 1:
-                    s = projected_update(x, weight, h, bias, **kwargs)
+                    s = projected_update(x, weight, h, bias, rectified_input=rectified_input, **kwargs)
                 else:
                     s = deconv_update(x, s, h, None, relu_input=False, **kwargs)
         return s, h
@@ -271,9 +271,30 @@ class Deconv(nn.Module):
         ``iterative_update`` passes them."""
         return ops_general.relative_error(x, self.conv(s, h))
 
-    def forward(self, x: Tensor) -> Tensor:
-        route = self._fit_fast if self.fast_path_applicable(x) else self._fit_general
-        return route(x)[0]
+    def forward(self, x: Tensor, rectified_input: bool = False) -> Tensor:
+        """The layer's sources.  ``rectified_input`` (not in the reference; see
+        ``takes_rectified_input``): ``x`` is a rectifier's output whose producer leaves that
+        rectifier's backward to this layer."""
+        if rectified_input and not self.takes_rectified_input(x):
+            # the producer has already dropped its rectifier's backward: refusing is the only
+            # answer that cannot return a wrong gradient
+            raise RuntimeError("Deconv.forward(rectified_input=True) on a call that takes_rectified_input() declines")
+        if self.fast_path_applicable(x):
+            return self._fit_fast(x, rectified_input)[0]
+        return self._fit_general(x)[0]
+
+    def takes_rectified_input(self, x: Tensor) -> bool:
+        """Whether ``forward(x, rectified_input=True)`` returns the gradient of ``x`` already
+        zero where ``x`` is: the HIP route with a single update, whose one node forms that
+        gradient in a GEMM.  A caller that rectifies ``x`` may then skip the rectifier's own
+        backward pass; otherwise it must not."""
+        if self.num_iters != 1 or not self.fast_path_applicable(x) or self._hip_dtype(x) != torch.bfloat16:
+            return False
+        # ... and that GEMM is the library's own, which masks in its epilogue (elsewhere the
+        # mask would be a pass of its own again)
+        n = math.prod(x.shape[2:])
+        return get_library().pointwise_gemm_supported(self.groups * self.source_channels, self.channels, n,
+                                                      ops.dtype_tag(torch.bfloat16))
 
 
 NDC = Deconv

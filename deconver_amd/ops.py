@@ -305,11 +305,18 @@ def pointwise_pack(lib: _lib.NdcLibrary, weight: Tensor, transposed: bool = Fals
 
 
 def pointwise_gemm(lib: _lib.NdcLibrary, x: Tensor, wfrag: Tensor, cout: int, bias: Optional[Tensor] = None,
-                   residual: Optional[Tensor] = None, act: Optional[str] = None, keep_z: bool = False):
+                   residual: Optional[Tensor] = None, act: Optional[str] = None, keep_z: bool = False,
+                   mask: Optional[Tensor] = None):
     """``y = act(W x + bias) + residual`` for contiguous bfloat16 ``x`` (B, cin, n) and packed
     ``W`` (``pointwise_pack``); returns ``(y, z)`` with ``z`` the product before bias and
-    activation when ``keep_z``, else None."""
+    activation when ``keep_z``, else None.  With ``mask`` (of the output's shape; no activation,
+    nothing kept): ``y = W x + bias + residual`` where ``mask > 0``, else 0."""
     B, cin, n = x.shape
+    if mask is not None:
+        if act is not None or keep_z:
+            raise ValueError("the masked form takes no activation and keeps nothing")
+        if mask.shape != (B, cout, n) or mask.dtype != x.dtype or not mask.is_contiguous():
+            raise ValueError("mask must be contiguous, of the output's shape and dtype")
     if wfrag.numel() != cin * cout or wfrag.dtype != torch.bfloat16:
         raise ValueError("wfrag does not belong to this projection")
     if bias is not None and (bias.dtype != torch.float32 or bias.numel() != cout or not bias.is_contiguous()):
@@ -319,6 +326,10 @@ def pointwise_gemm(lib: _lib.NdcLibrary, x: Tensor, wfrag: Tensor, cout: int, bi
         raise ValueError("residual must be contiguous, of the output's shape and dtype")
     y = x.new_empty(B, cout, n)
     z = x.new_empty(B, cout, n) if keep_z else None
+    if mask is not None:
+        lib.pointwise_gemm_masked(_ptr(x), _ptr(wfrag), _ptr(bias), _ptr(residual), _ptr(mask), _ptr(y), B, cin,
+                                  cout, n, _lib.NDC_BF16, _stream_of(x))
+        return y, None
     lib.pointwise_gemm(_ptr(x), _ptr(wfrag), _ptr(bias), _ptr(residual), _ptr(y), _ptr(z), B, cin, cout, n,
                        ACTS[act], _lib.NDC_BF16, _stream_of(x))
     return y, z

@@ -321,7 +321,7 @@ int ndc_bias_act_backward(const void *gy, const void *z, const float *bias, void
  * A streaming kernel on the matrix units: x is read once, y written once, float32 accumulation,
  * one rounding of the result.
  *   ndc_pointwise_gemm_supported  1 where the kernel applies: NDC_BF16; cin 64, 128 or 256, or a
- *                  larger multiple of 128 with cout <= 128; cout a multiple of 32;
+ *                  larger multiple of 64 with cout <= 128; cout a multiple of 32;
  *                  cin * cout * 2 <= 128 KiB; n a multiple of 64; else 0 (callers then use a
  *                  library GEMM and ndc_bias_act)
  *   ndc_pointwise_pack  writes W in the order the kernel reads it into wfrag
@@ -344,6 +344,16 @@ int ndc_pointwise_pack(const void *w, int w_dtype, int transposed, void *wfrag, 
 int ndc_pointwise_gemm(const void *x, const void *wfrag, const float *bias, const void *residual, void *y,
                        void *zkeep, int64_t batch, int64_t cin, int64_t cout, int64_t n, int act, int dtype,
                        void *stream);
+/*
+ * ndc_pointwise_gemm_masked: y = (W x + bias + residual) where mask > 0, else 0; mask of y's shape.
+ * The input gradient of a projection whose input is a rectifier's output (mask), with another
+ * gradient of the same tensor (residual) accumulated on the way: DeconvMixer's ReLU between
+ * in_proj and the layer (deconver/deconver.py:29-46), whose backward is then no pass of its own.
+ * Shapes and alignment as for ndc_pointwise_gemm; y may be residual.
+ */
+int ndc_pointwise_gemm_masked(const void *x, const void *wfrag, const float *bias, const void *residual,
+                              const void *mask, void *y, int64_t batch, int64_t cin, int64_t cout, int64_t n,
+                              int dtype, void *stream);
 /*
  * The input gradient of a projection whose INPUT was act(z + bias) (the second projection of
  * the MLP, deconver/layers/mlp.py:40-63, whose input is the GELU of the first one's output),

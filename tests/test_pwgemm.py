@@ -38,7 +38,7 @@ def test_support_predicate():
     assert lib.pointwise_gemm_supported(256, 64, 64, bf) and lib.pointwise_gemm_supported(128, 512, 4096, bf)
     assert not lib.pointwise_gemm_supported(64, 256, 128 ** 3, f32)       # bfloat16 only
     assert lib.pointwise_gemm_supported(512, 128, 4096, bf)               # many input channels: up to 128 out
-    assert not lib.pointwise_gemm_supported(512, 256, 4096, bf) and not lib.pointwise_gemm_supported(320, 64, 4096, bf)
+    assert not lib.pointwise_gemm_supported(512, 256, 4096, bf) and not lib.pointwise_gemm_supported(336, 64, 4096, bf)
     assert not lib.pointwise_gemm_supported(256, 512, 4096, bf)           # weights beyond 128 KiB
     assert not lib.pointwise_gemm_supported(64, 48, 4096, bf)             # cout not a multiple of 32
     assert not lib.pointwise_gemm_supported(64, 64, 100, bf)              # n not a multiple of 64
@@ -97,7 +97,7 @@ def test_bad_arguments_are_refused():
 @pytest.mark.parametrize("B,cin,cout,n", [
     (2, 64, 256, 64 * 64 * 8), (2, 256, 64, 64 * 64 * 8), (1, 64, 64, 4096), (2, 128, 512, 32 ** 3),
     (3, 128, 128, 64 * 33), (1, 256, 256, 64 * 7), (2, 64, 32, 64),
-    (2, 512, 128, 64 * 64 * 4), (1, 512, 64, 64 * 5), (1, 1024, 32, 128), (2, 384, 96, 64 * 3)])
+    (2, 512, 128, 64 * 64 * 4), (1, 512, 64, 64 * 5), (1, 1024, 32, 128), (2, 320, 96, 64 * 3)])
 @pytest.mark.parametrize("act,with_bias,with_res,keep", [(None, False, False, False), (None, True, True, False),
                                                           ("gelu", True, False, True), ("relu", False, False, False)])
 def test_gpu_matches_float64(B, cin, cout, n, act, with_bias, with_res, keep):
@@ -203,3 +203,70 @@ def test_mlp_as_one_node_matches_float64(with_residual):
         assert _rel(r.grad, rr.grad) < 1e-2
     for (name, p), (_, q) in zip(mlp.named_parameters(), ref.named_parameters()):
         assert p.grad.dtype == torch.float32 and _rel(p.grad, q.grad) < 2e-2, name
+
+
+def _masked_reference(x, w, bias, res, mask):
+    z, y = _reference(x, w, bias, res, None)
+    return torch.where(mask.double() > 0, y, torch.zeros_like(y))
+
+
+@pytest.mark.parametrize("cin,cout", [(64, 96), (384, 64)])
+def test_masked_form_on_the_host_build(cin, cout):
+    lib = hostcheck_library()
+    x, w, bias, res = _case(2, cin, cout, 128, seed=7)
+    mask = torch.randn(2, cout, 128, generator=torch.Generator().manual_seed(8)).bfloat16()
+    mask[0, 0, :5] = 0      # zero counts as off
+    y, none = ops.pointwise_gemm(lib, x, ops.pointwise_pack(lib, w), cout, bias, res, mask=mask)
+    assert none is None and _rel(y, _masked_reference(x, w, bias, res, mask)) < 1e-2
+    assert bool((y[mask <= 0] == 0).all())
+    with pytest.raises(ValueError):
+        ops.pointwise_gemm(lib, x, ops.pointwise_pack(lib, w), cout, act="relu", mask=mask)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("B,cin,cout,n,with_res", [(2, 256, 64, 64 * 64 * 4, True), (2, 512, 128, 64 * 33, True),
+                                                   (1, 64, 64, 4096, False), (2, 128, 512, 64 * 9, True)])
+def test_gpu_masked_form(B, cin, cout, n, with_res):
+    lib = _lib.get_library()
+    x, w, bias, res = _case(B, cin, cout, n, seed=9)
+    res = res if with_res else None
+    mask = torch.relu(torch.randn(B, cout, n, generator=torch.Generator().manual_seed(10))).bfloat16()
+    dev = [t.cuda() if t is not None else None for t in (x, w, res, mask)]
+    y, _ = ops.pointwise_gemm(lib, dev[0], ops.pointwise_pack(lib, dev[1]), cout, None, dev[2], mask=dev[3])
+    assert _rel(y, _masked_reference(x, w, None, res, mask)) < 1e-2
+    assert bool((y[dev[3] <= 0] == 0).all())
+    # where the mask is on, the masked form equals the plain one bit for bit
+    plain, _ = ops.pointwise_gemm(lib, dev[0], ops.pointwise_pack(lib, dev[1]), cout, None, dev[2])
+    assert torch.equal(y[dev[3] > 0], plain[dev[3] > 0])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("channels,size", [(64, (8, 8, 64)), (128, (4, 8, 64))])
+def test_mixer_with_the_rectifier_on_its_neighbours_matches_float64(channels, size):
+    """DeconvMixer under bf16 autocast: the ReLU's forward on in_proj, its backward in the layer's
+    input-gradient GEMM (no pass of its own) -- output and every gradient against the same mixer
+    in float64 on the CPU, on a case a float64 screen keeps clear of the rectifiers' kinks."""
+    import copy
+    import deconver_amd as dc
+    torch.manual_seed(11)
+    mixer = dc.DeconvMixer(channels, channels, kernel_size=(3, 3, 3), ratio=4, groups=-1)
+    with torch.no_grad():
+        mixer.deconv.init.linear.linear.bias.add_(1.0)
+    ref = copy.deepcopy(mixer).double()
+    mixer = mixer.cuda()
+    x0 = torch.randn(2, channels, *size)
+    g0 = torch.randn(2, channels, *size)
+    x = x0.cuda().bfloat16().requires_grad_(True)
+    assert mixer.deconv.takes_rectified_input(x)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        y = mixer(x)
+    y.backward(g0.cuda().bfloat16())
+    xr = x.detach().double().cpu().requires_grad_(True)
+    yr = ref(xr)
+    yr.backward(g0.bfloat16().double())
+    assert _rel(y.detach(), yr.detach()) < 2e-2
+    cos = torch.nn.functional.cosine_similarity(x.grad.double().cpu().flatten(), xr.grad.flatten(), dim=0)
+    assert cos > 0.999, float(cos)
+    for (name, p), (_, q) in zip(mixer.named_parameters(), ref.named_parameters()):
+        c = torch.nn.functional.cosine_similarity(p.grad.double().cpu().flatten(), q.grad.flatten(), dim=0)
+        assert c > 0.998, (name, float(c))
