@@ -179,8 +179,11 @@ class ProjectedUpdate(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, weight, h, bias, groups, m, sc, eps, taps=None, rectified_input=False):
         from .layers import project
-        w = weight.detach().to(x.dtype)
-        z = project(weight.detach(), x.flatten(2)).view(x.shape[0], w.shape[0], *x.shape[2:])
+        # (kept in its own dtype where the GEMMs pack it themselves, cast once otherwise)
+        w = weight.detach()
+        if not ops.pointwise_gemm_applies(_lib.get_library(), x.flatten(2), w.shape[0]):
+            w = w.to(x.dtype)
+        z = project(w, x.flatten(2)).view(x.shape[0], w.shape[0], *x.shape[2:])
         need_x, need_w, need_h, need_b = ctx.needs_input_grad[:4]
         out, saved = _node_forward(ctx, (need_x, need_x or need_w, need_h, need_b), x, z, h,
                                    bias, groups, m, sc, eps, True, taps)

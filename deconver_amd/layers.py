@@ -85,7 +85,7 @@ def project_back(weight: torch.Tensor, gz: torch.Tensor, accumulate: Optional[to
             with torch.cuda.device(gz.device):
                 wfrag = ops.pointwise_pack(lib, weight.contiguous(), transposed=True)
                 return ops.pointwise_gemm(lib, gz, wfrag, weight.shape[1], residual=accumulate, mask=mask)[0]
-        wt = weight.t().unsqueeze(0).expand(B, -1, -1)
+        wt = weight.to(gz.dtype).t().unsqueeze(0).expand(B, -1, -1)
         if accumulate is not None:
             gx = accumulate.baddbmm_(wt, gz)
         else:
@@ -117,7 +117,7 @@ class _PointwiseLinear(torch.autograd.Function):
         # (the weight arrives in its own dtype -- float32 under autocast -- and is cast here, so
         # that its gradient leaves backward as the float32 sum it is, not rounded to bf16 first)
         B = x.shape[0]
-        w = weight.detach().to(x.dtype)
+        w = weight.detach()
         bias32 = None if bias is None else bias.detach().float().contiguous()
         # the activation's gradient needs z + bias: gelu keeps z; relu alone needs only the
         # sign of its output, which may then overwrite z
@@ -127,9 +127,12 @@ class _PointwiseLinear(torch.autograd.Function):
             # the library's streaming GEMM: product, bias, activation and residual in one
             # kernel that reads x once and writes the result (and z where it is kept) once
             with torch.cuda.device(x.device):
-                y, z = ops.pointwise_gemm(lib, x, ops.pointwise_pack(lib, weight.detach().contiguous()),
+                y, z = ops.pointwise_gemm(lib, x, ops.pointwise_pack(lib, w.contiguous()),
                                           w.shape[0], bias32, residual, act, keep_z=keep_z)
+            # (the packing reads the weight in its own dtype, and so does the backward's: no
+            # cast copy of it is made or kept)
         else:
+            w = w.to(x.dtype)
             z = x.new_empty(B, w.shape[0], x.shape[2])
             torch.bmm(w.unsqueeze(0).expand(B, -1, -1), x, out=z)
             y = z
@@ -492,7 +495,7 @@ class _FusedMLP(torch.autograd.Function):
                                       None, "gelu", keep_z=any(ctx.needs_input_grad))
             y, _ = ops.pointwise_gemm(lib, a, ops.pointwise_pack(lib, w2.detach().contiguous()), cout, b2f,
                                       residual, None)
-        ctx.save_for_backward(x, z, a, w1.detach().to(x.dtype), w2.detach().to(x.dtype), b1f)
+        ctx.save_for_backward(x, z, a, w1.detach(), w2.detach(), b1f)
         ctx.dtypes = (w1.dtype, w2.dtype)
         return y
 
@@ -510,7 +513,7 @@ class _FusedMLP(torch.autograd.Function):
             if need_w2:
                 gw2 = projection_weight_grad(gy, a, ctx.dtypes[1])
             if need_x or need_w1 or need_b1:
-                gz, gb1 = ops.pointwise_gemm_actgrad(lib, gy, ops.pointwise_pack(lib, w2, transposed=True),
+                gz, gb1 = ops.pointwise_gemm_actgrad(lib, gy, ops.pointwise_pack(lib, w2.contiguous(), transposed=True),
                                                      w2.shape[1], z, b1f, "gelu", need_bias_grad=need_b1)
                 if need_w1:
                     gw1 = projection_weight_grad(gz, x, ctx.dtypes[0])

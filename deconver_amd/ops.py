@@ -292,11 +292,13 @@ def pointwise_gemm_applies(lib: _lib.NdcLibrary, x: Tensor, cout: int, act: Opti
 
 def pointwise_pack(lib: _lib.NdcLibrary, weight: Tensor, transposed: bool = False) -> Tensor:
     """The weight of a 1x1 projection in the order ``pointwise_gemm`` reads it (bf16).
-    ``weight``: ``(cout, cin)``, float32 or bfloat16, contiguous; with ``transposed`` it is
-    taken as the ``(cin, cout)`` storage of the matrix to apply (the input gradient's ``W^T``
-    from ``W`` as it lies)."""
+    ``weight``: ``(cout, cin)``, contiguous, float32 or bfloat16 (another floating dtype is cast
+    to bfloat16 first); with ``transposed`` it is taken as the ``(cin, cout)`` storage of the
+    matrix to apply (the input gradient's ``W^T`` from ``W`` as it lies)."""
+    if weight.is_floating_point() and weight.dtype not in _DTYPES:
+        weight = weight.to(torch.bfloat16)
     if weight.dim() != 2 or not weight.is_contiguous() or weight.dtype not in _DTYPES:
-        raise ValueError("pointwise_pack wants a contiguous float32 or bfloat16 matrix")
+        raise ValueError("pointwise_pack wants a contiguous floating-point matrix")
     cout, cin = (weight.shape[1], weight.shape[0]) if transposed else weight.shape
     wfrag = torch.empty(cout * cin, dtype=torch.bfloat16, device=weight.device)
     lib.pointwise_pack(_ptr(weight), dtype_tag(weight.dtype), transposed, _ptr(wfrag), cin, cout,
