@@ -19,17 +19,24 @@ from torch.nn.modules.utils import _pair
 from . import _lib, ops
 
 
-_CHUNKED_WGRAD_FROM = 1 << 17   # voxels per sample from which the weight gradient is chunked
-
-
-def _wgrad_chunks(batch: int, n: int) -> int:
+def _wgrad_chunks(batch: int, n: int, min_chunk: int = 2048) -> int:
     """Number of equal chunks the voxel axis is cut into for the weight-gradient GEMM: a power
-    of two that divides ``n``, leaves chunks of at least 2048 voxels and at most 128 GEMMs in
-    the batch (measured on an MI355X: 64 chunks at 64^3 and 128^3 with batch 2, 16 at 32^3)."""
+    of two that divides ``n``, leaves chunks of at least ``min_chunk`` voxels and at most 128
+    GEMMs in the batch."""
     s = 1
-    while s < 64 and n % (2 * s) == 0 and n // (2 * s) >= 2048 and batch * 2 * s <= 128:
+    while s < 64 and n % (2 * s) == 0 and n // (2 * s) >= min_chunk and batch * 2 * s <= 128:
         s *= 2
     return s
+
+
+def _wgrad_plan(batch: int, n: int, dtype: torch.dtype) -> int:
+    """The chunk count ``projection_weight_grad`` uses, from timings on an MI355X with batch 2
+    in bfloat16 (64 chunks at 128^3; 32 at 64^3, where 64 cost 0.05 ms more on the 128 x 128
+    result; 16 at 32^3: 0.056 ms against 0.11-0.13 ms unchunked; none at 16^3) and batch 8 in
+    float32 (none up to 256^2 voxels: there every chunked form was slower)."""
+    if dtype == torch.bfloat16:
+        return 1 if n < (1 << 15) else _wgrad_chunks(batch, n, 2048 if n < (1 << 17) else 8192)
+    return 1 if n < (1 << 17) else _wgrad_chunks(batch, n)
 
 
 def projection_weight_grad(gz: torch.Tensor, x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
@@ -40,7 +47,7 @@ def projection_weight_grad(gz: torch.Tensor, x: torch.Tensor, dtype: torch.dtype
     (strided views, no copies).  The partial results are added in float32, in one reduction."""
     B, cout, n = gz.shape
     cin = x.shape[1]
-    s = _wgrad_chunks(B, n) if n >= _CHUNKED_WGRAD_FROM else 1
+    s = _wgrad_plan(B, n, gz.dtype)
     if s == 1:
         parts = torch.bmm(gz, x.transpose(1, 2))
     else:

@@ -5,7 +5,7 @@ import pytest
 import torch
 import torch.nn.functional as F
 
-from deconver_amd.layers import Linear, _wgrad_chunks, pointwise_linear
+from deconver_amd.layers import Linear, _wgrad_chunks, _wgrad_plan, pointwise_linear
 
 pytestmark = pytest.mark.gpu
 
@@ -48,6 +48,10 @@ def test_chunk_rule():
     assert _wgrad_chunks(2, 64 ** 3) == 64 and _wgrad_chunks(2, 128 ** 3) == 64
     assert _wgrad_chunks(2, 32 ** 3) == 16 and _wgrad_chunks(3, 7 * 9 * 11) == 1
     assert _wgrad_chunks(8, 256 * 256) == 16 and _wgrad_chunks(1, 2048) == 1
+    bf16, f32 = torch.bfloat16, torch.float32
+    assert [_wgrad_plan(2, s ** 3, bf16) for s in (16, 32, 64, 128)] == [1, 16, 32, 64]
+    assert [_wgrad_plan(8, s ** 2, f32) for s in (64, 128, 256, 512)] == [1, 1, 1, 16]
+    assert _wgrad_plan(2, 64 ** 3, f32) == 64 and _wgrad_plan(3, 7 * 9 * 11, bf16) == 1
 
 
 def test_linear_module_under_autocast_keeps_float32_parameter_gradients():
