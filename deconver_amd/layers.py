@@ -44,18 +44,22 @@ def projection_weight_grad(gz: torch.Tensor, x: torch.Tensor, dtype: torch.dtype
     ``(B, Cin, N)``: the weight gradient of a 1x1 projection, a ``Cout x Cin`` result summed
     over all voxels.  Short rows (the 2-D network's levels) take one batched GEMM and a sum over
     the batch; long rows are cut into equal chunks of the voxel axis that become batch entries
-    (strided views, no copies).  The partial results are added in float32, in one reduction."""
+    (strided views, no copies).  The partial results -- float32 also for bfloat16 operands -- are
+    added in float32, in one reduction."""
     B, cout, n = gz.shape
     cin = x.shape[1]
     s = _wgrad_plan(B, n, gz.dtype)
+    # bfloat16 operands: the GEMMs hand out their float32 accumulators (same speed, and the
+    # partial results are then not rounded to bfloat16 before they are added)
+    f32 = {"out_dtype": torch.float32} if gz.is_cuda and gz.dtype == torch.bfloat16 else {}
     if s == 1:
-        parts = torch.bmm(gz, x.transpose(1, 2))
+        parts = torch.bmm(gz, x.transpose(1, 2), **f32)
     else:
-        parts = gz.new_empty(B * s, cout, cin)
+        parts = gz.new_empty(B * s, cout, cin, dtype=torch.float32 if f32 else gz.dtype)
         for b in range(B):
             a = gz[b].view(cout, s, n // s).transpose(0, 1)
             c = x[b].view(cin, s, n // s).permute(1, 2, 0)
-            torch.bmm(a, c, out=parts[b * s:(b + 1) * s])
+            torch.bmm(a, c, out=parts[b * s:(b + 1) * s], **f32)
     return parts.sum(0, dtype=torch.float32).to(dtype)
 
 
